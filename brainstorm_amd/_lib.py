@@ -1,0 +1,122 @@
+"""ctypes binding of libbship.so (declarations in include/bship.h).
+
+The library is loaded from the package directory (or ``$BSHIP_LIB``). There is
+no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import (POINTER, c_char_p, c_double, c_float, c_int, c_int64,
+                    c_size_t, c_uint32, c_void_p)
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+DEFAULT_LIB_PATH = os.path.join(HERE, "libbship.so")
+
+# op codes of include/bship.h
+ADD, SUB, MUL, DIV, FMOD = 0, 1, 2, 3, 4
+ADD_ST, MULT_ST, MULT_ADD_ST = 0, 1, 2
+ABS, SIGN, SQRT, LOG, SIGMOID, TANH, REL, EL = 0, 1, 2, 3, 4, 5, 6, 7
+SIGMOID_DERIV, TANH_DERIV, REL_DERIV, EL_DERIV = 0, 1, 2, 3
+COPY_IF, FILL_IF, ADD_IF = 0, 1, 2
+
+ERR_OUT_OF_MEMORY = -5
+
+_P = c_void_p          # device pointers travel as plain integers
+_I64 = c_int64
+
+# name -> argtypes; every function returns an int status except the two noted.
+SIGNATURES = {
+    "bship_init": [c_int],
+    "bship_shutdown": [],
+    "bship_sync": [],
+    "bship_device_info": [ctypes.c_char_p, c_size_t, POINTER(c_int)],
+    "bship_timer_start": [],
+    "bship_timer_stop": [],
+    "bship_timer_elapsed_ms": [POINTER(c_float)],
+    "bship_malloc": [c_size_t, POINTER(c_void_p)],
+    "bship_free": [_P],
+    "bship_pool_trim": [],
+    "bship_pool_stats": [POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)],
+    "bship_h2d": [_P, c_void_p, c_size_t],
+    "bship_d2h": [c_void_p, _P, c_size_t],
+    "bship_d2d": [_P, _P, c_size_t],
+    "bship_fill_f32": [_P, c_float, c_size_t],
+    "bship_binary_f32": [c_int, _P, _P, _P, c_size_t],
+    "bship_mult_add_tt_f32": [_P, _P, _P, c_size_t],
+    "bship_scalar_f32": [c_int, c_float, _P, _P, c_size_t],
+    "bship_unary_f32": [c_int, _P, _P, c_size_t],
+    "bship_deriv_f32": [c_int, _P, _P, _P, c_size_t],
+    "bship_clip_f32": [_P, c_float, c_float, _P, c_size_t],
+    "bship_cond_f32": [c_int, _P, c_float, _P, _P, c_size_t],
+    "bship_mv_f32": [c_int, _P, _P, _P, _I64, _I64, c_int, c_int],
+    "bship_broadcast_f32": [_P, _P, _I64, _I64, _I64],
+    "bship_merge_f32": [_P, _P, _P, _I64, _I64, _I64],
+    "bship_split_add_f32": [_P, _P, _P, _I64, _I64, _I64],
+    "bship_sum_f32": [_P, _P, _I64, _I64, c_int],
+    "bship_softmax_rows_f32": [_P, _P, _I64, _I64],
+    "bship_isfinite_f32": [_P, c_size_t, POINTER(c_int)],
+    "bship_binarize_f32": [_P, _P, _I64, _I64],
+    "bship_index_m_by_v_f32": [_P, _P, _P, _I64, _I64],
+    "bship_rng_seed": [c_uint32],
+    "bship_prob_mask_f32": [_P, c_size_t, c_double],
+    "bship_fill_gaussian_f32": [_P, c_size_t, c_double, c_double],
+    "bship_rng_get_state": [POINTER(c_uint32), POINTER(c_int), POINTER(c_int), POINTER(c_double)],
+    "bship_gemm_f32": [c_int, c_int, _I64, _I64, _I64, c_float, _P, _I64, _P, _I64, c_float, _P, _I64],
+    "bship_im2col_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
+    "bship_col2im_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
+    "bship_maxpool_fwd_nhwc_f32": [_P, _P, _P, _I64] + [c_int] * 10,
+    "bship_maxpool_bwd_nhwc_f32": [_P, _P, _P, _I64] + [c_int] * 10,
+    "bship_avgpool_fwd_nhwc_f32": [_P, _P, _I64] + [c_int] * 10,
+    "bship_avgpool_bwd_nhwc_f32": [_P, _P, _I64] + [c_int] * 10,
+}
+# functions that do not return a status
+SPECIAL_RESTYPES = {"bship_version": (c_int, []), "bship_last_error": (c_char_p, [])}
+
+EXPORTED_SYMBOLS = tuple(sorted(list(SIGNATURES) + list(SPECIAL_RESTYPES)))
+
+
+class BshipError(RuntimeError):
+    """A libbship call returned a non-zero status."""
+
+    def __init__(self, status, message):
+        super().__init__("libbship error %d: %s" % (status, message))
+        self.status = status
+
+
+def lib_path() -> str:
+    return os.environ.get("BSHIP_LIB") or DEFAULT_LIB_PATH
+
+
+_LIB = None
+
+
+def load():
+    """Loads libbship.so once and declares every prototype."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = lib_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            "libbship.so not found at %s; build it with `python -m brainstorm_amd.build` "
+            "(hipcc, gfx950). There is no CPU fallback." % path)
+    lib = ctypes.CDLL(path)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    for name, (restype, argtypes) in SPECIAL_RESTYPES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = restype
+    _LIB = lib
+    return lib
+
+
+def raise_for_status(lib, status):
+    msg = lib.bship_last_error()
+    msg = msg.decode("utf-8", "replace") if msg else ""
+    if status == ERR_OUT_OF_MEMORY:
+        raise MemoryError("libbship: " + msg)
+    raise BshipError(status, msg)

@@ -1,0 +1,256 @@
+// Broadcast operations: matrix (op) vector with a row vector (1,N) or a column
+// vector (M,1), broadcast_t along a size-1 axis, and merge/split on the last
+// axis. All are HBM-bound; the vector operand is read once per workgroup and
+// kept in registers (row vector) or fetched once per row tile (column vector).
+#pragma clang fp contract(off)
+
+#include "common.h"
+
+namespace bship {
+
+// ---- small helpers so one kernel body serves float and 4-wide vectors ----
+template <typename F> __device__ __forceinline__ float vmap(F f, float a, float b, float c) {
+    return f.apply(a, b, c);
+}
+template <typename F> __device__ __forceinline__ f4 vmap(F f, f4 a, f4 b, f4 c) {
+    f4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = f.apply(a[k], b[k], c[k]);
+    return o;
+}
+__device__ __forceinline__ f4 splat(f4, float s) { f4 r = {s, s, s, s}; return r; }
+__device__ __forceinline__ float splat(float, float s) { return s; }
+
+// functors: apply(m, v, old_out)
+template <bool ACC> struct MvAdd { __device__ float apply(float m, float v, float o) const { float r = m + v; return ACC ? o + r : r; } };
+template <bool ACC> struct MvSub { __device__ float apply(float m, float v, float o) const { float r = m - v; return ACC ? o + r : r; } };
+template <bool ACC> struct MvMul { __device__ float apply(float m, float v, float o) const { float r = m * v; return ACC ? o + r : r; } };
+template <bool ACC> struct MvDiv { __device__ float apply(float m, float v, float o) const { float r = m / v; return ACC ? o + r : r; } };
+
+constexpr int kMvUnroll = 4;
+
+// Row vector: a thread owns W consecutive columns and walks down a band of rows
+// with its slice of v in registers. grid.x tiles the columns, grid.y the row
+// bands. NW = N / W.
+template <int W, bool AL, bool ACC, typename F>
+__global__ __launch_bounds__(kBlock) void mv_rowvec_kernel(F f, const float* m, const float* v,
+                                                           float* out, int64_t M, int64_t NW,
+                                                           int64_t rows_per_block) {
+    typedef typename VecT<W>::type R;
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (c >= NW) return;
+    const R vv = vload<W, AL>(v + c * W);
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_block;
+    const int64_t r1 = (r0 + rows_per_block < M) ? r0 + rows_per_block : M;
+    for (int64_t r = r0; r < r1; r += kMvUnroll) {
+        R a[kMvUnroll], o[kMvUnroll];
+#pragma unroll
+        for (int u = 0; u < kMvUnroll; ++u) {
+            if (r + u < r1) {
+                const int64_t e = ((r + u) * NW + c) * W;
+                a[u] = vload<W, AL>(m + e);
+                if (ACC) o[u] = vload<W, AL>(out + e);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kMvUnroll; ++u) {
+            if (r + u < r1) {
+                const int64_t e = ((r + u) * NW + c) * W;
+                vstore<W, AL>(out + e, vmap(f, a[u], vv, ACC ? o[u] : a[u]));
+            }
+        }
+    }
+}
+
+// Column vector: the matrix is cut into tiles of kBlock*W columns of one row; a
+// workgroup strides over groups of kMvUnroll tiles and fetches v[row] per tile.
+template <int W, bool AL, bool ACC, typename F>
+__global__ __launch_bounds__(kBlock) void mv_colvec_kernel(F f, const float* m, const float* v,
+                                                           float* out, int64_t M, int64_t NW,
+                                                           int64_t tiles_per_row) {
+    typedef typename VecT<W>::type R;
+    const int64_t ntiles = M * tiles_per_row;
+    for (int64_t t0 = static_cast<int64_t>(blockIdx.x) * kMvUnroll; t0 < ntiles;
+         t0 += static_cast<int64_t>(gridDim.x) * kMvUnroll) {
+        R a[kMvUnroll], o[kMvUnroll];
+        float s[kMvUnroll];
+        int64_t idx[kMvUnroll];
+#pragma unroll
+        for (int u = 0; u < kMvUnroll; ++u) {
+            const int64_t t = t0 + u;
+            const int64_t row = t / tiles_per_row;
+            const int64_t c = (t - row * tiles_per_row) * kBlock + threadIdx.x;
+            idx[u] = (t < ntiles && c < NW) ? (row * NW + c) * W : -1;
+            if (idx[u] >= 0) {
+                s[u] = v[row];
+                a[u] = vload<W, AL>(m + idx[u]);
+                if (ACC) o[u] = vload<W, AL>(out + idx[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kMvUnroll; ++u) {
+            if (idx[u] >= 0)
+                vstore<W, AL>(out + idx[u], vmap(f, a[u], splat(a[u], s[u]), ACC ? o[u] : a[u]));
+        }
+    }
+}
+
+template <bool ACC, typename F>
+int launch_mv(const char* name, F f, const float* m, const float* v, float* out, int64_t M,
+              int64_t N, int v_is_col) {
+    const Context& c = ctx();
+    const bool vec = (N % 4 == 0);
+    const int64_t NW = vec ? N / 4 : N;
+    const dim3 blk(kBlock);
+    if (!v_is_col) {
+        const bool al = aligned16(m) && aligned16(out) && aligned16(v);
+        const int64_t target = static_cast<int64_t>(c.num_cus) * c.blocks_per_cu;
+        const int64_t gx = ceil_div(NW, kBlock);
+        int64_t bands = target / gx;
+        if (bands < 1) bands = 1;
+        int64_t rpb = ceil_div(M, bands);
+        if (rpb < 2 * kMvUnroll) rpb = 2 * kMvUnroll;
+        if (ceil_div(M, rpb) > 65535) rpb = ceil_div(M, 65535);
+        dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ceil_div(M, rpb)));
+        if (vec && al)
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+        else if (vec)
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+        else
+            hipLaunchKernelGGL((mv_rowvec_kernel<1, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+    } else {
+        const bool al = aligned16(m) && aligned16(out);
+        const int64_t tpr = ceil_div(NW, kBlock);
+        const int64_t groups = ceil_div(M * tpr, kMvUnroll);
+        dim3 grid(stream_grid(groups));
+        if (vec && al)
+            hipLaunchKernelGGL((mv_colvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+        else if (vec)
+            hipLaunchKernelGGL((mv_colvec_kernel<4, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+        else
+            hipLaunchKernelGGL((mv_colvec_kernel<1, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+    }
+    return check_launch(name);
+}
+
+// out(outer, bdim, inner) = a(outer, 1, inner)
+__global__ __launch_bounds__(kBlock) void broadcast_kernel(const float* __restrict__ a,
+                                                           float* __restrict__ out, int64_t outer,
+                                                           int64_t bdim, int64_t inner) {
+    const int64_t n = outer * bdim * inner;
+    const int64_t slab = bdim * inner;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < n;
+         e += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const int64_t o = e / slab;
+        const int64_t i = (e - o * slab) % inner;
+        out[e] = a[o * inner + i];
+    }
+}
+
+// out(rows, na+nb): [:, :na] = a, [:, na:] = b
+__global__ __launch_bounds__(kBlock) void merge_kernel(const float* __restrict__ a,
+                                                       const float* __restrict__ b,
+                                                       float* __restrict__ out, int64_t rows,
+                                                       int64_t na, int64_t nb) {
+    const int64_t w = na + nb;
+    const int64_t n = rows * w;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < n;
+         e += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const int64_t r = e / w;
+        const int64_t c = e - r * w;
+        out[e] = c < na ? a[r * na + c] : b[r * nb + (c - na)];
+    }
+}
+
+// oa += x[:, :na]; ob += x[:, na:]
+__global__ __launch_bounds__(kBlock) void split_add_kernel(const float* __restrict__ x, float* oa,
+                                                           float* ob, int64_t rows, int64_t na,
+                                                           int64_t nb) {
+    const int64_t w = na + nb;
+    const int64_t n = rows * w;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < n;
+         e += static_cast<int64_t>(gridDim.x) * kBlock) {
+        const int64_t r = e / w;
+        const int64_t c = e - r * w;
+        if (c < na) oa[r * na + c] += x[e];
+        else ob[r * nb + (c - na)] += x[e];
+    }
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" {
+
+int bship_mv_f32(int op, const float* m, const float* v, float* out, int64_t M, int64_t N,
+                 int v_is_col, int accumulate) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    if (M == 0 || N == 0) return 0;
+    BSHIP_REQUIRE_PTR(m);
+    BSHIP_REQUIRE_PTR(v);
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(m);
+    BSHIP_REQUIRE_F32_ALIGNED(v);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    if (accumulate) {
+        switch (op) {
+            case BSHIP_ADD: return launch_mv<true>("add_mv(acc)", MvAdd<true>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_SUB: return launch_mv<true>("subtract_mv(acc)", MvSub<true>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_MUL: return launch_mv<true>("mult_add_mv", MvMul<true>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_DIV: return launch_mv<true>("divide_mv(acc)", MvDiv<true>{}, m, v, out, M, N, v_is_col);
+        }
+    } else {
+        switch (op) {
+            case BSHIP_ADD: return launch_mv<false>("add_mv", MvAdd<false>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_SUB: return launch_mv<false>("subtract_mv", MvSub<false>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_MUL: return launch_mv<false>("mult_mv", MvMul<false>{}, m, v, out, M, N, v_is_col);
+            case BSHIP_DIV: return launch_mv<false>("divide_mv", MvDiv<false>{}, m, v, out, M, N, v_is_col);
+        }
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_mv_f32: unknown op %d", op);
+}
+
+int bship_broadcast_f32(const float* a, float* out, int64_t outer, int64_t bdim, int64_t inner) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(outer >= 0 && bdim >= 0 && inner >= 0);
+    const int64_t n = outer * bdim * inner;
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(a);
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_DIM(a != out);
+    hipLaunchKernelGGL(broadcast_kernel, dim3(stream_grid(ceil_div(n, kBlock))), dim3(kBlock), 0,
+                       ctx().stream, a, out, outer, bdim, inner);
+    return check_launch("broadcast_t");
+}
+
+int bship_merge_f32(const float* a, const float* b, float* out, int64_t rows, int64_t na,
+                    int64_t nb) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(rows >= 0 && na >= 0 && nb >= 0);
+    const int64_t n = rows * (na + nb);
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(out);
+    if (na > 0) BSHIP_REQUIRE_PTR(a);
+    if (nb > 0) BSHIP_REQUIRE_PTR(b);
+    hipLaunchKernelGGL(merge_kernel, dim3(stream_grid(ceil_div(n, kBlock))), dim3(kBlock), 0,
+                       ctx().stream, a, b, out, rows, na, nb);
+    return check_launch("merge_tt");
+}
+
+int bship_split_add_f32(const float* x, float* oa, float* ob, int64_t rows, int64_t na,
+                        int64_t nb) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(rows >= 0 && na >= 0 && nb >= 0);
+    const int64_t n = rows * (na + nb);
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(x);
+    if (na > 0) BSHIP_REQUIRE_PTR(oa);
+    if (nb > 0) BSHIP_REQUIRE_PTR(ob);
+    hipLaunchKernelGGL(split_add_kernel, dim3(stream_grid(ceil_div(n, kBlock))), dim3(kBlock), 0,
+                       ctx().stream, x, oa, ob, rows, na, nb);
+    return check_launch("split_add_tt");
+}
+
+}  // extern "C"

@@ -1,0 +1,134 @@
+// Shared plumbing of libbship: library context (device, stream), error
+// reporting, launch-shape helpers and the 128-bit vector types used by every
+// streaming kernel. gfx950 only: wavefronts are 64 lanes wide.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "../../include/bship.h"
+
+namespace bship {
+
+constexpr int kWave = 64;      // lanes per wavefront on CDNA
+constexpr int kBlock = 256;    // default workgroup: 4 wavefronts
+
+struct Context {
+    bool inited = false;
+    int device = -1;
+    int num_cus = 256;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    bool debug_sync = false;   // BSHIP_DEBUG_SYNC=1: sync + check after every launch
+    int blocks_per_cu = 8;     // streaming kernels launch num_cus*blocks_per_cu blocks
+    char name[256] = {0};
+};
+
+Context& ctx();
+
+// Records a formatted message for bship_last_error() and returns `code`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// 0 if e == hipSuccess, else records "<what>: <hip error string>" and returns e.
+int check_hip(hipError_t e, const char* what);
+// To be called right after a kernel launch.
+int check_launch(const char* what);
+
+#define BSHIP_REQUIRE_INIT()                                                     \
+    do {                                                                         \
+        if (!::bship::ctx().inited)                                              \
+            return ::bship::set_error(BSHIP_ERR_NOT_INITIALIZED,                 \
+                                      "%s: bship_init() has not been called",    \
+                                      __func__);                                 \
+    } while (0)
+
+#define BSHIP_REQUIRE_PTR(p)                                                     \
+    do {                                                                         \
+        if ((p) == nullptr)                                                      \
+            return ::bship::set_error(BSHIP_ERR_NULL_POINTER,                    \
+                                      "%s: argument '%s' is NULL", __func__, #p);\
+    } while (0)
+
+#define BSHIP_REQUIRE_F32_ALIGNED(p)                                             \
+    do {                                                                         \
+        if ((reinterpret_cast<uintptr_t>(p) & 3u) != 0)                          \
+            return ::bship::set_error(BSHIP_ERR_BAD_POINTER,                     \
+                                      "%s: argument '%s' is not 4-byte aligned", \
+                                      __func__, #p);                             \
+    } while (0)
+
+#define BSHIP_REQUIRE_DIM(cond)                                                  \
+    do {                                                                         \
+        if (!(cond))                                                             \
+            return ::bship::set_error(BSHIP_ERR_BAD_DIMENSION,                   \
+                                      "%s: requirement '%s' violated", __func__, \
+                                      #cond);                                    \
+    } while (0)
+
+#define BSHIP_HIP(call)                                                          \
+    do {                                                                         \
+        int _st = ::bship::check_hip((call), #call);                             \
+        if (_st != 0) return _st;                                                \
+    } while (0)
+
+// 128-bit vectors. f4 promises 16-byte alignment; f4u only 4-byte alignment --
+// the compiler still emits one global_load_dwordx4 for it (the memory system
+// accepts dword-aligned wide accesses), so views that start at an odd element
+// of the flat buffer keep wide transactions. The alignment of f4u lives in the
+// typedef, not in the type, so it must not be passed as a template argument:
+// kernels are parameterised by <W, AL> and go through vload/vstore below.
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef f4 f4u __attribute__((aligned(4)));
+
+template <int W> struct VecT { typedef float type; };
+template <> struct VecT<4> { typedef f4 type; };
+
+// Streaming (non-temporal) load/store of W floats starting at p.
+template <int W, bool AL>
+__device__ __forceinline__ typename VecT<W>::type vload(const float* p) {
+    if constexpr (W == 1) return __builtin_nontemporal_load(p);
+    else if constexpr (AL) return __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
+    else return __builtin_nontemporal_load(reinterpret_cast<const f4u*>(p));
+}
+template <int W, bool AL>
+__device__ __forceinline__ void vstore(float* p, typename VecT<W>::type v) {
+    if constexpr (W == 1) __builtin_nontemporal_store(v, p);
+    else if constexpr (AL) __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+    else __builtin_nontemporal_store(v, reinterpret_cast<f4u*>(p));
+}
+
+static inline bool aligned16(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Number of workgroups for a grid-stride streaming kernel over `tiles` tiles.
+static inline unsigned stream_grid(int64_t tiles) {
+    const Context& c = ctx();
+    int64_t cap = static_cast<int64_t>(c.num_cus) * c.blocks_per_cu;
+    int64_t g = tiles < cap ? tiles : cap;
+    return static_cast<unsigned>(g < 1 ? 1 : g);
+}
+
+// Scratch from the pool without zero-fill (internal partial-result buffers).
+int pool_alloc_raw(size_t nbytes, void** out);
+int pool_free_raw(void* p);
+// Enqueues mem[0:n] = val.
+int launch_fill(float* mem, float val, size_t n);
+
+// ---- wavefront / workgroup reductions (device) ----
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+}  // namespace bship

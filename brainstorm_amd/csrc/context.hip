@@ -1,0 +1,133 @@
+// Library lifecycle, error state and stream timers.
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "common.h"
+
+namespace bship {
+
+static Context g_ctx;
+static std::mutex g_ctx_mutex;
+static thread_local char t_error[512] = {0};
+
+Context& ctx() { return g_ctx; }
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_error, sizeof(t_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    return set_error(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return check_hip(e, what);
+    if (g_ctx.debug_sync) return check_hip(hipStreamSynchronize(g_ctx.stream), what);
+    return 0;
+}
+
+void pool_release_all();   // pool.hip
+void rng_release();        // rng.hip
+void gemm_release();       // gemm.hip
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" {
+
+int bship_version(void) { return BSHIP_VERSION; }
+
+const char* bship_last_error(void) { return t_error; }
+
+int bship_init(int device) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    if (g_ctx.inited) {
+        if (g_ctx.device == device) return 0;
+        return set_error(BSHIP_ERR_UNSUPPORTED,
+                         "bship_init: already initialised on device %d (asked for %d); "
+                         "call bship_shutdown() first", g_ctx.device, device);
+    }
+    int count = 0;
+    BSHIP_HIP(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count)
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_init: device %d not in [0,%d)",
+                         device, count);
+    BSHIP_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    BSHIP_HIP(hipGetDeviceProperties(&prop, device));
+    g_ctx.num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    snprintf(g_ctx.name, sizeof(g_ctx.name), "%s (%s)", prop.name, prop.gcnArchName);
+    // One stream at the default priority; every kernel and copy goes here in call order.
+    BSHIP_HIP(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking));
+    BSHIP_HIP(hipEventCreate(&g_ctx.ev_start));
+    BSHIP_HIP(hipEventCreate(&g_ctx.ev_stop));
+    const char* dbg = getenv("BSHIP_DEBUG_SYNC");
+    g_ctx.debug_sync = dbg && dbg[0] && dbg[0] != '0';
+    const char* bpc = getenv("BSHIP_BLOCKS_PER_CU");
+    if (bpc && atoi(bpc) > 0 && atoi(bpc) <= 64) g_ctx.blocks_per_cu = atoi(bpc);
+    g_ctx.device = device;
+    g_ctx.inited = true;
+    return 0;
+}
+
+int bship_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_ctx_mutex);
+    if (!g_ctx.inited) return 0;
+    (void)hipStreamSynchronize(g_ctx.stream);
+    gemm_release();
+    rng_release();
+    pool_release_all();
+    (void)hipEventDestroy(g_ctx.ev_start);
+    (void)hipEventDestroy(g_ctx.ev_stop);
+    (void)hipStreamDestroy(g_ctx.stream);
+    g_ctx = Context();
+    return 0;
+}
+
+int bship_sync(void) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_HIP(hipStreamSynchronize(g_ctx.stream));
+    return 0;
+}
+
+int bship_device_info(char* name_host, size_t name_len, int* compute_units) {
+    BSHIP_REQUIRE_INIT();
+    if (name_host && name_len) {
+        strncpy(name_host, g_ctx.name, name_len - 1);
+        name_host[name_len - 1] = 0;
+    }
+    if (compute_units) *compute_units = g_ctx.num_cus;
+    return 0;
+}
+
+int bship_timer_start(void) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_HIP(hipEventRecord(g_ctx.ev_start, g_ctx.stream));
+    return 0;
+}
+
+int bship_timer_stop(void) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_HIP(hipEventRecord(g_ctx.ev_stop, g_ctx.stream));
+    return 0;
+}
+
+int bship_timer_elapsed_ms(float* ms_host) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(ms_host);
+    BSHIP_HIP(hipEventSynchronize(g_ctx.ev_stop));
+    BSHIP_HIP(hipEventElapsedTime(ms_host, g_ctx.ev_start, g_ctx.ev_stop));
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,261 @@
+// Elementwise handler operations: one streaming kernel template, instantiated
+// per operation. Every operation is HBM-bound; the kernel moves 128 bits per
+// lane per access, keeps kUnroll independent accesses in flight per lane and
+// uses a grid of a few workgroups per compute unit that strides over tiles.
+//
+// Arithmetic follows NumPy's float32 evaluation order exactly (each NumPy
+// temporary is one float32 rounding), so products are never fused into adds.
+#pragma clang fp contract(off)
+
+#include "common.h"
+
+namespace bship {
+
+constexpr int kUnroll = 4;
+constexpr size_t kTile = static_cast<size_t>(kBlock) * 4 * kUnroll;   // floats per tile
+
+// F::apply(v0, v1, v2) -> result. NIN pointers are read (p0..), `out` is written.
+// `out` may alias any input, so nothing here is __restrict__; all loads of a
+// tile are issued before its stores.
+template <int NIN, bool AL, typename F>
+__global__ __launch_bounds__(kBlock) void ew_kernel(F f, const float* p0, const float* p1,
+                                                    const float* p2, float* out, size_t n) {
+    const size_t ntiles = n / kTile;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * kTile + threadIdx.x * 4;
+        f4 r0[kUnroll], r1[kUnroll], r2[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t q = base + u * (kBlock * 4);
+            r0[u] = vload<4, AL>(p0 + q);
+            if (NIN > 1) r1[u] = vload<4, AL>(p1 + q);
+            if (NIN > 2) r2[u] = vload<4, AL>(p2 + q);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            f4 o;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                o[k] = f.apply(r0[u][k], NIN > 1 ? r1[u][k] : 0.0f, NIN > 2 ? r2[u][k] : 0.0f);
+            vstore<4, AL>(out + base + u * (kBlock * 4), o);
+        }
+    }
+    // tail shorter than one tile: last workgroup, scalar
+    if (blockIdx.x == gridDim.x - 1) {
+        for (size_t i = ntiles * kTile + threadIdx.x; i < n; i += kBlock)
+            out[i] = f.apply(p0[i], NIN > 1 ? p1[i] : 0.0f, NIN > 2 ? p2[i] : 0.0f);
+    }
+}
+
+template <int NIN, typename F>
+int launch_ew(const char* name, F f, const float* p0, const float* p1, const float* p2,
+              float* out, size_t n) {
+    if (n == 0) return 0;
+    unsigned grid = stream_grid(static_cast<int64_t>(n / kTile));
+    bool al = aligned16(p0) && aligned16(out) && (NIN < 2 || aligned16(p1)) &&
+              (NIN < 3 || aligned16(p2));
+    if (al)
+        hipLaunchKernelGGL((ew_kernel<NIN, true, F>), dim3(grid), dim3(kBlock), 0, ctx().stream, f,
+                           p0, p1, p2, out, n);
+    else
+        hipLaunchKernelGGL((ew_kernel<NIN, false, F>), dim3(grid), dim3(kBlock), 0, ctx().stream, f,
+                           p0, p1, p2, out, n);
+    return check_launch(name);
+}
+
+// ------------------------------- functors ---------------------------------
+// Inputs arrive as (v0, v1, v2) in the order the launcher passes pointers.
+
+struct AddOp  { __device__ float apply(float a, float b, float) const { return a + b; } };
+struct SubOp  { __device__ float apply(float a, float b, float) const { return a - b; } };
+struct MulOp  { __device__ float apply(float a, float b, float) const { return a * b; } };
+struct DivOp  { __device__ float apply(float a, float b, float) const { return a / b; } };
+struct FmodOp { __device__ float apply(float a, float b, float) const { return fmodf(a, b); } };
+// (a, b, old out): out + a*b with the product rounded first
+struct MultAddOp {
+    __device__ float apply(float a, float b, float o) const { float p = a * b; return o + p; }
+};
+
+struct AddStOp  { float s; __device__ float apply(float t, float, float) const { return t + s; } };
+struct MultStOp { float s; __device__ float apply(float t, float, float) const { return s * t; } };
+// (t, old out)
+struct MultAddStOp {
+    float s;
+    __device__ float apply(float t, float o, float) const { float p = s * t; return o + p; }
+};
+
+struct AbsOp  { __device__ float apply(float x, float, float) const { return fabsf(x); } };
+// np.sign: 1, -1, 0 (also for -0.0), NaN stays NaN
+struct SignOp {
+    __device__ float apply(float x, float, float) const {
+        return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : (x == 0.0f ? 0.0f : x));
+    }
+};
+struct SqrtOp { __device__ float apply(float x, float, float) const { return sqrtf(x); } };
+// Transcendentals are evaluated in float64 and rounded once, which gives the
+// correctly rounded float32 value; the kernels stay memory-bound.
+struct LogOp {
+    __device__ float apply(float x, float, float) const { return static_cast<float>(log(static_cast<double>(x))); }
+};
+struct TanhOp {
+    __device__ float apply(float x, float, float) const { return static_cast<float>(tanh(static_cast<double>(x))); }
+};
+// numpy 283-287: 1/(1+exp(-x)) for x >= 0, exp(x)/(1+exp(x)) for x < 0
+struct SigmoidOp {
+    __device__ float apply(float x, float, float) const {
+        double xd = static_cast<double>(x);
+        double e = exp(-fabs(xd));
+        double r = (x >= 0.0f ? 1.0 : e) / (1.0 + e);
+        return (x != x) ? x : static_cast<float>(r);
+    }
+};
+// numpy 277-278: x*(x>0); the mask is 1.0 or 0.0, so negatives give -0.0
+struct RelOp {
+    __device__ float apply(float x, float, float) const { return x > 0.0f ? x : x * 0.0f; }
+};
+// numpy 303-305: x*(x>=0) + (exp(x)-1)*(x<0), every step in float32
+struct ElOp {
+    __device__ float apply(float x, float, float) const {
+        float e = static_cast<float>(exp(static_cast<double>(x)));
+        float t1 = x * (x >= 0.0f ? 1.0f : 0.0f);
+        float t2 = (e - 1.0f) * (x < 0.0f ? 1.0f : 0.0f);
+        return t1 + t2;
+    }
+};
+
+// derivatives take (y, dy)
+struct SigmoidDerivOp {
+    __device__ float apply(float y, float dy, float) const { float p = dy * y; float q = 1.0f - y; return p * q; }
+};
+struct TanhDerivOp {
+    __device__ float apply(float y, float dy, float) const { float p = y * y; float q = 1.0f - p; return dy * q; }
+};
+struct RelDerivOp {
+    __device__ float apply(float y, float dy, float) const { return dy * (y > 0.0f ? 1.0f : 0.0f); }
+};
+struct ElDerivOp {
+    __device__ float apply(float y, float dy, float) const {
+        float t1 = dy * (y >= 0.0f ? 1.0f : 0.0f);
+        float q = y + 1.0f;
+        float p = dy * q;
+        float t2 = p * (y < 0.0f ? 1.0f : 0.0f);
+        return t1 + t2;
+    }
+};
+
+// np.clip = minimum(maximum(a, lo), hi) with NaN in `a` propagating
+struct ClipOp {
+    float lo, hi;
+    __device__ float apply(float a, float, float) const {
+        float t = (a != a || a > lo) ? a : lo;
+        return (t != t || t < hi) ? t : hi;
+    }
+};
+
+// conditional ops; cond != 0 is true for NaN as in NumPy
+struct CopyIfOp {  // (a, cond, old out)
+    __device__ float apply(float a, float c, float o) const { return c != 0.0f ? a : o; }
+};
+struct FillIfOp {  // (cond, old out)
+    float val;
+    __device__ float apply(float c, float o, float) const { return c != 0.0f ? val : o; }
+};
+struct AddIfOp {   // (a, cond, old out)
+    __device__ float apply(float a, float c, float o) const { return c != 0.0f ? o + a : o; }
+};
+
+}  // namespace bship
+
+using namespace bship;
+
+#define BSHIP_EW_PROLOGUE(first, outp)        \
+    BSHIP_REQUIRE_INIT();                     \
+    if (n == 0) return 0;                     \
+    BSHIP_REQUIRE_PTR(first);                 \
+    BSHIP_REQUIRE_PTR(outp);                  \
+    BSHIP_REQUIRE_F32_ALIGNED(first);         \
+    BSHIP_REQUIRE_F32_ALIGNED(outp)
+
+extern "C" {
+
+int bship_binary_f32(int op, const float* a, const float* b, float* out, size_t n) {
+    BSHIP_EW_PROLOGUE(a, out);
+    BSHIP_REQUIRE_PTR(b);
+    BSHIP_REQUIRE_F32_ALIGNED(b);
+    switch (op) {
+        case BSHIP_ADD:  return launch_ew<2>("add_tt", AddOp{}, a, b, nullptr, out, n);
+        case BSHIP_SUB:  return launch_ew<2>("subtract_tt", SubOp{}, a, b, nullptr, out, n);
+        case BSHIP_MUL:  return launch_ew<2>("mult_tt", MulOp{}, a, b, nullptr, out, n);
+        case BSHIP_DIV:  return launch_ew<2>("divide_tt", DivOp{}, a, b, nullptr, out, n);
+        case BSHIP_FMOD: return launch_ew<2>("modulo_tt", FmodOp{}, a, b, nullptr, out, n);
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_binary_f32: unknown op %d", op);
+}
+
+int bship_mult_add_tt_f32(const float* a, const float* b, float* out, size_t n) {
+    BSHIP_EW_PROLOGUE(a, out);
+    BSHIP_REQUIRE_PTR(b);
+    BSHIP_REQUIRE_F32_ALIGNED(b);
+    return launch_ew<3>("mult_add_tt", MultAddOp{}, a, b, out, out, n);
+}
+
+int bship_scalar_f32(int op, float s, const float* t, float* out, size_t n) {
+    BSHIP_EW_PROLOGUE(t, out);
+    switch (op) {
+        case BSHIP_ADD_ST:      return launch_ew<1>("add_st", AddStOp{s}, t, nullptr, nullptr, out, n);
+        case BSHIP_MULT_ST:     return launch_ew<1>("mult_st", MultStOp{s}, t, nullptr, nullptr, out, n);
+        case BSHIP_MULT_ADD_ST: return launch_ew<2>("mult_add_st", MultAddStOp{s}, t, out, nullptr, out, n);
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_scalar_f32: unknown op %d", op);
+}
+
+int bship_unary_f32(int op, const float* x, float* y, size_t n) {
+    BSHIP_EW_PROLOGUE(x, y);
+    switch (op) {
+        case BSHIP_ABS:     return launch_ew<1>("abs_t", AbsOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_SIGN:    return launch_ew<1>("sign_t", SignOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_SQRT:    return launch_ew<1>("sqrt_t", SqrtOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_LOG:     return launch_ew<1>("log_t", LogOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_SIGMOID: return launch_ew<1>("sigmoid", SigmoidOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_TANH:    return launch_ew<1>("tanh", TanhOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_REL:     return launch_ew<1>("rel", RelOp{}, x, nullptr, nullptr, y, n);
+        case BSHIP_EL:      return launch_ew<1>("el", ElOp{}, x, nullptr, nullptr, y, n);
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_unary_f32: unknown op %d", op);
+}
+
+int bship_deriv_f32(int op, const float* y, const float* dy, float* dx, size_t n) {
+    BSHIP_EW_PROLOGUE(y, dx);
+    BSHIP_REQUIRE_PTR(dy);
+    BSHIP_REQUIRE_F32_ALIGNED(dy);
+    switch (op) {
+        case BSHIP_SIGMOID_DERIV: return launch_ew<2>("sigmoid_deriv", SigmoidDerivOp{}, y, dy, nullptr, dx, n);
+        case BSHIP_TANH_DERIV:    return launch_ew<2>("tanh_deriv", TanhDerivOp{}, y, dy, nullptr, dx, n);
+        case BSHIP_REL_DERIV:     return launch_ew<2>("rel_deriv", RelDerivOp{}, y, dy, nullptr, dx, n);
+        case BSHIP_EL_DERIV:      return launch_ew<2>("el_deriv", ElDerivOp{}, y, dy, nullptr, dx, n);
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_deriv_f32: unknown op %d", op);
+}
+
+int bship_clip_f32(const float* a, float lo, float hi, float* out, size_t n) {
+    BSHIP_EW_PROLOGUE(a, out);
+    return launch_ew<1>("clip_t", ClipOp{lo, hi}, a, nullptr, nullptr, out, n);
+}
+
+int bship_cond_f32(int op, const float* a, float val, float* out, const float* cond, size_t n) {
+    BSHIP_EW_PROLOGUE(cond, out);
+    BSHIP_REQUIRE_F32_ALIGNED(a);
+    switch (op) {
+        case BSHIP_COPY_IF:
+            BSHIP_REQUIRE_PTR(a);
+            return launch_ew<3>("copy_to_if", CopyIfOp{}, a, cond, out, out, n);
+        case BSHIP_FILL_IF:
+            return launch_ew<2>("fill_if", FillIfOp{val}, cond, out, nullptr, out, n);
+        case BSHIP_ADD_IF:
+            BSHIP_REQUIRE_PTR(a);
+            return launch_ew<3>("add_into_if", AddIfOp{}, a, cond, out, out, n);
+    }
+    return set_error(BSHIP_ERR_BAD_OP, "bship_cond_f32: unknown op %d", op);
+}
+
+}  // extern "C"

@@ -1,0 +1,137 @@
+// dot_mm / dot_add_mm through hipBLASLt. The handler's matrices are row-major;
+// hipBLASLt is column-major, so C = op(A) op(B) is issued as
+// C^T = op(B)^T op(A)^T by swapping the operands. Descriptors and the algorithm
+// chosen by the heuristic are cached per problem shape, because recurrent
+// networks issue the same small product thousands of times per step.
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "common.h"
+
+namespace bship {
+
+namespace {
+
+struct GemmPlan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+};
+
+typedef std::tuple<int, int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t> GemmKey;
+
+std::mutex g_gemm_mutex;
+hipblasLtHandle_t g_handle = nullptr;
+std::map<GemmKey, GemmPlan> g_plans;
+void* g_workspace = nullptr;
+constexpr size_t kWorkspaceBytes = 64u << 20;
+
+int blas_error(hipblasStatus_t s, const char* what) {
+    return set_error(BSHIP_ERR_BLAS, "%s failed with hipblasStatus %d", what, static_cast<int>(s));
+}
+
+#define BSHIP_BLAS(call)                                       \
+    do {                                                       \
+        hipblasStatus_t _s = (call);                           \
+        if (_s != HIPBLAS_STATUS_SUCCESS) return blas_error(_s, #call); \
+    } while (0)
+
+void destroy_plan(GemmPlan& p) {
+    if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
+    if (p.lb) hipblasLtMatrixLayoutDestroy(p.lb);
+    if (p.lc) hipblasLtMatrixLayoutDestroy(p.lc);
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    p = GemmPlan();
+}
+
+// Column-major problem: D(m x n) = opA(A) opB(B), leading dimensions lda/ldb/ldc.
+int make_plan(GemmPlan& p, hipblasOperation_t opa, hipblasOperation_t opb, int64_t m, int64_t n,
+              int64_t k, int64_t lda, int64_t ldb, int64_t ldc) {
+    BSHIP_BLAS(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+    int32_t ta = static_cast<int32_t>(opa), tb = static_cast<int32_t>(opb);
+    BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)));
+    BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)));
+    const bool na = (opa == HIPBLAS_OP_N), nb = (opb == HIPBLAS_OP_N);
+    BSHIP_BLAS(hipblasLtMatrixLayoutCreate(&p.la, HIP_R_32F, na ? m : k, na ? k : m, lda));
+    BSHIP_BLAS(hipblasLtMatrixLayoutCreate(&p.lb, HIP_R_32F, nb ? k : n, nb ? n : k, ldb));
+    BSHIP_BLAS(hipblasLtMatrixLayoutCreate(&p.lc, HIP_R_32F, m, n, ldc));
+    hipblasLtMatmulPreference_t pref = nullptr;
+    BSHIP_BLAS(hipblasLtMatmulPreferenceCreate(&pref));
+    uint64_t ws = kWorkspaceBytes;
+    hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(
+        pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
+    hipblasLtMatmulHeuristicResult_t res[1];
+    int found = 0;
+    if (s == HIPBLAS_STATUS_SUCCESS)
+        s = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, res, &found);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    if (s != HIPBLAS_STATUS_SUCCESS) return blas_error(s, "hipblasLtMatmulAlgoGetHeuristic");
+    if (found < 1)
+        return set_error(BSHIP_ERR_BLAS,
+                         "hipBLASLt has no float32 algorithm for m=%lld n=%lld k=%lld opA=%d opB=%d",
+                         (long long)m, (long long)n, (long long)k, (int)opa, (int)opb);
+    p.algo = res[0].algo;
+    p.workspace = res[0].workspaceSize;
+    return 0;
+}
+
+}  // namespace
+
+void gemm_release() {
+    std::lock_guard<std::mutex> lock(g_gemm_mutex);
+    for (auto& kv : g_plans) destroy_plan(kv.second);
+    g_plans.clear();
+    if (g_workspace) { pool_free_raw(g_workspace); g_workspace = nullptr; }
+    if (g_handle) { hipblasLtDestroy(g_handle); g_handle = nullptr; }
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
+                              const float* A, int64_t lda, const float* B, int64_t ldb, float beta,
+                              float* C, int64_t ldc) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0 && K >= 0);
+    if (M == 0 || N == 0) return 0;
+    BSHIP_REQUIRE_PTR(C);
+    BSHIP_REQUIRE_DIM(ldc >= N);
+    if (K == 0) {
+        // empty inner dimension: C = beta * C
+        if (beta == 1.0f) return 0;
+        if (ldc != N) return set_error(BSHIP_ERR_UNSUPPORTED, "bship_gemm_f32: K == 0 needs a dense C");
+        return beta == 0.0f ? bship_fill_f32(C, 0.0f, static_cast<size_t>(M * N))
+                            : bship_scalar_f32(BSHIP_MULT_ST, beta, C, C, static_cast<size_t>(M * N));
+    }
+    BSHIP_REQUIRE_PTR(A);
+    BSHIP_REQUIRE_PTR(B);
+    BSHIP_REQUIRE_DIM(lda >= (transa ? M : K));
+    BSHIP_REQUIRE_DIM(ldb >= (transb ? K : N));
+    std::lock_guard<std::mutex> lock(g_gemm_mutex);
+    if (!g_handle) BSHIP_BLAS(hipblasLtCreate(&g_handle));
+    if (!g_workspace) {
+        int st = pool_alloc_raw(kWorkspaceBytes, &g_workspace);
+        if (st != 0) return st;
+    }
+    // Row-major C(MxN) = op(A) op(B)  <=>  column-major C^T(NxM) = op(B)^T op(A)^T.
+    // A row-major matrix read as column-major is its transpose, so the first
+    // column-major operand is B with opB, the second is A with opA.
+    const GemmKey key(transa != 0, transb != 0, M, N, K, lda, ldb, ldc);
+    auto it = g_plans.find(key);
+    if (it == g_plans.end()) {
+        GemmPlan plan;
+        int st = make_plan(plan, transb ? HIPBLAS_OP_T : HIPBLAS_OP_N, transa ? HIPBLAS_OP_T : HIPBLAS_OP_N,
+                           N, M, K, ldb, lda, ldc);
+        if (st != 0) { destroy_plan(plan); return st; }
+        it = g_plans.emplace(key, plan).first;
+    }
+    const GemmPlan& p = it->second;
+    BSHIP_BLAS(hipblasLtMatmul(g_handle, p.desc, &alpha, B, p.la, A, p.lb, &beta, C, p.lc, C, p.lc,
+                               &p.algo, g_workspace, kWorkspaceBytes, ctx().stream));
+    return check_launch("gemm");
+}

@@ -1,0 +1,240 @@
+// Caching device-memory pool, host<->device copies, copy_to and fill.
+//
+// The pool never returns memory to the driver while the library is in use:
+// freed blocks go to a per-size free list and are handed out again. Because
+// every kernel runs on the one library stream, a block that is reused is
+// touched by its new owner only after all work of the previous owner.
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace bship {
+
+namespace {
+std::mutex g_pool_mutex;
+std::map<size_t, std::vector<void*>> g_free;       // rounded size -> cached blocks
+std::unordered_map<void*, size_t> g_live;          // handed-out block -> rounded size
+size_t g_in_use = 0, g_cached = 0, g_device_allocs = 0;
+
+size_t round_size(size_t n) {
+    size_t q = n < (64u << 10) ? 256 : (n < (1u << 20) ? 4096 : (2u << 20));
+    return (n + q - 1) / q * q;
+}
+
+size_t pool_limit() {
+    const char* s = getenv("BSHIP_POOL_LIMIT_BYTES");
+    return s && s[0] ? static_cast<size_t>(strtoull(s, nullptr, 10)) : 0;
+}
+
+void trim_locked() {
+    for (auto& kv : g_free)
+        for (void* p : kv.second) (void)hipFree(p);
+    g_free.clear();
+    g_cached = 0;
+}
+}  // namespace
+
+int pool_alloc_raw(size_t nbytes, void** out) {
+    *out = nullptr;
+    if (nbytes == 0) return 0;
+    size_t sz = round_size(nbytes);
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_free.find(sz);
+    if (it != g_free.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        g_cached -= sz;
+    } else {
+        size_t limit = pool_limit();
+        if (limit && g_in_use + g_cached + sz > limit) {
+            // Give cached blocks back before refusing.
+            (void)hipStreamSynchronize(ctx().stream);
+            trim_locked();
+            if (g_in_use + sz > limit)
+                return set_error(BSHIP_ERR_OUT_OF_MEMORY,
+                                 "pool limit of %zu bytes reached (in use %zu, asked %zu)",
+                                 limit, g_in_use, sz);
+        }
+        hipError_t e = hipMalloc(out, sz);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipStreamSynchronize(ctx().stream);
+            trim_locked();
+            e = hipMalloc(out, sz);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                *out = nullptr;
+                return set_error(BSHIP_ERR_OUT_OF_MEMORY,
+                                 "hipMalloc of %zu bytes failed: %s (in use %zu)", sz,
+                                 hipGetErrorString(e), g_in_use);
+            }
+        }
+        ++g_device_allocs;
+    }
+    g_live[*out] = sz;
+    g_in_use += sz;
+    return 0;
+}
+
+int pool_free_raw(void* p) {
+    if (!p) return 0;
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_live.find(p);
+    if (it == g_live.end())
+        return set_error(BSHIP_ERR_BAD_POINTER, "bship_free: %p was not allocated by the pool", p);
+    size_t sz = it->second;
+    g_live.erase(it);
+    g_in_use -= sz;
+    g_free[sz].push_back(p);
+    g_cached += sz;
+    return 0;
+}
+
+void pool_release_all() {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    trim_locked();
+    for (auto& kv : g_live) (void)hipFree(kv.first);
+    g_live.clear();
+    g_in_use = 0;
+    g_device_allocs = 0;
+}
+
+// ------------------------------- kernels ----------------------------------
+
+// Each block-iteration covers a tile of kBlock*4*kFillUnroll floats.
+constexpr int kFillUnroll = 4;
+
+template <bool AL>
+__global__ __launch_bounds__(kBlock) void fill_kernel(float* __restrict__ p, float val, size_t n) {
+    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
+    const size_t ntiles = n / tile;
+    const f4 vv = {val, val, val, val};
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        float* q = p + t * tile + threadIdx.x * 4;
+#pragma unroll
+        for (int u = 0; u < kFillUnroll; ++u) vstore<4, AL>(q + u * kBlock * 4, vv);
+    }
+    // tail (fewer than one tile), handled by the first block only
+    if (blockIdx.x == 0)
+        for (size_t i = ntiles * tile + threadIdx.x; i < n; i += kBlock) p[i] = val;
+}
+
+template <bool AL>
+__global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ s,
+                                                      float* __restrict__ d, size_t n) {
+    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
+    const size_t ntiles = n / tile;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t off = t * tile + threadIdx.x * 4;
+        f4 r[kFillUnroll];
+#pragma unroll
+        for (int u = 0; u < kFillUnroll; ++u) r[u] = vload<4, AL>(s + off + u * kBlock * 4);
+#pragma unroll
+        for (int u = 0; u < kFillUnroll; ++u) vstore<4, AL>(d + off + u * kBlock * 4, r[u]);
+    }
+    if (blockIdx.x == 0)
+        for (size_t i = ntiles * tile + threadIdx.x; i < n; i += kBlock) d[i] = s[i];
+}
+
+int launch_fill(float* p, float val, size_t n) {
+    if (n == 0) return 0;
+    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
+    unsigned grid = stream_grid(static_cast<int64_t>(n / tile));
+    if (aligned16(p))
+        hipLaunchKernelGGL(fill_kernel<true>, dim3(grid), dim3(kBlock), 0, ctx().stream, p, val, n);
+    else
+        hipLaunchKernelGGL(fill_kernel<false>, dim3(grid), dim3(kBlock), 0, ctx().stream, p, val, n);
+    return check_launch("fill_kernel");
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" {
+
+int bship_malloc(size_t nbytes, void** out) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(out);
+    int st = pool_alloc_raw(nbytes, out);
+    if (st != 0 || *out == nullptr) return st;
+    // Blocks are rounded to a multiple of 256 bytes, so clearing whole floats covers nbytes.
+    return launch_fill(static_cast<float*>(*out), 0.0f, (nbytes + 3) / 4);
+}
+
+int bship_free(void* p) {
+    BSHIP_REQUIRE_INIT();
+    return pool_free_raw(p);
+}
+
+int bship_pool_trim(void) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_HIP(hipStreamSynchronize(ctx().stream));
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    trim_locked();
+    return 0;
+}
+
+int bship_pool_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_allocations) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    if (bytes_in_use) *bytes_in_use = g_in_use;
+    if (bytes_cached) *bytes_cached = g_cached;
+    if (device_allocations) *device_allocations = g_device_allocs;
+    return 0;
+}
+
+int bship_h2d(void* dst, const void* src_host, size_t nbytes) {
+    BSHIP_REQUIRE_INIT();
+    if (nbytes == 0) return 0;
+    BSHIP_REQUIRE_PTR(dst);
+    BSHIP_REQUIRE_PTR(src_host);
+    BSHIP_HIP(hipMemcpyAsync(dst, src_host, nbytes, hipMemcpyHostToDevice, ctx().stream));
+    BSHIP_HIP(hipStreamSynchronize(ctx().stream));
+    return 0;
+}
+
+int bship_d2h(void* dst_host, const void* src, size_t nbytes) {
+    BSHIP_REQUIRE_INIT();
+    if (nbytes == 0) return 0;
+    BSHIP_REQUIRE_PTR(dst_host);
+    BSHIP_REQUIRE_PTR(src);
+    BSHIP_HIP(hipMemcpyAsync(dst_host, src, nbytes, hipMemcpyDeviceToHost, ctx().stream));
+    BSHIP_HIP(hipStreamSynchronize(ctx().stream));
+    return 0;
+}
+
+int bship_d2d(void* dst, const void* src, size_t nbytes) {
+    BSHIP_REQUIRE_INIT();
+    if (nbytes == 0 || dst == src) return 0;
+    BSHIP_REQUIRE_PTR(dst);
+    BSHIP_REQUIRE_PTR(src);
+    uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | nbytes;
+    if (bits & 3u) {  // not float-granular: let the runtime copy bytes
+        BSHIP_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, ctx().stream));
+        return 0;
+    }
+    const size_t n = nbytes / 4;
+    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
+    unsigned grid = stream_grid(static_cast<int64_t>(n / tile));
+    const float* s = static_cast<const float*>(src);
+    float* d = static_cast<float*>(dst);
+    if (aligned16(s) && aligned16(d))
+        hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(kBlock), 0, ctx().stream, s, d, n);
+    else
+        hipLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(kBlock), 0, ctx().stream, s, d, n);
+    return check_launch("copy_kernel");
+}
+
+int bship_fill_f32(float* mem, float val, size_t n) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(mem);
+    BSHIP_REQUIRE_F32_ALIGNED(mem);
+    return launch_fill(mem, val, n);
+}
+
+}  // extern "C"

@@ -1,0 +1,424 @@
+// Reductions: sum_t over axis 0, axis 1 or everything, the fused one-pass row
+// softmax, and the is_fully_finite check. Each input element is read from HBM
+// exactly once. Results are deterministic: partial sums are combined in a
+// fixed order (no floating-point atomics).
+#pragma clang fp contract(off)
+
+#include "common.h"
+
+namespace bship {
+
+__device__ __forceinline__ float hsum(float v) { return v; }
+__device__ __forceinline__ float hsum(f4 v) { return (v[0] + v[1]) + (v[2] + v[3]); }
+__device__ __forceinline__ float hmax(float v) { return v; }
+__device__ __forceinline__ float hmax(f4 v) { return fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])); }
+template <typename R> __device__ __forceinline__ R vzero();
+template <> __device__ __forceinline__ float vzero<float>() { return 0.0f; }
+template <> __device__ __forceinline__ f4 vzero<f4>() { f4 z = {0.0f, 0.0f, 0.0f, 0.0f}; return z; }
+
+// ============================ sum over axis 0 ==============================
+// Column sums of a row-major (M,N) matrix. A workgroup is 64 column-lanes x 4
+// row-lanes (one wavefront per row-lane): each wavefront reads 64*W consecutive
+// columns of one row per access, walks down its band of rows with 4 independent
+// accumulators, and the 4 wavefronts are combined through LDS. grid.x tiles the
+// columns, grid.y splits the rows; with more than one row band the bands write
+// partial sums that a second launch of the same kernel adds up. NW = N / W.
+template <int W, bool AL>
+__global__ __launch_bounds__(kBlock) void colsum_kernel(const float* __restrict__ a,
+                                                        float* __restrict__ out, int64_t M,
+                                                        int64_t NW, int64_t rows_per_block) {
+    typedef typename VecT<W>::type R;
+    __shared__ R lds[kBlock];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wv = threadIdx.x / kWave;                      // 0..3: row-lane
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kWave + lane;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_block;
+    const int64_t r1 = (r0 + rows_per_block < M) ? r0 + rows_per_block : M;
+    R acc0 = vzero<R>(), acc1 = vzero<R>(), acc2 = vzero<R>(), acc3 = vzero<R>();
+    if (c < NW) {
+        const float* p = a + c * W;
+        const int64_t pitch = NW * W;
+        int64_t r = r0 + wv;
+        for (; r + 12 < r1; r += 16) {
+            R x0 = vload<W, AL>(p + r * pitch);
+            R x1 = vload<W, AL>(p + (r + 4) * pitch);
+            R x2 = vload<W, AL>(p + (r + 8) * pitch);
+            R x3 = vload<W, AL>(p + (r + 12) * pitch);
+            acc0 += x0; acc1 += x1; acc2 += x2; acc3 += x3;
+        }
+        for (; r < r1; r += 4) acc0 += vload<W, AL>(p + r * pitch);
+    }
+    lds[threadIdx.x] = (acc0 + acc1) + (acc2 + acc3);
+    __syncthreads();
+    if (wv == 0 && c < NW) {
+        R t = (lds[lane] + lds[lane + kWave]) + (lds[lane + 2 * kWave] + lds[lane + 3 * kWave]);
+        vstore<W, AL>(out + (static_cast<int64_t>(blockIdx.y) * NW + c) * W, t);
+    }
+}
+
+static void launch_colsum_kernel(bool vec, bool al, dim3 grid, const float* a, float* dst,
+                                 int64_t M, int64_t NW, int64_t rpb) {
+    hipStream_t s = ctx().stream;
+    if (vec && al) hipLaunchKernelGGL((colsum_kernel<4, true>), grid, dim3(kBlock), 0, s, a, dst, M, NW, rpb);
+    else if (vec)  hipLaunchKernelGGL((colsum_kernel<4, false>), grid, dim3(kBlock), 0, s, a, dst, M, NW, rpb);
+    else           hipLaunchKernelGGL((colsum_kernel<1, false>), grid, dim3(kBlock), 0, s, a, dst, M, NW, rpb);
+}
+
+static int launch_colsum(const float* a, float* out, int64_t M, int64_t N) {
+    const Context& c = ctx();
+    const bool vec = (N % 4 == 0);
+    const int64_t NW = vec ? N / 4 : N;
+    const int64_t gx = ceil_div(NW, kWave);
+    const int64_t target = static_cast<int64_t>(c.num_cus) * 4;
+    int64_t bands = target / gx;
+    if (bands < 1) bands = 1;
+    const int64_t min_rows = 64;             // at least 4 unrolled steps per wavefront
+    if (bands > ceil_div(M, min_rows)) bands = ceil_div(M, min_rows);
+    if (bands > 1024) bands = 1024;
+    const int64_t rpb = ceil_div(M, bands);
+    bands = ceil_div(M, rpb);
+    float* dst = out;
+    float* partial = nullptr;
+    if (bands > 1) {
+        void* p = nullptr;
+        int st = pool_alloc_raw(static_cast<size_t>(bands) * N * sizeof(float), &p);
+        if (st != 0) return st;
+        partial = static_cast<float*>(p);
+        dst = partial;
+    }
+    launch_colsum_kernel(vec, aligned16(a) && aligned16(dst),
+                         dim3(static_cast<unsigned>(gx), static_cast<unsigned>(bands)), a, dst, M, NW, rpb);
+    int st = check_launch("sum_t(axis=0)");
+    if (partial) {
+        if (st == 0) {
+            // second stage: column sums of the (bands, N) partials in one band
+            launch_colsum_kernel(vec, aligned16(partial) && aligned16(out),
+                                 dim3(static_cast<unsigned>(gx), 1), partial, out, bands, NW, bands);
+            st = check_launch("sum_t(axis=0) stage 2");
+        }
+        pool_free_raw(partial);   // a later owner of the block runs after this launch
+    }
+    return st;
+}
+
+// ============================ sum over axis 1 ==============================
+// Row sums. THREADS lanes cooperate on one row (64 = one wavefront, 4 rows per
+// workgroup; 256 = the whole workgroup). Lanes stride over the row, W floats
+// per access; a row tail that does not fill W floats is added scalar-wise.
+template <int W, bool AL, int THREADS>
+__global__ __launch_bounds__(kBlock) void rowsum_kernel(const float* __restrict__ a,
+                                                        float* __restrict__ out, int64_t M,
+                                                        int64_t N) {
+    constexpr int ROWS = kBlock / THREADS;
+    typedef typename VecT<W>::type R;
+    __shared__ float lds[kBlock / kWave];
+    const int t = threadIdx.x % THREADS;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / THREADS;
+    float total = 0.0f;
+    if (row < M) {
+        const int64_t NW = N / W;
+        const float* p = a + row * N;
+        R acc0 = vzero<R>(), acc1 = vzero<R>(), acc2 = vzero<R>(), acc3 = vzero<R>();
+        int64_t i = t;
+        for (; i + 3 * THREADS < NW; i += 4 * THREADS) {
+            R x0 = vload<W, AL>(p + i * W);
+            R x1 = vload<W, AL>(p + (i + THREADS) * W);
+            R x2 = vload<W, AL>(p + (i + 2 * THREADS) * W);
+            R x3 = vload<W, AL>(p + (i + 3 * THREADS) * W);
+            acc0 += x0; acc1 += x1; acc2 += x2; acc3 += x3;
+        }
+        for (; i < NW; i += THREADS) acc0 += vload<W, AL>(p + i * W);
+        total = hsum((acc0 + acc1) + (acc2 + acc3));
+        for (int64_t j = NW * W + t; j < N; j += THREADS) total += p[j];
+    }
+    total = wave_sum(total);
+    if (THREADS == kWave) {
+        if (t == 0 && row < M) out[row] = total;
+    } else {
+        const int wv = threadIdx.x / kWave;
+        if ((threadIdx.x & (kWave - 1)) == 0) lds[wv] = total;
+        __syncthreads();
+        if (threadIdx.x == 0 && row < M) out[row] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    }
+}
+
+// One thread per row, for very short rows.
+__global__ __launch_bounds__(kBlock) void rowsum_small_kernel(const float* __restrict__ a,
+                                                              float* __restrict__ out, int64_t M,
+                                                              int64_t N) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (row >= M) return;
+    float s = 0.0f;
+    for (int64_t j = 0; j < N; ++j) s += a[row * N + j];
+    out[row] = s;
+}
+
+template <int THREADS>
+static void launch_rowsum_kernel(bool vec, bool al, dim3 grid, const float* a, float* out,
+                                 int64_t M, int64_t N) {
+    hipStream_t s = ctx().stream;
+    if (vec && al) hipLaunchKernelGGL((rowsum_kernel<4, true, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
+    else if (vec)  hipLaunchKernelGGL((rowsum_kernel<4, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
+    else           hipLaunchKernelGGL((rowsum_kernel<1, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
+}
+
+static int launch_rowsum(const float* a, float* out, int64_t M, int64_t N) {
+    if (N <= 16) {
+        hipLaunchKernelGGL(rowsum_small_kernel, dim3(static_cast<unsigned>(ceil_div(M, kBlock))),
+                           dim3(kBlock), 0, ctx().stream, a, out, M, N);
+        return check_launch("sum_t(axis=1) small");
+    }
+    // every row starts on a 16-byte boundary only if N % 4 == 0 and the base does
+    const bool vec = (N % 4 == 0);
+    const bool al = aligned16(a);
+    if (N <= 2048)
+        launch_rowsum_kernel<kWave>(vec, al, dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), a, out, M, N);
+    else
+        launch_rowsum_kernel<kBlock>(vec, al, dim3(static_cast<unsigned>(M)), a, out, M, N);
+    return check_launch("sum_t(axis=1)");
+}
+
+// ============================== sum of all =================================
+// Stage 1: `chunks` workgroups each sum one contiguous chunk (a row of the
+// (chunks, len) view of the data) with the row-sum kernel; stage 2 sums the
+// partials with one workgroup.
+static int launch_sumall(const float* a, float* out, int64_t n) {
+    const Context& c = ctx();
+    const int64_t min_chunk = 16384;
+    int64_t chunks = static_cast<int64_t>(c.num_cus) * 8;
+    if (chunks > n / min_chunk) chunks = n / min_chunk;
+    if (chunks <= 1) {
+        // vector width 4 over the whole array; the kernel adds the n % 4 tail itself
+        launch_rowsum_kernel<kBlock>(true, aligned16(a), dim3(1), a, out, 1, n);
+        return check_launch("sum_t(axis=None)");
+    }
+    const int64_t len = (n / chunks) & ~int64_t(3);   // chunk starts keep the base alignment
+    const int64_t body = len * chunks;
+    const int64_t rest = n - body;                     // summed as one extra short row
+    void* p = nullptr;
+    int st = pool_alloc_raw(static_cast<size_t>(chunks + 1) * sizeof(float), &p);
+    if (st != 0) return st;
+    float* partial = static_cast<float*>(p);
+    launch_rowsum_kernel<kBlock>(true, aligned16(a), dim3(static_cast<unsigned>(chunks)), a, partial, chunks, len);
+    st = check_launch("sum_t(axis=None) stage 1");
+    int64_t np = chunks;
+    if (st == 0 && rest > 0) {
+        launch_rowsum_kernel<kBlock>(false, false, dim3(1), a + body, partial + chunks, 1, rest);
+        st = check_launch("sum_t(axis=None) tail");
+        np = chunks + 1;
+    }
+    if (st == 0) {
+        launch_rowsum_kernel<kBlock>(false, false, dim3(1), partial, out, 1, np);
+        st = check_launch("sum_t(axis=None) stage 2");
+    }
+    pool_free_raw(partial);
+    return st;
+}
+
+// ================================ softmax ==================================
+// One pass over HBM: THREADS lanes hold a whole row in registers (PER accesses
+// of W floats each), reduce max and sum across the lanes, then write e/sum.
+// out = exp(m - rowmax) / sum(exp(m - rowmax))      (numpy 292-295)
+// The launcher guarantees N % W == 0 and N / W <= THREADS * PER.
+template <int W, bool AL, int THREADS, int PER>
+__global__ __launch_bounds__(kBlock) void softmax_reg_kernel(const float* m, float* out, int64_t M,
+                                                             int64_t N) {
+    constexpr int ROWS = kBlock / THREADS;
+    typedef typename VecT<W>::type R;
+    __shared__ float lds[2][kBlock / kWave];
+    const int t = threadIdx.x % THREADS;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / THREADS;
+    const bool live = row < M;
+    const int64_t NW = N / W;
+    const float* p = m + (live ? row : 0) * N;
+    float* q = out + (live ? row : 0) * N;
+    R x[PER];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int64_t i = t + static_cast<int64_t>(k) * THREADS;
+        if (live && i < NW) {
+            x[k] = vload<W, AL>(p + i * W);
+            mx = fmaxf(mx, hmax(x[k]));
+        }
+    }
+    mx = wave_max(mx);
+    if (THREADS > kWave) {
+        if ((threadIdx.x & (kWave - 1)) == 0) lds[0][threadIdx.x / kWave] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(lds[0][0], lds[0][1]), fmaxf(lds[0][2], lds[0][3]));
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int64_t i = t + static_cast<int64_t>(k) * THREADS;
+        if (live && i < NW) {
+            if constexpr (W == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) x[k][j] = expf(x[k][j] - mx);
+            } else {
+                x[k] = expf(x[k] - mx);
+            }
+            sum += hsum(x[k]);
+        }
+    }
+    sum = wave_sum(sum);
+    if (THREADS > kWave) {
+        if ((threadIdx.x & (kWave - 1)) == 0) lds[1][threadIdx.x / kWave] = sum;
+        __syncthreads();
+        sum = (lds[1][0] + lds[1][1]) + (lds[1][2] + lds[1][3]);
+    }
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int64_t i = t + static_cast<int64_t>(k) * THREADS;
+        if (live && i < NW) {
+            R r;
+            if constexpr (W == 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r[j] = x[k][j] / sum;
+            } else {
+                r = x[k] / sum;
+            }
+            vstore<W, AL>(q + i * W, r);
+        }
+    }
+}
+
+// Rows too long for registers: a workgroup per row, three sweeps (max, sum of
+// exponentials, normalise); the second and third sweeps mostly hit the caches.
+__global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, float* out, int64_t M,
+                                                              int64_t N) {
+    __shared__ float lds[kBlock / kWave];
+    const int wv = threadIdx.x / kWave;
+    const int64_t row = blockIdx.x;
+    const float* p = m + row * N;
+    float* q = out + row * N;
+    float mx = -INFINITY;
+    for (int64_t i = threadIdx.x; i < N; i += kBlock) mx = fmaxf(mx, p[i]);
+    mx = wave_max(mx);
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[wv] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+    __syncthreads();
+    float sum = 0.0f;
+    for (int64_t i = threadIdx.x; i < N; i += kBlock) sum += expf(p[i] - mx);
+    sum = wave_sum(sum);
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[wv] = sum;
+    __syncthreads();
+    sum = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    for (int64_t i = threadIdx.x; i < N; i += kBlock) q[i] = expf(p[i] - mx) / sum;
+}
+
+template <int W, bool AL, int THREADS>
+static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N) {
+    hipStream_t s = ctx().stream;
+    const dim3 b(kBlock);
+    switch (per) {
+        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 1>), grid, b, 0, s, m, out, M, N); break;
+        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 2>), grid, b, 0, s, m, out, M, N); break;
+        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 4>), grid, b, 0, s, m, out, M, N); break;
+        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 8>), grid, b, 0, s, m, out, M, N); break;
+        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 16>), grid, b, 0, s, m, out, M, N); break;
+    }
+}
+
+template <int THREADS>
+static void launch_softmax_threads(bool vec, bool al, int per, dim3 grid, const float* m, float* out,
+                                   int64_t M, int64_t N) {
+    if (vec && al) launch_softmax_per<4, true, THREADS>(per, grid, m, out, M, N);
+    else if (vec)  launch_softmax_per<4, false, THREADS>(per, grid, m, out, M, N);
+    else           launch_softmax_per<1, false, THREADS>(per, grid, m, out, M, N);
+}
+
+static int launch_softmax(const float* m, float* out, int64_t M, int64_t N) {
+    const bool vec = (N % 4 == 0);
+    const bool al = aligned16(m) && aligned16(out);
+    const int64_t NW = vec ? N / 4 : N;
+    // smallest power-of-two number of accesses per lane that covers the row
+    auto per_for = [&](int threads) {
+        int per = 1;
+        while (per < 16 && static_cast<int64_t>(per) * threads < NW) per *= 2;
+        return per;
+    };
+    if (NW <= static_cast<int64_t>(kWave) * 16) {
+        launch_softmax_threads<kWave>(vec, al, per_for(kWave),
+                                      dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N);
+    } else if (NW <= static_cast<int64_t>(kBlock) * 16) {
+        launch_softmax_threads<kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N);
+    } else {
+        hipLaunchKernelGGL(softmax_long_kernel, dim3(static_cast<unsigned>(M)), dim3(kBlock), 0,
+                           ctx().stream, m, out, M, N);
+    }
+    return check_launch("softmax_m");
+}
+
+// ============================== is finite ==================================
+__global__ __launch_bounds__(kBlock) void nonfinite_kernel(const float* __restrict__ a, size_t n,
+                                                           int* __restrict__ flag) {
+    bool bad = false;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * kBlock) {
+        const uint32_t bits = __float_as_uint(a[i]);
+        bad |= ((bits & 0x7f800000u) == 0x7f800000u);
+    }
+    if (bad) *flag = 1;    // every writer stores the same value
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" {
+
+int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    BSHIP_REQUIRE_DIM(axis == 0 || axis == 1 || axis == -1);
+    const int64_t out_n = axis == 0 ? N : (axis == 1 ? M : 1);
+    if (out_n == 0) return 0;
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    if (M == 0 || N == 0) return launch_fill(out, 0.0f, static_cast<size_t>(out_n));  // empty sum
+    BSHIP_REQUIRE_PTR(a);
+    BSHIP_REQUIRE_F32_ALIGNED(a);
+    BSHIP_REQUIRE_DIM(a != out);
+    BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
+    if (axis == 0) return M == 1 ? bship_d2d(out, a, static_cast<size_t>(N) * 4) : launch_colsum(a, out, M, N);
+    if (axis == 1) return N == 1 ? bship_d2d(out, a, static_cast<size_t>(M) * 4) : launch_rowsum(a, out, M, N);
+    return launch_sumall(a, out, M * N);
+}
+
+int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    if (M == 0 || N == 0) return 0;
+    BSHIP_REQUIRE_PTR(m);
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(m);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
+    return launch_softmax(m, out, M, N);
+}
+
+int bship_isfinite_f32(const float* a, size_t n, int* result_host) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(result_host);
+    *result_host = 1;
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(a);
+    BSHIP_REQUIRE_F32_ALIGNED(a);
+    void* p = nullptr;
+    int st = bship_malloc(sizeof(int), &p);     // zero-filled
+    if (st != 0) return st;
+    hipLaunchKernelGGL(nonfinite_kernel,
+                       dim3(stream_grid(ceil_div(static_cast<int64_t>(n), kBlock * 4))),
+                       dim3(kBlock), 0, ctx().stream, a, n, static_cast<int*>(p));
+    st = check_launch("is_fully_finite");
+    int flag = 0;
+    if (st == 0) st = bship_d2h(&flag, p, sizeof(int));
+    bship_free(p);
+    if (st == 0) *result_host = flag ? 0 : 1;
+    return st;
+}
+
+}  // extern "C"

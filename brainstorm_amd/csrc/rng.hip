@@ -1,0 +1,383 @@
+// Device-resident MT19937 that reproduces numpy.random.RandomState bit for bit.
+//
+// The reference draws dropout masks from the handler's RandomState
+// (numpy_handler.py 199-200: rnd.uniform(size) < p). To give the same masks
+// the generator state (624 words + position + the cached gaussian of the legacy
+// polar method) lives in device memory and one workgroup advances it:
+//  - the twist of a 624-word block has only distance-1 and distance-397
+//    dependencies, so it is done in three data-parallel phases in LDS
+//    (words 0..226, 227..453, 454..623);
+//  - tempering and the 53-bit double construction
+//    ((a >> 5) * 2^26 + (b >> 6)) / 2^53 are element-parallel.
+// Nothing is copied to the host, so mask generation stays asynchronous.
+#include <mutex>
+
+#include "common.h"
+
+namespace bship {
+
+constexpr int kMtN = 624;
+constexpr int kMtM = 397;
+
+struct RngState {
+    uint32_t key[kMtN];
+    int32_t pos;          // next unread word of key; kMtN means "regenerate first"
+    int32_t has_gauss;    // legacy_gauss cache flag
+    double gauss;         // cached second variate of the polar method
+};
+
+static RngState* g_state = nullptr;   // device memory
+static std::mutex g_rng_mutex;
+
+__device__ __forceinline__ uint32_t mt_twist(uint32_t u, uint32_t v) {
+    const uint32_t y = (u & 0x80000000u) | (v & 0x7fffffffu);
+    return (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+}
+
+__device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
+    y ^= (y >> 11);
+    y ^= (y << 7) & 0x9d2c5680u;
+    y ^= (y << 15) & 0xefc60000u;
+    y ^= (y >> 18);
+    return y;
+}
+
+// Replaces the 624 words in `cur` by the next block, written to `nxt`.
+// Must be called by all kBlock threads of the workgroup.
+__device__ __forceinline__ void mt_next_block(const uint32_t* cur, uint32_t* nxt) {
+    const int t = threadIdx.x;
+    // phase 1: words 0..226 depend on old words only
+    if (t < kMtN - kMtM) nxt[t] = cur[t + kMtM] ^ mt_twist(cur[t], cur[t + 1]);
+    __syncthreads();
+    // phase 2: words 227..453 use new words 0..226
+    {
+        const int i = t + (kMtN - kMtM);
+        if (i < 2 * (kMtN - kMtM)) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], cur[i + 1]);
+    }
+    __syncthreads();
+    // phase 3: words 454..623 use new words 227..396; the last one wraps to new word 0
+    {
+        const int i = t + 2 * (kMtN - kMtM);
+        if (i < kMtN - 1) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], cur[i + 1]);
+        else if (i == kMtN - 1) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], nxt[0]);
+    }
+    __syncthreads();
+}
+static_assert(kBlock >= kMtN - kMtM, "one thread per word of a twist phase");
+
+// Word stream shared by the consumers below: LDS copy of the state, double
+// buffered, plus at most one tempered word carried over a block boundary when a
+// 53-bit double straddles it.
+struct MtStream {
+    uint32_t buf[2][kMtN];
+    uint32_t carry;
+};
+
+// mask[i] = (next_double() < p) ? 1 : 0 for i in [0,n). Single workgroup.
+__global__ __launch_bounds__(kBlock) void mt_mask_kernel(RngState* st, float* __restrict__ mask,
+                                                         size_t n, double p) {
+    __shared__ MtStream s;
+    int cur = 0;
+    for (int i = threadIdx.x; i < kMtN; i += kBlock) s.buf[0][i] = st->key[i];
+    int pos = st->pos;                 // same value in every thread
+    __syncthreads();
+    bool have_carry = false;
+    size_t done = 0;
+    while (done < n) {
+        if (pos >= kMtN) {
+            mt_next_block(s.buf[cur], s.buf[cur ^ 1]);
+            cur ^= 1;
+            pos = 0;
+        }
+        const uint32_t* key = s.buf[cur];
+        // logical word L of this round: the carried word (if any) followed by key[pos...]
+        const int avail = kMtN - pos + (have_carry ? 1 : 0);
+        size_t pairs = static_cast<size_t>(avail / 2);
+        const bool finishing = pairs >= n - done;
+        if (finishing) pairs = n - done;
+        for (size_t j = threadIdx.x; j < pairs; j += kBlock) {
+            const int l0 = static_cast<int>(2 * j);
+            uint32_t w0, w1;
+            if (have_carry) {
+                w0 = (l0 == 0) ? s.carry : mt_temper(key[pos + l0 - 1]);
+                w1 = mt_temper(key[pos + l0]);
+            } else {
+                w0 = mt_temper(key[pos + l0]);
+                w1 = mt_temper(key[pos + l0 + 1]);
+            }
+            const double r = (static_cast<double>(w0 >> 5) * 67108864.0 + static_cast<double>(w1 >> 6)) /
+                             9007199254740992.0;
+            mask[done + j] = (r < p) ? 1.0f : 0.0f;
+        }
+        const int used = static_cast<int>(2 * pairs) - (have_carry ? 1 : 0);   // words taken from key
+        __syncthreads();                       // everyone has read s.carry
+        pos += used;
+        done += pairs;
+        have_carry = false;
+        if (!finishing && pos == kMtN - 1) {   // odd word left: carry it into the next block
+            if (threadIdx.x == 0) s.carry = mt_temper(key[kMtN - 1]);
+            have_carry = true;
+            pos = kMtN;
+            __syncthreads();
+        }
+    }
+    for (int i = threadIdx.x; i < kMtN; i += kBlock) st->key[i] = s.buf[cur][i];
+    if (threadIdx.x == 0) st->pos = pos;
+}
+
+// Writes `count` raw doubles of the stream to `u` (used by fill_gaussian).
+// Single workgroup; same structure as the mask kernel.
+__global__ __launch_bounds__(kBlock) void mt_doubles_kernel(RngState* st, double* __restrict__ u,
+                                                            size_t n) {
+    __shared__ MtStream s;
+    int cur = 0;
+    for (int i = threadIdx.x; i < kMtN; i += kBlock) s.buf[0][i] = st->key[i];
+    int pos = st->pos;
+    __syncthreads();
+    bool have_carry = false;
+    size_t done = 0;
+    while (done < n) {
+        if (pos >= kMtN) {
+            mt_next_block(s.buf[cur], s.buf[cur ^ 1]);
+            cur ^= 1;
+            pos = 0;
+        }
+        const uint32_t* key = s.buf[cur];
+        const int avail = kMtN - pos + (have_carry ? 1 : 0);
+        size_t pairs = static_cast<size_t>(avail / 2);
+        const bool finishing = pairs >= n - done;
+        if (finishing) pairs = n - done;
+        for (size_t j = threadIdx.x; j < pairs; j += kBlock) {
+            const int l0 = static_cast<int>(2 * j);
+            uint32_t w0, w1;
+            if (have_carry) {
+                w0 = (l0 == 0) ? s.carry : mt_temper(key[pos + l0 - 1]);
+                w1 = mt_temper(key[pos + l0]);
+            } else {
+                w0 = mt_temper(key[pos + l0]);
+                w1 = mt_temper(key[pos + l0 + 1]);
+            }
+            u[done + j] = (static_cast<double>(w0 >> 5) * 67108864.0 + static_cast<double>(w1 >> 6)) /
+                          9007199254740992.0;
+        }
+        const int used = static_cast<int>(2 * pairs) - (have_carry ? 1 : 0);
+        __syncthreads();
+        pos += used;
+        done += pairs;
+        have_carry = false;
+        if (!finishing && pos == kMtN - 1) {
+            if (threadIdx.x == 0) s.carry = mt_temper(key[kMtN - 1]);
+            have_carry = true;
+            pos = kMtN;
+            __syncthreads();
+        }
+    }
+    for (int i = threadIdx.x; i < kMtN; i += kBlock) st->key[i] = s.buf[cur][i];
+    if (threadIdx.x == 0) st->pos = pos;
+}
+
+// Legacy polar method (RandomState.standard_normal): trial t uses doubles
+// u[2t], u[2t+1]; x1 = 2u0-1, x2 = 2u1-1, r2 = x1^2+x2^2; rejected if r2 >= 1 or
+// r2 == 0; an accepted trial yields f*x2 first and caches f*x1 for the next
+// call, f = sqrt(-2 ln(r2) / r2). One workgroup scans the trials in order and
+// compacts the accepted ones with a prefix sum, so output k comes from the
+// same trial as in the sequential algorithm.
+// result[0] = number of trials consumed, result[1] = outputs written.
+__global__ __launch_bounds__(kBlock) void gauss_polar_kernel(RngState* st, const double* __restrict__ u,
+                                                             size_t trials, float* __restrict__ out,
+                                                             size_t n, size_t start, double mean,
+                                                             double stdv, unsigned long long* result) {
+    __shared__ unsigned int counts[kBlock];
+    __shared__ size_t used_s;
+    size_t produced = start;          // outputs already written (from the cache or earlier chunks)
+    size_t t0 = 0;
+    if (threadIdx.x == 0) { used_s = 0; }
+    __syncthreads();
+    while (t0 < trials && produced < n) {
+        const size_t t = t0 + threadIdx.x;
+        double x1 = 0.0, x2 = 0.0, r2 = 2.0;
+        if (t < trials) {
+            x1 = 2.0 * u[2 * t] - 1.0;
+            x2 = 2.0 * u[2 * t + 1] - 1.0;
+            r2 = x1 * x1 + x2 * x2;
+        }
+        const bool acc = (t < trials) && !(r2 >= 1.0 || r2 == 0.0);
+        counts[threadIdx.x] = acc ? 1u : 0u;
+        __syncthreads();
+        // inclusive scan over the workgroup (Hillis-Steele; 8 steps)
+        for (int off = 1; off < kBlock; off <<= 1) {
+            unsigned int v = counts[threadIdx.x];
+            if (threadIdx.x >= static_cast<unsigned>(off)) v += counts[threadIdx.x - off];
+            __syncthreads();
+            counts[threadIdx.x] = v;
+            __syncthreads();
+        }
+        const unsigned int incl = counts[threadIdx.x];
+        const unsigned int total = counts[kBlock - 1];
+        if (acc) {
+            const size_t k = produced + 2 * static_cast<size_t>(incl - 1);   // index of first output
+            if (k < n) {
+                const double f = sqrt(-2.0 * log(r2) / r2);
+                out[k] = static_cast<float>(stdv * (f * x2) + mean);
+                if (k + 1 < n) {
+                    out[k + 1] = static_cast<float>(stdv * (f * x1) + mean);
+                } else {
+                    // the last output is the first of its pair: cache the second
+                    st->gauss = f * x1;
+                    st->has_gauss = 1;
+                }
+                // the trial that produced output n-1 or n-2 is the last one consumed
+                if (k + 2 >= n) used_s = t + 1;
+            }
+        }
+        __syncthreads();
+        produced += 2 * static_cast<size_t>(total);
+        t0 += kBlock;
+    }
+    if (threadIdx.x == 0) {
+        const bool complete = produced >= n;
+        result[0] = complete ? used_s : trials;
+        result[1] = complete ? n : produced;
+    }
+}
+
+// Emits the cached gaussian (if any) as output 0 and clears the cache flag.
+__global__ void gauss_cache_kernel(RngState* st, float* out, size_t n, double mean, double stdv,
+                                   unsigned long long* result) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        unsigned long long start = 0;
+        if (n > 0 && st->has_gauss) {
+            out[0] = static_cast<float>(stdv * st->gauss + mean);
+            st->has_gauss = 0;
+            st->gauss = 0.0;
+            start = 1;
+        }
+        result[2] = start;
+    }
+}
+
+// Copies the word stream position only (key and pos); the gaussian cache is left alone.
+__global__ void rng_copy_state_kernel(const RngState* src, RngState* dst) {
+    for (int i = threadIdx.x; i < kMtN; i += blockDim.x) dst->key[i] = src->key[i];
+    if (threadIdx.x == 0) { dst->pos = src->pos; }
+}
+
+void rng_release() {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (g_state) { pool_free_raw(g_state); g_state = nullptr; }
+}
+
+static int rng_ensure_state() {
+    if (g_state) return 0;
+    void* p = nullptr;
+    int st = pool_alloc_raw(sizeof(RngState), &p);
+    if (st != 0) return st;
+    g_state = static_cast<RngState*>(p);
+    return 0;
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" {
+
+int bship_rng_seed(uint32_t seed) {
+    BSHIP_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    int st = rng_ensure_state();
+    if (st != 0) return st;
+    // init_genrand of the MT19937 reference code, as used by RandomState(int)
+    RngState h;
+    h.key[0] = seed;
+    for (int i = 1; i < kMtN; ++i)
+        h.key[i] = 1812433253u * (h.key[i - 1] ^ (h.key[i - 1] >> 30)) + static_cast<uint32_t>(i);
+    h.pos = kMtN;
+    h.has_gauss = 0;
+    h.gauss = 0.0;
+    return bship_h2d(g_state, &h, sizeof(RngState));
+}
+
+int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) {
+    BSHIP_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_rng_get_state: bship_rng_seed() has not been called");
+    RngState h;
+    int st = bship_d2h(&h, g_state, sizeof(RngState));
+    if (st != 0) return st;
+    if (key_host) for (int i = 0; i < kMtN; ++i) key_host[i] = h.key[i];
+    if (pos_host) *pos_host = h.pos;
+    if (has_gauss_host) *has_gauss_host = h.has_gauss;
+    if (gauss_host) *gauss_host = h.gauss;
+    return 0;
+}
+
+int bship_prob_mask_f32(float* mask, size_t n, double p) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(mask);
+    BSHIP_REQUIRE_F32_ALIGNED(mask);
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_prob_mask_f32: bship_rng_seed() has not been called");
+    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kBlock), 0, ctx().stream, g_state, mask, n, p);
+    return check_launch("generate_probability_mask");
+}
+
+int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_fill_gaussian_f32: bship_rng_seed() has not been called");
+    hipStream_t s = ctx().stream;
+    // device scalars: [0] trials consumed, [1] outputs written, [2] outputs taken from the cache
+    void* rp = nullptr;
+    int st = pool_alloc_raw(3 * sizeof(unsigned long long), &rp);
+    if (st != 0) return st;
+    unsigned long long* result = static_cast<unsigned long long*>(rp);
+    void* snap_p = nullptr;
+    st = pool_alloc_raw(sizeof(RngState), &snap_p);
+    if (st != 0) { pool_free_raw(rp); return st; }
+    RngState* snap = static_cast<RngState*>(snap_p);
+
+    hipLaunchKernelGGL(gauss_cache_kernel, dim3(1), dim3(64), 0, s, g_state, out, n, mean, stdv, result);
+    st = check_launch("fill_gaussian cache");
+    unsigned long long host_res[3] = {0, 0, 0};
+    if (st == 0) st = bship_d2h(host_res, result, sizeof(host_res));
+    size_t produced = static_cast<size_t>(host_res[2]);
+    while (st == 0 && produced < n) {
+        // Acceptance rate is pi/4; draw a generous batch of trials, then rewind the
+        // generator to exactly the number of trials the sequential algorithm consumes.
+        const size_t need = (n - produced + 1) / 2;
+        const size_t trials = need + need / 2 + 1024;
+        void* up = nullptr;
+        st = pool_alloc_raw(2 * trials * sizeof(double), &up);
+        if (st != 0) break;
+        double* u = static_cast<double*>(up);
+        hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, s, g_state, snap);
+        hipLaunchKernelGGL(mt_doubles_kernel, dim3(1), dim3(kBlock), 0, s, g_state, u, 2 * trials);
+        hipLaunchKernelGGL(gauss_polar_kernel, dim3(1), dim3(kBlock), 0, s, g_state, u, trials, out, n,
+                           produced, mean, stdv, result);
+        st = check_launch("fill_gaussian");
+        if (st == 0) st = bship_d2h(host_res, result, sizeof(host_res));
+        if (st == 0) {
+            const size_t used = static_cast<size_t>(host_res[0]);
+            produced = static_cast<size_t>(host_res[1]);
+            if (used < trials) {
+                // rewind: restore the snapshot and skip exactly 2*used doubles
+                hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, s, snap, g_state);
+                if (used > 0)
+                    hipLaunchKernelGGL(mt_doubles_kernel, dim3(1), dim3(kBlock), 0, s, g_state, u, 2 * used);
+                st = check_launch("fill_gaussian rewind");
+            }
+        }
+        pool_free_raw(up);
+    }
+    pool_free_raw(snap_p);
+    pool_free_raw(rp);
+    if (st == 0) st = bship_sync();
+    return st;
+}
+
+}  // extern "C"

@@ -1,0 +1,183 @@
+"""DeviceArray: the array type HipHandler works on.
+
+A dense, C-contiguous float32 array in device memory, described by a raw device
+address and a shape. brainstorm's buffer manager allocates one flat array per
+network and carves every layer's inputs, outputs, parameters and internals out
+of it by slicing and reshaping (brainstorm/structure/buffers.py:79-83,
+buffer_structure.py:218-245), and the recurrent layers index time steps with
+negative integers (lstm_layer.py:117), so this type supports exactly that:
+integer / slice / tuple indexing (step 1 only), ``reshape``, zero-sized and
+0-d arrays -- all returning views that alias the parent. The minimal array
+contract is the one brainstorm's DebugArray states (debug_handler.py:12-35).
+
+Only views that stay dense are representable. A slice that would need a row
+pitch (e.g. ``a[:, 1:3]`` of a wider matrix) raises NotImplementedError.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+ITEMSIZE = 4
+
+
+class _Block:
+    """Owner of one pool block; returns it to the pool when the last view dies."""
+
+    __slots__ = ("ptr", "_free")
+
+    def __init__(self, ptr, free_fn):
+        self.ptr = ptr
+        self._free = free_fn
+
+    def __del__(self):
+        if self.ptr and self._free is not None:
+            try:
+                self._free(self.ptr)
+            except Exception:   # interpreter shutdown
+                pass
+            self.ptr = 0
+
+
+def _prod(shape):
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+class DeviceArray:
+    __slots__ = ("ptr", "shape", "size", "_owner", "_handler")
+
+    dtype = np.dtype(np.float32)
+
+    def __init__(self, ptr, shape, owner, handler=None):
+        self.ptr = ptr              # device address of element 0 (int; 0 for empty arrays)
+        self.shape = shape          # tuple of ints
+        self.size = _prod(shape)
+        self._owner = owner         # keeps the pool block alive
+        self._handler = handler     # for get()
+
+    # ---------------------------------------------------------------- basics
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def nbytes(self):
+        return self.size * ITEMSIZE
+
+    def __len__(self):
+        if not self.shape:
+            raise TypeError("len() of a 0-d array")
+        return self.shape[0]
+
+    def __repr__(self):
+        return "DeviceArray(shape=%r, ptr=0x%x)" % (self.shape, self.ptr or 0)
+
+    def get(self):
+        """NumPy copy of the contents (blocks until the device has caught up)."""
+        return self._handler.get_numpy_copy(self)
+
+    # --------------------------------------------------------------- reshape
+    def reshape(self, *new_shape):
+        if len(new_shape) == 1 and not isinstance(new_shape[0], (int, np.integer)):
+            new_shape = tuple(new_shape[0])
+        new_shape = tuple(int(s) for s in new_shape)
+        if -1 in new_shape:
+            if new_shape.count(-1) > 1:
+                raise ValueError("can only specify one unknown dimension")
+            known = _prod(s for s in new_shape if s != -1)
+            if known == 0 or self.size % known:
+                raise ValueError("cannot reshape array of size %d into shape %r"
+                                 % (self.size, new_shape))
+            new_shape = tuple(self.size // known if s == -1 else s for s in new_shape)
+        if any(s < 0 for s in new_shape) or _prod(new_shape) != self.size:
+            raise ValueError("cannot reshape array of size %d into shape %r"
+                             % (self.size, new_shape))
+        return DeviceArray(self.ptr, new_shape, self._owner, self._handler)
+
+    # -------------------------------------------------------------- indexing
+    def __getitem__(self, key):
+        shape = self.shape
+        # fast paths: a[i] and a[i:j] on the first axis (the recurrent layers' inner loop)
+        if type(key) is int:
+            if not shape:
+                raise IndexError("too many indices for a 0-d array")
+            n = shape[0]
+            if key < 0:
+                key += n
+            if not 0 <= key < n:
+                raise IndexError("index out of bounds for axis 0 with size %d" % n)
+            rest = shape[1:]
+            inner = self.size // n
+            return DeviceArray(self.ptr + key * inner * ITEMSIZE if self.ptr else 0, rest,
+                               self._owner, self._handler)
+        if type(key) is slice:
+            if not shape:
+                raise IndexError("too many indices for a 0-d array")
+            if key.step not in (None, 1):
+                raise NotImplementedError("DeviceArray slices must have step 1")
+            n = shape[0]
+            start, stop, _ = key.indices(n)
+            length = max(0, stop - start)
+            inner = self.size // n if n else _prod(shape[1:])
+            return DeviceArray(self.ptr + start * inner * ITEMSIZE if self.ptr else 0,
+                               (length,) + shape[1:], self._owner, self._handler)
+        return self._getitem_general(key)
+
+    def _getitem_general(self, key):
+        if not isinstance(key, tuple):
+            key = (key,)
+        shape = self.shape
+        if any(k is Ellipsis for k in key):
+            if sum(1 for k in key if k is Ellipsis) > 1:
+                raise IndexError("an index can only have a single ellipsis")
+            pos = next(i for i, k in enumerate(key) if k is Ellipsis)
+            fill = len(shape) - (len(key) - 1)
+            if fill < 0:
+                raise IndexError("too many indices for array")
+            key = key[:pos] + (slice(None),) * fill + key[pos + 1:]
+        if len(key) > len(shape):
+            raise IndexError("too many indices for array: array is %d-dimensional, "
+                             "but %d were indexed" % (len(shape), len(key)))
+        key = key + (slice(None),) * (len(shape) - len(key))
+        # element strides of the dense parent
+        strides = [0] * len(shape)
+        acc = 1
+        for ax in range(len(shape) - 1, -1, -1):
+            strides[ax] = acc
+            acc *= shape[ax]
+        offset = 0
+        new_shape, new_strides = [], []
+        for ax, k in enumerate(key):
+            n = shape[ax]
+            if isinstance(k, (int, np.integer)):
+                k = int(k)
+                if k < 0:
+                    k += n
+                if not 0 <= k < n:
+                    raise IndexError("index out of bounds for axis %d with size %d" % (ax, n))
+                offset += k * strides[ax]
+            elif isinstance(k, slice):
+                if k.step not in (None, 1):
+                    raise NotImplementedError("DeviceArray slices must have step 1")
+                start, stop, _ = k.indices(n)
+                length = max(0, stop - start)
+                if length:
+                    offset += start * strides[ax]
+                new_shape.append(length)
+                new_strides.append(strides[ax])
+            else:
+                raise IndexError("DeviceArray indices must be integers or slices, not %s"
+                                 % type(k).__name__)
+        new_shape = tuple(new_shape)
+        if _prod(new_shape) != 0:
+            expect = 1
+            for n, st in zip(reversed(new_shape), reversed(new_strides)):
+                if n != 1 and st != expect:
+                    raise NotImplementedError(
+                        "slicing %r out of shape %r needs a row pitch; DeviceArray views "
+                        "must stay dense" % (key, shape))
+                expect *= n
+        return DeviceArray(self.ptr + offset * ITEMSIZE if self.ptr else 0, new_shape,
+                           self._owner, self._handler)

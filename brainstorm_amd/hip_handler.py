@@ -1,0 +1,413 @@
+"""HipHandler: brainstorm's Handler interface on one MI355X.
+
+Every method forwards to one (sometimes two) C calls of libbship.so, which
+enqueue hand-written gfx950 kernels on the library's stream and return at
+once. Only ``get_numpy_copy``, ``set_from_numpy``/``create_from_numpy``,
+``is_fully_finite`` and ``fill_gaussian`` wait for the device.
+
+Semantics follow brainstorm's NumpyHandler (brainstorm/handlers/numpy_handler.py)
+operation by operation; the line of the reference each method mirrors is given
+next to it. The handler computes in float32 only, like the reference's GPU
+handler (pycuda_handler.py:31).
+"""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import (ABS, ADD, ADD_IF, ADD_ST, COPY_IF, DIV, EL, EL_DERIV, FILL_IF, FMOD, LOG, MUL,
+                   MULT_ADD_ST, MULT_ST, REL, REL_DERIV, SIGMOID, SIGMOID_DERIV, SIGN, SQRT, SUB,
+                   TANH, TANH_DERIV)
+from .device_array import DeviceArray, _Block, _prod
+from .handler_api import Handler
+
+SEED_RANGE = (0, 1000000000)   # brainstorm/randomness.py:16
+
+
+class HipRandomState:
+    """The handler's random state: an MT19937 stream kept in device memory.
+
+    Mirrors the seed bookkeeping of brainstorm.randomness.RandomState
+    (randomness.py:10-64): it remembers its seed, can be re-seeded and reset.
+    The stream equals numpy.random.RandomState(seed)'s, so masks drawn here
+    equal the ones NumpyHandler draws from the same seed.
+    """
+
+    def __init__(self, handler, seed=None):
+        self._handler = handler
+        if seed is None:
+            seed = int(np.random.randint(*SEED_RANGE))
+        self.seed(seed)
+
+    def seed(self, seed=None):
+        if seed is None:
+            seed = int(np.random.randint(*SEED_RANGE))
+        seed = int(seed)
+        if not 0 <= seed < 2 ** 32:
+            raise ValueError("seed must be between 0 and 2**32 - 1")
+        self._handler._call(self._handler._lib.bship_rng_seed(seed))
+        self._seed = seed
+
+    def get_seed(self):
+        return self._seed
+
+    def set_seed(self, seed):
+        self.seed(seed)
+
+    def reset(self):
+        self.seed(self._seed)
+
+    def get_state(self):
+        """('MT19937', key, pos, has_gauss, cached_gaussian) like RandomState.get_state()."""
+        key = (ctypes.c_uint32 * 624)()
+        pos, has_gauss, gauss = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
+        h = self._handler
+        h._call(h._lib.bship_rng_get_state(key, ctypes.byref(pos), ctypes.byref(has_gauss),
+                                           ctypes.byref(gauss)))
+        return ('MT19937', np.frombuffer(key, dtype=np.uint32).copy(), pos.value,
+                has_gauss.value, gauss.value)
+
+
+class HipHandler(Handler):
+    __undescribed__ = {'context', 'dtype', 'EMPTY', 'rnd'}
+
+    array_type = DeviceArray
+
+    def __init__(self, seed=None, device=0):
+        super(HipHandler, self).__init__()
+        self._lib = _lib.load()
+        self._call(self._lib.bship_init(int(device)))
+        self.dtype = np.float32
+        self.device = int(device)
+        self.context = self._lib
+        self._free = self._lib.bship_free
+        self.EMPTY = DeviceArray(0, (0,), None, self)
+        self.rnd = HipRandomState(self, seed)
+
+    def __describe__(self):
+        return {'@type': self.__class__.__name__}
+
+    def __init_from_description__(self, description):
+        self.__init__()
+
+    # ------------------------------------------------------------- plumbing
+    def _call(self, status):
+        if status:
+            _lib.raise_for_status(self._lib, status)
+
+    def synchronize(self):
+        """Waits until every operation issued so far has finished."""
+        self._call(self._lib.bship_sync())
+
+    def device_info(self):
+        name = ctypes.create_string_buffer(256)
+        cus = ctypes.c_int()
+        self._call(self._lib.bship_device_info(name, 256, ctypes.byref(cus)))
+        return name.value.decode(), cus.value
+
+    # ------------------------------------------------- allocate new memory
+    def allocate(self, shape):
+        # numpy 36-37 / pycuda 70-71: "allocate" hands out zeros
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        shape = tuple(int(s) for s in shape)
+        n = _prod(shape)
+        if n == 0:
+            return DeviceArray(0, shape, None, self)
+        p = ctypes.c_void_p()
+        self._call(self._lib.bship_malloc(n * 4, ctypes.byref(p)))
+        return DeviceArray(p.value, shape, _Block(p.value, self._free), self)
+
+    def zeros(self, shape):
+        return self.allocate(shape)
+
+    def ones(self, shape):
+        a = self.allocate(shape)
+        self.fill(a, 1.0)
+        return a
+
+    # --------------------------------------------------------- copy and fill
+    def copy_to(self, src, dest):
+        # numpy 47-52 / pycuda 83-85
+        if src.size != dest.size:
+            raise ValueError("copy_to: size mismatch %r -> %r" % (src.shape, dest.shape))
+        self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
+
+    def copy_to_if(self, src, dest, cond):
+        self._call(self._lib.bship_cond_f32(COPY_IF, src.ptr, 0.0, dest.ptr, cond.ptr, dest.size))
+
+    def create_from_numpy(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        out = self.allocate(arr.shape)
+        if out.size:
+            self._call(self._lib.bship_h2d(out.ptr, arr.ctypes.data, arr.nbytes))
+        return out
+
+    def fill(self, mem, val):
+        self._call(self._lib.bship_fill_f32(mem.ptr, val, mem.size))
+
+    def fill_if(self, mem, val, cond):
+        self._call(self._lib.bship_cond_f32(FILL_IF, None, val, mem.ptr, cond.ptr, mem.size))
+
+    def get_numpy_copy(self, mem):
+        assert type(mem) == self.array_type
+        out = np.empty(mem.shape, dtype=np.float32)
+        if mem.size:
+            self._call(self._lib.bship_d2h(out.ctypes.data, mem.ptr, mem.size * 4))
+        return out
+
+    def set_from_numpy(self, mem, arr):
+        # numpy 64-65: mem[:] = arr.astype(dtype), which broadcasts
+        arr = np.asarray(arr)
+        if arr.shape != mem.shape:
+            arr = np.broadcast_to(arr, mem.shape)
+        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        if mem.size:
+            self._call(self._lib.bship_h2d(mem.ptr, arr.ctypes.data, arr.nbytes))
+
+    # --------------------------------------------------------- debug helper
+    def is_fully_finite(self, a):
+        res = ctypes.c_int(1)
+        self._call(self._lib.bship_isfinite_f32(a.ptr, a.size, ctypes.byref(res)))
+        return bool(res.value)
+
+    # ------------------------------------------------ elementwise operations
+    def abs_t(self, a, out):
+        self._call(self._lib.bship_unary_f32(ABS, a.ptr, out.ptr, out.size))
+
+    def add_into_if(self, a, out, cond):
+        self._call(self._lib.bship_cond_f32(ADD_IF, a.ptr, 0.0, out.ptr, cond.ptr, out.size))
+
+    def add_st(self, s, t, out):
+        self._call(self._lib.bship_scalar_f32(ADD_ST, s, t.ptr, out.ptr, out.size))
+
+    def add_tt(self, a, b, out):
+        self._call(self._lib.bship_binary_f32(ADD, a.ptr, b.ptr, out.ptr, out.size))
+
+    def clip_t(self, a, a_min, a_max, out):
+        self._call(self._lib.bship_clip_f32(a.ptr, a_min, a_max, out.ptr, out.size))
+
+    def divide_tt(self, a, b, out):
+        self._call(self._lib.bship_binary_f32(DIV, a.ptr, b.ptr, out.ptr, out.size))
+
+    def log_t(self, a, out):
+        self._call(self._lib.bship_unary_f32(LOG, a.ptr, out.ptr, out.size))
+
+    def modulo_tt(self, a, b, out):
+        self._call(self._lib.bship_binary_f32(FMOD, a.ptr, b.ptr, out.ptr, out.size))
+
+    def mult_add_st(self, s, t, out):
+        self._call(self._lib.bship_scalar_f32(MULT_ADD_ST, s, t.ptr, out.ptr, out.size))
+
+    def mult_add_tt(self, a, b, out):
+        self._call(self._lib.bship_mult_add_tt_f32(a.ptr, b.ptr, out.ptr, out.size))
+
+    def mult_st(self, s, t, out):
+        self._call(self._lib.bship_scalar_f32(MULT_ST, s, t.ptr, out.ptr, out.size))
+
+    def mult_tt(self, a, b, out):
+        self._call(self._lib.bship_binary_f32(MUL, a.ptr, b.ptr, out.ptr, out.size))
+
+    def sign_t(self, a, out):
+        self._call(self._lib.bship_unary_f32(SIGN, a.ptr, out.ptr, out.size))
+
+    def sqrt_t(self, a, out):
+        self._call(self._lib.bship_unary_f32(SQRT, a.ptr, out.ptr, out.size))
+
+    def subtract_tt(self, a, b, out):
+        assert a.shape == b.shape == out.shape     # numpy 265
+        self._call(self._lib.bship_binary_f32(SUB, a.ptr, b.ptr, out.ptr, out.size))
+
+    # -------------------------------------------------- broadcast operations
+    def _mv(self, op, m, v, out, accumulate):
+        """out (+)= m (op) v with v a row vector (1,N)/(N,) or a column vector (M,1)."""
+        if v.shape == m.shape:
+            if accumulate:
+                assert op == MUL
+                return self._call(self._lib.bship_mult_add_tt_f32(m.ptr, v.ptr, out.ptr, out.size))
+            return self._call(self._lib.bship_binary_f32(op, m.ptr, v.ptr, out.ptr, out.size))
+        n_cols = m.shape[-1] if m.shape else 1
+        n_rows = m.size // n_cols if n_cols else 0
+        vs = v.shape
+        if v.size == n_cols and (len(vs) == 1 or vs[0] == 1 or n_rows == 1):
+            is_col = 0
+        elif v.size == n_rows and vs[-1] == 1:
+            is_col = 1
+        else:
+            raise ValueError("cannot broadcast vector of shape %r against matrix of shape %r"
+                             % (vs, m.shape))
+        self._call(self._lib.bship_mv_f32(op, m.ptr, v.ptr, out.ptr, n_rows, n_cols, is_col,
+                                          accumulate))
+
+    def add_mv(self, m, v, out):
+        self._mv(ADD, m, v, out, 0)
+
+    def subtract_mv(self, m, v, out):
+        self._mv(SUB, m, v, out, 0)
+
+    def mult_mv(self, m, v, out):
+        self._mv(MUL, m, v, out, 0)
+
+    def divide_mv(self, m, v, out):
+        self._mv(DIV, m, v, out, 0)
+
+    def mult_add_mv(self, m, v, out):
+        # numpy 239-240; not declared by the abstract class but called by the LSTM layers
+        self._mv(MUL, m, v, out, 1)
+
+    def broadcast_t(self, a, axis, out):
+        # numpy 103-105
+        assert (out.shape[:axis] + (1,) + out.shape[axis + 1:]) == a.shape
+        outer = _prod(out.shape[:axis])
+        inner = _prod(out.shape[axis + 1:])
+        self._call(self._lib.bship_broadcast_f32(a.ptr, out.ptr, outer, out.shape[axis], inner))
+
+    def merge_tt(self, a, b, out):
+        # numpy 221-225
+        na, nb = a.shape[-1], b.shape[-1]
+        assert na + nb == out.shape[-1]
+        rows = out.size // out.shape[-1] if out.shape[-1] else 0
+        self._call(self._lib.bship_merge_f32(a.ptr, b.ptr, out.ptr, rows, na, nb))
+
+    def split_add_tt(self, x, out_a, out_b):
+        # numpy 251-256
+        na, nb = out_a.shape[-1], out_b.shape[-1]
+        assert na + nb == x.shape[-1]
+        rows = x.size // x.shape[-1] if x.shape[-1] else 0
+        self._call(self._lib.bship_split_add_f32(x.ptr, out_a.ptr, out_b.ptr, rows, na, nb))
+
+    # ------------------------------------------------------------ reductions
+    def sum_t(self, a, axis, out):
+        # numpy 268-273; the shape of `out` decides keepdims, which does not change the layout
+        if axis is None or a.ndim <= 1:
+            rows, cols, ax = 1, a.size, -1
+        elif a.ndim == 2 and axis in (0, 1):
+            rows, cols = a.shape
+            ax = axis
+        else:
+            raise NotImplementedError("sum_t over axis %r of a %d-d array" % (axis, a.ndim))
+        self._call(self._lib.bship_sum_f32(a.ptr, out.ptr, rows, cols, ax))
+
+    def softmax_m(self, m, out):
+        n_cols = m.shape[-1]
+        self._call(self._lib.bship_softmax_rows_f32(m.ptr, out.ptr, m.size // n_cols if n_cols else 0,
+                                                    n_cols))
+
+    # -------------------------------------------------------------- indexing
+    def binarize_v(self, v, out):
+        self._call(self._lib.bship_binarize_f32(v.ptr, out.ptr, out.shape[0], out.shape[1]))
+
+    def index_m_by_v(self, m, v, out):
+        self._call(self._lib.bship_index_m_by_v_f32(m.ptr, v.ptr, out.ptr, m.shape[0], m.shape[1]))
+
+    # ------------------------------------------------------------------- RNG
+    def fill_gaussian(self, mean, std, out):
+        self._call(self._lib.bship_fill_gaussian_f32(out.ptr, out.size, mean, std))
+
+    def generate_probability_mask(self, mask, probability):
+        self._call(self._lib.bship_prob_mask_f32(mask.ptr, mask.size, probability))
+
+    # ------------------------------------------------------- dense products
+    def _gemm(self, a, b, out, transa, transb, beta):
+        m, k = (a.shape[1], a.shape[0]) if transa else a.shape
+        kb, n = (b.shape[1], b.shape[0]) if transb else b.shape
+        if k != kb or out.shape != (m, n):
+            raise ValueError("shapes %r%s . %r%s -> %r do not match"
+                             % (a.shape, "^T" if transa else "", b.shape, "^T" if transb else "",
+                                out.shape))
+        self._call(self._lib.bship_gemm_f32(int(bool(transa)), int(bool(transb)), m, n, k, 1.0,
+                                            a.ptr, a.shape[1], b.ptr, b.shape[1], beta,
+                                            out.ptr, n))
+
+    def dot_mm(self, a, b, out, transa=False, transb=False):
+        self._gemm(a, b, out, transa, transb, 0.0)
+
+    def dot_add_mm(self, a, b, out, transa=False, transb=False):
+        self._gemm(a, b, out, transa, transb, 1.0)
+
+    def conv2d_forward_batch(self, inputs, weights, bias, outputs, padding, stride):
+        # numpy 149-171, with the per-image loop folded into one im2col and one product:
+        # col (N*oh*ow, kh*kw*C) . W(F, kh*kw*C)^T -> outputs (N*oh*ow, F), then + bias
+        n, h, w, c = inputs.shape
+        f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
+        oh, ow = outputs.shape[1], outputs.shape[2]
+        kc = kh * kw * c
+        rows = n * oh * ow
+        col = self.allocate((rows, kc))
+        self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
+                                                   padding, stride[0], stride[1]))
+        out2d = outputs.reshape((rows, f))
+        self._gemm(col, weights.reshape((f, kc)), out2d, False, True, 0.0)
+        self._mv(ADD, out2d, bias.reshape((1, f)), out2d, 0)
+
+    def conv2d_backward_batch(self, inputs, weights, padding, stride, in_deltas, out_deltas,
+                              weight_deltas, bias_deltas):
+        # numpy 110-147: weight_deltas and bias_deltas are overwritten, in_deltas accumulated
+        n, h, w, c = inputs.shape
+        f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
+        oh, ow = out_deltas.shape[1], out_deltas.shape[2]
+        kc = kh * kw * c
+        rows = n * oh * ow
+        col = self.allocate((rows, kc))
+        self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
+                                                   padding, stride[0], stride[1]))
+        dy = out_deltas.reshape((rows, f))
+        self._gemm(dy, col, weight_deltas.reshape((f, kc)), True, False, 0.0)
+        self._call(self._lib.bship_sum_f32(dy.ptr, bias_deltas.ptr, rows, f, 0))
+        self._gemm(dy, weights.reshape((f, kc)), col, False, False, 0.0)
+        self._call(self._lib.bship_col2im_nhwc_f32(col.ptr, in_deltas.ptr, n, h, w, c, kh, kw,
+                                                   padding, stride[0], stride[1]))
+
+    # --------------------------------------------------------------- pooling
+    def maxpool2d_forward_batch(self, inputs, window, outputs, padding, stride, argmax):
+        n, h, w, c = inputs.shape
+        self._call(self._lib.bship_maxpool_fwd_nhwc_f32(
+            inputs.ptr, outputs.ptr, argmax.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
+            window[0], window[1], padding, stride[0], stride[1]))
+
+    def maxpool2d_backward_batch(self, inputs, window, outputs, padding, stride, argmax,
+                                 in_deltas, out_deltas):
+        n, h, w, c = inputs.shape
+        self._call(self._lib.bship_maxpool_bwd_nhwc_f32(
+            argmax.ptr, out_deltas.ptr, in_deltas.ptr, n, h, w, c, outputs.shape[1],
+            outputs.shape[2], window[0], window[1], padding, stride[0], stride[1]))
+
+    def avgpool2d_forward_batch(self, inputs, window, outputs, padding, stride):
+        n, h, w, c = inputs.shape
+        self._call(self._lib.bship_avgpool_fwd_nhwc_f32(
+            inputs.ptr, outputs.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
+            window[0], window[1], padding, stride[0], stride[1]))
+
+    def avgpool2d_backward_batch(self, inputs, window, outputs, padding, stride, in_deltas,
+                                 out_deltas):
+        n, h, w, c = inputs.shape
+        self._call(self._lib.bship_avgpool_bwd_nhwc_f32(
+            out_deltas.ptr, in_deltas.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
+            window[0], window[1], padding, stride[0], stride[1]))
+
+    # -------------------------------------------------- activation functions
+    def rel(self, x, y):
+        self._call(self._lib.bship_unary_f32(REL, x.ptr, y.ptr, y.size))
+
+    def rel_deriv(self, x, y, dy, dx):
+        self._call(self._lib.bship_deriv_f32(REL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+
+    def sigmoid(self, x, y):
+        self._call(self._lib.bship_unary_f32(SIGMOID, x.ptr, y.ptr, y.size))
+
+    def sigmoid_deriv(self, x, y, dy, dx):
+        self._call(self._lib.bship_deriv_f32(SIGMOID_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+
+    def tanh(self, x, y):
+        self._call(self._lib.bship_unary_f32(TANH, x.ptr, y.ptr, y.size))
+
+    def tanh_deriv(self, x, y, dy, dx):
+        self._call(self._lib.bship_deriv_f32(TANH_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+
+    def el(self, x, y):
+        self._call(self._lib.bship_unary_f32(EL, x.ptr, y.ptr, y.size))
+
+    def el_deriv(self, x, y, dy, dx):
+        self._call(self._lib.bship_deriv_f32(EL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))

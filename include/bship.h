@@ -1,0 +1,256 @@
+/*
+ * bship.h - C ABI of libbship.so, the MI355X (gfx950) compute back end behind
+ * brainstorm's Handler interface.
+ *
+ * Every entry point is what a ctypes/cffi binding of the reference's handler
+ * would bind for one handler operation; the comment above each declaration
+ * names the reference method it stands in for
+ * (brainstorm/handlers/numpy_handler.py = "numpy", pycuda_handler.py = "pycuda",
+ * base_handler.py = "base", _cpuop.pyx = "_cpuop").
+ *
+ * Conventions
+ *  - extern "C", C99 types only, no exceptions cross the boundary.
+ *  - Every function returns an int status: 0 = OK, > 0 = a hipError_t,
+ *    < 0 = one of the BSHIP_ERR_* argument/state errors below. The message of
+ *    the last failure on the calling thread is returned by bship_last_error().
+ *  - Pointers named float* / void* are raw DEVICE addresses (already offset to
+ *    the first element of the view) unless the parameter is called `host`.
+ *    All arrays are dense, C-contiguous float32. Only 4-byte alignment is
+ *    required; 16-byte aligned pointers take the fastest kernels.
+ *  - An output may be the same array as an input for every elementwise and
+ *    broadcast operation (in-place use); partial overlap is not supported.
+ *  - All work is enqueued, in call order, on one stream owned by the library.
+ *    Calls return without waiting unless stated ("blocks").
+ *  - Zero-sized arrays (n == 0, M == 0 ...) are legal and do nothing.
+ */
+#ifndef BSHIP_H
+#define BSHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BSHIP_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* argument / state errors (negative so they never collide with hipError_t) */
+#define BSHIP_ERR_NOT_INITIALIZED (-1)
+#define BSHIP_ERR_NULL_POINTER    (-2)
+#define BSHIP_ERR_BAD_DIMENSION   (-3)
+#define BSHIP_ERR_BAD_OP          (-4)
+#define BSHIP_ERR_OUT_OF_MEMORY   (-5)
+#define BSHIP_ERR_UNSUPPORTED     (-6)
+#define BSHIP_ERR_BAD_POINTER     (-7)
+#define BSHIP_ERR_BLAS            (-8)
+
+/* ------------------------------ lifecycle -------------------------------- */
+
+/* Selects the device, creates the stream and the memory pool. Idempotent for
+ * the same device. Replaces `import pycuda.autoinit` + culinalg.init()
+ * (pycuda 18; brainstorm/optional.py 32). */
+int bship_init(int device);
+/* Frees every pool block and destroys the stream. Blocks. */
+int bship_shutdown(void);
+/* Waits for all enqueued work. Blocks. */
+int bship_sync(void);
+int bship_version(void);
+/* Message of the last failed call on this thread ("" if none). The string is
+ * owned by the library and valid until the next failing call on the thread. */
+const char* bship_last_error(void);
+/* Device name and compute-unit count of the initialised device. */
+int bship_device_info(char* name_host, size_t name_len, int* compute_units);
+
+/* Timing on the library's stream (hipEvent pair); used to measure kernels
+ * where they actually run. start/stop enqueue events, elapsed blocks. */
+int bship_timer_start(void);
+int bship_timer_stop(void);
+int bship_timer_elapsed_ms(float* ms_host);
+
+/* ------------------------------- memory ---------------------------------- */
+
+/* allocate/zeros (numpy 36-43, pycuda 70-79): a block of at least `nbytes`
+ * from the caching pool, 256-byte aligned and ZERO-FILLED (both reference
+ * handlers return zeros from allocate, and lstm_layer.py 167/258 depends on
+ * it). nbytes == 0 yields *out = NULL and status 0. */
+int bship_malloc(size_t nbytes, void** out);
+/* Returns a block to the pool cache (no hipFree). NULL is a no-op. */
+int bship_free(void* p);
+/* hipFree()s every cached (unused) block. Blocks. */
+int bship_pool_trim(void);
+int bship_pool_stats(size_t* bytes_in_use, size_t* bytes_cached,
+                     size_t* device_allocations);
+
+/* set_from_numpy / create_from_numpy (numpy 54-65, pycuda 90-107). Blocks
+ * until the host buffer may be reused. */
+int bship_h2d(void* dst, const void* src_host, size_t nbytes);
+/* get_numpy_copy (numpy 60-62, pycuda 99-101). Blocks. */
+int bship_d2h(void* dst_host, const void* src, size_t nbytes);
+/* copy_to (numpy 47-52, pycuda 83-85). */
+int bship_d2d(void* dst, const void* src, size_t nbytes);
+/* fill (numpy 57-58, pycuda 93-94). */
+int bship_fill_f32(float* mem, float val, size_t n);
+
+/* ----------------------------- elementwise ------------------------------- */
+
+enum {
+    BSHIP_ADD = 0,  /* add_tt       numpy 86-87   pycuda 130-131 */
+    BSHIP_SUB = 1,  /* subtract_tt  numpy 264-266 pycuda 372-373 */
+    BSHIP_MUL = 2,  /* mult_tt      numpy 245-246 pycuda 351-352 */
+    BSHIP_DIV = 3,  /* divide_tt    numpy 190-191 pycuda 272-273 */
+    BSHIP_FMOD = 4  /* modulo_tt    numpy 227-228 (np.fmod: sign of dividend) */
+};
+/* out = a (op) b */
+int bship_binary_f32(int op, const float* a, const float* b, float* out, size_t n);
+
+/* mult_add_tt (numpy 233-234, pycuda 331-332): out += a*b, the product rounded
+ * to float32 before the add exactly as NumPy evaluates it (no fused multiply-add). */
+int bship_mult_add_tt_f32(const float* a, const float* b, float* out, size_t n);
+
+enum {
+    BSHIP_ADD_ST = 0,      /* add_st       numpy 83-84   : out = t + s   */
+    BSHIP_MULT_ST = 1,     /* mult_st      numpy 242-243 : out = s * t   */
+    BSHIP_MULT_ADD_ST = 2  /* mult_add_st  numpy 230-231 : out += s * t  */
+};
+/* The Python float scalar is rounded to float32 first, which is what NumPy
+ * does for a float32 array combined with a Python scalar. */
+int bship_scalar_f32(int op, float s, const float* t, float* out, size_t n);
+
+enum {
+    BSHIP_ABS = 0,     /* abs_t   numpy 74-75   */
+    BSHIP_SIGN = 1,    /* sign_t  numpy 248-249 */
+    BSHIP_SQRT = 2,    /* sqrt_t  numpy 258-259 */
+    BSHIP_LOG = 3,     /* log_t   numpy 207-208 */
+    BSHIP_SIGMOID = 4, /* sigmoid numpy 283-287 */
+    BSHIP_TANH = 5,    /* tanh    numpy 297-298 */
+    BSHIP_REL = 6,     /* rel     numpy 277-278 : x*(x>0), negatives give -0.0 */
+    BSHIP_EL = 7       /* el      numpy 303-305 */
+};
+int bship_unary_f32(int op, const float* x, float* y, size_t n);
+
+enum {
+    BSHIP_SIGMOID_DERIV = 0, /* numpy 289-290 : dx = (dy*y)*(1-y)          */
+    BSHIP_TANH_DERIV = 1,    /* numpy 300-301 : dx = dy*(1-y*y)            */
+    BSHIP_REL_DERIV = 2,     /* numpy 280-281 : dx = dy*(y>0)              */
+    BSHIP_EL_DERIV = 3       /* numpy 307-309 : dx = dy*(y>=0)+dy*(y+1)*(y<0) */
+};
+/* The reference never reads `x` in a derivative, so it is not passed. */
+int bship_deriv_f32(int op, const float* y, const float* dy, float* dx, size_t n);
+
+/* clip_t (numpy 107-108, pycuda 171-172) */
+int bship_clip_f32(const float* a, float lo, float hi, float* out, size_t n);
+
+enum {
+    BSHIP_COPY_IF = 0, /* copy_to_if  numpy 173-174 : if cond!=0: out = a    */
+    BSHIP_FILL_IF = 1, /* fill_if     numpy 196-197 : if cond!=0: out = val  */
+    BSHIP_ADD_IF = 2   /* add_into_if numpy 77-78   : if cond!=0: out += a   */
+};
+/* `a` is ignored for FILL_IF, `val` for the other two. */
+int bship_cond_f32(int op, const float* a, float val, float* out,
+                   const float* cond, size_t n);
+
+/* ------------------------------ broadcast -------------------------------- */
+
+/* add_mv / subtract_mv / mult_mv / divide_mv (numpy 80-81, 261-262, 236-237,
+ * 187-188; pycuda 124-125, 369-370, 334-338, 269-270) and mult_add_mv
+ * (numpy 239-240): m is (M,N); v is (1,N) when v_is_col == 0, (M,1) otherwise.
+ * op is BSHIP_ADD/SUB/MUL/DIV. accumulate != 0 computes out += m (op) v. */
+int bship_mv_f32(int op, const float* m, const float* v, float* out,
+                 int64_t M, int64_t N, int v_is_col, int accumulate);
+
+/* broadcast_t (numpy 103-105, pycuda 166-169): a has shape (outer,1,inner),
+ * out has shape (outer,bdim,inner). */
+int bship_broadcast_f32(const float* a, float* out, int64_t outer,
+                        int64_t bdim, int64_t inner);
+
+/* merge_tt (numpy 221-225, pycuda 317-323): out[:, :na] = a, out[:, na:] = b */
+int bship_merge_f32(const float* a, const float* b, float* out, int64_t rows,
+                    int64_t na, int64_t nb);
+/* split_add_tt (numpy 251-256, pycuda 357-364): oa += x[:, :na]; ob += x[:, na:] */
+int bship_split_add_f32(const float* x, float* oa, float* ob, int64_t rows,
+                        int64_t na, int64_t nb);
+
+/* ------------------------------ reductions ------------------------------- */
+
+/* sum_t (numpy 268-273, pycuda 375-381) of a (M,N): axis 0 -> out[N],
+ * axis 1 -> out[M], axis -1 (None) -> out[1]. Deterministic (no float atomics). */
+int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis);
+/* softmax_m (numpy 292-295, pycuda 403-408): row-wise, one pass over HBM. */
+int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N);
+/* is_fully_finite (numpy 69-70, pycuda 111-114). *result_host = 1 if every
+ * element is finite. Blocks. */
+int bship_isfinite_f32(const float* a, size_t n, int* result_host);
+
+/* ------------------------------- indexing -------------------------------- */
+
+/* binarize_v (numpy 99-101, pycuda 163-164): out[i,j] = (j == (int)v[i]) */
+int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K);
+/* index_m_by_v (numpy 202-203, pycuda 284-285): out[i] = m[i, (int)v[i]].
+ * Labels outside [0,K) are undefined in the reference; here they read as 0. */
+int bship_index_m_by_v_f32(const float* m, const float* v, float* out,
+                           int64_t M, int64_t K);
+
+/* --------------------------------- RNG ----------------------------------- */
+
+/* Seeds the device-resident MT19937 state the way
+ * numpy.random.RandomState(seed) does (randomness.py 66-80, numpy 21). Blocks. */
+int bship_rng_seed(uint32_t seed);
+/* generate_probability_mask (numpy 199-200): mask = (uniform[0,1) < p), drawing
+ * the same 53-bit doubles, in the same order, as RandomState.uniform. */
+int bship_prob_mask_f32(float* mask, size_t n, double p);
+/* fill_gaussian (numpy 193-194): out = std*standard_normal + mean with the
+ * legacy polar method of RandomState.standard_normal. Blocks. */
+int bship_fill_gaussian_f32(float* out, size_t n, double mean, double std);
+/* Copies the 624 state words, position, has_gauss flag and cached gaussian to
+ * the host (for tests and for saving the stream position). Blocks. */
+int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host,
+                        double* gauss_host);
+
+/* -------------------------------- dense ---------------------------------- */
+
+/* dot_mm / dot_add_mm (numpy 176-185, pycuda 259-267): row-major
+ * C(MxN) = alpha * op(A) * op(B) + beta * C through hipBLASLt.
+ * op(A) is MxK: A is stored MxK (transa == 0) or KxM (transa != 0); ld* are
+ * row pitches in elements. */
+int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int64_t K,
+                   float alpha, const float* A, int64_t lda, const float* B,
+                   int64_t ldb, float beta, float* C, int64_t ldc);
+
+/* im2col of a whole NHWC batch (_cpuop 251-277 applied per image by numpy
+ * 158-166): col is (n*out_h*out_w, kh*kw*c). */
+int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w,
+                          int c, int kh, int kw, int pad, int stride_h,
+                          int stride_w);
+/* col2im (_cpuop 282-309 applied per image by numpy 142-147): in_deltas +=
+ * scatter of col, summed in the reference's (out_y, out_x) scan order. */
+int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h,
+                          int w, int c, int kh, int kw, int pad, int stride_h,
+                          int stride_w);
+
+/* maxpool2d_forward_batch (numpy 216-219, _cpuop 27-80). argmax holds the
+ * per-image flat (y*w+x)*c+ch index as float32, -1 for an empty window. */
+int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax,
+                               int64_t n, int h, int w, int c, int out_h,
+                               int out_w, int pool_h, int pool_w, int pad,
+                               int stride_h, int stride_w);
+/* maxpool2d_backward_batch (numpy 210-214, _cpuop 84-115); gather form that
+ * adds in the reference's scan order, so the result is deterministic. */
+int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas,
+                               float* in_deltas, int64_t n, int h, int w, int c,
+                               int out_h, int out_w, int pool_h, int pool_w,
+                               int pad, int stride_h, int stride_w);
+/* avgpool2d_forward_batch (numpy 94-97, _cpuop 120-162) */
+int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h,
+                               int w, int c, int out_h, int out_w, int pool_h,
+                               int pool_w, int pad, int stride_h, int stride_w);
+/* avgpool2d_backward_batch (numpy 89-92, _cpuop 167-202) */
+int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
+                               int64_t n, int h, int w, int c, int out_h,
+                               int out_w, int pool_h, int pool_w, int pad,
+                               int stride_h, int stride_w);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSHIP_H */

@@ -1,0 +1,661 @@
+"""GPU parity: HipHandler against the CPU oracle, operation by operation.
+
+Structured like brainstorm/tests/test_handlers_against_reference.py: every
+ndarray argument is uploaded, the operation runs on both handlers, and EVERY
+array argument is compared afterwards (so in-place side effects are pinned
+too). Where the reference compares with allclose(rtol=1e-5), this file uses the
+stricter bars the operation allows:
+
+  exact   bit-for-bit (all arithmetic made of single IEEE float32 operations,
+          integer/indexing operations, the MT19937 mask stream)
+  ulp     transcendentals, see test_transcendentals for the stated bound
+  rel     1e-5 relative for reductions, softmax and matrix products
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from util import assert_bit_equal, assert_max_ulp, sum_tolerance, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+# the reference's shapes (test_handlers_against_reference.py:24-25) ...
+some_2d_shapes = ((1, 1), (4, 1), (1, 4), (5, 5), (3, 4), (4, 3))
+some_nd_shapes = ((1, 1, 4), (1, 1, 3, 3), (3, 4, 2, 1))
+# ... plus shapes that exercise whole tiles, tile tails and odd row lengths
+big_shapes = ((64, 64), (37, 1031), (4096,), (3, 5000), (1000, 205), (100, 1200), (513, 2048))
+
+
+def rand(rng, shape):
+    return np.asarray(rng.standard_normal(shape), dtype=F32)
+
+
+def operation_check(hip, ref, op_name, ref_args, compare="exact", **tol):
+    """Runs op_name on both handlers; returns the list of (ref_array, hip_array_as_numpy)."""
+    args = [hip.create_from_numpy(a) if isinstance(a, np.ndarray) else a for a in ref_args]
+    getattr(ref, op_name)(*ref_args)
+    getattr(hip, op_name)(*args)
+    pairs = []
+    for i, (r, a) in enumerate(zip(ref_args, args)):
+        if not isinstance(r, np.ndarray):
+            continue
+        got = hip.get_numpy_copy(a)
+        what = "%s arg %d shape %r" % (op_name, i, r.shape)
+        if compare == "exact":
+            assert_bit_equal(got, r, what)
+        elif compare == "ulp":
+            assert_max_ulp(got, r, tol["max_ulp"], what)
+        elif compare == "rel":
+            np.testing.assert_allclose(got, r, rtol=tol.get("rtol", 1e-5), atol=tol.get("atol", 0),
+                                       err_msg=what)
+        pairs.append((r, got))
+    return pairs
+
+
+# ------------------------------------------------------------------ elementwise
+BINARY_OPS = ["add_tt", "subtract_tt", "mult_tt", "divide_tt", "modulo_tt", "mult_add_tt"]
+
+
+@pytest.mark.parametrize("op", BINARY_OPS)
+def test_binary_tt_exact(hip, ref, op):
+    rng = np.random.RandomState(0)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        a, b, out = rand(rng, shape), rand(rng, shape), rand(rng, shape)
+        operation_check(hip, ref, op, (a, b, out))
+
+
+@pytest.mark.parametrize("op", BINARY_OPS)
+def test_binary_tt_in_place(hip, ref, op):
+    # out aliases an input, as the layers do (e.g. add_tt(dbi, tmp, dbi), lstm_layer.py:228)
+    rng = np.random.RandomState(1)
+    for shape in ((5, 5), (37, 1031)):
+        a, b = rand(rng, shape), rand(rng, shape)
+        want_a, want_b = a.copy(), b.copy()
+        getattr(ref, op)(want_a, want_b, want_a)
+        da, db = hip.create_from_numpy(a), hip.create_from_numpy(b)
+        getattr(hip, op)(da, db, da)
+        assert_bit_equal(da.get(), want_a, op + " out is a")
+        want_a2, want_b2 = a.copy(), b.copy()
+        getattr(ref, op)(want_a2, want_b2, want_b2)
+        da, db = hip.create_from_numpy(a), hip.create_from_numpy(b)
+        getattr(hip, op)(da, db, db)
+        assert_bit_equal(db.get(), want_b2, op + " out is b")
+
+
+def test_special_values_exact(hip, ref):
+    special = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38,
+                        -3.4e38, 1.17549435e-38, 0.5, -2.5, 7.0, 1e-20], dtype=F32)
+    a, b = np.meshgrid(special, special)
+    a, b = a.copy(), b.copy()
+    with np.errstate(all="ignore"):
+        for op in ("add_tt", "subtract_tt", "mult_tt", "divide_tt", "modulo_tt", "mult_add_tt"):
+            operation_check(hip, ref, op, (a.copy(), b.copy(), np.ones_like(a)))
+        for op in ("abs_t", "sign_t", "sqrt_t", "rel"):
+            operation_check(hip, ref, op, (a.copy(), np.zeros_like(a)))
+        operation_check(hip, ref, "clip_t", (a.copy(), -1.0, 1.0, np.zeros_like(a)))
+        for op in ("rel_deriv", "sigmoid_deriv", "tanh_deriv", "el_deriv"):
+            operation_check(hip, ref, op, (None, a.copy(), b.copy(), np.zeros_like(a)))
+
+
+@pytest.mark.parametrize("op,scalar", [("add_st", 0.1), ("mult_st", 0.5), ("mult_add_st", 0.5),
+                                       ("mult_st", -1.0), ("mult_add_st", -0.0125), ("add_st", 1e-8)])
+def test_scalar_ops_exact(hip, ref, op, scalar):
+    rng = np.random.RandomState(2)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        t, out = rand(rng, shape), rand(rng, shape)
+        operation_check(hip, ref, op, (scalar, t, out))
+
+
+@pytest.mark.parametrize("op", ["abs_t", "sign_t", "rel"])
+def test_unary_exact(hip, ref, op):
+    rng = np.random.RandomState(3)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        a = rand(rng, shape)
+        a.ravel()[::7] = 0.0          # sign_t of zeros (test_handlers_against_reference.py:305-313)
+        operation_check(hip, ref, op, (a, np.zeros_like(a)))
+
+
+def test_sqrt_exact(hip, ref):
+    # IEEE-correct square root: identical bits. Inputs as in the reference's test (x + 10)
+    # and the U(0.1, 10) of the op sweep.
+    rng = np.random.RandomState(4)
+    for shape in some_2d_shapes + big_shapes:
+        a = (rand(rng, shape) + 10).astype(F32)
+        operation_check(hip, ref, "sqrt_t", (a, np.zeros_like(a)))
+        a = rng.uniform(0.1, 10, shape).astype(F32)
+        operation_check(hip, ref, "sqrt_t", (a, np.zeros_like(a)))
+
+
+def test_clip_exact(hip, ref):
+    rng = np.random.RandomState(5)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        a = rand(rng, shape)
+        operation_check(hip, ref, "clip_t", (a, -1.0, 1.0, np.zeros_like(a)))
+        operation_check(hip, ref, "clip_t", (np.abs(a), 1e-6, 1.0, np.zeros_like(a)))
+
+
+@pytest.mark.parametrize("op", ["rel_deriv", "sigmoid_deriv", "tanh_deriv", "el_deriv"])
+def test_derivs_exact(hip, ref, op):
+    rng = np.random.RandomState(6)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        y, dy = rand(rng, shape), rand(rng, shape)
+        # x is never read by a derivative (debug_handler.py:489 passes None)
+        operation_check(hip, ref, op, (None, y, dy, np.zeros_like(y)))
+    # in-place form used by the layers: f(y, y, dy, dy)   (base_handler.py:50-56)
+    y, dy = rand(rng, (37, 1031)), rand(rng, (37, 1031))
+    want = dy.copy()
+    getattr(ref, op)(y, y, want, want)
+    dyd, yd = hip.create_from_numpy(dy), hip.create_from_numpy(y)
+    getattr(hip, op)(yd, yd, dyd, dyd)
+    assert_bit_equal(dyd.get(), want, op + " in place")
+
+
+@pytest.mark.parametrize("op", ["copy_to_if", "add_into_if"])
+def test_cond_ops_exact(hip, ref, op):
+    rng = np.random.RandomState(7)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes:
+        a, out = rand(rng, shape), rand(rng, shape)
+        cond = (rng.uniform(size=shape) < 0.5).astype(F32) * rand(rng, shape)
+        operation_check(hip, ref, op, (a, out, cond))
+
+
+def test_fill_if_exact(hip, ref):
+    rng = np.random.RandomState(8)
+    for shape in some_2d_shapes + big_shapes:
+        mem = rand(rng, shape)
+        cond = (rng.uniform(size=shape) < 0.5).astype(F32)
+        operation_check(hip, ref, "fill_if", (mem, 2.5, cond))
+
+
+def test_fill_copy_allocate(hip, ref):
+    rng = np.random.RandomState(9)
+    for shape in some_2d_shapes + some_nd_shapes + big_shapes + ((0,), (1, 0, 7), ()):
+        a = rand(rng, shape)
+        operation_check(hip, ref, "fill", (a, -3.25))
+        operation_check(hip, ref, "copy_to", (rand(rng, shape), a))
+        for maker in ("allocate", "zeros", "ones"):
+            got = getattr(hip, maker)(shape)
+            want = getattr(ref, maker)(shape)
+            assert got.shape == want.shape
+            assert_bit_equal(hip.get_numpy_copy(got), want, maker)
+
+
+def test_allocate_reuses_blocks_zeroed(hip):
+    # a pool block that comes back must be handed out zero-filled again
+    for _ in range(3):
+        a = hip.allocate((1000, 33))
+        hip.fill(a, 7.0)
+        del a
+        b = hip.allocate((1000, 33))
+        assert not hip.get_numpy_copy(b).any()
+        del b
+
+
+def test_set_from_numpy_casts_and_broadcasts(hip, ref):
+    mem = hip.allocate((3, 4))
+    hip.set_from_numpy(mem, np.arange(12, dtype=np.float64).reshape(3, 4))
+    assert_bit_equal(mem.get(), np.arange(12, dtype=F32).reshape(3, 4))
+    hip.set_from_numpy(mem, np.arange(4, dtype=np.int32))       # numpy_handler.py:65 broadcasts
+    assert_bit_equal(mem.get(), np.broadcast_to(np.arange(4, dtype=F32), (3, 4)))
+
+
+# -------------------------------------------------------------- transcendentals
+def _check_transcendental(hip, ref, op, x, exact_f64, label):
+    """Stated bound for float32 transcendentals.
+
+    HIP evaluates in float64 and rounds once, so it must be within 1 ulp of the float64
+    evaluation of the reference formula rounded to float32 (`truth`). NumPy's own float32
+    SIMD routines are measurably 1-4 ulp away from that truth (depending on the host CPU),
+    so the distance to the float32 oracle is bounded elementwise by 2 ulp + the oracle's own
+    distance from the truth; wherever the oracle is within 2 ulp of the truth this is the
+    plain "<= 2 ulp to NumpyHandler" bar... and the distance to the oracle is reported.
+    """
+    want32 = np.zeros_like(x)
+    getattr(ref, op)(x.copy(), want32)
+    xd = hip.create_from_numpy(x)
+    yd = hip.allocate(x.shape)
+    getattr(hip, op)(xd, yd)
+    got = yd.get()
+    with np.errstate(all="ignore"):
+        truth = exact_f64(x.astype(np.float64)).astype(F32)
+    d_truth = ulp_distance(got, truth)
+    d_oracle = ulp_distance(got, want32)
+    oracle_err = ulp_distance(want32, truth)
+    assert d_truth.max() <= 1, "%s %s: %d ulp from the float64 evaluation" % (op, label, d_truth.max())
+    assert np.all(d_oracle <= 2 + oracle_err), "%s %s: too far from the float32 oracle" % (op, label)
+    print("%s %s: max ulp to float32 oracle %d (oracle itself %d from float64 truth), "
+          "fraction within 2 ulp %.6f" % (op, label, d_oracle.max(), oracle_err.max(),
+                                           np.mean(d_oracle <= 2)))
+    # in place must give the same bits
+    getattr(hip, op)(xd, xd)
+    assert_bit_equal(xd.get(), got, op + " in place")
+
+
+def _sigmoid64(x):
+    e = np.exp(-np.abs(x))
+    return np.where(x >= 0, 1.0 / (1.0 + e), e / (1.0 + e))
+
+
+@pytest.mark.parametrize("shape", [(5, 5), (37, 1031), (1024, 1024)])
+def test_transcendentals(hip, ref, shape):
+    rng = np.random.RandomState(10)
+    x = rand(rng, shape)
+    _check_transcendental(hip, ref, "tanh", x, np.tanh, "N(0,1)")
+    _check_transcendental(hip, ref, "sigmoid", x, _sigmoid64, "N(0,1)")
+    _check_transcendental(hip, ref, "tanh", (x * 8).astype(F32), np.tanh, "N(0,64)")
+    _check_transcendental(hip, ref, "sigmoid", (x * 30).astype(F32), _sigmoid64, "N(0,900)")
+    u = rng.uniform(0.1, 10, shape).astype(F32)
+    _check_transcendental(hip, ref, "log_t", u, np.log, "U(0.1,10)")
+    _check_transcendental(hip, ref, "log_t", (x + 10).astype(F32), np.log, "N(10,1)")
+
+
+def test_el(hip, ref):
+    # el = x*(x>=0) + (exp(x)-1)*(x<0) in float32 steps (numpy_handler.py:305). exp(x)-1 cancels,
+    # so an ulp of exp(x) (<= 2^-24 for x<0) is an ABSOLUTE error of the result: the bound is
+    # 3 ulp of 1.0 = 3 * 2^-24 absolute (2 for NumPy's exp, 1 for the rounding of ours) or 2 ulp.
+    rng = np.random.RandomState(11)
+    for shape in ((5, 5), (37, 1031)):
+        x = rand(rng, shape)
+        want = np.zeros_like(x)
+        ref.el(x, want)
+        xd, yd = hip.create_from_numpy(x), hip.allocate(shape)
+        hip.el(xd, yd)
+        got = yd.get()
+        ok = (np.abs(got.astype(np.float64) - want) <= 3 * 2.0 ** -24) | (ulp_distance(got, want).reshape(shape) <= 2)
+        assert ok.all()
+
+
+# ----------------------------------------------------------------- broadcast
+MV_OPS = ["add_mv", "subtract_mv", "mult_mv", "divide_mv", "mult_add_mv"]
+
+
+@pytest.mark.parametrize("op", MV_OPS)
+def test_mv_row_and_column_exact(hip, ref, op):
+    rng = np.random.RandomState(12)
+    shapes = some_2d_shapes + ((64, 64), (37, 1031), (100, 1200), (1000, 205), (513, 2048), (100, 10),
+                               (2048, 4096), (7, 16384))
+    for shape in shapes:
+        m, out = rand(rng, shape), rand(rng, shape)
+        row = (rand(rng, (1, shape[1])) + 3).astype(F32)
+        col = (rand(rng, (shape[0], 1)) + 3).astype(F32)
+        operation_check(hip, ref, op, (m, row, out))
+        operation_check(hip, ref, op, (m.copy(), col, out.copy()))
+    # in place: out is m (FullyConnected: add_mv(y, bias, y))
+    m = rand(rng, (100, 1200))
+    row = rand(rng, (1, 1200))
+    want = m.copy()
+    getattr(ref, op)(want, row, want)
+    md = hip.create_from_numpy(m)
+    getattr(hip, op)(md, hip.create_from_numpy(row), md)
+    assert_bit_equal(md.get(), want, op + " in place")
+
+
+def test_mv_one_dimensional_vector_is_a_row(hip, ref):
+    # conv bias arrives as a 1-D (F,) vector (pycuda_handler.py:256-257)
+    rng = np.random.RandomState(13)
+    m, v = rand(rng, (50, 32)), rand(rng, (32,))
+    out = np.zeros_like(m)
+    ref.add_mv(m, v, out)
+    od = hip.allocate(m.shape)
+    hip.add_mv(hip.create_from_numpy(m), hip.create_from_numpy(v), od)
+    assert_bit_equal(od.get(), out)
+
+
+def test_mult_mv_same_shape(hip, ref):
+    rng = np.random.RandomState(14)
+    m, v = rand(rng, (5, 7)), rand(rng, (5, 7))
+    operation_check(hip, ref, "mult_mv", (m, v, np.zeros_like(m)))
+
+
+def test_broadcast_t_exact(hip, ref):
+    # the 7 cases of test_handlers_against_reference.py:242-257 and larger ones
+    rng = np.random.RandomState(15)
+    cases = [((1, 4), 0, (3, 4)), ((3, 1), 1, (3, 4)), ((1, 3, 4), 0, (2, 3, 4)),
+             ((2, 1, 4), 1, (2, 5, 4)), ((2, 3, 1), 2, (2, 3, 6)), ((1, 1, 3, 3), 0, (4, 1, 3, 3)),
+             ((3, 4, 2, 1), 3, (3, 4, 2, 5)), ((1, 1000), 0, (100, 1000)), ((20, 30, 1), 2, (20, 30, 17))]
+    for a_shape, axis, out_shape in cases:
+        operation_check(hip, ref, "broadcast_t", (rand(rng, a_shape), axis, np.zeros(out_shape, F32)))
+
+
+def test_merge_split_exact(hip, ref):
+    rng = np.random.RandomState(16)
+    for rows, na, nb in [((4,), 1, 1), ((3, 2), 3, 5), ((2049,), 3, 1025), ((7, 5), 128, 64)]:
+        a, b = rand(rng, rows + (na,)), rand(rng, rows + (nb,))
+        out = np.zeros(rows + (na + nb,), F32)
+        operation_check(hip, ref, "merge_tt", (a, b, out))
+        x = rand(rng, rows + (na + nb,))
+        operation_check(hip, ref, "split_add_tt", (x, a.copy(), b.copy()))
+
+
+# ------------------------------------------------------------------ reductions
+def _check_sum(hip, ref, a, axis, out_shape):
+    want = np.zeros(out_shape, F32)
+    ref.sum_t(a, axis, want)
+    od = hip.create_from_numpy(np.full(out_shape, 99.0, F32))
+    hip.sum_t(hip.create_from_numpy(a), axis, od)
+    got = od.get()
+    assert got.shape == want.shape
+    truth = np.sum(a.astype(np.float64), axis=axis)
+    tol = sum_tolerance(want, a, axis)
+    err = np.abs(got.astype(np.float64).reshape(tol.shape) - want.astype(np.float64).reshape(tol.shape))
+    assert np.all(err <= tol), "sum_t axis=%r shape %r: error %g over tolerance" % (
+        axis, a.shape, float(np.max(err / tol)))
+    # and no further from the float64 sum than the float32 oracle is (up to the same bound)
+    err_truth = np.abs(got.astype(np.float64).reshape(tol.shape) - truth.reshape(tol.shape))
+    assert np.all(err_truth <= tol)
+
+
+def test_sum_t(hip, ref):
+    rng = np.random.RandomState(17)
+    shapes = some_2d_shapes + ((64, 64), (37, 1031), (100, 1200), (1000, 205), (10000, 10), (7, 16384),
+                               (2048, 4096), (513, 2049), (100, 1), (1, 100), (3000, 17), (70000, 3))
+    for shape in shapes:
+        for a in (rand(rng, shape), np.abs(rand(rng, shape))):
+            _check_sum(hip, ref, a, 0, (1, shape[1]))
+            _check_sum(hip, ref, a, 0, (shape[1],))
+            _check_sum(hip, ref, a, 1, (shape[0],))
+            _check_sum(hip, ref, a, 1, (shape[0], 1))
+            _check_sum(hip, ref, a, None, ())
+    # Loss layer: 3-D array, axis None, 0-d output (loss_layer.py:44-46)
+    _check_sum(hip, ref, rand(rng, (1, 100, 1)), None, ())
+    _check_sum(hip, ref, rand(rng, (1 << 22,)), None, ())
+    _check_sum(hip, ref, rand(rng, ((1 << 22) + 13,)), None, ())
+
+
+def test_sum_t_is_deterministic(hip):
+    rng = np.random.RandomState(18)
+    a = hip.create_from_numpy(rand(rng, (2048, 4096)))
+    outs = []
+    for _ in range(3):
+        o = hip.allocate((4096,))
+        hip.sum_t(a, 0, o)
+        outs.append(o.get())
+    assert_bit_equal(outs[0], outs[1])
+    assert_bit_equal(outs[0], outs[2])
+
+
+def test_softmax_m(hip, ref):
+    rng = np.random.RandomState(19)
+    shapes = some_2d_shapes + ((100, 10), (10000, 205), (64, 64), (37, 1031), (16, 4096), (5, 5000),
+                               (3, 16384), (2, 70001), (2, 70000), (300, 256), (9, 1024), (9, 1025))
+    for shape in shapes:
+        for scale in (1.0, 20.0):
+            m = (rand(rng, shape) * scale).astype(F32)
+            pairs = operation_check(hip, ref, "softmax_m", (m, np.zeros_like(m)), compare="rel", rtol=1e-5, atol=1e-37)
+            got = pairs[1][1]
+            # invariant the domain gives: rows sum to one
+            np.testing.assert_allclose(got.astype(np.float64).sum(axis=1), 1.0, rtol=0, atol=1e-5)
+    # in place (softmax_ce_layer.py calls it out of place, but aliasing must be safe)
+    m = rand(rng, (100, 205))
+    want = np.zeros_like(m)
+    ref.softmax_m(m, want)
+    md = hip.create_from_numpy(m)
+    hip.softmax_m(md, md)
+    np.testing.assert_allclose(md.get(), want, rtol=1e-5)
+
+
+def test_is_fully_finite(hip, ref):
+    rng = np.random.RandomState(20)
+    for shape in ((5, 5), (37, 1031), (1 << 20,)):
+        a = rand(rng, shape)
+        assert hip.is_fully_finite(hip.create_from_numpy(a)) is True
+        for bad in (np.nan, np.inf, -np.inf):
+            b = a.copy()
+            b.ravel()[b.size // 3] = bad
+            assert hip.is_fully_finite(hip.create_from_numpy(b)) is False
+            assert bool(ref.is_fully_finite(b)) is False
+
+
+# -------------------------------------------------------------------- indexing
+def test_binarize_v_exact(hip, ref):
+    rng = np.random.RandomState(21)
+    for rows, k in [(1, 1), (5, 3), (100, 10), (10000, 205), (64, 64), (300, 1031), (512, 4096)]:
+        v = rng.randint(0, k, (rows, 1)).astype(F32)
+        operation_check(hip, ref, "binarize_v", (v, np.full((rows, k), 7.0, F32)))
+
+
+def test_index_m_by_v_exact(hip, ref):
+    rng = np.random.RandomState(22)
+    for rows, k in [(1, 1), (5, 3), (100, 10), (10000, 205), (4096, 4096)]:
+        m = rand(rng, (rows, k))
+        v = rng.randint(0, k, (rows, 1)).astype(F32)
+        operation_check(hip, ref, "index_m_by_v", (m, v, np.zeros((rows, 1), F32)))
+
+
+# ------------------------------------------------------------------------- RNG
+def test_generate_probability_mask_matches_randomstate(hip):
+    # Sizes chosen so that consecutive calls start at even and odd positions of the 624-word
+    # MT19937 block and cross block boundaries (a 53-bit double takes two words).
+    from brainstorm_amd import HipHandler  # noqa: F401  (same library instance)
+    for seed in (0, 1, 42, 4294967295):
+        hip.rnd.seed(seed)
+        rs = np.random.RandomState(seed)
+        for shape, p in [((7, 5), 0.8), ((1,), 0.5), ((311,), 0.5), ((312,), 0.3), ((313,), 0.9),
+                         ((1, 100, 784), 0.8), ((1, 100, 1200), 0.5), ((3,), 0.5), ((100000,), 0.123)]:
+            mask = hip.allocate(shape)
+            hip.generate_probability_mask(mask, p)
+            want = (rs.uniform(size=shape) < p).astype(F32)
+            assert_bit_equal(mask.get(), want, "mask seed %d shape %r" % (seed, shape))
+        # the generator state itself must agree with NumPy's afterwards
+        _, key, pos, _, _ = hip.rnd.get_state()
+        st = rs.get_state()
+        assert pos == st[2]
+        np.testing.assert_array_equal(key, st[1])
+
+
+def test_fill_gaussian_matches_randomstate(hip):
+    for seed in (0, 7):
+        hip.rnd.seed(seed)
+        rs = np.random.RandomState(seed)
+        for shape, mean, std in [((5,), 0.0, 1.0), ((4,), 1.5, 0.1), ((1000, 37), -2.0, 3.0), ((1,), 0.0, 1.0),
+                                 ((2,), 0.0, 1.0)]:
+            out = hip.allocate(shape)
+            hip.fill_gaussian(mean, std, out)
+            want = (std * rs.standard_normal(shape) + mean).astype(F32)
+            # float64 log/sqrt of the device maths library vs the host's: at most 1 float32 ulp
+            assert_max_ulp(out.get(), want, 1, "fill_gaussian seed %d shape %r" % (seed, shape))
+        # interleave with masks: both draw from the one stream
+        mask = hip.allocate((11,))
+        hip.generate_probability_mask(mask, 0.5)
+        assert_bit_equal(mask.get(), (rs.uniform(size=(11,)) < 0.5).astype(F32))
+        _, key, pos, has_gauss, _ = hip.rnd.get_state()
+        st = rs.get_state()
+        assert (pos, has_gauss) == (st[2], st[3])
+        np.testing.assert_array_equal(key, st[1])
+
+
+# ----------------------------------------------------------------------- dense
+def test_dot_mm_and_dot_add_mm(hip, ref):
+    rng = np.random.RandomState(23)
+    dims = [(1, 1, 1), (4, 1, 3), (5, 5, 5), (3, 4, 2), (100, 784, 1200), (100, 1200, 10), (64, 205, 1000),
+            (257, 129, 65)]
+    for (m, k, n), ta, tb in itertools.product(dims, (False, True), (False, True)):
+        a = rand(rng, (k, m) if ta else (m, k))
+        b = rand(rng, (n, k) if tb else (k, n))
+        out = rand(rng, (m, n))
+        for op in ("dot_mm", "dot_add_mm"):
+            want = out.copy()
+            getattr(ref, op)(a, b, want, ta, tb)
+            od = hip.create_from_numpy(out)
+            getattr(hip, op)(hip.create_from_numpy(a), hip.create_from_numpy(b), od, ta, tb)
+            # 1e-5 relative to the magnitude of a length-k inner product
+            scale = np.sqrt(k) + np.abs(want)
+            assert np.max(np.abs(od.get() - want) / scale) <= 1e-5, (op, m, k, n, ta, tb)
+
+
+# -------------------------------------------------------------- conv / pooling
+def _out_size(n, k, pad, stride):
+    return (n + 2 * pad - k) // stride + 1
+
+
+POOL_CASES = [(n, h, w, c, win, pad, stride)
+              for (n, h, w, c) in [(1, 4, 4, 1), (2, 5, 7, 3), (3, 32, 32, 32), (2, 15, 15, 64)]
+              for win in [(1, 1), (2, 2), (3, 3), (2, 3), (3, 2)]
+              for pad in (0, 1, 2)
+              for stride in [(1, 1), (2, 2), (1, 2), (3, 3)]
+              if win[0] <= h + 2 * pad and win[1] <= w + 2 * pad]
+
+
+def test_maxpool_forward_backward_exact(hip, ref):
+    rng = np.random.RandomState(24)
+    for n, h, w, c, win, pad, stride in POOL_CASES:
+        oh, ow = _out_size(h, win[0], pad, stride[0]), _out_size(w, win[1], pad, stride[1])
+        x = rand(rng, (n, h, w, c))
+        x[rng.uniform(size=x.shape) < 0.3] = 0.5          # ties: the first maximum must win
+        out = np.zeros((n, oh, ow, c), F32)
+        arg = np.zeros((n, oh, ow, c), F32)
+        ref.maxpool2d_forward_batch(x, win, out, pad, stride, arg)
+        xd = hip.create_from_numpy(x)
+        outd, argd = hip.allocate(out.shape), hip.allocate(arg.shape)
+        hip.maxpool2d_forward_batch(xd, win, outd, pad, stride, argd)
+        what = "maxpool %r" % ((n, h, w, c, win, pad, stride),)
+        assert_bit_equal(outd.get(), out, what + " values")
+        assert_bit_equal(argd.get(), arg, what + " argmax")
+        dout = rand(rng, out.shape)
+        din = rand(rng, x.shape)
+        want = din.copy()
+        ref.maxpool2d_backward_batch(x, win, out, pad, stride, arg, want, dout)
+        dind = hip.create_from_numpy(din)
+        hip.maxpool2d_backward_batch(xd, win, outd, pad, stride, argd, dind, hip.create_from_numpy(dout))
+        assert_bit_equal(dind.get(), want, what + " backward")
+
+
+def test_avgpool_forward_backward_exact(hip, ref):
+    rng = np.random.RandomState(25)
+    for n, h, w, c, win, pad, stride in POOL_CASES:
+        oh, ow = _out_size(h, win[0], pad, stride[0]), _out_size(w, win[1], pad, stride[1])
+        x = rand(rng, (n, h, w, c))
+        out = np.zeros((n, oh, ow, c), F32)
+        ref.avgpool2d_forward_batch(x, win, out, pad, stride)
+        xd = hip.create_from_numpy(x)
+        outd = hip.allocate(out.shape)
+        hip.avgpool2d_forward_batch(xd, win, outd, pad, stride)
+        what = "avgpool %r" % ((n, h, w, c, win, pad, stride),)
+        assert_bit_equal(outd.get(), out, what + " values")
+        dout, din = rand(rng, out.shape), rand(rng, x.shape)
+        want = din.copy()
+        ref.avgpool2d_backward_batch(x, win, out, pad, stride, want, dout)
+        dind = hip.create_from_numpy(din)
+        hip.avgpool2d_backward_batch(xd, win, outd, pad, stride, dind, hip.create_from_numpy(dout))
+        assert_bit_equal(dind.get(), want, what + " backward")
+
+
+CONV_CASES = [(2, 5, 4, 3, 2, 3, 3, 0, (1, 1)), (2, 5, 4, 3, 2, 3, 3, 1, (2, 1)), (1, 3, 3, 1, 1, 1, 1, 0, (1, 1)),
+              (4, 9, 9, 3, 4, 5, 5, 2, (1, 1)), (3, 9, 6, 1, 3, 3, 2, 1, (2, 3)),
+              (10, 32, 32, 3, 32, 5, 5, 2, (1, 1)), (10, 15, 15, 32, 64, 5, 5, 2, (1, 1))]
+
+
+def test_conv2d_forward_backward(hip, ref):
+    rng = np.random.RandomState(26)
+    for n, h, w, c, f, kh, kw, pad, stride in CONV_CASES:
+        oh, ow = _out_size(h, kh, pad, stride[0]), _out_size(w, kw, pad, stride[1])
+        x = rand(rng, (n, h, w, c))
+        wts = rand(rng, (f, kh, kw, c))
+        bias = rand(rng, (f,))
+        out = np.zeros((n, oh, ow, f), F32)
+        ref.conv2d_forward_batch(x, wts, bias, out, pad, stride)
+        xd, wd, bd = hip.create_from_numpy(x), hip.create_from_numpy(wts), hip.create_from_numpy(bias)
+        outd = hip.allocate(out.shape)
+        hip.conv2d_forward_batch(xd, wd, bd, outd, pad, stride)
+        k = kh * kw * c
+        scale = np.sqrt(k) + np.abs(out)
+        assert np.max(np.abs(outd.get() - out) / scale) <= 1e-5, ("conv fwd", n, h, w, c, f)
+        dout = rand(rng, out.shape)
+        din = rand(rng, x.shape)
+        want_din, dw, db = din.copy(), np.full_like(wts, 5.0), np.full_like(bias, 5.0)
+        ref.conv2d_backward_batch(x, wts, pad, stride, want_din, dout, dw, db)
+        dind = hip.create_from_numpy(din)
+        dwd, dbd = hip.create_from_numpy(np.full_like(wts, 5.0)), hip.create_from_numpy(np.full_like(bias, 5.0))
+        hip.conv2d_backward_batch(xd, wd, pad, stride, dind, hip.create_from_numpy(dout), dwd, dbd)
+        assert np.max(np.abs(dind.get() - want_din) / (np.sqrt(f * kh * kw) + np.abs(want_din))) <= 1e-5
+        assert np.max(np.abs(dwd.get() - dw) / (np.sqrt(n * oh * ow) + np.abs(dw))) <= 1e-5
+        assert np.max(np.abs(dbd.get() - db) / (np.sqrt(n * oh * ow) + np.abs(db))) <= 1e-5
+
+
+def test_im2col_col2im_exact(hip, ref):
+    # through the C ABI directly: the batched kernels against the oracle's per-image routines
+    rng = np.random.RandomState(27)
+    lib = hip._lib
+    for n, h, w, c, f, kh, kw, pad, stride in CONV_CASES:
+        oh, ow = _out_size(h, kh, pad, stride[0]), _out_size(w, kw, pad, stride[1])
+        x = rand(rng, (n, h, w, c))
+        col = np.zeros((n, oh * ow, kh * kw * c), F32)
+        for i in range(n):
+            ref._im2col(x[i], kh, kw, pad, stride, col[i])
+        xd = hip.create_from_numpy(x)
+        cold = hip.allocate(col.shape)
+        hip._call(lib.bship_im2col_nhwc_f32(xd.ptr, cold.ptr, n, h, w, c, kh, kw, pad, stride[0], stride[1]))
+        assert_bit_equal(cold.get(), col, "im2col")
+        cols = rand(rng, col.shape)
+        din = rand(rng, x.shape)
+        want = din.copy()
+        for i in range(n):
+            ref._col2im(cols[i], kh, kw, pad, stride, want[i])
+        dind = hip.create_from_numpy(din)
+        colsd = hip.create_from_numpy(cols)
+        hip._call(lib.bship_col2im_nhwc_f32(colsd.ptr, dind.ptr, n, h, w, c, kh, kw, pad,
+                                            stride[0], stride[1]))
+        assert_bit_equal(dind.get(), want, "col2im")
+
+
+# ---------------------------------------------------------- views of one buffer
+def test_ops_on_unaligned_views(hip, ref):
+    # Layer buffers are slices of one flat array (buffers.py:79-83) and may start at any element,
+    # so only 4-byte alignment can be assumed.
+    rng = np.random.RandomState(28)
+    flat = rand(rng, (3 * 5000 + 16,))
+    fd = hip.create_from_numpy(flat)
+    for off in (1, 2, 3, 5):
+        a, b, o = (flat[off:off + 5000], flat[5003 + off:5003 + off + 5000], flat[10007:10007 + 5000])
+        want = flat.copy()
+        wa, wb, wo = want[off:off + 5000], want[5003 + off:5003 + off + 5000], want[10007:10007 + 5000]
+        ref.add_tt(wa, wb, wo)
+        ref.sigmoid_deriv(None, wa, wb, wo[:5000])
+        fd2 = hip.create_from_numpy(flat)
+        da, db, do = fd2[off:off + 5000], fd2[5003 + off:5003 + off + 5000], fd2[10007:10007 + 5000]
+        hip.add_tt(da, db, do)
+        hip.sigmoid_deriv(None, da, db, do)
+        assert_bit_equal(fd2.get(), want, "offset %d" % off)
+        # 2-D views with odd row length, row vector add + row/col sums + softmax
+        m = flat[off:off + 4800].reshape(40, 120)
+        md = fd[off:off + 4800].reshape((40, 120))
+        v = flat[9000 + off:9000 + off + 120].reshape(1, 120)
+        vd = fd[9000 + off:9000 + off + 120].reshape((1, 120))
+        want_o = np.zeros_like(m)
+        ref.add_mv(m, v, want_o)
+        od = hip.allocate((40, 120))
+        hip.add_mv(md, vd, od)
+        assert_bit_equal(od.get(), want_o)
+        _check_sum(hip, ref, m.copy(), 0, (120,))
+        s0 = hip.allocate((120,))
+        hip.sum_t(md, 0, s0)
+        np.testing.assert_allclose(s0.get(), m.sum(axis=0), rtol=1e-4, atol=1e-5)
+        s1 = hip.allocate((40,))
+        hip.sum_t(md, 1, s1)
+        np.testing.assert_allclose(s1.get(), m.sum(axis=1), rtol=1e-4, atol=1e-5)
+        sm = hip.allocate((40, 120))
+        hip.softmax_m(md, sm)
+        want_sm = np.zeros_like(m)
+        ref.softmax_m(m, want_sm)
+        np.testing.assert_allclose(sm.get(), want_sm, rtol=1e-5)
+    assert_bit_equal(fd.get(), flat, "inputs untouched")
+
+
+def test_device_array_views_alias(hip):
+    base = hip.create_from_numpy(np.arange(2 * 3 * 4, dtype=F32).reshape(2, 3, 4))
+    host = np.arange(24, dtype=F32).reshape(2, 3, 4)
+    np.testing.assert_array_equal(base[1].get(), host[1])
+    np.testing.assert_array_equal(base[-1, 1:].get(), host[-1, 1:])
+    np.testing.assert_array_equal(base[0, 2].get(), host[0, 2])
+    np.testing.assert_array_equal(base[1, 2, 3].get(), host[1, 2, 3])
+    np.testing.assert_array_equal(base.reshape((6, 4))[2:5].get(), host.reshape(6, 4)[2:5])
+    np.testing.assert_array_equal(base[:, :, :].get(), host)
+    hip.fill(base[1, 1:], -1.0)                 # writes through a view reach the parent
+    host[1, 1:] = -1.0
+    np.testing.assert_array_equal(base.get(), host)
+    flat = base.reshape(24)
+    hip.fill(flat[3:5], 9.0)
+    host.reshape(24)[3:5] = 9.0
+    np.testing.assert_array_equal(base.get(), host)
