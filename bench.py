@@ -1,0 +1,248 @@
+#!/usr/bin/env python
+"""Benchmark of the handler hot path on one MI355X.
+
+A "step" is one pass of the handler-operation sweep (the operations named by
+the op-sweep configuration: elementwise, activations and derivatives,
+reductions, softmax, matrix-vector broadcasts, label indexing) over synthetic
+float32 tensors that are already resident in HBM. The headline value is the
+sweep's aggregate algorithmic throughput in GB/s: the sum over operations of
+the minimum number of bytes each must move (bytes read + bytes written,
+ALG_BYTES below) divided by the wall time of the step.
+
+Prints ONE JSON line. Besides the required keys it carries
+  roofline      for the operation that takes the largest share of a step:
+                algorithmic bytes / mean kernel time (HIP events on the library's
+                stream, taken inside the timed steps) against 8 TB/s HBM peak
+  cpu_baseline  the CPU oracle (NumpyHandler semantics, NumPy) timed on this
+                machine's host cores on a bounded sample (the 4096x4096 sweep)
+  ops           per-operation GB/s and fraction of peak
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size S] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+F32 = np.float32
+
+
+def alg_bytes(rows, cols):
+    """Minimum HBM traffic of each sweep operation on a (rows, cols) float32 tensor."""
+    n = rows * cols
+    return {
+        "add_tt": 12 * n, "mult_tt": 12 * n, "divide_tt": 12 * n,
+        "mult_add_st": 12 * n,
+        "sigmoid": 8 * n, "tanh": 8 * n, "rel": 8 * n,
+        "sigmoid_deriv": 12 * n, "tanh_deriv": 12 * n, "rel_deriv": 12 * n,
+        "clip_t": 8 * n, "sqrt_t": 8 * n, "log_t": 8 * n,
+        "sum_t_axis0": 4 * n + 4 * cols, "sum_t_axis1": 4 * n + 4 * rows, "sum_t_all": 4 * n + 4,
+        "softmax_m": 8 * n,
+        "add_mv_row": 8 * n + 4 * cols, "mult_mv_row": 8 * n + 4 * cols,
+        "add_mv_col": 8 * n + 4 * rows, "mult_mv_col": 8 * n + 4 * rows,
+        "binarize_v": 4 * n + 4 * rows,
+        "index_m_by_v": 12 * rows,          # label + gathered element + result per row
+    }
+
+
+def sweep_ops(h, t):
+    """(name, thunk) for every operation of the sweep on handler h and tensor set t."""
+    return [
+        ("add_tt", lambda: h.add_tt(t["a"], t["b"], t["out"])),
+        ("mult_tt", lambda: h.mult_tt(t["a"], t["b"], t["out"])),
+        ("divide_tt", lambda: h.divide_tt(t["a"], t["u"], t["out"])),
+        ("mult_add_st", lambda: h.mult_add_st(0.5, t["a"], t["acc"])),
+        ("sigmoid", lambda: h.sigmoid(t["a"], t["out"])),
+        ("tanh", lambda: h.tanh(t["a"], t["out"])),
+        ("rel", lambda: h.rel(t["a"], t["out"])),
+        ("sigmoid_deriv", lambda: h.sigmoid_deriv(None, t["y"], t["b"], t["out"])),
+        ("tanh_deriv", lambda: h.tanh_deriv(None, t["y"], t["b"], t["out"])),
+        ("rel_deriv", lambda: h.rel_deriv(None, t["y"], t["b"], t["out"])),
+        ("clip_t", lambda: h.clip_t(t["a"], -1.0, 1.0, t["out"])),
+        ("sqrt_t", lambda: h.sqrt_t(t["u"], t["out"])),
+        ("log_t", lambda: h.log_t(t["u"], t["out"])),
+        ("sum_t_axis0", lambda: h.sum_t(t["a"], 0, t["row_out"])),
+        ("sum_t_axis1", lambda: h.sum_t(t["a"], 1, t["col_out"])),
+        ("sum_t_all", lambda: h.sum_t(t["a"], None, t["scalar_out"])),
+        ("softmax_m", lambda: h.softmax_m(t["a"], t["out"])),
+        ("add_mv_row", lambda: h.add_mv(t["a"], t["row"], t["out"])),
+        ("mult_mv_row", lambda: h.mult_mv(t["a"], t["row"], t["out"])),
+        ("add_mv_col", lambda: h.add_mv(t["a"], t["col"], t["out"])),
+        ("mult_mv_col", lambda: h.mult_mv(t["a"], t["col"], t["out"])),
+        ("binarize_v", lambda: h.binarize_v(t["labels"], t["out"])),
+        ("index_m_by_v", lambda: h.index_m_by_v(t["a"], t["labels"], t["picked"])),
+    ]
+
+
+def host_tensors(size, seed=0):
+    """The op-sweep inputs: N(0,1) tensors, U(0.1,10) denominators, integer labels; seed 0."""
+    rng = np.random.RandomState(seed)
+    shape = (size, size)
+    t = {
+        "a": rng.standard_normal(shape).astype(F32),
+        "b": rng.standard_normal(shape).astype(F32),
+        "u": rng.uniform(0.1, 10, shape).astype(F32),
+        "row": rng.standard_normal((1, size)).astype(F32),
+        "col": rng.standard_normal((size, 1)).astype(F32),
+        "labels": rng.randint(0, size, (size, 1)).astype(F32),
+    }
+    t["y"] = np.tanh(t["b"])          # a plausible activation output for the derivatives
+    return t
+
+
+def add_outputs(h, t, size):
+    t["out"] = h.allocate((size, size))
+    t["acc"] = h.allocate((size, size))
+    t["row_out"] = h.allocate((1, size))
+    t["col_out"] = h.allocate((size, 1))
+    t["scalar_out"] = h.allocate(())
+    t["picked"] = h.allocate((size, 1))
+    return t
+
+
+def device_tensors(hip, size, base=4096):
+    """Tensors of (size, size) on the device, tiled from the seeded (base, base) host inputs
+    with the handler's own broadcast_t so that no multi-GiB host arrays are needed."""
+    base = min(base, size)
+    src = host_tensors(base)
+    reps = (size * size) // (base * base)
+    t = {}
+    for name in ("a", "b", "u", "y"):
+        small = hip.create_from_numpy(src[name].reshape(1, base * base))
+        big = hip.allocate((reps, base * base))
+        hip.broadcast_t(small, 0, big)
+        t[name] = big.reshape((size, size))
+    rng = np.random.RandomState(1)
+    t["row"] = hip.create_from_numpy(rng.standard_normal((1, size)).astype(F32))
+    t["col"] = hip.create_from_numpy(rng.standard_normal((size, 1)).astype(F32))
+    t["labels"] = hip.create_from_numpy(rng.randint(0, size, (size, 1)).astype(F32))
+    return add_outputs(hip, t, size)
+
+
+def run_gpu(size, steps, warmup):
+    from brainstorm_amd import HipHandler
+    hip = HipHandler(seed=0)
+    lib = hip._lib
+    name, cus = hip.device_info()
+    t = device_tensors(hip, size)
+    ops = sweep_ops(hip, t)
+    nops = len(ops)
+    assert steps * (nops + 1) <= 1024, "too many steps for the event slots"
+    for _ in range(warmup):
+        for _, fn in ops:
+            fn()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    slot = 0
+    for _ in range(steps):
+        # one event before every operation and one after the last: kernel times are read
+        # after the timed region, nothing waits inside it
+        for _, fn in ops:
+            lib.bship_event_record(slot)
+            slot += 1
+            fn()
+        lib.bship_event_record(slot)
+        slot += 1
+    hip.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms = ctypes.c_float()
+    per_op_ms = {n: [] for n, _ in ops}
+    for s in range(steps):
+        base = s * (nops + 1)
+        for i, (n, _) in enumerate(ops):
+            hip._call(lib.bship_event_elapsed_ms(base + i, base + i + 1, ctypes.byref(ms)))
+            per_op_ms[n].append(ms.value)
+    return hip, name, cus, elapsed, {n: float(np.mean(v)) for n, v in per_op_ms.items()}
+
+
+def run_cpu(size, budget_s):
+    """Times the CPU oracle on the (size, size) sweep: whole passes until ~budget_s is spent."""
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from oracle.numpy_ref_handler import NumpyRefHandler
+    ref = NumpyRefHandler(F32, seed=0)
+    t = add_outputs(ref, host_tensors(size), size)
+    ops = sweep_ops(ref, t)
+    for _, fn in ops[:2]:
+        fn()                                   # touch the output pages once
+    per_op = {n: [] for n, _ in ops}
+    passes = 0
+    start = time.perf_counter()
+    while passes < 1 or (time.perf_counter() - start < budget_s and passes < 20):
+        for n, fn in ops:
+            t0 = time.perf_counter()
+            fn()
+            per_op[n].append(time.perf_counter() - t0)
+        passes += 1
+    return passes, {n: float(np.median(v)) for n, v in per_op.items()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=16384, help="tensors are size x size float32")
+    ap.add_argument("--cpu-size", type=int, default=4096)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the handler path has no multi-GPU part "
+                 "(got --gpus %d); run it with --gpus 1" % args.gpus)
+    if args.size % 4096 and args.size > 4096:
+        sys.exit("--size must be a multiple of 4096")
+
+    hip, dev_name, cus, elapsed, op_ms = run_gpu(args.size, args.steps, args.warmup)
+    ab = alg_bytes(args.size, args.size)
+    total_bytes = sum(ab[n] for n in op_ms)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = total_bytes / (elapsed / args.steps) / 1e9
+    ops = {}
+    for n, ms in op_ms.items():
+        gbps = ab[n] / (ms * 1e-3) / 1e9
+        ops[n] = {"ms": round(ms, 4), "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    dominant = max(op_ms, key=lambda n: op_ms[n])
+    roofline = {
+        "kernel": dominant, "bound": "hbm",
+        "achieved": ops[dominant]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": ops[dominant]["frac"], "traffic": None,
+        "alg_bytes_per_launch": ab[dominant], "ms_per_launch": ops[dominant]["ms"],
+    }
+    out = {
+        "metric": "handler-op HBM GB/s", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "handler op sweep (%d operations) on float32 %dx%d tensors (2^%d "
+                               "elements each), inputs resident in HBM"
+                               % (len(op_ms), args.size, args.size,
+                                  int(round(np.log2(args.size * args.size)))),
+                   "device": dev_name, "compute_units": cus},
+        "roofline": roofline,
+        "ops": ops,
+    }
+    if not args.no_cpu:
+        passes, cpu_s = run_cpu(args.cpu_size, args.cpu_seconds)
+        cab = alg_bytes(args.cpu_size, args.cpu_size)
+        cpu_total = sum(cpu_s.values())
+        out["cpu_baseline"] = {
+            "value": round(sum(cab[n] for n in cpu_s) / cpu_total / 1e9, 3), "unit": "GB/s",
+            "cores": 1, "kind": "port",
+            "sample": "%d passes of the same %d-operation sweep on %dx%d float32 tensors with the "
+                      "NumPy oracle (median per operation; NumPy elementwise and reduction "
+                      "routines run on one core); host has %d cores, numpy %s"
+                      % (passes, len(cpu_s), args.cpu_size, args.cpu_size, os.cpu_count(), np.__version__),
+            "ops_gbps": {n: round(cab[n] / s / 1e9, 3) for n, s in cpu_s.items()},
+        }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -31,9 +31,8 @@ SIGNATURES = {
     "bship_shutdown": [],
     "bship_sync": [],
     "bship_device_info": [ctypes.c_char_p, c_size_t, POINTER(c_int)],
-    "bship_timer_start": [],
-    "bship_timer_stop": [],
-    "bship_timer_elapsed_ms": [POINTER(c_float)],
+    "bship_event_record": [c_int],
+    "bship_event_elapsed_ms": [c_int, c_int, POINTER(c_float)],
     "bship_malloc": [c_size_t, POINTER(c_void_p)],
     "bship_free": [_P],
     "bship_pool_trim": [],

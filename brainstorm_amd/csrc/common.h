@@ -21,7 +21,7 @@ struct Context {
     int device = -1;
     int num_cus = 256;
     hipStream_t stream = nullptr;
-    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    hipEvent_t events[BSHIP_MAX_EVENTS] = {nullptr};   // created on first use
     bool debug_sync = false;   // BSHIP_DEBUG_SYNC=1: sync + check after every launch
     int blocks_per_cu = 8;     // streaming kernels launch num_cus*blocks_per_cu blocks
     char name[256] = {0};

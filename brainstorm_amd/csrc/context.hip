@@ -69,8 +69,6 @@ int bship_init(int device) {
     snprintf(g_ctx.name, sizeof(g_ctx.name), "%s (%s)", prop.name, prop.gcnArchName);
     // One stream at the default priority; every kernel and copy goes here in call order.
     BSHIP_HIP(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking));
-    BSHIP_HIP(hipEventCreate(&g_ctx.ev_start));
-    BSHIP_HIP(hipEventCreate(&g_ctx.ev_stop));
     const char* dbg = getenv("BSHIP_DEBUG_SYNC");
     g_ctx.debug_sync = dbg && dbg[0] && dbg[0] != '0';
     const char* bpc = getenv("BSHIP_BLOCKS_PER_CU");
@@ -87,8 +85,8 @@ int bship_shutdown(void) {
     gemm_release();
     rng_release();
     pool_release_all();
-    (void)hipEventDestroy(g_ctx.ev_start);
-    (void)hipEventDestroy(g_ctx.ev_stop);
+    for (hipEvent_t e : g_ctx.events)
+        if (e) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(g_ctx.stream);
     g_ctx = Context();
     return 0;
@@ -110,23 +108,23 @@ int bship_device_info(char* name_host, size_t name_len, int* compute_units) {
     return 0;
 }
 
-int bship_timer_start(void) {
+int bship_event_record(int slot) {
     BSHIP_REQUIRE_INIT();
-    BSHIP_HIP(hipEventRecord(g_ctx.ev_start, g_ctx.stream));
+    BSHIP_REQUIRE_DIM(slot >= 0 && slot < BSHIP_MAX_EVENTS);
+    if (!g_ctx.events[slot]) BSHIP_HIP(hipEventCreate(&g_ctx.events[slot]));
+    BSHIP_HIP(hipEventRecord(g_ctx.events[slot], g_ctx.stream));
     return 0;
 }
 
-int bship_timer_stop(void) {
-    BSHIP_REQUIRE_INIT();
-    BSHIP_HIP(hipEventRecord(g_ctx.ev_stop, g_ctx.stream));
-    return 0;
-}
-
-int bship_timer_elapsed_ms(float* ms_host) {
+int bship_event_elapsed_ms(int start_slot, int stop_slot, float* ms_host) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_PTR(ms_host);
-    BSHIP_HIP(hipEventSynchronize(g_ctx.ev_stop));
-    BSHIP_HIP(hipEventElapsedTime(ms_host, g_ctx.ev_start, g_ctx.ev_stop));
+    BSHIP_REQUIRE_DIM(start_slot >= 0 && start_slot < BSHIP_MAX_EVENTS);
+    BSHIP_REQUIRE_DIM(stop_slot >= 0 && stop_slot < BSHIP_MAX_EVENTS);
+    if (!g_ctx.events[start_slot] || !g_ctx.events[stop_slot])
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_event_elapsed_ms: slot never recorded");
+    BSHIP_HIP(hipEventSynchronize(g_ctx.events[stop_slot]));
+    BSHIP_HIP(hipEventElapsedTime(ms_host, g_ctx.events[start_slot], g_ctx.events[stop_slot]));
     return 0;
 }
 

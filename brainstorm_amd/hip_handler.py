@@ -139,7 +139,7 @@ class HipHandler(Handler):
         self._call(self._lib.bship_cond_f32(COPY_IF, src.ptr, 0.0, dest.ptr, cond.ptr, dest.size))
 
     def create_from_numpy(self, arr):
-        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        arr = np.asarray(arr, dtype=np.float32, order='C')    # keeps 0-d arrays 0-d
         out = self.allocate(arr.shape)
         if out.size:
             self._call(self._lib.bship_h2d(out.ptr, arr.ctypes.data, arr.nbytes))
@@ -163,7 +163,7 @@ class HipHandler(Handler):
         arr = np.asarray(arr)
         if arr.shape != mem.shape:
             arr = np.broadcast_to(arr, mem.shape)
-        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        arr = np.asarray(arr, dtype=np.float32, order='C')
         if mem.size:
             self._call(self._lib.bship_h2d(mem.ptr, arr.ctypes.data, arr.nbytes))
 

@@ -62,11 +62,12 @@ const char* bship_last_error(void);
 /* Device name and compute-unit count of the initialised device. */
 int bship_device_info(char* name_host, size_t name_len, int* compute_units);
 
-/* Timing on the library's stream (hipEvent pair); used to measure kernels
- * where they actually run. start/stop enqueue events, elapsed blocks. */
-int bship_timer_start(void);
-int bship_timer_stop(void);
-int bship_timer_elapsed_ms(float* ms_host);
+/* Timing on the library's stream, where the kernels actually run: record
+ * enqueues a hipEvent into one of BSHIP_MAX_EVENTS slots (no waiting);
+ * elapsed waits for slot `stop` and returns the time between the two records. */
+#define BSHIP_MAX_EVENTS 1024
+int bship_event_record(int slot);
+int bship_event_elapsed_ms(int start_slot, int stop_slot, float* ms_host);
 
 /* ------------------------------- memory ---------------------------------- */
 

@@ -608,13 +608,13 @@ def test_ops_on_unaligned_views(hip, ref):
     flat = rand(rng, (3 * 5000 + 16,))
     fd = hip.create_from_numpy(flat)
     for off in (1, 2, 3, 5):
-        a, b, o = (flat[off:off + 5000], flat[5003 + off:5003 + off + 5000], flat[10007:10007 + 5000])
+        a, b, o = (flat[off:off + 5000], flat[5003 + off:5003 + off + 5000], flat[10012:10012 + 5000])
         want = flat.copy()
-        wa, wb, wo = want[off:off + 5000], want[5003 + off:5003 + off + 5000], want[10007:10007 + 5000]
+        wa, wb, wo = want[off:off + 5000], want[5003 + off:5003 + off + 5000], want[10012:10012 + 5000]
         ref.add_tt(wa, wb, wo)
         ref.sigmoid_deriv(None, wa, wb, wo[:5000])
         fd2 = hip.create_from_numpy(flat)
-        da, db, do = fd2[off:off + 5000], fd2[5003 + off:5003 + off + 5000], fd2[10007:10007 + 5000]
+        da, db, do = fd2[off:off + 5000], fd2[5003 + off:5003 + off + 5000], fd2[10012:10012 + 5000]
         hip.add_tt(da, db, do)
         hip.sigmoid_deriv(None, da, db, do)
         assert_bit_equal(fd2.get(), want, "offset %d" % off)
