@@ -49,7 +49,8 @@ def sources() -> list[str]:
 
 def _compile_one(hipcc: str, src: str, verbose: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+    extra = os.environ.get("BSHIP_EXTRA_HIPCC_FLAGS", "").split()   # e.g. -DNAME=VALUE for experiments
+    cmd = [hipcc] + HIPCC_FLAGS + extra + ["-c", src, "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

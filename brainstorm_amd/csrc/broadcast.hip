@@ -1,7 +1,7 @@
 // Broadcast operations: matrix (op) vector with a row vector (1,N) or a column
 // vector (M,1), broadcast_t along a size-1 axis, and merge/split on the last
-// axis. All are HBM-bound; the vector operand is read once per workgroup and
-// kept in registers (row vector) or fetched once per row tile (column vector).
+// axis. All are HBM-bound; the matrix is streamed once, the vector operand is
+// small and comes out of the caches.
 #pragma clang fp contract(off)
 
 #include "common.h"
@@ -27,73 +27,56 @@ template <bool ACC> struct MvSub { __device__ float apply(float m, float v, floa
 template <bool ACC> struct MvMul { __device__ float apply(float m, float v, float o) const { float r = m * v; return ACC ? o + r : r; } };
 template <bool ACC> struct MvDiv { __device__ float apply(float m, float v, float o) const { float r = m / v; return ACC ? o + r : r; } };
 
-constexpr int kMvUnroll = 4;
-
-// Row vector: a thread owns W consecutive columns and walks down a band of rows
-// with its slice of v in registers. grid.x tiles the columns, grid.y the row
-// bands. NW = N / W.
-template <int W, bool AL, bool ACC, typename F>
+// Row vector: a workgroup handles R consecutive rows of one tile of kBlock*W
+// columns; each lane loads its slice of v once and applies it to R rows.
+// One workgroup per tile (see elementwise.hip for why). NW = N / W.
+template <int W, bool AL, bool ACC, int R, typename F>
 __global__ __launch_bounds__(kBlock) void mv_rowvec_kernel(F f, const float* m, const float* v,
                                                            float* out, int64_t M, int64_t NW,
-                                                           int64_t rows_per_block) {
-    typedef typename VecT<W>::type R;
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+                                                           unsigned col_tiles) {
+    typedef typename VecT<W>::type T;
+    const unsigned ct = blockIdx.x % col_tiles;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x / col_tiles) * R;
+    const int64_t c = static_cast<int64_t>(ct) * kBlock + threadIdx.x;
     if (c >= NW) return;
-    const R vv = vload<W, AL>(v + c * W);
-    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_block;
-    const int64_t r1 = (r0 + rows_per_block < M) ? r0 + rows_per_block : M;
-    for (int64_t r = r0; r < r1; r += kMvUnroll) {
-        R a[kMvUnroll], o[kMvUnroll];
+    const T vv = vload<W, AL>(v + c * W);
+    T a[R], o[R];
 #pragma unroll
-        for (int u = 0; u < kMvUnroll; ++u) {
-            if (r + u < r1) {
-                const int64_t e = ((r + u) * NW + c) * W;
-                a[u] = vload<W, AL>(m + e);
-                if (ACC) o[u] = vload<W, AL>(out + e);
-            }
+    for (int u = 0; u < R; ++u) {
+        if (r0 + u < M) {
+            const int64_t e = ((r0 + u) * NW + c) * W;
+            a[u] = vload<W, AL>(m + e);
+            if (ACC) o[u] = vload<W, AL>(out + e);
         }
+    }
 #pragma unroll
-        for (int u = 0; u < kMvUnroll; ++u) {
-            if (r + u < r1) {
-                const int64_t e = ((r + u) * NW + c) * W;
-                vstore<W, AL>(out + e, vmap(f, a[u], vv, ACC ? o[u] : a[u]));
-            }
+    for (int u = 0; u < R; ++u) {
+        if (r0 + u < M) {
+            const int64_t e = ((r0 + u) * NW + c) * W;
+            vstore<W, AL>(out + e, vmap(f, a[u], vv, ACC ? o[u] : a[u]));
         }
     }
 }
 
-// Column vector: the matrix is cut into tiles of kBlock*W columns of one row; a
-// workgroup strides over groups of kMvUnroll tiles and fetches v[row] per tile.
+// Column vector: one workgroup per tile of kBlock*W columns of one row; v[row]
+// is one broadcast load per tile.
 template <int W, bool AL, bool ACC, typename F>
 __global__ __launch_bounds__(kBlock) void mv_colvec_kernel(F f, const float* m, const float* v,
                                                            float* out, int64_t M, int64_t NW,
-                                                           int64_t tiles_per_row) {
-    typedef typename VecT<W>::type R;
-    const int64_t ntiles = M * tiles_per_row;
-    for (int64_t t0 = static_cast<int64_t>(blockIdx.x) * kMvUnroll; t0 < ntiles;
-         t0 += static_cast<int64_t>(gridDim.x) * kMvUnroll) {
-        R a[kMvUnroll], o[kMvUnroll];
-        float s[kMvUnroll];
-        int64_t idx[kMvUnroll];
-#pragma unroll
-        for (int u = 0; u < kMvUnroll; ++u) {
-            const int64_t t = t0 + u;
-            const int64_t row = t / tiles_per_row;
-            const int64_t c = (t - row * tiles_per_row) * kBlock + threadIdx.x;
-            idx[u] = (t < ntiles && c < NW) ? (row * NW + c) * W : -1;
-            if (idx[u] >= 0) {
-                s[u] = v[row];
-                a[u] = vload<W, AL>(m + idx[u]);
-                if (ACC) o[u] = vload<W, AL>(out + idx[u]);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kMvUnroll; ++u) {
-            if (idx[u] >= 0)
-                vstore<W, AL>(out + idx[u], vmap(f, a[u], splat(a[u], s[u]), ACC ? o[u] : a[u]));
-        }
-    }
+                                                           unsigned tiles_per_row) {
+    typedef typename VecT<W>::type T;
+    const int64_t row = blockIdx.x / tiles_per_row;
+    const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
+    if (c >= NW) return;
+    const int64_t e = (row * NW + c) * W;
+    const float s = v[row];
+    const T a = vload<W, AL>(m + e);
+    T o = a;
+    if (ACC) o = vload<W, AL>(out + e);
+    vstore<W, AL>(out + e, vmap(f, a, splat(a, s), o));
 }
+
+constexpr int kMvRows = 4;
 
 template <bool ACC, typename F>
 int launch_mv(const char* name, F f, const float* m, const float* v, float* out, int64_t M,
@@ -102,27 +85,27 @@ int launch_mv(const char* name, F f, const float* m, const float* v, float* out,
     const bool vec = (N % 4 == 0);
     const int64_t NW = vec ? N / 4 : N;
     const dim3 blk(kBlock);
+    const int64_t col_tiles = ceil_div(NW, kBlock);
     if (!v_is_col) {
         const bool al = aligned16(m) && aligned16(out) && aligned16(v);
-        const int64_t target = static_cast<int64_t>(c.num_cus) * c.blocks_per_cu;
-        const int64_t gx = ceil_div(NW, kBlock);
-        int64_t bands = target / gx;
-        if (bands < 1) bands = 1;
-        int64_t rpb = ceil_div(M, bands);
-        if (rpb < 2 * kMvUnroll) rpb = 2 * kMvUnroll;
-        if (ceil_div(M, rpb) > 65535) rpb = ceil_div(M, 65535);
-        dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(ceil_div(M, rpb)));
+        const int64_t blocks = col_tiles * ceil_div(M, kMvRows);
+        if (blocks > 0x7fffffff || col_tiles > 0x7fffffff)
+            return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: matrix too large for one launch", name);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        const unsigned ctl = static_cast<unsigned>(col_tiles);
         if (vec && al)
-            hipLaunchKernelGGL((mv_rowvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, true, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
         else if (vec)
-            hipLaunchKernelGGL((mv_rowvec_kernel<4, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
         else
-            hipLaunchKernelGGL((mv_rowvec_kernel<1, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, rpb);
+            hipLaunchKernelGGL((mv_rowvec_kernel<1, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
     } else {
         const bool al = aligned16(m) && aligned16(out);
-        const int64_t tpr = ceil_div(NW, kBlock);
-        const int64_t groups = ceil_div(M * tpr, kMvUnroll);
-        dim3 grid(stream_grid(groups));
+        const int64_t blocks = col_tiles * M;
+        if (blocks > 0x7fffffff)
+            return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: matrix too large for one launch", name);
+        const dim3 grid(static_cast<unsigned>(blocks));
+        const unsigned tpr = static_cast<unsigned>(col_tiles);
         if (vec && al)
             hipLaunchKernelGGL((mv_colvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
         else if (vec)

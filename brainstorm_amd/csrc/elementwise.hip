@@ -1,64 +1,78 @@
 // Elementwise handler operations: one streaming kernel template, instantiated
-// per operation. Every operation is HBM-bound; the kernel moves 128 bits per
-// lane per access, keeps kUnroll independent accesses in flight per lane and
-// uses a grid of a few workgroups per compute unit that strides over tiles.
+// per operation. Every operation is HBM-bound. Measured on MI355X, the fastest
+// shape for such kernels is the simplest one: each lane moves one 128-bit
+// vector per operand with non-temporal accesses, a workgroup of 256 lanes
+// covers one tile of 1024 floats, and the grid has one workgroup per tile
+// (hundreds of thousands of short workgroups, dispatched in address order)
+// rather than a few long-running ones that stride over the tiles.
 //
 // Arithmetic follows NumPy's float32 evaluation order exactly (each NumPy
 // temporary is one float32 rounding), so products are never fused into adds.
 #pragma clang fp contract(off)
 
 #include "common.h"
+#include "fastmath64.h"
 
 namespace bship {
 
-constexpr int kUnroll = 4;
-constexpr size_t kTile = static_cast<size_t>(kBlock) * 4 * kUnroll;   // floats per tile
+constexpr size_t kTile = static_cast<size_t>(kBlock) * 4;   // floats per workgroup and vector
 
 // F::apply(v0, v1, v2) -> result. NIN pointers are read (p0..), `out` is written.
-// `out` may alias any input, so nothing here is __restrict__; all loads of a
-// tile are issued before its stores.
-template <int NIN, bool AL, typename F>
+// `out` may alias any input, so nothing here is __restrict__; a lane loads all
+// of its operands before it stores. VPL = 128-bit vectors per lane: 1 for the
+// cheap operations, more for the float64 transcendentals so that a wavefront
+// has enough loads in flight to hide its long arithmetic phase.
+template <int NIN, bool AL, int VPL, typename F>
 __global__ __launch_bounds__(kBlock) void ew_kernel(F f, const float* p0, const float* p1,
                                                     const float* p2, float* out, size_t n) {
-    const size_t ntiles = n / kTile;
-    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const size_t base = t * kTile + threadIdx.x * 4;
-        f4 r0[kUnroll], r1[kUnroll], r2[kUnroll];
+    const size_t base = static_cast<size_t>(blockIdx.x) * (kTile * VPL) + threadIdx.x * 4;
+    f4 r0[VPL], r1[VPL], r2[VPL];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const size_t q = base + u * (kBlock * 4);
-            r0[u] = vload<4, AL>(p0 + q);
-            if (NIN > 1) r1[u] = vload<4, AL>(p1 + q);
-            if (NIN > 2) r2[u] = vload<4, AL>(p2 + q);
+    for (int u = 0; u < VPL; ++u) {
+        const size_t i = base + u * kTile;
+        if (i + 4 <= n) {
+            r0[u] = vload<4, AL>(p0 + i);
+            if (NIN > 1) r1[u] = vload<4, AL>(p1 + i);
+            if (NIN > 2) r2[u] = vload<4, AL>(p2 + i);
         }
+    }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < VPL; ++u) {
+        const size_t i = base + u * kTile;
+        if (i + 4 <= n) {
             f4 o;
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 o[k] = f.apply(r0[u][k], NIN > 1 ? r1[u][k] : 0.0f, NIN > 2 ? r2[u][k] : 0.0f);
-            vstore<4, AL>(out + base + u * (kBlock * 4), o);
+            vstore<4, AL>(out + i, o);
+        } else {
+            for (size_t j = i; j < n; ++j)     // the last, partial vector of the array
+                out[j] = f.apply(p0[j], NIN > 1 ? p1[j] : 0.0f, NIN > 2 ? p2[j] : 0.0f);
         }
     }
-    // tail shorter than one tile: last workgroup, scalar
-    if (blockIdx.x == gridDim.x - 1) {
-        for (size_t i = ntiles * kTile + threadIdx.x; i < n; i += kBlock)
-            out[i] = f.apply(p0[i], NIN > 1 ? p1[i] : 0.0f, NIN > 2 ? p2[i] : 0.0f);
-    }
 }
+
+template <typename F, typename = void> struct VectorsPerLane { static constexpr int value = 1; };
+template <typename F> struct VectorsPerLane<F, std::void_t<decltype(F::kVectorsPerLane)>> {
+    static constexpr int value = F::kVectorsPerLane;
+};
 
 template <int NIN, typename F>
 int launch_ew(const char* name, F f, const float* p0, const float* p1, const float* p2,
               float* out, size_t n) {
     if (n == 0) return 0;
-    unsigned grid = stream_grid(static_cast<int64_t>(n / kTile));
+    constexpr int VPL = VectorsPerLane<F>::value;
+    const size_t tiles = (n + kTile * VPL - 1) / (kTile * VPL);
+    if (tiles > 0x7fffffffu)
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", name, n);
+    const dim3 grid(static_cast<unsigned>(tiles));
     bool al = aligned16(p0) && aligned16(out) && (NIN < 2 || aligned16(p1)) &&
               (NIN < 3 || aligned16(p2));
     if (al)
-        hipLaunchKernelGGL((ew_kernel<NIN, true, F>), dim3(grid), dim3(kBlock), 0, ctx().stream, f,
+        hipLaunchKernelGGL((ew_kernel<NIN, true, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
                            p0, p1, p2, out, n);
     else
-        hipLaunchKernelGGL((ew_kernel<NIN, false, F>), dim3(grid), dim3(kBlock), 0, ctx().stream, f,
+        hipLaunchKernelGGL((ew_kernel<NIN, false, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
                            p0, p1, p2, out, n);
     return check_launch(name);
 }
@@ -92,22 +106,21 @@ struct SignOp {
     }
 };
 struct SqrtOp { __device__ float apply(float x, float, float) const { return sqrtf(x); } };
-// Transcendentals are evaluated in float64 and rounded once, which gives the
-// correctly rounded float32 value; the kernels stay memory-bound.
+// Transcendentals are evaluated in float64 and rounded once (fastmath64.h).
+#ifndef BSHIP_HEAVY_VPL
+#define BSHIP_HEAVY_VPL 2
+#endif
 struct LogOp {
-    __device__ float apply(float x, float, float) const { return static_cast<float>(log(static_cast<double>(x))); }
+    static constexpr int kVectorsPerLane = BSHIP_HEAVY_VPL;
+    __device__ float apply(float x, float, float) const { return log_f32(x); }
 };
 struct TanhOp {
-    __device__ float apply(float x, float, float) const { return static_cast<float>(tanh(static_cast<double>(x))); }
+    static constexpr int kVectorsPerLane = BSHIP_HEAVY_VPL;
+    __device__ float apply(float x, float, float) const { return tanh_f32(x); }
 };
-// numpy 283-287: 1/(1+exp(-x)) for x >= 0, exp(x)/(1+exp(x)) for x < 0
 struct SigmoidOp {
-    __device__ float apply(float x, float, float) const {
-        double xd = static_cast<double>(x);
-        double e = exp(-fabs(xd));
-        double r = (x >= 0.0f ? 1.0 : e) / (1.0 + e);
-        return (x != x) ? x : static_cast<float>(r);
-    }
+    static constexpr int kVectorsPerLane = BSHIP_HEAVY_VPL;
+    __device__ float apply(float x, float, float) const { return sigmoid_f32(x); }
 };
 // numpy 277-278: x*(x>0); the mask is 1.0 or 0.0, so negatives give -0.0
 struct RelOp {
@@ -116,7 +129,7 @@ struct RelOp {
 // numpy 303-305: x*(x>=0) + (exp(x)-1)*(x<0), every step in float32
 struct ElOp {
     __device__ float apply(float x, float, float) const {
-        float e = static_cast<float>(exp(static_cast<double>(x)));
+        float e = exp_f32(x);
         float t1 = x * (x >= 0.0f ? 1.0f : 0.0f);
         float t2 = (e - 1.0f) * (x < 0.0f ? 1.0f : 0.0f);
         return t1 + t2;

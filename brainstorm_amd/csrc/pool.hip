@@ -105,49 +105,40 @@ void pool_release_all() {
 
 // ------------------------------- kernels ----------------------------------
 
-// Each block-iteration covers a tile of kBlock*4*kFillUnroll floats.
-constexpr int kFillUnroll = 4;
+// One workgroup per tile of kBlock*4 floats, one 128-bit access per lane.
+constexpr size_t kCopyTile = static_cast<size_t>(kBlock) * 4;
 
 template <bool AL>
 __global__ __launch_bounds__(kBlock) void fill_kernel(float* __restrict__ p, float val, size_t n) {
-    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
-    const size_t ntiles = n / tile;
-    const f4 vv = {val, val, val, val};
-    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        float* q = p + t * tile + threadIdx.x * 4;
-#pragma unroll
-        for (int u = 0; u < kFillUnroll; ++u) vstore<4, AL>(q + u * kBlock * 4, vv);
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i + 4 <= n) {
+        const f4 vv = {val, val, val, val};
+        vstore<4, AL>(p + i, vv);
+    } else {
+        for (size_t j = i; j < n; ++j) p[j] = val;
     }
-    // tail (fewer than one tile), handled by the first block only
-    if (blockIdx.x == 0)
-        for (size_t i = ntiles * tile + threadIdx.x; i < n; i += kBlock) p[i] = val;
 }
 
 template <bool AL>
 __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ s,
                                                       float* __restrict__ d, size_t n) {
-    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
-    const size_t ntiles = n / tile;
-    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const size_t off = t * tile + threadIdx.x * 4;
-        f4 r[kFillUnroll];
-#pragma unroll
-        for (int u = 0; u < kFillUnroll; ++u) r[u] = vload<4, AL>(s + off + u * kBlock * 4);
-#pragma unroll
-        for (int u = 0; u < kFillUnroll; ++u) vstore<4, AL>(d + off + u * kBlock * 4, r[u]);
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i + 4 <= n) {
+        vstore<4, AL>(d + i, vload<4, AL>(s + i));
+    } else {
+        for (size_t j = i; j < n; ++j) d[j] = s[j];
     }
-    if (blockIdx.x == 0)
-        for (size_t i = ntiles * tile + threadIdx.x; i < n; i += kBlock) d[i] = s[i];
 }
 
 int launch_fill(float* p, float val, size_t n) {
     if (n == 0) return 0;
-    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
-    unsigned grid = stream_grid(static_cast<int64_t>(n / tile));
+    const size_t tiles = (n + kCopyTile - 1) / kCopyTile;
+    if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "fill: %zu elements exceed one launch", n);
+    const dim3 grid(static_cast<unsigned>(tiles));
     if (aligned16(p))
-        hipLaunchKernelGGL(fill_kernel<true>, dim3(grid), dim3(kBlock), 0, ctx().stream, p, val, n);
+        hipLaunchKernelGGL(fill_kernel<true>, grid, dim3(kBlock), 0, ctx().stream, p, val, n);
     else
-        hipLaunchKernelGGL(fill_kernel<false>, dim3(grid), dim3(kBlock), 0, ctx().stream, p, val, n);
+        hipLaunchKernelGGL(fill_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, p, val, n);
     return check_launch("fill_kernel");
 }
 
@@ -218,14 +209,15 @@ int bship_d2d(void* dst, const void* src, size_t nbytes) {
         return 0;
     }
     const size_t n = nbytes / 4;
-    const size_t tile = static_cast<size_t>(kBlock) * 4 * kFillUnroll;
-    unsigned grid = stream_grid(static_cast<int64_t>(n / tile));
+    const size_t tiles = (n + kCopyTile - 1) / kCopyTile;
+    if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "copy: %zu bytes exceed one launch", nbytes);
+    const dim3 grid(static_cast<unsigned>(tiles));
     const float* s = static_cast<const float*>(src);
     float* d = static_cast<float*>(dst);
     if (aligned16(s) && aligned16(d))
-        hipLaunchKernelGGL(copy_kernel<true>, dim3(grid), dim3(kBlock), 0, ctx().stream, s, d, n);
+        hipLaunchKernelGGL(copy_kernel<true>, grid, dim3(kBlock), 0, ctx().stream, s, d, n);
     else
-        hipLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(kBlock), 0, ctx().stream, s, d, n);
+        hipLaunchKernelGGL(copy_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, s, d, n);
     return check_launch("copy_kernel");
 }
 

@@ -1,0 +1,113 @@
+"""CPU-only: DeviceArray view arithmetic (no device memory is touched).
+
+The array contract is the one brainstorm/tests/test_array.py states for its DebugArray (integer
+multi-indexing gives the same type with reduced shape, out-of-range raises IndexError) plus what
+the buffer manager and the recurrent layers do with arrays: slices, negative indices, reshape,
+zero-sized arrays (buffers.py:67-83, lstm_layer.py:106-117)."""
+import itertools
+
+import numpy as np
+import pytest
+
+from brainstorm_amd.device_array import DeviceArray
+
+BASE_PTR = 0x7f0000001000
+
+
+def make(shape):
+    return DeviceArray(BASE_PTR, tuple(shape), None, None), np.zeros(shape, dtype=np.float32)
+
+
+def offset_of(view, base):
+    return (view.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // 4
+
+
+def npview(host, key):
+    """host[key] as an array view even when every axis is indexed (NumPy would return a scalar)."""
+    key = key if isinstance(key, tuple) else (key,)
+    if not any(k is Ellipsis for k in key):
+        key = key + (Ellipsis,)
+    return host[key]
+
+
+def check_same(dev, host, host_base):
+    assert dev.shape == host.shape
+    assert dev.size == host.size
+    if host.size:
+        assert (dev.ptr - BASE_PTR) // 4 == offset_of(host, host_base)
+
+
+KEYS = [0, 1, -1, slice(None), slice(1, 3), slice(-2, None), slice(0, 0), slice(None, -1),
+        (0, 1), (1, 2, 3), (-1, -1), (1, slice(None)), (1, slice(1, 2)), (-1, slice(1, None)),
+        (slice(None), slice(None)), (slice(1, 2), slice(None)), (0, 2, slice(1, 3)), (Ellipsis,),
+        (1, Ellipsis), (slice(2, 5), Ellipsis)]
+
+
+@pytest.mark.parametrize("shape", [(5,), (4, 3), (3, 4, 5), (2, 1, 3, 4), (6, 1)])
+def test_dense_views_match_numpy(shape):
+    dev, host = make(shape)
+    for key in KEYS:
+        try:
+            want = npview(host, key)
+        except IndexError:
+            with pytest.raises(IndexError):
+                dev[key]
+            continue
+        if want.size > 1 and not want.flags["C_CONTIGUOUS"]:
+            with pytest.raises(NotImplementedError):
+                dev[key]
+            continue
+        check_same(dev[key], want, host)
+
+
+def test_integer_multi_indexing_like_debug_array():
+    # brainstorm/tests/test_array.py:16-63
+    dev, host = make((2, 3, 4, 5))
+    for key in itertools.product(range(2), range(3)):
+        check_same(dev[key], npview(host, key), host)
+    check_same(dev[1, 2, 3], npview(host, (1, 2, 3)), host)
+    assert dev[1, 2, 3, 4].shape == ()
+    for bad in (2, (0, 3), (0, 0, 4), (0, 0, 0, 5), -3):
+        with pytest.raises(IndexError):
+            dev[bad]
+    with pytest.raises(IndexError):
+        dev[0, 0, 0, 0, 0]
+
+
+def test_views_of_views_and_reshape_alias():
+    dev, host = make((101, 100, 8))
+    v, h = dev[:-1], host[:-1]
+    check_same(v, h, host)
+    check_same(v.reshape((100 * 100, 8)), h.reshape(100 * 100, 8), host)
+    check_same(dev[-1], host[-1], host)                      # context slot of a time-major buffer
+    check_same(dev[3].reshape(800), host[3].reshape(800), host)
+    check_same(dev.reshape(-1, 8)[200:300], host.reshape(-1, 8)[200:300], host)
+    check_same(dev.reshape((101, 800))[5:7].reshape((2, 100, 8)), host[5:7], host)
+    with pytest.raises(ValueError):
+        dev.reshape((7, 7))
+    with pytest.raises(ValueError):
+        dev.reshape((-1, -1))
+
+
+def test_row_pitched_views_are_refused():
+    dev, _ = make((4, 6))
+    for key in [(slice(None), slice(1, 3)), (slice(0, 2), 0), (slice(None), 2)]:
+        with pytest.raises(NotImplementedError):
+            dev[key]
+    dev[:, 0:6]                     # the full feature range of a hub stays dense
+    dev[2:3, 1:3]                   # a single row is dense whatever its columns
+    with pytest.raises(NotImplementedError):
+        dev[::2]
+
+
+def test_zero_sized_and_zero_dimensional():
+    empty = DeviceArray(0, (1, 0, 7), None, None)
+    assert empty.size == 0 and empty[0].shape == (0, 7) and empty[:, :, 2:4].shape == (1, 0, 2)
+    assert empty.reshape((0,)).shape == (0,)
+    scalar = DeviceArray(BASE_PTR, (), None, None)
+    assert scalar.size == 1 and scalar.ndim == 0 and scalar.reshape((1, 1)).shape == (1, 1)
+    with pytest.raises(IndexError):
+        scalar[0]
+    dev, host = make((3, 4))
+    check_same(dev[1:1], host[1:1], host)
+    assert dev.nbytes == 48 and len(dev) == 3
