@@ -1,0 +1,159 @@
+"""GPU parity of the four network workloads: the same op-trace drivers
+(brainstorm_amd/drivers) run on HipHandler and on the float32 CPU oracle with
+identical seeded inputs, weights and dropout masks.
+
+What is compared and to which bar:
+  * dropout masks and max-pooling argmax: bit-exact;
+  * loss: 1e-5 relative;
+  * every other buffer (activations, deltas, the flat gradient vector, parameters
+    after momentum steps): max |hip - oracle| <= TOL * max |oracle| per buffer. The
+    two sides sum the same float32 products in different orders inside the matrix
+    products (hipBLASLt tiles vs OpenBLAS), so single elements of a long
+    back-propagated chain cannot be held to 1e-5 of their own magnitude; the bar
+    is 1e-5 of the buffer's scale for single passes and 1e-4 for gradients that
+    went through a 100-step recurrence or through training steps.
+"""
+import numpy as np
+import pytest
+
+from brainstorm_amd.drivers import configs
+from brainstorm_amd.drivers.net import MomentumStepper
+from oracle.numpy_ref_handler import NumpyRefHandler
+from util import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+def scaled_err(got, want):
+    scale = float(np.max(np.abs(want)))
+    return float(np.max(np.abs(got.astype(np.float64) - want))) / (scale if scale > 0 else 1.0)
+
+
+def both(builder, hip, seed_rng, **kw):
+    ref = NumpyRefHandler(F32, seed=seed_rng)
+    hip.rnd.seed(seed_rng)
+    net_h, data = builder(hip, **kw)
+    net_r, data_r = builder(ref, **kw)
+    for k in data:
+        assert np.array_equal(data[k], data_r[k])
+    net_h.provide_external_data(data)
+    net_r.provide_external_data(data_r)
+    return net_h, net_r
+
+
+def compare_all(net_h, net_r, tol, exact=()):
+    worst = {}
+    for name in net_r.layers:
+        bh, br = net_h.buffers[name], net_r.buffers[name]
+        for group in ("outputs", "internals", "output_deltas"):
+            for key, want in getattr(br, group).items():
+                got = net_h.handler.get_numpy_copy(getattr(bh, group)[key])
+                tag = "%s.%s.%s" % (name, group, key)
+                if (name, key) in exact:
+                    assert_bit_equal(got, want, tag)
+                else:
+                    worst[tag] = scaled_err(got, want)
+    bad = {k: v for k, v in worst.items() if v > tol}
+    assert not bad, "buffers over %g: %r" % (tol, bad)
+    return max(worst.values())
+
+
+def test_mlp_training_steps(hip):
+    net_h, net_r = both(configs.build_mlp, hip, 21)
+    net_h.forward_pass(training_pass=True)
+    net_r.forward_pass(training_pass=True)
+    net_h.backward_pass()
+    net_r.backward_pass()
+    exact = {("drop1", "mask"), ("drop2", "mask"), ("drop3", "mask")}
+    worst = compare_all(net_h, net_r, 1e-5, exact)
+    loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
+    assert abs(loss_h - loss_r) <= 1e-5 * abs(loss_r)
+    g_err = scaled_err(net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients)
+    assert g_err <= 1e-5, g_err
+    # 20 momentum steps (lr 0.1, momentum 0.9 as in examples/mnist_pi.py:46) with fresh masks
+    st_h, st_r = MomentumStepper(0.1, 0.9), MomentumStepper(0.1, 0.9)
+    st_h.start(net_h)
+    st_r.start(net_r)
+    for _ in range(20):
+        st_h.run()
+        st_r.run()
+    for k in ("drop1", "drop2", "drop3"):
+        assert_bit_equal(net_h.get(k, "internals", "mask"), net_r.get(k, "internals", "mask"), k)
+    p_err = scaled_err(net_h.handler.get_numpy_copy(net_h.parameters), net_r.parameters)
+    assert p_err <= 1e-4, p_err
+    loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
+    assert abs(loss_h - loss_r) <= 1e-4 * abs(loss_r)
+    print("mlp: worst buffer %.2e, gradient %.2e, parameters after 20 steps %.2e" % (worst, g_err, p_err))
+
+
+def test_lstm_full_size_forward_backward(hip):
+    # the full configuration: T=100, batch 100, 205 symbols, 1000 cells, full BPTT
+    net_h, net_r = both(configs.build_lstm, hip, 22)
+    net_h.forward_pass(training_pass=True)
+    net_r.forward_pass(training_pass=True)
+    loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
+    assert abs(loss_h - loss_r) <= 1e-5 * abs(loss_r), (loss_h, loss_r)
+    for key in ("Za", "Ib", "Ca", "Cb"):
+        err = scaled_err(net_h.get("lstm", "internals", key), net_r.get("lstm", "internals", key))
+        assert err <= 1e-5, (key, err)
+    assert scaled_err(net_h.get("lstm", "outputs", "default"), net_r.get("lstm", "outputs", "default")) <= 1e-5
+    net_h.backward_pass()
+    net_r.backward_pass()
+    g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
+    worst = 0.0
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        err = scaled_err(g_h[a:b], g_r[a:b])
+        worst = max(worst, err)
+        assert err <= 1e-4, (name, err)
+    d_err = scaled_err(net_h.get("Input", "output_deltas", "default"), net_r.get("Input", "output_deltas", "default"))
+    assert d_err <= 1e-4, d_err
+    print("lstm: worst gradient block %.2e, input deltas %.2e" % (worst, d_err))
+
+
+def test_highway_batchnorm_blocks(hip):
+    # two blocks at the configuration's width and batch (the oracle's matrix products bound the size)
+    net_h, net_r = both(configs.build_highway, hip, 23, blocks=2)
+    net_h.forward_pass(training_pass=True)
+    net_r.forward_pass(training_pass=True)
+    net_h.backward_pass()
+    net_r.backward_pass()
+    worst = compare_all(net_h, net_r, 2e-5)
+    loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
+    assert abs(loss_h - loss_r) <= 1e-5 * abs(loss_r)
+    g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        assert scaled_err(g_h[a:b], g_r[a:b]) <= 2e-5, name
+    # the running statistics (parameters mu, sigma) moved identically
+    assert scaled_err(net_h.handler.get_numpy_copy(net_h.parameters), net_r.parameters) <= 1e-6
+    print("highway: worst buffer %.2e" % worst)
+
+
+def test_cnn_forward_backward(hip):
+    net_h, net_r = both(configs.build_cnn, hip, 24)
+    net_h.forward_pass(training_pass=True)
+    net_r.forward_pass(training_pass=True)
+    # Pooling must agree exactly GIVEN the same input: feed the oracle's conv outputs to the GPU pool
+    for conv, pool in (("conv1", "pool1"), ("conv2", "pool2")):
+        x = net_r.get(conv, "outputs", "default")
+        bh = net_h.buffers[pool]
+        saved = net_h.handler.get_numpy_copy(bh.inputs["default"])
+        net_h.handler.set_from_numpy(bh.inputs["default"], x)
+        net_h.layers[pool].forward_pass(bh, True)
+        assert_bit_equal(net_h.get(pool, "outputs", "default"), net_r.get(pool, "outputs", "default"), pool)
+        assert_bit_equal(net_h.get(pool, "internals", "argmax"), net_r.get(pool, "internals", "argmax"), pool + " argmax")
+        net_h.handler.set_from_numpy(bh.inputs["default"], saved)
+        net_h.layers[pool].forward_pass(bh, True)
+    loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
+    assert abs(loss_h - loss_r) <= 1e-5 * abs(loss_r)
+    for name in ("conv1", "conv2", "fc", "out"):
+        assert scaled_err(net_h.get(name, "outputs", "default"), net_r.get(name, "outputs", "default")) <= 1e-5, name
+    net_h.backward_pass()
+    net_r.backward_pass()
+    g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
+    worst = 0.0
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        err = scaled_err(g_h[a:b], g_r[a:b])
+        worst = max(worst, err)
+        assert err <= 5e-5, (name, err)
+    print("cnn: worst gradient block %.2e" % worst)
