@@ -49,6 +49,7 @@ def alg_bytes(rows, cols):
         "add_mv_col": 8 * n + 4 * rows, "mult_mv_col": 8 * n + 4 * rows,
         "binarize_v": 4 * n + 4 * rows,
         "index_m_by_v": 12 * rows,          # label + gathered element + result per row
+        "copy_to": 8 * n, "fill": 4 * n,
     }
 
 
@@ -78,6 +79,8 @@ def sweep_ops(h, t):
         ("mult_mv_col", lambda: h.mult_mv(t["a"], t["col"], t["out"])),
         ("binarize_v", lambda: h.binarize_v(t["labels"], t["out"])),
         ("index_m_by_v", lambda: h.index_m_by_v(t["a"], t["labels"], t["picked"])),
+        ("copy_to", lambda: h.copy_to(t["a"], t["out"])),
+        ("fill", lambda: h.fill(t["out"], 0.5)),
     ]
 
 
@@ -162,6 +165,44 @@ def run_gpu(size, steps, warmup):
     return hip, name, cus, elapsed, {n: float(np.mean(v)) for n, v in per_op_ms.items()}
 
 
+def time_net(handler, builder, steps, warmup, sync, **kw):
+    """Training steps per second of one network workload (forward + backward + momentum update,
+    inputs uploaded once; the per-step loss read-back of a Trainer is included)."""
+    from brainstorm_amd.drivers.net import MomentumStepper
+    net, data = builder(handler, **kw)
+    net.provide_external_data(data)
+    stepper = MomentumStepper(0.1, 0.9)
+    stepper.start(net)
+    for _ in range(warmup):
+        stepper.run()
+        net.get("loss", "outputs", "loss")
+    sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        stepper.run()
+        net.get("loss", "outputs", "loss")      # device-to-host copy + wait, as trainer.py:100 does
+    sync()
+    dt = (time.perf_counter() - t0) / steps
+    samples = data["default"].shape[0] * data["default"].shape[1]
+    return {"ms_per_step": round(dt * 1e3, 3), "samples_per_s": round(samples / dt, 1)}
+
+
+def run_nets_gpu(hip):
+    from brainstorm_amd.drivers import configs
+    return {
+        "mlp_784-1200-1200-10_batch100": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize),
+        "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
+    }
+
+
+def run_nets_cpu(ref):
+    from brainstorm_amd.drivers import configs
+    return {
+        "mlp_784-1200-1200-10_batch100": time_net(ref, configs.build_mlp, 10, 1, lambda: None),
+        "lstm_205-1000-205_T100_batch100": time_net(ref, configs.build_lstm, 1, 0, lambda: None),
+    }
+
+
 def run_cpu(size, budget_s):
     """Times the CPU oracle on the (size, size) sweep: whole passes until ~budget_s is spent."""
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
@@ -192,6 +233,7 @@ def main():
     ap.add_argument("--cpu-size", type=int, default=4096)
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-nets", action="store_true", help="skip the MLP/LSTM samples/s runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the handler path has no multi-GPU part "
@@ -228,6 +270,9 @@ def main():
         "roofline": roofline,
         "ops": ops,
     }
+    if not args.no_nets:
+        # second part of the metric: training samples/s of the MLP and LSTM workloads
+        out["nets"] = run_nets_gpu(hip)
     if not args.no_cpu:
         passes, cpu_s = run_cpu(args.cpu_size, args.cpu_seconds)
         cab = alg_bytes(args.cpu_size, args.cpu_size)
@@ -241,6 +286,9 @@ def main():
                       % (passes, len(cpu_s), args.cpu_size, args.cpu_size, os.cpu_count(), np.__version__),
             "ops_gbps": {n: round(cab[n] / s / 1e9, 3) for n, s in cpu_s.items()},
         }
+        if not args.no_nets:
+            from oracle.numpy_ref_handler import NumpyRefHandler
+            out["cpu_baseline"]["nets"] = run_nets_cpu(NumpyRefHandler(F32, seed=0))
     print(json.dumps(out))
 
 

@@ -12,6 +12,11 @@ What is compared and to which bar:
     back-propagated chain cannot be held to 1e-5 of their own magnitude; the bar
     is 1e-5 of the buffer's scale for single passes and 1e-4 for gradients that
     went through a 100-step recurrence or through training steps.
+  * deltas behind a ReLU: `rel_deriv` is a discrete decision (y > 0). A pre-activation
+    within rounding distance of zero can land on different sides on the two handlers
+    (about one unit in a million at width 4096 x batch 2048); such a unit's delta then
+    differs by its full size. The Highway test therefore compares the backward pass
+    from one common forward state (the oracle's activations uploaded to the GPU).
 """
 import numpy as np
 import pytest
@@ -116,17 +121,32 @@ def test_highway_batchnorm_blocks(hip):
     net_h, net_r = both(configs.build_highway, hip, 23, blocks=2)
     net_h.forward_pass(training_pass=True)
     net_r.forward_pass(training_pass=True)
-    net_h.backward_pass()
-    net_r.backward_pass()
-    worst = compare_all(net_h, net_r, 2e-5)
+    worst_fwd = 0.0
+    for name in net_r.layers:
+        for group in ("outputs", "internals"):
+            for key, want in getattr(net_r.buffers[name], group).items():
+                err = scaled_err(net_h.get(name, group, key), want)
+                worst_fwd = max(worst_fwd, err)
+                assert err <= 1e-5, (name, group, key, err)
     loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
     assert abs(loss_h - loss_r) <= 1e-5 * abs(loss_r)
-    g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
-    for name, (a, b, _) in net_r.parameter_slices().items():
-        assert scaled_err(g_h[a:b], g_r[a:b]) <= 2e-5, name
     # the running statistics (parameters mu, sigma) moved identically
     assert scaled_err(net_h.handler.get_numpy_copy(net_h.parameters), net_r.parameters) <= 1e-6
-    print("highway: worst buffer %.2e" % worst)
+    # Backward from the SAME forward state: rel_deriv is a discrete decision (y > 0), and with
+    # 2 x 8M ReLU units a few pre-activations lie within rounding distance of zero and land on
+    # different sides on the two handlers; each such unit changes a whole row of upstream deltas.
+    # Giving both sides the oracle's activations removes that (and nothing else) from the comparison.
+    for name in net_r.layers:
+        for group in ("outputs", "internals"):
+            for key, want in getattr(net_r.buffers[name], group).items():
+                net_h.handler.set_from_numpy(getattr(net_h.buffers[name], group)[key], want)
+    net_h.backward_pass()
+    net_r.backward_pass()
+    worst = compare_all(net_h, net_r, 1e-5)
+    g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        assert scaled_err(g_h[a:b], g_r[a:b]) <= 1e-5, name
+    print("highway: worst forward buffer %.2e, worst backward buffer %.2e" % (worst_fwd, worst))
 
 
 def test_cnn_forward_backward(hip):
