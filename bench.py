@@ -34,6 +34,20 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 F32 = np.float32
 
 
+# HBM bytes per launch at the default 16384x16384 workload, measured with
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (two runs of this script) and scaled by what
+# the same counters read for the sweep's 1 GiB copy_to (factors 2.000 and 0.999); the table and
+# the commands are in profiles/op_sweep_2p28_hbm_traffic.md. MiB per launch.
+MEASURED_TRAFFIC_MIB_2P28 = {
+    "add_tt": 3071.2, "mult_tt": 3071.2, "divide_tt": 3071.2, "mult_add_st": 3071.2,
+    "sigmoid_deriv": 3071.2, "tanh_deriv": 3071.2, "rel_deriv": 3071.2,
+    "sigmoid": 2047.3, "tanh": 2047.3, "log_t": 2047.3, "rel": 2047.9, "clip_t": 2047.3,
+    "sqrt_t": 2047.2, "copy_to": 2048.0, "fill": 1024.0, "softmax_m": 2047.4,
+    "add_mv_row": 2047.5, "mult_mv_row": 2047.5, "add_mv_col": 2049.4, "mult_mv_col": 2049.4,
+    "sum_t_axis0": 1025.0, "sum_t_axis1": 1024.5, "sum_t_all": 1024.5, "binarize_v": 1025.1,
+}
+
+
 def alg_bytes(rows, cols):
     """Minimum HBM traffic of each sweep operation on a (rows, cols) float32 tensor."""
     n = rows * cols
@@ -254,7 +268,9 @@ def main():
     roofline = {
         "kernel": dominant, "bound": "hbm",
         "achieved": ops[dominant]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": ops[dominant]["frac"], "traffic": None,
+        "frac": ops[dominant]["frac"],
+        "traffic": (int(MEASURED_TRAFFIC_MIB_2P28[dominant] * 2 ** 20)
+                    if args.size == 16384 and dominant in MEASURED_TRAFFIC_MIB_2P28 else None),
         "alg_bytes_per_launch": ab[dominant], "ms_per_launch": ops[dominant]["ms"],
     }
     out = {
