@@ -69,7 +69,10 @@ static int launch_colsum(const float* a, float* out, int64_t M, int64_t N) {
     const bool vec = (N % 4 == 0);
     const int64_t NW = vec ? N / 4 : N;
     const int64_t gx = ceil_div(NW, kWave);
-    const int64_t target = static_cast<int64_t>(c.num_cus) * 4;
+#ifndef BSHIP_COLSUM_TARGET
+#define BSHIP_COLSUM_TARGET 4
+#endif
+    const int64_t target = static_cast<int64_t>(c.num_cus) * BSHIP_COLSUM_TARGET;
     int64_t bands = target / gx;
     if (bands < 1) bands = 1;
     const int64_t min_rows = 64;             // at least 4 unrolled steps per wavefront

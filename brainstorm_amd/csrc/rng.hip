@@ -3,13 +3,20 @@
 // The reference draws dropout masks from the handler's RandomState
 // (numpy_handler.py 199-200: rnd.uniform(size) < p). To give the same masks
 // the generator state (624 words + position + the cached gaussian of the legacy
-// polar method) lives in device memory and one workgroup advances it:
-//  - the twist of a 624-word block has only distance-1 and distance-397
-//    dependencies, so it is done in three data-parallel phases in LDS
-//    (words 0..226, 227..453, 454..623);
-//  - tempering and the 53-bit double construction
-//    ((a >> 5) * 2^26 + (b >> 6)) / 2^53 are element-parallel.
-// Nothing is copied to the host, so mask generation stays asynchronous.
+// polar method) lives in device memory and one workgroup advances it. Nothing
+// is copied to the host, so mask generation stays asynchronous.
+//
+// The generator is treated as one linear stream of raw words r[0], r[1], ...:
+// the 624 words of the current block are r[0..623] and every later word follows
+// from
+//     r[n] = r[n-227] ^ twist(r[n-624], r[n-623])
+// (the block-wise regeneration of the MT19937 reference code, unrolled). One
+// "step" produces 227 consecutive words with one lane per word: r[n-227] is the
+// word the SAME lane produced in the previous step, so it stays in a register,
+// and r[n-624], r[n-623] were written at least two steps earlier, so they are
+// fetched from LDS one step ahead. The serial chain per step is a handful of
+// ALU instructions and one barrier. Tempering and the 53-bit double
+// construction ((a >> 5) * 2^26 + (b >> 6)) / 2^53 are element-parallel.
 #include <mutex>
 
 #include "common.h"
@@ -42,138 +49,82 @@ __device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
     return y;
 }
 
-// Replaces the 624 words in `cur` by the next block, written to `nxt`.
-// Must be called by all kBlock threads of the workgroup.
-__device__ __forceinline__ void mt_next_block(const uint32_t* cur, uint32_t* nxt) {
+constexpr int kLag = kMtN - kMtM;             // 227
+constexpr int kRing = 4096;                   // LDS ring of raw words (power of two)
+constexpr int kRingMask = kRing - 1;
+constexpr int kStepsPerBatch = 9;             // 9 * 227 = 2043 new words between consume phases
+static_assert(kBlock >= kLag, "one lane per word of a step");
+static_assert(kStepsPerBatch * kLag + kMtN + kLag + 2 <= kRing, "ring holds history, backlog and a batch");
+
+// Draws n (> 0) 53-bit doubles from the stream, in order, and hands double number
+// i to sink(i, value); leaves the state as numpy's RandomState would have it
+// (whole blocks regenerated, position inside the last one). One workgroup of
+// kBlock threads; every control decision is the same in all threads, so the
+// barriers are reached uniformly.
+template <typename Sink>
+__device__ __forceinline__ void mt_generate(RngState* st, size_t n, Sink sink) {
+    __shared__ uint32_t ring[kRing];
     const int t = threadIdx.x;
-    // phase 1: words 0..226 depend on old words only
-    if (t < kMtN - kMtM) nxt[t] = cur[t + kMtM] ^ mt_twist(cur[t], cur[t + 1]);
+    for (int i = t; i < kMtN; i += kBlock) ring[i] = st->key[i];
+    const size_t pos0 = static_cast<size_t>(st->pos);        // 0..624, next unread word
     __syncthreads();
-    // phase 2: words 227..453 use new words 0..226
-    {
-        const int i = t + (kMtN - kMtM);
-        if (i < 2 * (kMtN - kMtM)) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], cur[i + 1]);
+    const size_t end_word = pos0 + 2 * n;                     // first word NOT consumed
+    const size_t gen_end = (end_word + kMtN - 1) / kMtN * kMtN;   // whole blocks
+    size_t have = kMtN;                                       // words r[0..have) exist
+    size_t done = 0;                                          // doubles emitted
+    const bool gen_lane = t < kLag;
+    uint32_t carry = 0, a = 0, b = 0;
+    if (gen_lane) {
+        carry = ring[have + t - kLag];                        // r[n-227] of the first step
+        a = ring[(have + t - kMtN) & kRingMask];
+        b = ring[(have + t - kMtN + 1) & kRingMask];
+    }
+    while (true) {
+        size_t steps = (gen_end - have + kLag - 1) / kLag;
+        if (steps > kStepsPerBatch) steps = kStepsPerBatch;
+        for (size_t s = 0; s < steps; ++s) {
+            if (gen_lane) {
+                carry ^= mt_twist(a, b);
+                ring[(have + t) & kRingMask] = carry;
+                // operands of the next step: written two or more steps ago
+                a = ring[(have + kLag + t - kMtN) & kRingMask];
+                b = ring[(have + kLag + t - kMtN + 1) & kRingMask];
+            }
+            have += kLag;
+            __syncthreads();
+        }
+        // consume every complete pair of words that exists by now
+        const size_t first = pos0 + 2 * done;
+        size_t pairs = have > first ? (have - first) / 2 : 0;
+        if (pairs > n - done) pairs = n - done;
+        for (size_t j = t; j < pairs; j += kBlock) {
+            const size_t w = first + 2 * j;
+            const uint32_t w0 = mt_temper(ring[w & kRingMask]);
+            const uint32_t w1 = mt_temper(ring[(w + 1) & kRingMask]);
+            sink(done + j, (static_cast<double>(w0 >> 5) * 67108864.0 + static_cast<double>(w1 >> 6)) /
+                               9007199254740992.0);
+        }
+        done += pairs;
+        if (done >= n && have >= gen_end) break;
+        __syncthreads();                                      // ring slots may be overwritten next
     }
     __syncthreads();
-    // phase 3: words 454..623 use new words 227..396; the last one wraps to new word 0
-    {
-        const int i = t + 2 * (kMtN - kMtM);
-        if (i < kMtN - 1) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], cur[i + 1]);
-        else if (i == kMtN - 1) nxt[i] = nxt[i - (kMtN - kMtM)] ^ mt_twist(cur[i], nxt[0]);
-    }
-    __syncthreads();
+    // numpy keeps the block that holds the last consumed word and the position inside it
+    const size_t block0 = gen_end - kMtN;
+    for (int i = t; i < kMtN; i += kBlock) st->key[i] = ring[(block0 + i) & kRingMask];
+    if (t == 0) st->pos = static_cast<int32_t>(end_word - block0);
 }
-static_assert(kBlock >= kMtN - kMtM, "one thread per word of a twist phase");
 
-// Word stream shared by the consumers below: LDS copy of the state, double
-// buffered, plus at most one tempered word carried over a block boundary when a
-// 53-bit double straddles it.
-struct MtStream {
-    uint32_t buf[2][kMtN];
-    uint32_t carry;
-};
-
-// mask[i] = (next_double() < p) ? 1 : 0 for i in [0,n). Single workgroup.
+// mask[i] = (next_double() < p) ? 1 : 0 for i in [0,n).
 __global__ __launch_bounds__(kBlock) void mt_mask_kernel(RngState* st, float* __restrict__ mask,
                                                          size_t n, double p) {
-    __shared__ MtStream s;
-    int cur = 0;
-    for (int i = threadIdx.x; i < kMtN; i += kBlock) s.buf[0][i] = st->key[i];
-    int pos = st->pos;                 // same value in every thread
-    __syncthreads();
-    bool have_carry = false;
-    size_t done = 0;
-    while (done < n) {
-        if (pos >= kMtN) {
-            mt_next_block(s.buf[cur], s.buf[cur ^ 1]);
-            cur ^= 1;
-            pos = 0;
-        }
-        const uint32_t* key = s.buf[cur];
-        // logical word L of this round: the carried word (if any) followed by key[pos...]
-        const int avail = kMtN - pos + (have_carry ? 1 : 0);
-        size_t pairs = static_cast<size_t>(avail / 2);
-        const bool finishing = pairs >= n - done;
-        if (finishing) pairs = n - done;
-        for (size_t j = threadIdx.x; j < pairs; j += kBlock) {
-            const int l0 = static_cast<int>(2 * j);
-            uint32_t w0, w1;
-            if (have_carry) {
-                w0 = (l0 == 0) ? s.carry : mt_temper(key[pos + l0 - 1]);
-                w1 = mt_temper(key[pos + l0]);
-            } else {
-                w0 = mt_temper(key[pos + l0]);
-                w1 = mt_temper(key[pos + l0 + 1]);
-            }
-            const double r = (static_cast<double>(w0 >> 5) * 67108864.0 + static_cast<double>(w1 >> 6)) /
-                             9007199254740992.0;
-            mask[done + j] = (r < p) ? 1.0f : 0.0f;
-        }
-        const int used = static_cast<int>(2 * pairs) - (have_carry ? 1 : 0);   // words taken from key
-        __syncthreads();                       // everyone has read s.carry
-        pos += used;
-        done += pairs;
-        have_carry = false;
-        if (!finishing && pos == kMtN - 1) {   // odd word left: carry it into the next block
-            if (threadIdx.x == 0) s.carry = mt_temper(key[kMtN - 1]);
-            have_carry = true;
-            pos = kMtN;
-            __syncthreads();
-        }
-    }
-    for (int i = threadIdx.x; i < kMtN; i += kBlock) st->key[i] = s.buf[cur][i];
-    if (threadIdx.x == 0) st->pos = pos;
+    mt_generate(st, n, [=](size_t i, double r) { mask[i] = (r < p) ? 1.0f : 0.0f; });
 }
 
-// Writes `count` raw doubles of the stream to `u` (used by fill_gaussian).
-// Single workgroup; same structure as the mask kernel.
+// u[i] = next_double() for i in [0,n) (used by fill_gaussian, also to skip ahead).
 __global__ __launch_bounds__(kBlock) void mt_doubles_kernel(RngState* st, double* __restrict__ u,
                                                             size_t n) {
-    __shared__ MtStream s;
-    int cur = 0;
-    for (int i = threadIdx.x; i < kMtN; i += kBlock) s.buf[0][i] = st->key[i];
-    int pos = st->pos;
-    __syncthreads();
-    bool have_carry = false;
-    size_t done = 0;
-    while (done < n) {
-        if (pos >= kMtN) {
-            mt_next_block(s.buf[cur], s.buf[cur ^ 1]);
-            cur ^= 1;
-            pos = 0;
-        }
-        const uint32_t* key = s.buf[cur];
-        const int avail = kMtN - pos + (have_carry ? 1 : 0);
-        size_t pairs = static_cast<size_t>(avail / 2);
-        const bool finishing = pairs >= n - done;
-        if (finishing) pairs = n - done;
-        for (size_t j = threadIdx.x; j < pairs; j += kBlock) {
-            const int l0 = static_cast<int>(2 * j);
-            uint32_t w0, w1;
-            if (have_carry) {
-                w0 = (l0 == 0) ? s.carry : mt_temper(key[pos + l0 - 1]);
-                w1 = mt_temper(key[pos + l0]);
-            } else {
-                w0 = mt_temper(key[pos + l0]);
-                w1 = mt_temper(key[pos + l0 + 1]);
-            }
-            u[done + j] = (static_cast<double>(w0 >> 5) * 67108864.0 + static_cast<double>(w1 >> 6)) /
-                          9007199254740992.0;
-        }
-        const int used = static_cast<int>(2 * pairs) - (have_carry ? 1 : 0);
-        __syncthreads();
-        pos += used;
-        done += pairs;
-        have_carry = false;
-        if (!finishing && pos == kMtN - 1) {
-            if (threadIdx.x == 0) s.carry = mt_temper(key[kMtN - 1]);
-            have_carry = true;
-            pos = kMtN;
-            __syncthreads();
-        }
-    }
-    for (int i = threadIdx.x; i < kMtN; i += kBlock) st->key[i] = s.buf[cur][i];
-    if (threadIdx.x == 0) st->pos = pos;
+    mt_generate(st, n, [=](size_t i, double r) { u[i] = r; });
 }
 
 // Legacy polar method (RandomState.standard_normal): trial t uses doubles
