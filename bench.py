@@ -206,6 +206,9 @@ def run_nets_gpu(hip):
     return {
         "mlp_784-1200-1200-10_batch100": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize),
         "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
+        # same network, the elementwise part of each time step in one launch (same bits)
+        "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,
+                                                               hip.synchronize, fused=True),
     }
 
 

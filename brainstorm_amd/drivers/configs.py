@@ -66,7 +66,7 @@ def build_mlp(handler, seed=1, batch=100, in_size=784, hidden=1200, classes=10):
     return _finish(net, data, _init_parameters(net, rng, 0.01))
 
 
-def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1000):
+def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1000, fused=False):
     rng = np.random.RandomState(seed)
     ids = rng.randint(0, symbols, (time_steps, batch, 1))
     onehot = np.zeros((time_steps, batch, symbols), dtype=F32)     # like data_iterators.OneHot
@@ -74,7 +74,7 @@ def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1
     data = {"default": onehot, "targets": ids.astype(F32)}
     net = Net(handler, [
         ("Input", Input({"default": (symbols,), "targets": (1,)}), {}),
-        ("lstm", Lstm(hidden, "tanh"), {"default": "Input.default"}),
+        ("lstm", Lstm(hidden, "tanh", fused=fused), {"default": "Input.default"}),
         ("out", FullyConnected(symbols, "linear"), {"default": "lstm.default"}),
         ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),

@@ -222,9 +222,15 @@ class Lstm(Layer):
     PARAMS = ("Wz", "Wi", "Wf", "Wo", "pi", "pf", "po", "Rz", "Ri", "Rf", "Ro", "bz", "bi", "bf", "bo")
     INTERNALS = ("Za", "Zb", "Ia", "Ib", "Fa", "Fb", "Oa", "Ob", "Ca", "Cb")
 
-    def __init__(self, size, activation="tanh"):
+    def __init__(self, size, activation="tanh", fused=False):
         self.size = int(size)
         self.activation = activation
+        # fused=True: the elementwise part of each time step goes through the handler's
+        # lstm_forward_step / lstm_backward_step (one launch each, same bits) when it has them
+        self.fused = bool(fused)
+
+    def _use_fused(self):
+        return self.fused and hasattr(self.handler, "lstm_forward_step")
 
     def setup(self, in_shapes):
         in_size = _prod(in_shapes["default"].feature_shape)
@@ -253,6 +259,18 @@ class Lstm(Layer):
         _h.dot_mm(flat_x, Wi, flatten_time(Ia[:-1]), transb=True)
         _h.dot_mm(flat_x, Wf, flatten_time(Fa[:-1]), transb=True)
         _h.dot_mm(flat_x, Wo, flatten_time(Oa[:-1]), transb=True)
+
+        if self._use_fused():
+            for t in range(time_size):
+                y_prev = y[t - 1]
+                _h.dot_add_mm(y_prev, Rz, Za[t], transb=True)
+                _h.dot_add_mm(y_prev, Ri, Ia[t], transb=True)
+                _h.dot_add_mm(y_prev, Rf, Fa[t], transb=True)
+                _h.dot_add_mm(y_prev, Ro, Oa[t], transb=True)
+                _h.lstm_forward_step(self.activation, Za[t], Zb[t], Ia[t], Ib[t], Fa[t], Fb[t],
+                                     Oa[t], Ob[t], Ca[t], Cb[t], Ca[t - 1], y[t],
+                                     pi, pf, po, bz, bi, bf, bo)
+            return
 
         for t in range(time_size):
             # block input
@@ -296,7 +314,20 @@ class Lstm(Layer):
         dy = _h.allocate(y.shape)          # zeros: dy[-1] is read below without ever being written
         _h.fill(dCa, 0.0)
         time_size = x.shape[0]
+        fused = self._use_fused()
         for t in range(time_size - 1, -1, -1):
+            if fused:
+                dy_t = dy[t]
+                _h.copy_to(deltas[t], dy_t)
+                _h.dot_add_mm(dIa[t + 1], Ri, dy_t)
+                _h.dot_add_mm(dFa[t + 1], Rf, dy_t)
+                _h.dot_add_mm(dOa[t + 1], Ro, dy_t)
+                _h.dot_add_mm(dZa[t + 1], Rz, dy_t)
+                _h.lstm_backward_step(self.activation, dy_t, Zb[t], Ib[t], Fb[t], Ob[t], Cb[t],
+                                      Ca[t - 1], Fb[t + 1], dIa[t + 1], dFa[t + 1], dCa[t + 1],
+                                      dZa[t], dZb[t], dIa[t], dIb[t], dFa[t], dFb[t], dOa[t],
+                                      dOb[t], dCa[t], dCb[t], pi, pf, po)
+                continue
             # accumulate recurrent deltas
             _h.copy_to(deltas[t], dy[t])
             _h.dot_add_mm(dIa[t + 1], Ri, dy[t])

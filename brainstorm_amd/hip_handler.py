@@ -411,3 +411,34 @@ class HipHandler(Handler):
 
     def el_deriv(self, x, y, dy, dx):
         self._call(self._lib.bship_deriv_f32(EL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+
+    # ------------------------------------------------ fused layer-level steps
+    # Extensions beyond the Handler interface. A layer may test for them with
+    # hasattr() and fall back on the single operations, which give the same bits.
+    _ACT_CODES = {"sigmoid": 0, "tanh": 1, "rel": 2, "linear": 3, "el": 4}
+
+    def lstm_forward_step(self, activation, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, Ca_prev, y,
+                          pi, pf, po, bz, bi, bf, bo):
+        """Everything lstm_layer.py:121-145 does at one time step after its four
+        dot_add_mm calls; the arrays are the [t] (and Ca[t-1]) slices."""
+        batch, n = Za.shape
+        mats = (Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, Ca_prev, y)
+        vecs = (pi, pf, po, bz, bi, bf, bo)
+        if any(m.shape != (batch, n) for m in mats) or any(v.size != n for v in vecs):
+            raise ValueError("lstm_forward_step: inconsistent shapes")
+        self._call(self._lib.bship_lstm_fwd_step_f32(
+            self._ACT_CODES[activation], batch, n, *[a.ptr for a in mats + vecs]))
+
+    def lstm_backward_step(self, activation, dy, Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next,
+                           dFa_next, dCa_next, dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb,
+                           pi, pf, po):
+        """Everything lstm_layer.py:186-214 does at one time step between the
+        dot_add_mm calls into dy[t] and the end of the loop body."""
+        batch, n = dy.shape
+        mats = (dy, Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next,
+                dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb)
+        vecs = (pi, pf, po)
+        if any(m.shape != (batch, n) for m in mats) or any(v.size != n for v in vecs):
+            raise ValueError("lstm_backward_step: inconsistent shapes")
+        self._call(self._lib.bship_lstm_bwd_step_f32(
+            self._ACT_CODES[activation], batch, n, *[a.ptr for a in mats + vecs]))

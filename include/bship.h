@@ -251,6 +251,45 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
                                int out_w, int pool_h, int pool_w, int pad,
                                int stride_h, int stride_w);
 
+/* --------------------------- fused layer steps --------------------------- */
+
+/* Extensions beyond the handler interface: one launch for the elementwise
+ * part of one LSTM time step, chaining the same float32 operations in the
+ * order the layer issues them as single handler calls, so the results are
+ * bit-identical to that sequence. All matrices are (batch, n) dense; the
+ * peephole vectors p* and the biases b* hold n elements.
+ * Activation codes: the act_func table of base_handler.py 57-63. */
+enum {
+    BSHIP_ACT_SIGMOID = 0,
+    BSHIP_ACT_TANH = 1,
+    BSHIP_ACT_REL = 2,
+    BSHIP_ACT_LINEAR = 3,
+    BSHIP_ACT_EL = 4
+};
+/* LstmLayerImpl.forward_pass, the part of the loop body after the four
+ * dot_add_mm calls (lstm_layer.py 121-145). Za, Ia, Fa, Oa hold the
+ * accumulated products on entry and the biased pre-activations on return. */
+int bship_lstm_fwd_step_f32(int act, int64_t batch, int64_t n, float* Za,
+                            float* Zb, float* Ia, float* Ib, float* Fa,
+                            float* Fb, float* Oa, float* Ob, float* Ca,
+                            float* Cb, const float* Ca_prev, float* y,
+                            const float* pi, const float* pf, const float* po,
+                            const float* bz, const float* bi, const float* bf,
+                            const float* bo);
+/* LstmLayerImpl.backward_pass, the part of the loop body between the
+ * recurrent dot_add_mm calls into dy and the dot_add_mm calls that follow
+ * (lstm_layer.py 186-214). dCa holds its initial content on entry (the layer
+ * accumulates into it); the *_next arguments are the buffers of time t+1. */
+int bship_lstm_bwd_step_f32(int act, int64_t batch, int64_t n, const float* dy,
+                            const float* Zb, const float* Ib, const float* Fb,
+                            const float* Ob, const float* Cb,
+                            const float* Ca_prev, const float* Fb_next,
+                            const float* dIa_next, const float* dFa_next,
+                            const float* dCa_next, float* dZa, float* dZb,
+                            float* dIa, float* dIb, float* dFa, float* dFb,
+                            float* dOa, float* dOb, float* dCa, float* dCb,
+                            const float* pi, const float* pf, const float* po);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,130 @@
+"""GPU: the fused LSTM time-step entry points against the sequence of single
+handler operations they replace. Both run on the GPU with the same matrix-product
+kernels, so every buffer must agree bit for bit; the unfused sequence itself is
+held to the CPU oracle in test_gpu_configs.py."""
+import numpy as np
+import pytest
+
+from brainstorm_amd.drivers import configs
+from util import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+def run_lstm(hip, fused, **kw):
+    hip.rnd.seed(5)
+    net, data = configs.build_lstm(hip, fused=fused, **kw)
+    net.provide_external_data(data)
+    net.forward_pass(training_pass=True)
+    net.backward_pass()
+    return net
+
+
+@pytest.mark.parametrize("shape", [dict(time_steps=7, batch=5, symbols=11, hidden=13),
+                                   dict(time_steps=20, batch=33, symbols=50, hidden=257)])
+def test_fused_lstm_network_is_bit_identical(hip, shape):
+    plain = run_lstm(hip, False, **shape)
+    fused = run_lstm(hip, True, **shape)
+    assert fused.layers["lstm"]._use_fused()
+    for group in ("outputs", "internals", "output_deltas"):
+        for key in getattr(plain.buffers["lstm"], group):
+            assert_bit_equal(fused.get("lstm", group, key), plain.get("lstm", group, key),
+                             "lstm.%s.%s" % (group, key))
+    assert_bit_equal(hip.get_numpy_copy(fused.gradients), hip.get_numpy_copy(plain.gradients), "gradients")
+    assert_bit_equal(fused.get("Input", "output_deltas", "default"),
+                     plain.get("Input", "output_deltas", "default"), "input deltas")
+
+
+@pytest.mark.parametrize("activation", ["tanh", "sigmoid", "rel", "el", "linear"])
+def test_fused_steps_match_single_operations(hip, activation):
+    rng = np.random.RandomState(17)
+    batch, n = 37, 129                       # odd sizes: views start at unaligned addresses
+
+    def mats(count, scale=1.0):
+        flat = hip.create_from_numpy((scale * rng.standard_normal((count, batch, n))).astype(F32))
+        return [flat[k] for k in range(count)]
+
+    def vecs(count):
+        return [hip.create_from_numpy(rng.standard_normal((1, n)).astype(F32)) for _ in range(count)]
+
+    pi, pf, po = vecs(3)
+    bz, bi, bf, bo = [v.reshape((n,)) for v in vecs(4)]
+    h = hip
+
+    # ---- forward
+    acc = [m for m in mats(4)]                                  # Za, Ia, Fa, Oa as the products left them
+    ca_prev = mats(1)[0]
+    init = [h.get_numpy_copy(a) for a in acc]
+    Za, Ia, Fa, Oa = acc
+    Zb, Ib, Fb, Ob, Ca, Cb, y = mats(7)
+    h.lstm_forward_step(activation, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, ca_prev, y,
+                        pi, pf, po, bz, bi, bf, bo)
+    got = [h.get_numpy_copy(a) for a in (Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y)]
+
+    for a, v in zip(acc, init):
+        h.set_from_numpy(a, v)
+    h.add_mv(Za, bz.reshape((1, n)), Za)
+    h.act_func[activation](Za, Zb)
+    h.mult_add_mv(ca_prev, pi, Ia)
+    h.add_mv(Ia, bi.reshape((1, n)), Ia)
+    h.sigmoid(Ia, Ib)
+    h.mult_add_mv(ca_prev, pf, Fa)
+    h.add_mv(Fa, bf.reshape((1, n)), Fa)
+    h.sigmoid(Fa, Fb)
+    h.mult_tt(Ib, Zb, Ca)
+    h.mult_add_tt(Fb, ca_prev, Ca)
+    h.mult_add_mv(Ca, po, Oa)
+    h.add_mv(Oa, bo.reshape((1, n)), Oa)
+    h.sigmoid(Oa, Ob)
+    h.act_func[activation](Ca, Cb)
+    h.mult_tt(Ob, Cb, y)
+    names = "Za Zb Ia Ib Fa Fb Oa Ob Ca Cb y".split()
+    for name, g, a in zip(names, got, (Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y)):
+        assert_bit_equal(g, h.get_numpy_copy(a), "forward " + name)
+
+    # ---- backward, on the forward state just computed
+    dy, fb_next, dia_next, dfa_next, dca_next = mats(5, 0.5)
+    dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb = mats(10)
+    dca_init = h.get_numpy_copy(dCa)
+    h.lstm_backward_step(activation, dy, Zb, Ib, Fb, Ob, Cb, ca_prev, fb_next, dia_next, dfa_next,
+                         dca_next, dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po)
+    outs = (dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb)
+    got = [h.get_numpy_copy(a) for a in outs]
+
+    h.set_from_numpy(dCa, dca_init)
+    h.mult_add_mv(dia_next, pi, dCa)
+    h.mult_add_mv(dfa_next, pf, dCa)
+    h.mult_tt(dy, Cb, dOb)
+    h.sigmoid_deriv(Oa, Ob, dOb, dOa)
+    h.mult_add_mv(dOa, po, dCa)
+    h.mult_tt(dy, Ob, dCb)
+    h.act_func_deriv[activation](Ca, Cb, dCb, dCb)
+    h.add_tt(dCa, dCb, dCa)
+    h.mult_add_tt(dca_next, fb_next, dCa)
+    h.mult_tt(dCa, ca_prev, dFb)
+    h.sigmoid_deriv(Fa, Fb, dFb, dFa)
+    h.mult_tt(dCa, Zb, dIb)
+    h.sigmoid_deriv(Ia, Ib, dIb, dIa)
+    h.mult_tt(dCa, Ib, dZb)
+    h.act_func_deriv[activation](Za, Zb, dZb, dZa)
+    names = "dZa dZb dIa dIb dFa dFb dOa dOb dCa dCb".split()
+    for name, g, a in zip(names, got, outs):
+        assert_bit_equal(g, h.get_numpy_copy(a), "backward " + name)
+
+
+def test_fused_step_argument_errors(hip):
+    a = hip.allocate((4, 8))
+    v = hip.allocate((1, 8))
+    b = hip.allocate((8,))
+    with pytest.raises(ValueError):
+        hip.lstm_forward_step("tanh", a, a, a, a, a, a, a, a, a, a, hip.allocate((4, 9)), a,
+                              v, v, v, b, b, b, b)
+    with pytest.raises(KeyError):
+        hip.lstm_forward_step("softplus", a, a, a, a, a, a, a, a, a, a, a, a, v, v, v, b, b, b, b)
+    lib = hip._lib
+    p = a.ptr
+    assert lib.bship_lstm_fwd_step_f32(9, 4, 8, *([p] * 19)) == -4
+    assert lib.bship_lstm_fwd_step_f32(1, 4, 8, *([p] * 18 + [None])) == -2
+    assert lib.bship_lstm_bwd_step_f32(1, -1, 8, *([p] * 24)) == -3
+    assert lib.bship_lstm_bwd_step_f32(1, 0, 8, *([p] * 24)) == 0
