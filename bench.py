@@ -209,6 +209,9 @@ def run_nets_gpu(hip):
         # same network, the elementwise part of each time step in one launch (same bits)
         "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,
                                                                hip.synchronize, fused=True),
+        # ... and the four recurrent matrix products of a step as one over the stacked matrices
+        "lstm_205-1000-205_T100_batch100_fused_packed": time_net(hip, configs.build_lstm, 5, 1,
+                                                                hip.synchronize, fused="packed"),
     }
 
 

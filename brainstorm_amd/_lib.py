@@ -70,6 +70,8 @@ SIGNATURES = {
     "bship_avgpool_bwd_nhwc_f32": [_P, _P, _I64] + [c_int] * 10,
     "bship_lstm_fwd_step_f32": [c_int, _I64, _I64] + [_P] * 19,
     "bship_lstm_bwd_step_f32": [c_int, _I64, _I64] + [_P] * 24,
+    "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,
+    "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
 }
 # functions that do not return a status
 SPECIAL_RESTYPES = {"bship_version": (c_int, []), "bship_last_error": (c_char_p, [])}

@@ -225,12 +225,21 @@ class Lstm(Layer):
     def __init__(self, size, activation="tanh", fused=False):
         self.size = int(size)
         self.activation = activation
-        # fused=True: the elementwise part of each time step goes through the handler's
-        # lstm_forward_step / lstm_backward_step (one launch each, same bits) when it has them
-        self.fused = bool(fused)
+        # fused="steps" (or True): the elementwise part of each time step goes through the
+        # handler's lstm_forward_step / lstm_backward_step (one launch each, same bits) when it
+        # has them. fused="packed": additionally the four recurrent products of a step become
+        # one product over the stacked matrices [Rz;Ri;Rf;Ro] (same values up to the summation
+        # order inside the matrix product).
+        self.fused = "steps" if fused is True else (fused or False)
+        assert self.fused in (False, "steps", "packed")
 
     def _use_fused(self):
-        return self.fused and hasattr(self.handler, "lstm_forward_step")
+        return bool(self.fused) and hasattr(self.handler, "lstm_forward_step")
+
+    def _stacked_recurrent(self, Rz, Ri, Rf, Ro):
+        if self.fused != "packed" or not hasattr(self.handler, "stack_adjacent"):
+            return None
+        return self.handler.stack_adjacent([Rz, Ri, Rf, Ro])
 
     def setup(self, in_shapes):
         in_size = _prod(in_shapes["default"].feature_shape)
@@ -260,6 +269,15 @@ class Lstm(Layer):
         _h.dot_mm(flat_x, Wf, flatten_time(Fa[:-1]), transb=True)
         _h.dot_mm(flat_x, Wo, flatten_time(Oa[:-1]), transb=True)
 
+        R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
+        if R_all is not None:
+            rec = _h.allocate((x.shape[1], 4 * n))
+            for t in range(time_size):
+                _h.dot_mm(y[t - 1], R_all, rec, transb=True)
+                _h.lstm_forward_step_packed(self.activation, rec, Za[t], Zb[t], Ia[t], Ib[t], Fa[t],
+                                            Fb[t], Oa[t], Ob[t], Ca[t], Cb[t], Ca[t - 1], y[t],
+                                            pi, pf, po, bz, bi, bf, bo)
+            return
         if self._use_fused():
             for t in range(time_size):
                 y_prev = y[t - 1]
@@ -315,7 +333,20 @@ class Lstm(Layer):
         _h.fill(dCa, 0.0)
         time_size = x.shape[0]
         fused = self._use_fused()
+        R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
+        if R_all is not None:
+            # [dZa|dIa|dFa|dOa] of the step after the current one, double-buffered; zero beyond the end
+            packed = [_h.allocate((x.shape[1], 4 * self.size)) for _ in range(2)]
         for t in range(time_size - 1, -1, -1):
+            if R_all is not None:
+                dy_t = dy[t]
+                _h.dot_mm(packed[(t + 1) % 2], R_all, dy_t)
+                _h.lstm_backward_step_packed(self.activation, deltas[t], dy_t, packed[t % 2],
+                                             Zb[t], Ib[t], Fb[t], Ob[t], Cb[t], Ca[t - 1],
+                                             Fb[t + 1], dIa[t + 1], dFa[t + 1], dCa[t + 1],
+                                             dZa[t], dZb[t], dIa[t], dIb[t], dFa[t], dFb[t],
+                                             dOa[t], dOb[t], dCa[t], dCb[t], pi, pf, po)
+                continue
             if fused:
                 dy_t = dy[t]
                 _h.copy_to(deltas[t], dy_t)

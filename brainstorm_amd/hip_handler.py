@@ -442,3 +442,44 @@ class HipHandler(Handler):
             raise ValueError("lstm_backward_step: inconsistent shapes")
         self._call(self._lib.bship_lstm_bwd_step_f32(
             self._ACT_CODES[activation], batch, n, *[a.ptr for a in mats + vecs]))
+
+    def stack_adjacent(self, arrays):
+        """One (k*rows, ...) array over k equally shaped arrays that lie back to back in
+        device memory (as the four recurrent matrices of an LSTM do in brainstorm's
+        parameter vector), or None if they do not."""
+        first = arrays[0]
+        for k, a in enumerate(arrays):
+            if a.shape != first.shape or a.ptr != first.ptr + k * first.nbytes or not a.ptr:
+                return None
+        shape = (len(arrays) * first.shape[0],) + tuple(first.shape[1:])
+        return DeviceArray(first.ptr, shape, [a._owner for a in arrays], self)
+
+    def lstm_forward_step_packed(self, activation, rec, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb,
+                                 Ca_prev, y, pi, pf, po, bz, bi, bf, bo):
+        """lstm_forward_step with the four recurrent products given as one matrix
+        rec (batch, 4n) = y[t-1] . [Rz;Ri;Rf;Ro]^T instead of accumulated into Za..Oa."""
+        batch, n = Za.shape
+        mats = (Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, Ca_prev, y)
+        vecs = (pi, pf, po, bz, bi, bf, bo)
+        if (rec.shape != (batch, 4 * n) or any(m.shape != (batch, n) for m in mats)
+                or any(v.size != n for v in vecs)):
+            raise ValueError("lstm_forward_step_packed: inconsistent shapes")
+        self._call(self._lib.bship_lstm_fwd_step_packed_f32(
+            self._ACT_CODES[activation], batch, n, rec.ptr, *[a.ptr for a in mats + vecs]))
+
+    def lstm_backward_step_packed(self, activation, deltas, dy, packed_out, Zb, Ib, Fb, Ob, Cb,
+                                  Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next, dZa, dZb, dIa,
+                                  dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po):
+        """lstm_backward_step for one stacked recurrent product: dy holds
+        packed[t+1] . [Rz;Ri;Rf;Ro] on entry and deltas + that afterwards;
+        packed_out (batch, 4n) receives [dZa|dIa|dFa|dOa] of this step."""
+        batch, n = dy.shape
+        mats = (deltas, dy, Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next,
+                dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb)
+        vecs = (pi, pf, po)
+        if (packed_out.shape != (batch, 4 * n) or any(m.shape != (batch, n) for m in mats)
+                or any(v.size != n for v in vecs)):
+            raise ValueError("lstm_backward_step_packed: inconsistent shapes")
+        self._call(self._lib.bship_lstm_bwd_step_packed_f32(
+            self._ACT_CODES[activation], batch, n, deltas.ptr, dy.ptr, packed_out.ptr,
+            *[a.ptr for a in mats[2:] + vecs]))

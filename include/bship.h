@@ -289,6 +289,38 @@ int bship_lstm_bwd_step_f32(int act, int64_t batch, int64_t n, const float* dy,
                             float* dIa, float* dIb, float* dFa, float* dFb,
                             float* dOa, float* dOb, float* dCa, float* dCb,
                             const float* pi, const float* pf, const float* po);
+/* The same two steps for a caller that forms the four recurrent products of a
+ * time step as ONE matrix product over the stacked recurrent weights
+ * [Rz;Ri;Rf;Ro] (4n x n, as they lie in brainstorm's parameter vector,
+ * lstm_layer.py 62-65) instead of four accumulating ones:
+ *  - forward: rec (batch, 4n) = y[t-1] [Rz;Ri;Rf;Ro]^T, columns [z|i|f|o], is
+ *    added to Za, Ia, Fa, Oa before the step proper;
+ *  - backward: dy holds packed[t+1] [Rz;Ri;Rf;Ro] on entry and receives
+ *    deltas + that (lstm_layer.py 181-185); packed_out (batch, 4n) receives
+ *    [dZa|dIa|dFa|dOa] of this step, the left operand of the next product.
+ * The elementwise arithmetic is the same; the matrix products sum in another
+ * order than four separate ones, so results agree to rounding, not bit for bit. */
+int bship_lstm_fwd_step_packed_f32(int act, int64_t batch, int64_t n,
+                                   const float* rec, float* Za, float* Zb,
+                                   float* Ia, float* Ib, float* Fa, float* Fb,
+                                   float* Oa, float* Ob, float* Ca, float* Cb,
+                                   const float* Ca_prev, float* y,
+                                   const float* pi, const float* pf,
+                                   const float* po, const float* bz,
+                                   const float* bi, const float* bf,
+                                   const float* bo);
+int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n,
+                                   const float* deltas, float* dy,
+                                   float* packed_out, const float* Zb,
+                                   const float* Ib, const float* Fb,
+                                   const float* Ob, const float* Cb,
+                                   const float* Ca_prev, const float* Fb_next,
+                                   const float* dIa_next, const float* dFa_next,
+                                   const float* dCa_next, float* dZa, float* dZb,
+                                   float* dIa, float* dIb, float* dFa,
+                                   float* dFb, float* dOa, float* dOb,
+                                   float* dCa, float* dCb, const float* pi,
+                                   const float* pf, const float* po);
 
 #ifdef __cplusplus
 }

@@ -114,6 +114,28 @@ def test_lstm_full_size_forward_backward(hip):
     d_err = scaled_err(net_h.get("Input", "output_deltas", "default"), net_r.get("Input", "output_deltas", "default"))
     assert d_err <= 1e-4, d_err
     print("lstm: worst gradient block %.2e, input deltas %.2e" % (worst, d_err))
+    # the same network through the fused time-step kernels with one stacked recurrent
+    # product per step: held to the oracle at the same bars
+    hip.rnd.seed(22)
+    net_p, data = configs.build_lstm(hip, fused="packed")
+    net_p.provide_external_data(data)
+    net_p.forward_pass(training_pass=True)
+    net_p.backward_pass()
+    loss_p = net_p.get("loss", "outputs", "loss")[0]
+    assert abs(loss_p - loss_r) <= 1e-5 * abs(loss_r), (loss_p, loss_r)
+    for key in ("Za", "Ib", "Ca", "Cb"):
+        err = scaled_err(net_p.get("lstm", "internals", key), net_r.get("lstm", "internals", key))
+        assert err <= 1e-5, (key, err)
+    g_p = hip.get_numpy_copy(net_p.gradients)
+    worst_p = 0.0
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        err = scaled_err(g_p[a:b], g_r[a:b])
+        worst_p = max(worst_p, err)
+        assert err <= 1e-4, (name, err)
+    d_err = scaled_err(net_p.get("Input", "output_deltas", "default"), net_r.get("Input", "output_deltas", "default"))
+    assert d_err <= 1e-4, d_err
+    print("lstm, fused steps + stacked recurrent product: worst gradient block %.2e, input deltas %.2e"
+          % (worst_p, d_err))
 
 
 def test_highway_batchnorm_blocks(hip):

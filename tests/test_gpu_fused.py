@@ -113,6 +113,34 @@ def test_fused_steps_match_single_operations(hip, activation):
         assert_bit_equal(g, h.get_numpy_copy(a), "backward " + name)
 
 
+def test_packed_lstm_network_matches_to_rounding(hip):
+    # one stacked recurrent product per step instead of four: same values up to the
+    # summation order inside the matrix products
+    shape = dict(time_steps=20, batch=33, symbols=50, hidden=257)
+    plain = run_lstm(hip, False, **shape)
+    packed = run_lstm(hip, "packed", **shape)
+    assert packed.layers["lstm"]._stacked_recurrent(*list(packed.buffers["lstm"].parameters.values())[7:11]) is not None
+    for group in ("outputs", "internals", "output_deltas"):
+        for key in getattr(plain.buffers["lstm"], group):
+            want = plain.get("lstm", group, key)
+            got = packed.get("lstm", group, key)
+            scale = float(np.max(np.abs(want))) or 1.0
+            assert float(np.max(np.abs(got - want))) <= 1e-5 * scale, (group, key)
+    g_want, g_got = hip.get_numpy_copy(plain.gradients), hip.get_numpy_copy(packed.gradients)
+    for name, (a, b, _) in plain.parameter_slices().items():
+        scale = float(np.max(np.abs(g_want[a:b]))) or 1.0
+        assert float(np.max(np.abs(g_got[a:b] - g_want[a:b]))) <= 1e-5 * scale, name
+
+
+def test_stack_adjacent(hip):
+    flat = hip.allocate((4 * 6 + 5,))
+    parts = [flat[k * 6:(k + 1) * 6].reshape((2, 3)) for k in range(4)]
+    whole = hip.stack_adjacent(parts)
+    assert whole.shape == (8, 3) and whole.ptr == parts[0].ptr
+    assert hip.stack_adjacent([parts[0], parts[2]]) is None
+    assert hip.stack_adjacent([parts[0], flat[6:11].reshape((5,))]) is None
+
+
 def test_fused_step_argument_errors(hip):
     a = hip.allocate((4, 8))
     v = hip.allocate((1, 8))
