@@ -72,6 +72,11 @@ SIGNATURES = {
     "bship_lstm_bwd_step_f32": [c_int, _I64, _I64] + [_P] * 24,
     "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,
     "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
+    "bship_highway_fwd_f32": [_P, _P, _P, _P, c_size_t],
+    "bship_highway_bwd_f32": [_P] * 7 + [c_size_t],
+    "bship_bias_act_f32": [c_int, _P, _P, _P, _I64, _I64],
+    "bship_batchnorm_fwd_f32": [c_int, _P, _P, _P, _P, _P, c_double, c_double, _P, _P, _P, _P, _I64, _I64],
+    "bship_batchnorm_bwd_f32": [_P] * 7 + [_I64, _I64],
 }
 # functions that do not return a status
 SPECIAL_RESTYPES = {"bship_version": (c_int, []), "bship_last_error": (c_char_p, [])}

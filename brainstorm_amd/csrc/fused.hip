@@ -6,6 +6,7 @@
 // its results are bit-identical to the unfused sequence.
 #pragma clang fp contract(off)
 
+#include "colsum.h"
 #include "common.h"
 #include "functors.h"
 
@@ -146,10 +147,309 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
     }
 }
 
+
+// =================== generic multi-operand streaming kernels ===================
+// Bodies describe one element: apply(v, in, out) with v = the row-vector operands
+// at this column, in = the matrix operands at this element, out = the results.
+// A body provides the pointer tables vecs[kVecs], ins[kIn], outs[kOut]; an output
+// may be the same array as an input (every lane loads all operands first).
+constexpr int kFusedRows = 4;
+
+template <int W, bool AL, typename Body>
+__global__ __launch_bounds__(kBlock) void rowvec_fused_kernel(Body b, int64_t M, int64_t NW,
+                                                              unsigned col_tiles) {
+    typedef typename VecT<W>::type T;
+    constexpr int KV = Body::kVecs > 0 ? Body::kVecs : 1;
+    constexpr int R = kFusedRows;
+    const unsigned ct = blockIdx.x % col_tiles;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x / col_tiles) * R;
+    const int64_t c = static_cast<int64_t>(ct) * kBlock + threadIdx.x;
+    if (c >= NW) return;
+    T v[KV];
+#pragma unroll
+    for (int k = 0; k < Body::kVecs; ++k) v[k] = vload<W, AL>(b.vecs[k] + c * W);
+    T in[R][Body::kIn];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        if (r0 + u < M) {
+            const int64_t e = ((r0 + u) * NW + c) * W;
+#pragma unroll
+            for (int k = 0; k < Body::kIn; ++k) in[u][k] = vload<W, AL>(b.ins[k] + e);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        if (r0 + u < M) {
+            const int64_t e = ((r0 + u) * NW + c) * W;
+            T o[Body::kOut];
+            if constexpr (W == 1) {
+                float vs[KV], is[Body::kIn], os[Body::kOut];
+#pragma unroll
+                for (int k = 0; k < Body::kVecs; ++k) vs[k] = v[k];
+#pragma unroll
+                for (int k = 0; k < Body::kIn; ++k) is[k] = in[u][k];
+                b.apply(vs, is, os);
+#pragma unroll
+                for (int k = 0; k < Body::kOut; ++k) o[k] = os[k];
+            } else {
+#pragma unroll
+                for (int q = 0; q < W; ++q) {
+                    float vs[KV], is[Body::kIn], os[Body::kOut];
+#pragma unroll
+                    for (int k = 0; k < Body::kVecs; ++k) vs[k] = v[k][q];
+#pragma unroll
+                    for (int k = 0; k < Body::kIn; ++k) is[k] = in[u][k][q];
+                    b.apply(vs, is, os);
+#pragma unroll
+                    for (int k = 0; k < Body::kOut; ++k) o[k][q] = os[k];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < Body::kOut; ++k) vstore<W, AL>(b.outs[k] + e, o[k]);
+        }
+    }
+}
+
+template <typename Body>
+int launch_rowvec_fused(const char* name, const Body& b, int64_t M, int64_t N) {
+    if (M == 0 || N == 0) return 0;
+    const bool vec = (N % 4 == 0);
+    const int64_t NW = vec ? N / 4 : N;
+    const int64_t col_tiles = ceil_div(NW, kBlock);
+    const int64_t blocks = col_tiles * ceil_div(M, kFusedRows);
+    if (blocks > 0x7fffffff)
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: matrix too large for one launch", name);
+    bool al = true;
+    for (int k = 0; k < Body::kVecs; ++k) al = al && aligned16(b.vecs[k]);
+    for (int k = 0; k < Body::kIn; ++k) al = al && aligned16(b.ins[k]);
+    for (int k = 0; k < Body::kOut; ++k) al = al && aligned16(b.outs[k]);
+    const dim3 grid(static_cast<unsigned>(blocks)), blk(kBlock);
+    const unsigned ctl = static_cast<unsigned>(col_tiles);
+    hipStream_t s = ctx().stream;
+    if (vec && al) hipLaunchKernelGGL((rowvec_fused_kernel<4, true, Body>), grid, blk, 0, s, b, M, NW, ctl);
+    else if (vec)  hipLaunchKernelGGL((rowvec_fused_kernel<4, false, Body>), grid, blk, 0, s, b, M, NW, ctl);
+    else           hipLaunchKernelGGL((rowvec_fused_kernel<1, false, Body>), grid, blk, 0, s, b, M, NW, ctl);
+    return check_launch(name);
+}
+
+// Flat arrays: one workgroup per tile of 1024 floats, one 128-bit vector per lane
+// and operand; the array's last, partial vector is handled element by element.
+template <bool AL, typename Body>
+__global__ __launch_bounds__(kBlock) void flat_fused_kernel(Body b, size_t n) {
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {
+        f4 in[Body::kIn], o[Body::kOut];
+#pragma unroll
+        for (int k = 0; k < Body::kIn; ++k) in[k] = vload<4, AL>(b.ins[k] + i);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float is[Body::kIn], os[Body::kOut];
+#pragma unroll
+            for (int k = 0; k < Body::kIn; ++k) is[k] = in[k][q];
+            b.apply(nullptr, is, os);
+#pragma unroll
+            for (int k = 0; k < Body::kOut; ++k) o[k][q] = os[k];
+        }
+#pragma unroll
+        for (int k = 0; k < Body::kOut; ++k) vstore<4, AL>(b.outs[k] + i, o[k]);
+    } else {
+        for (size_t j = i; j < n; ++j) {
+            float is[Body::kIn], os[Body::kOut];
+#pragma unroll
+            for (int k = 0; k < Body::kIn; ++k) is[k] = b.ins[k][j];
+            b.apply(nullptr, is, os);
+#pragma unroll
+            for (int k = 0; k < Body::kOut; ++k) b.outs[k][j] = os[k];
+        }
+    }
+}
+
+template <typename Body>
+int launch_flat_fused(const char* name, const Body& b, size_t n) {
+    if (n == 0) return 0;
+    const size_t tiles = (n + static_cast<size_t>(kBlock) * 4 - 1) / (static_cast<size_t>(kBlock) * 4);
+    if (tiles > 0x7fffffffu)
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", name, n);
+    bool al = true;
+    for (int k = 0; k < Body::kIn; ++k) al = al && aligned16(b.ins[k]);
+    for (int k = 0; k < Body::kOut; ++k) al = al && aligned16(b.outs[k]);
+    const dim3 grid(static_cast<unsigned>(tiles)), blk(kBlock);
+    if (al) hipLaunchKernelGGL((flat_fused_kernel<true, Body>), grid, blk, 0, ctx().stream, b, n);
+    else    hipLaunchKernelGGL((flat_fused_kernel<false, Body>), grid, blk, 0, ctx().stream, b, n);
+    return check_launch(name);
+}
+
+// ---- Highway (highway_layer.py:40-71) ----
+// forward:  tmp = H - x; tmp = T * tmp; y = tmp + x
+struct HighwayFwdBody {
+    static constexpr int kVecs = 0, kIn = 3, kOut = 1;
+    const float* ins[3];   // H, T, x
+    float* outs[1];        // y
+    __device__ void apply(const float*, const float* in, float* o) const {
+        float tmp = in[0] - in[2];
+        tmp = in[1] * tmp;
+        o[0] = tmp + in[2];
+    }
+};
+// backward: tmp = 1 - T; dx += tmp * dy; dH += T * dy; tmp = H - x; dT += tmp * dy
+struct HighwayBwdBody {
+    static constexpr int kVecs = 0, kIn = 7, kOut = 3;
+    const float* ins[7];   // H, T, x, dy, dx, dH, dT
+    float* outs[3];        // dx, dH, dT
+    __device__ void apply(const float*, const float* in, float* o) const {
+        const float dy = in[3];
+        float tmp = 1.0f - in[1];
+        o[0] = MultAddOp{}.apply(tmp, dy, in[4]);
+        o[1] = MultAddOp{}.apply(in[1], dy, in[5]);
+        tmp = in[0] - in[2];
+        o[2] = MultAddOp{}.apply(tmp, dy, in[6]);
+    }
+};
+
+// ---- bias + activation of a fully connected layer (fully_connected_layer.py:62-64) ----
+template <typename Act>
+struct BiasActBody {
+    static constexpr int kVecs = 1, kIn = 1, kOut = 1;
+    const float* vecs[1];  // bias
+    const float* ins[1];   // the matrix product
+    float* outs[1];
+    __device__ void apply(const float* v, const float* in, float* o) const {
+        const float z = in[0] + v[0];
+        o[0] = Act{}.apply(z, 0.0f, 0.0f);
+    }
+};
+struct LinearOp { __device__ float apply(float x, float, float) const { return x; } };
+
+// ---- batch normalisation (batch_normalization_layer.py:54-152) ----
+// source of the variance reduction: centered = x + mu_b (stored), value = centered^2
+struct CenterSquareSrc {
+    const float* x;
+    const float* mu;
+    float* centered;
+    bool aligned() const { return aligned16(x) && aligned16(mu) && aligned16(centered); }
+    template <int W, bool AL> __device__ typename VecT<W>::type prep(int64_t col) const {
+        return vload<W, AL>(mu + col);
+    }
+    template <int W, bool AL>
+    __device__ typename VecT<W>::type load(int64_t off, typename VecT<W>::type m) const {
+        const typename VecT<W>::type c = vload<W, AL>(x + off) + m;
+        vstore<W, AL>(centered + off, c);
+        return c * c;
+    }
+};
+// source of the dgamma reduction: out_deltas * x_hat
+struct ProductSrc {
+    const float* a;
+    const float* b;
+    bool aligned() const { return aligned16(a) && aligned16(b); }
+    template <int W, bool AL> __device__ typename VecT<W>::type prep(int64_t) const {
+        return vzero<typename VecT<W>::type>();
+    }
+    template <int W, bool AL>
+    __device__ typename VecT<W>::type load(int64_t off, typename VecT<W>::type) const {
+        return vload<W, AL>(a + off) * vload<W, AL>(b + off);
+    }
+};
+
+// mu_b = (-1/m) * colsum; mu = decay * mu; mu += (1 - decay) * mu_b
+__global__ __launch_bounds__(kBlock) void bn_mean_update_kernel(float* mu_b, float* mu, float neg_inv_m,
+                                                                float decay, float one_minus_decay,
+                                                                int64_t n) {
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (j >= n) return;
+    const float b = MultStOp{neg_inv_m}.apply(mu_b[j], 0.0f, 0.0f);
+    mu_b[j] = b;
+    const float r = MultStOp{decay}.apply(mu[j], 0.0f, 0.0f);
+    mu[j] = MultAddStOp{one_minus_decay}.apply(b, r, 0.0f);
+}
+
+// sigma2 = (1/m) * colsum; sigma2 += eps; sigma_b = sqrt(sigma2);
+// sigma = decay * sigma; sigma += (1 - decay) * sigma_b
+__global__ __launch_bounds__(kBlock) void bn_sigma_update_kernel(float* sigma_b, float* sigma, float inv_m,
+                                                                 float eps, float decay,
+                                                                 float one_minus_decay, int64_t n) {
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (j >= n) return;
+    float s2 = MultStOp{inv_m}.apply(sigma_b[j], 0.0f, 0.0f);
+    s2 = AddStOp{eps}.apply(s2, 0.0f, 0.0f);
+    const float sb = SqrtOp{}.apply(s2, 0.0f, 0.0f);
+    sigma_b[j] = sb;
+    const float r = MultStOp{decay}.apply(sigma[j], 0.0f, 0.0f);
+    sigma[j] = MultAddStOp{one_minus_decay}.apply(sb, r, 0.0f);
+}
+
+// dgamma += s1; s1 *= 1/m; dbeta += s2; s2 *= 1/m; coeff = gamma / sigma_b
+__global__ __launch_bounds__(kBlock) void bn_bwd_vectors_kernel(float* s1, float* s2, float* coeff,
+                                                                float* dgamma, float* dbeta,
+                                                                const float* gamma, const float* sigma_b,
+                                                                float inv_m, int64_t n) {
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (j >= n) return;
+    const float a = s1[j], b = s2[j];
+    dgamma[j] = a + dgamma[j];
+    s1[j] = MultStOp{inv_m}.apply(a, 0.0f, 0.0f);
+    dbeta[j] = b + dbeta[j];
+    s2[j] = MultStOp{inv_m}.apply(b, 0.0f, 0.0f);
+    coeff[j] = gamma[j] / sigma_b[j];
+}
+
+// x_hat = centered / sigma; out = x_hat * gamma; out += beta
+struct BnNormBody {
+    static constexpr int kVecs = 3, kIn = 1, kOut = 2;
+    const float* vecs[3];  // sigma, gamma, beta
+    const float* ins[1];   // centered
+    float* outs[2];        // x_hat, out
+    __device__ void apply(const float* v, const float* in, float* o) const {
+        const float xh = in[0] / v[0];
+        const float t = xh * v[1];
+        o[0] = xh;
+        o[1] = t + v[2];
+    }
+};
+// the same with the centering in front (inference: running mean and deviation)
+struct BnInferBody {
+    static constexpr int kVecs = 4, kIn = 1, kOut = 3;
+    const float* vecs[4];  // mu (negative running mean), sigma, gamma, beta
+    const float* ins[1];   // inputs
+    float* outs[3];        // centered, x_hat, out
+    __device__ void apply(const float* v, const float* in, float* o) const {
+        const float c = in[0] + v[0];
+        const float xh = c / v[1];
+        const float t = xh * v[2];
+        o[0] = c;
+        o[1] = xh;
+        o[2] = t + v[3];
+    }
+};
+// term1 = x_hat * s1; term2 = dy - term1; term3 = term2 - s2; term4 = term3 * coeff;
+// in_deltas = term4 + in_deltas
+struct BnBwdBody {
+    static constexpr int kVecs = 3, kIn = 3, kOut = 1;
+    const float* vecs[3];  // s1 = colsum(dy * x_hat) / m, s2 = colsum(dy) / m, coeff = gamma / sigma_b
+    const float* ins[3];   // out_deltas, x_hat, in_deltas
+    float* outs[1];        // in_deltas
+    __device__ void apply(const float* v, const float* in, float* o) const {
+        const float t1 = in[1] * v[0];
+        const float t2 = in[0] - t1;
+        const float t3 = t2 - v[1];
+        const float t4 = t3 * v[2];
+        o[0] = t4 + in[2];
+    }
+};
 }  // namespace bship
 
 namespace bship {
 namespace {
+
+int check_pointers(const char* fn, const void* const* ptrs, int count) {
+    for (int i = 0; i < count; ++i) {
+        if (ptrs[i] == nullptr) return set_error(BSHIP_ERR_NULL_POINTER, "%s: an argument is NULL", fn);
+        if (reinterpret_cast<uintptr_t>(ptrs[i]) & 3u)
+            return set_error(BSHIP_ERR_BAD_POINTER, "%s: an argument is not 4-byte aligned", fn);
+    }
+    return 0;
+}
 
 int check_step_args(const char* fn, int act, int64_t batch, int64_t n, const void* const* ptrs,
                     int count) {
@@ -255,6 +555,116 @@ int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n, const floa
                   dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po,
                   deltas, dy, packed_out};
     return lstm_bwd_launch(__func__, true, act, batch, n, a);
+}
+
+int bship_highway_fwd_f32(const float* H, const float* T, const float* x, float* y, size_t n) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    const void* ptrs[] = {H, T, x, y};
+    int st = check_pointers(__func__, ptrs, 4);
+    if (st != 0) return st;
+    HighwayFwdBody b{{H, T, x}, {y}};
+    return launch_flat_fused("highway_forward", b, n);
+}
+
+int bship_highway_bwd_f32(const float* H, const float* T, const float* x, const float* dy, float* dx,
+                          float* dH, float* dT, size_t n) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    const void* ptrs[] = {H, T, x, dy, dx, dH, dT};
+    int st = check_pointers(__func__, ptrs, 7);
+    if (st != 0) return st;
+    HighwayBwdBody b{{H, T, x, dy, dx, dH, dT}, {dx, dH, dT}};
+    return launch_flat_fused("highway_backward", b, n);
+}
+
+int bship_bias_act_f32(int act, const float* in, const float* bias, float* out, int64_t M, int64_t N) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    if (act < kActSigmoid || act > kActEl)
+        return set_error(BSHIP_ERR_BAD_OP, "%s: unknown activation %d", __func__, act);
+    if (M == 0 || N == 0) return 0;
+    const void* ptrs[] = {in, bias, out};
+    int st = check_pointers(__func__, ptrs, 3);
+    if (st != 0) return st;
+    switch (act) {
+        case kActSigmoid: return launch_rowvec_fused("bias_act", BiasActBody<SigmoidOp>{{bias}, {in}, {out}}, M, N);
+        case kActTanh:    return launch_rowvec_fused("bias_act", BiasActBody<TanhOp>{{bias}, {in}, {out}}, M, N);
+        case kActRel:     return launch_rowvec_fused("bias_act", BiasActBody<RelOp>{{bias}, {in}, {out}}, M, N);
+        case kActEl:      return launch_rowvec_fused("bias_act", BiasActBody<ElOp>{{bias}, {in}, {out}}, M, N);
+        default:          return launch_rowvec_fused("bias_act", BiasActBody<LinearOp>{{bias}, {in}, {out}}, M, N);
+    }
+}
+
+int bship_batchnorm_fwd_f32(int training, const float* inputs, const float* gamma, const float* beta,
+                            float* mu, float* sigma, double decay, double epsilon, float* sigma_b,
+                            float* centered, float* x_hat, float* out, int64_t M, int64_t N) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    if (N == 0) return 0;
+    const void* ptrs[] = {inputs, gamma, beta, mu, sigma, sigma_b, centered, x_hat, out};
+    int st = check_pointers(__func__, ptrs, 9);
+    if (st != 0) return st;
+    if (!training) {
+        BnInferBody b{{mu, sigma, gamma, beta}, {inputs}, {centered, x_hat, out}};
+        return launch_rowvec_fused("batchnorm_forward", b, M, N);
+    }
+    BSHIP_REQUIRE_DIM(M >= 1);
+    // Python evaluates -1.0/m, 1.0/m and 1.0-decay in double; the handler then rounds to float32
+    const float neg_inv_m = static_cast<float>(-1.0 / static_cast<double>(M));
+    const float inv_m = static_cast<float>(1.0 / static_cast<double>(M));
+    const float dec = static_cast<float>(decay);
+    const float omd = static_cast<float>(1.0 - decay);
+    const float eps = static_cast<float>(epsilon);
+    const dim3 vgrid(static_cast<unsigned>(ceil_div(N, kBlock))), blk(kBlock);
+    hipStream_t s = ctx().stream;
+    // negative batch mean into sigma_b (the layer uses that buffer as scratch), running mean
+    st = M == 1 ? bship_d2d(sigma_b, inputs, static_cast<size_t>(N) * 4)
+                : launch_colsum(PlainSrc{inputs}, sigma_b, M, N);
+    if (st != 0) return st;
+    hipLaunchKernelGGL(bn_mean_update_kernel, vgrid, blk, 0, s, sigma_b, mu, neg_inv_m, dec, omd, N);
+    if ((st = check_launch("batchnorm mean")) != 0) return st;
+    // centered = inputs + mu_b while summing centered^2 down the columns
+    st = launch_colsum(CenterSquareSrc{inputs, sigma_b, centered}, sigma_b, M, N);
+    if (st != 0) return st;
+    hipLaunchKernelGGL(bn_sigma_update_kernel, vgrid, blk, 0, s, sigma_b, sigma, inv_m, eps, dec, omd, N);
+    if ((st = check_launch("batchnorm deviation")) != 0) return st;
+    BnNormBody b{{sigma_b, gamma, beta}, {centered}, {x_hat, out}};
+    return launch_rowvec_fused("batchnorm_forward", b, M, N);
+}
+
+int bship_batchnorm_bwd_f32(const float* out_deltas, const float* x_hat, const float* gamma,
+                            const float* sigma_b, float* dgamma, float* dbeta, float* in_deltas,
+                            int64_t M, int64_t N) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 1 && N >= 0);
+    if (N == 0) return 0;
+    const void* ptrs[] = {out_deltas, x_hat, gamma, sigma_b, dgamma, dbeta, in_deltas};
+    int st = check_pointers(__func__, ptrs, 7);
+    if (st != 0) return st;
+    void* raw = nullptr;
+    const size_t vec_bytes = (static_cast<size_t>(N) * 4 + 255) & ~static_cast<size_t>(255);
+    if ((st = pool_alloc_raw(3 * vec_bytes, &raw)) != 0) return st;
+    float* s1 = static_cast<float*>(raw);
+    float* s2 = reinterpret_cast<float*>(static_cast<char*>(raw) + vec_bytes);
+    float* coeff = reinterpret_cast<float*>(static_cast<char*>(raw) + 2 * vec_bytes);
+    const float inv_m = static_cast<float>(1.0 / static_cast<double>(M));
+    st = launch_colsum(ProductSrc{out_deltas, x_hat}, s1, M, N);
+    if (st == 0)
+        st = M == 1 ? bship_d2d(s2, out_deltas, static_cast<size_t>(N) * 4)
+                    : launch_colsum(PlainSrc{out_deltas}, s2, M, N);
+    if (st == 0) {
+        hipLaunchKernelGGL(bn_bwd_vectors_kernel, dim3(static_cast<unsigned>(ceil_div(N, kBlock))),
+                           dim3(kBlock), 0, ctx().stream, s1, s2, coeff, dgamma, dbeta, gamma, sigma_b,
+                           inv_m, N);
+        st = check_launch("batchnorm gradients");
+    }
+    if (st == 0) {
+        BnBwdBody b{{s1, s2, coeff}, {out_deltas, x_hat, in_deltas}, {in_deltas}};
+        st = launch_rowvec_fused("batchnorm_backward", b, M, N);
+    }
+    pool_free_raw(raw);   // a later owner of the block runs after these launches
+    return st;
 }
 
 }  // extern "C"

@@ -82,7 +82,7 @@ def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1
     return _finish(net, data, _init_parameters(net, rng, 0.05))
 
 
-def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10):
+def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10, fused=False):
     rng = np.random.RandomState(seed)
     data = {"default": rng.standard_normal((1, batch, width)).astype(F32),
             "targets": rng.randint(0, classes, (1, batch, 1)).astype(F32)}
@@ -90,10 +90,10 @@ def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10
     prev = "Input.default"
     for k in range(blocks):
         layers += [
-            ("bn%d" % k, BatchNorm(), {"default": prev}),
-            ("H%d" % k, FullyConnected(width, "rel"), {"default": "bn%d.default" % k}),
-            ("T%d" % k, FullyConnected(width, "sigmoid"), {"default": "bn%d.default" % k}),
-            ("hw%d" % k, Highway(), {"H": "H%d.default" % k, "T": "T%d.default" % k,
+            ("bn%d" % k, BatchNorm(fused=fused), {"default": prev}),
+            ("H%d" % k, FullyConnected(width, "rel", fused=fused), {"default": "bn%d.default" % k}),
+            ("T%d" % k, FullyConnected(width, "sigmoid", fused=fused), {"default": "bn%d.default" % k}),
+            ("hw%d" % k, Highway(fused=fused), {"H": "H%d.default" % k, "T": "T%d.default" % k,
                                      "x": "bn%d.default" % k}),
         ]
         prev = "hw%d.default" % k

@@ -98,9 +98,10 @@ class Input(Layer):
 class FullyConnected(Layer):
     """layers/fully_connected_layer.py:52-78"""
 
-    def __init__(self, size, activation="rel"):
+    def __init__(self, size, activation="rel", fused=False):
         self.size = int(size)
         self.activation = activation
+        self.fused = bool(fused)        # bias + activation through handler.bias_act when it exists
 
     def setup(self, in_shapes):
         in_size = _prod(in_shapes["default"].feature_shape)
@@ -114,6 +115,9 @@ class FullyConnected(Layer):
         inputs = flatten_time_and_features(buffers.inputs["default"])
         outputs = flatten_time_and_features(buffers.outputs["default"])
         _h.dot_mm(inputs, W, outputs, transb=True)
+        if self.fused and hasattr(_h, "bias_act"):
+            _h.bias_act(self.activation, outputs, bias, outputs)
+            return
         _h.add_mv(outputs, bias.reshape((1, bias.shape[0])), outputs)
         _h.inplace_act_func[self.activation](outputs)
 
@@ -459,9 +463,10 @@ class Lstm(Layer):
 class BatchNorm(Layer):
     """layers/batch_normalization_layer.py:54-152"""
 
-    def __init__(self, decay=0.9, epsilon=1.0e-5):
+    def __init__(self, decay=0.9, epsilon=1.0e-5, fused=False):
         self.decay = decay
         self.epsilon = epsilon
+        self.fused = bool(fused)        # whole passes through handler.batchnorm_* when they exist
 
     def setup(self, in_shapes):
         shape = in_shapes["default"].feature_shape
@@ -479,6 +484,10 @@ class BatchNorm(Layer):
         x_hat = flatten_all_but_last(buffers.internals["x_hat"])
         out = flatten_all_but_last(buffers.outputs["default"])
         m = inputs.shape[0]
+        if self.fused and hasattr(_h, "batchnorm_forward"):
+            _h.batchnorm_forward(training_pass, inputs, gamma, beta, mu, sigma, self.decay,
+                                 self.epsilon, sigma_b, centered, x_hat, out)
+            return
 
         if training_pass:
             mu_b = sigma_b                       # reused as scratch for the NEGATIVE batch mean
@@ -514,6 +523,9 @@ class BatchNorm(Layer):
         outdeltas = flatten_all_but_last(buffers.output_deltas["default"])
         indeltas = flatten_all_but_last(buffers.input_deltas["default"])
         m = outdeltas.shape[0]
+        if self.fused and hasattr(_h, "batchnorm_backward"):
+            _h.batchnorm_backward(outdeltas, x_hat, gamma, sigma_b, dgamma, dbeta, indeltas)
+            return
 
         big_tmp = _h.allocate(x_hat.shape)
         small_tmp = _h.allocate(gamma.shape)
@@ -538,6 +550,9 @@ class BatchNorm(Layer):
 class Highway(Layer):
     """layers/highway_layer.py:40-71: y = T*H + (1-T)*x with inputs 'H', 'T', 'x'."""
 
+    def __init__(self, fused=False):
+        self.fused = bool(fused)        # one pass each way through handler.highway_* when they exist
+
     def setup(self, in_shapes):
         return OrderedDict(default=Buf(in_shapes["x"].feature_shape)), OrderedDict(), OrderedDict()
 
@@ -545,6 +560,9 @@ class Highway(Layer):
         _h = self.handler
         x, H, T = buffers.inputs["x"], buffers.inputs["H"], buffers.inputs["T"]
         y = buffers.outputs["default"]
+        if self.fused and hasattr(_h, "highway_forward"):
+            _h.highway_forward(H, T, x, y)
+            return
         tmp = _h.zeros(x.shape)
         _h.subtract_tt(H, x, out=tmp)
         _h.mult_tt(T, tmp, out=tmp)
@@ -555,6 +573,9 @@ class Highway(Layer):
         x, H, T = buffers.inputs["x"], buffers.inputs["H"], buffers.inputs["T"]
         dx, dH, dT = buffers.input_deltas["x"], buffers.input_deltas["H"], buffers.input_deltas["T"]
         dy = buffers.output_deltas["default"]
+        if self.fused and hasattr(_h, "highway_backward"):
+            _h.highway_backward(H, T, x, dy, dx, dH, dT)
+            return
         tmp = _h.ones(dx.shape)
         _h.subtract_tt(tmp, T, out=tmp)
         _h.mult_add_tt(tmp, dy, out=dx)

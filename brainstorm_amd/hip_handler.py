@@ -483,3 +483,45 @@ class HipHandler(Handler):
         self._call(self._lib.bship_lstm_bwd_step_packed_f32(
             self._ACT_CODES[activation], batch, n, deltas.ptr, dy.ptr, packed_out.ptr,
             *[a.ptr for a in mats[2:] + vecs]))
+
+    def highway_forward(self, H, T, x, y):
+        """y = T * (H - x) + x with the roundings of highway_layer.py:48-51, one pass."""
+        if not (H.shape == T.shape == x.shape == y.shape):
+            raise ValueError("highway_forward: inconsistent shapes")
+        self._call(self._lib.bship_highway_fwd_f32(H.ptr, T.ptr, x.ptr, y.ptr, y.size))
+
+    def highway_backward(self, H, T, x, dy, dx, dH, dT):
+        """dx += (1-T)*dy; dH += T*dy; dT += (H-x)*dy (highway_layer.py:64-71), one pass."""
+        if any(a.shape != x.shape for a in (H, T, dy, dx, dH, dT)):
+            raise ValueError("highway_backward: inconsistent shapes")
+        self._call(self._lib.bship_highway_bwd_f32(H.ptr, T.ptr, x.ptr, dy.ptr, dx.ptr, dH.ptr,
+                                                   dT.ptr, x.size))
+
+    def bias_act(self, activation, m, bias, out):
+        """out = act(m + bias): add_mv followed by act_func[activation] in one pass
+        (fully_connected_layer.py:61-62). m and out are (M, N), bias has N elements."""
+        n_cols = m.shape[-1]
+        if out.shape != m.shape or bias.size != n_cols:
+            raise ValueError("bias_act: inconsistent shapes")
+        self._call(self._lib.bship_bias_act_f32(self._ACT_CODES[activation], m.ptr, bias.ptr, out.ptr,
+                                                m.size // n_cols if n_cols else 0, n_cols))
+
+    def batchnorm_forward(self, training_pass, inputs, gamma, beta, mu, sigma, decay, epsilon,
+                          sigma_b, centered, x_hat, out):
+        """batch_normalization_layer.py:54-105 on flattened (M, N) buffers."""
+        rows, n = inputs.shape
+        if (any(a.shape != (rows, n) for a in (centered, x_hat, out))
+                or any(v.size != n for v in (gamma, beta, mu, sigma, sigma_b))):
+            raise ValueError("batchnorm_forward: inconsistent shapes")
+        self._call(self._lib.bship_batchnorm_fwd_f32(
+            int(bool(training_pass)), inputs.ptr, gamma.ptr, beta.ptr, mu.ptr, sigma.ptr,
+            float(decay), float(epsilon), sigma_b.ptr, centered.ptr, x_hat.ptr, out.ptr, rows, n))
+
+    def batchnorm_backward(self, out_deltas, x_hat, gamma, sigma_b, dgamma, dbeta, in_deltas):
+        """batch_normalization_layer.py:107-152 on flattened (M, N) buffers."""
+        rows, n = out_deltas.shape
+        if (x_hat.shape != (rows, n) or in_deltas.shape != (rows, n)
+                or any(v.size != n for v in (gamma, sigma_b, dgamma, dbeta))):
+            raise ValueError("batchnorm_backward: inconsistent shapes")
+        self._call(self._lib.bship_batchnorm_bwd_f32(out_deltas.ptr, x_hat.ptr, gamma.ptr, sigma_b.ptr,
+                                                     dgamma.ptr, dbeta.ptr, in_deltas.ptr, rows, n))

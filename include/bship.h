@@ -322,6 +322,43 @@ int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n,
                                    float* dCa, float* dCb, const float* pi,
                                    const float* pf, const float* po);
 
+/* HighwayLayerImpl.forward_pass (highway_layer.py 48-51) in one pass:
+ * tmp = H - x; tmp = T * tmp; y = tmp + x. */
+int bship_highway_fwd_f32(const float* H, const float* T, const float* x,
+                          float* y, size_t n);
+/* HighwayLayerImpl.backward_pass (highway_layer.py 64-71) in one pass:
+ * dx += (1 - T) * dy; dH += T * dy; dT += (H - x) * dy. */
+int bship_highway_bwd_f32(const float* H, const float* T, const float* x,
+                          const float* dy, float* dx, float* dH, float* dT,
+                          size_t n);
+/* add_mv(outputs, bias, outputs) followed by inplace_act_func[act](outputs)
+ * (fully_connected_layer.py 61-62) in one pass: out = act(in + bias), in and
+ * out (M,N), bias N elements, act one of BSHIP_ACT_*. out may be in. */
+int bship_bias_act_f32(int act, const float* in, const float* bias, float* out,
+                       int64_t M, int64_t N);
+/* BatchNormLayerImpl.forward_pass (batch_normalization_layer.py 54-105) on
+ * (M,N) matrices and N-element vectors. training != 0: batch statistics (the
+ * negative batch mean and then the deviation go through sigma_b as in the
+ * layer), running averages mu and sigma updated with `decay`, three passes
+ * over the matrix instead of seven: column sums; centering fused with the
+ * column sums of squares; normalise + scale + shift. training == 0: one pass
+ * with the running mu and sigma. decay and epsilon arrive as the Python floats
+ * (the layer computes 1.0 - decay in double before the handler rounds it). */
+int bship_batchnorm_fwd_f32(int training, const float* inputs,
+                            const float* gamma, const float* beta, float* mu,
+                            float* sigma, double decay, double epsilon,
+                            float* sigma_b, float* centered, float* x_hat,
+                            float* out, int64_t M, int64_t N);
+/* BatchNormLayerImpl.backward_pass (batch_normalization_layer.py 107-152):
+ * dgamma += colsum(out_deltas * x_hat); dbeta += colsum(out_deltas);
+ * in_deltas += ((out_deltas - x_hat * dgamma_b / M) - dbeta_b / M) * gamma / sigma_b
+ * with the layer's order of float32 operations. Takes 3 N-element temporaries
+ * from the pool. */
+int bship_batchnorm_bwd_f32(const float* out_deltas, const float* x_hat,
+                            const float* gamma, const float* sigma_b,
+                            float* dgamma, float* dbeta, float* in_deltas,
+                            int64_t M, int64_t N);
+
 #ifdef __cplusplus
 }
 #endif

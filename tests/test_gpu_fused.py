@@ -1,4 +1,5 @@
-"""GPU: the fused LSTM time-step entry points against the sequence of single
+"""GPU: the fused layer-level entry points (LSTM time steps, Highway, BatchNorm, bias +
+activation) against the sequence of single
 handler operations they replace. Both run on the GPU with the same matrix-product
 kernels, so every buffer must agree bit for bit; the unfused sequence itself is
 held to the CPU oracle in test_gpu_configs.py."""
@@ -156,3 +157,130 @@ def test_fused_step_argument_errors(hip):
     assert lib.bship_lstm_fwd_step_f32(1, 4, 8, *([p] * 18 + [None])) == -2
     assert lib.bship_lstm_bwd_step_f32(1, -1, 8, *([p] * 24)) == -3
     assert lib.bship_lstm_bwd_step_f32(1, 0, 8, *([p] * 24)) == 0
+
+
+# ------------------------------------------------------------------ Highway / BatchNorm / bias
+def run_highway(hip, fused, training=True, **kw):
+    hip.rnd.seed(6)
+    net, data = configs.build_highway(hip, fused=fused, **kw)
+    net.provide_external_data(data)
+    net.forward_pass(training_pass=training)
+    net.backward_pass()
+    return net
+
+
+@pytest.mark.parametrize("shape", [dict(blocks=2, batch=37, width=101), dict(blocks=3, batch=256, width=512)])
+@pytest.mark.parametrize("training", [True, False])
+def test_fused_highway_batchnorm_network_is_bit_identical(hip, shape, training):
+    plain = run_highway(hip, False, training, **shape)
+    fused = run_highway(hip, True, training, **shape)
+    for name in plain.layers:
+        for group in ("outputs", "internals", "output_deltas"):
+            for key in getattr(plain.buffers[name], group):
+                if training is False and name.startswith("bn") and key == "sigma_b":
+                    continue        # not written by an inference pass
+                assert_bit_equal(fused.get(name, group, key), plain.get(name, group, key),
+                                 "%s.%s.%s" % (name, group, key))
+    assert_bit_equal(hip.get_numpy_copy(fused.parameters), hip.get_numpy_copy(plain.parameters), "parameters")
+    if training:                    # the backward pass uses the batch deviation of a training pass
+        assert_bit_equal(hip.get_numpy_copy(fused.gradients), hip.get_numpy_copy(plain.gradients), "gradients")
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 5), (37, 129), (300, 64), (2048, 260)])
+def test_fused_batchnorm_matches_single_operations(hip, rows, cols):
+    from brainstorm_amd.drivers.layers import BatchNorm
+    rng = np.random.RandomState(rows * 1000 + cols)
+    h = hip
+
+    class Bufs:
+        pass
+
+    def make(fused):
+        r = np.random.RandomState(99)
+        pad = h.allocate((1,))          # shifts what follows off 16-byte alignment in one variant
+        b = Bufs()
+        flat = h.create_from_numpy(r.standard_normal((6, 1, rows, cols)).astype(F32))
+        b.inputs = {"default": flat[0]}
+        b.outputs = {"default": flat[1]}
+        b.internals = {"sigma_b": h.create_from_numpy(r.standard_normal((cols,)).astype(F32)),
+                       "centered": flat[2], "x_hat": flat[3]}
+        b.output_deltas = {"default": flat[4]}
+        b.input_deltas = {"default": flat[5]}
+        vec = lambda lo, hi: h.create_from_numpy(r.uniform(lo, hi, (cols,)).astype(F32))
+        from collections import OrderedDict
+        b.parameters = OrderedDict([("gamma", vec(0.5, 2)), ("beta", vec(-1, 1)), ("mu", vec(-1, 1)),
+                                    ("sigma", vec(0.5, 2))])
+        b.gradients = OrderedDict([("gamma", vec(-1, 1)), ("beta", vec(-1, 1))])
+        layer = BatchNorm(fused=fused)
+        layer.handler = h
+        return layer, b, pad
+
+    for training in (True, False):
+        results = []
+        for fused in (False, True):
+            layer, b, _ = make(fused)
+            layer.forward_pass(b, training_pass=training)
+            if training:
+                layer.backward_pass(b)
+            got = {}
+            for group in ("outputs", "internals", "input_deltas", "parameters", "gradients"):
+                for key, arr in getattr(b, group).items():
+                    got[group + "." + key] = h.get_numpy_copy(arr)
+            results.append(got)
+        for key in results[0]:
+            assert_bit_equal(results[1][key], results[0][key], "training=%s %s" % (training, key))
+
+
+@pytest.mark.parametrize("activation", ["tanh", "sigmoid", "rel", "el", "linear"])
+@pytest.mark.parametrize("rows,cols", [(3, 7), (65, 1028)])
+def test_bias_act_matches_single_operations(hip, activation, rows, cols):
+    rng = np.random.RandomState(3)
+    x = rng.standard_normal((rows, cols)).astype(F32)
+    bias = hip.create_from_numpy(rng.standard_normal((cols,)).astype(F32))
+    a = hip.create_from_numpy(x)
+    b = hip.create_from_numpy(x)
+    hip.bias_act(activation, a, bias, a)
+    hip.add_mv(b, bias.reshape((1, cols)), b)
+    hip.inplace_act_func[activation](b)
+    assert_bit_equal(a.get(), b.get(), activation)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1024, 4099, 300001])
+def test_highway_steps_match_single_operations(hip, n):
+    rng = np.random.RandomState(n)
+    h = hip
+    flat = h.create_from_numpy(rng.standard_normal((8, n)).astype(F32))   # rows start at odd offsets
+    H, T, x, dy, dx, dH, dT, y = [flat[k] for k in range(8)]
+    init = flat.get()
+    h.highway_forward(H, T, x, y)
+    h.highway_backward(H, T, x, dy, dx, dH, dT)
+    got = flat.get()
+    h.set_from_numpy(flat, init)
+    tmp = h.zeros(x.shape)
+    h.subtract_tt(H, x, out=tmp)
+    h.mult_tt(T, tmp, out=tmp)
+    h.add_tt(tmp, x, out=y)
+    tmp = h.ones(dx.shape)
+    h.subtract_tt(tmp, T, out=tmp)
+    h.mult_add_tt(tmp, dy, out=dx)
+    h.mult_add_tt(T, dy, out=dH)
+    h.subtract_tt(H, x, out=tmp)
+    h.mult_add_tt(tmp, dy, out=dT)
+    assert_bit_equal(got, flat.get(), "highway n=%d" % n)
+
+
+def test_fused_layer_argument_errors(hip):
+    a = hip.allocate((4, 8))
+    v = hip.allocate((8,))
+    with pytest.raises(ValueError):
+        hip.highway_forward(a, a, a, hip.allocate((4, 9)))
+    with pytest.raises(ValueError):
+        hip.bias_act("rel", a, hip.allocate((7,)), a)
+    with pytest.raises(ValueError):
+        hip.batchnorm_forward(True, a, v, v, v, v, 0.9, 1e-5, v, a, a, hip.allocate((8, 4)))
+    lib = hip._lib
+    assert lib.bship_bias_act_f32(7, a.ptr, v.ptr, a.ptr, 4, 8) == -4
+    assert lib.bship_highway_fwd_f32(a.ptr, None, a.ptr, a.ptr, 32) == -2
+    assert lib.bship_batchnorm_bwd_f32(a.ptr, a.ptr, v.ptr, v.ptr, v.ptr, v.ptr, a.ptr, 0, 8) == -3
+    assert lib.bship_batchnorm_fwd_f32(1, a.ptr, v.ptr, v.ptr, v.ptr, v.ptr, 0.9, 1e-5, v.ptr, a.ptr,
+                                       a.ptr, a.ptr, 4, 0) == 0
