@@ -205,6 +205,9 @@ def run_nets_gpu(hip):
     from brainstorm_amd.drivers import configs
     return {
         "mlp_784-1200-1200-10_batch100": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize),
+        # same network, dropout and bias+activation through the fused entry points (same bits)
+        "mlp_784-1200-1200-10_batch100_fused": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize,
+                                                        fused=True),
         "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
         # same network, the elementwise part of each time step in one launch (same bits)
         "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,

@@ -74,6 +74,7 @@ SIGNATURES = {
     "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
     "bship_highway_fwd_f32": [_P, _P, _P, _P, c_size_t],
     "bship_highway_bwd_f32": [_P] * 7 + [c_size_t],
+    "bship_dropout_fwd_f32": [_P, _P, _P, c_size_t, c_double, c_float],
     "bship_bias_act_f32": [c_int, _P, _P, _P, _I64, _I64],
     "bship_batchnorm_fwd_f32": [c_int, _P, _P, _P, _P, _P, c_double, c_double, _P, _P, _P, _P, _I64, _I64],
     "bship_batchnorm_bwd_f32": [_P] * 7 + [_I64, _I64],

@@ -22,7 +22,11 @@
 // MI355X: 1.5 ns per double (a 100x1200 dropout mask in 0.16 ms); a minimal
 // LDS-read / write / barrier step of a 1024-lane workgroup costs 0.13 us there,
 // which bounds this single-stream design at roughly 0.4 ns per double.
+#include <cstdlib>
+#include <deque>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 
@@ -78,12 +82,17 @@ static_assert(kWideHistory + 2 * kWide + 2 <= kRing, "ring holds history, a step
 // RandomState would have it (whole blocks regenerated, position inside the last
 // one). One workgroup of kRngThreads threads; every control decision is the same
 // in all threads, so the barriers are reached uniformly.
+// If `before` is not null it receives the stream position (key, pos) as found.
 template <typename Sink>
-__device__ __forceinline__ void mt_generate(RngState* st, size_t n, Sink sink) {
+__device__ __forceinline__ void mt_generate(RngState* st, size_t n, Sink sink, RngState* before = nullptr) {
     __shared__ uint32_t ring[kRing];
     const unsigned t = threadIdx.x;
     for (unsigned i = t; i < kMtN; i += kRngThreads) ring[i] = st->key[i];
     const size_t pos0 = static_cast<size_t>(st->pos);        // 0..624, next unread word
+    if (before != nullptr) {
+        for (unsigned i = t; i < kMtN; i += kRngThreads) before->key[i] = ring[i];
+        if (t == 0) before->pos = static_cast<int32_t>(pos0);
+    }
     __syncthreads();
     const size_t end_word = pos0 + 2 * n;                     // first word NOT consumed
     const size_t gen_end = (end_word + kMtN - 1) / kMtN * kMtN;   // whole blocks
@@ -142,14 +151,14 @@ __device__ __forceinline__ void mt_generate(RngState* st, size_t n, Sink sink) {
 
 // mask[i] = (next_double() < p) ? 1 : 0 for i in [0,n).
 __global__ __launch_bounds__(kRngThreads) void mt_mask_kernel(RngState* st, float* __restrict__ mask,
-                                                         size_t n, double p) {
+                                                         size_t n, double p, RngState* before) {
     // k / 2^53 < p  <=>  k < ceil(p * 2^53): p * 2^53 is exact in float64, so the reference's
     // float64 compare of the stream's double with p becomes an integer compare.
     uint64_t threshold;
     if (!(p > 0.0)) threshold = 0;                                   // p <= 0 or NaN: never
     else if (p >= 1.0) threshold = ~static_cast<uint64_t>(0);        // every k is below 2^53
     else threshold = static_cast<uint64_t>(ceil(p * 9007199254740992.0));
-    mt_generate(st, n, [=](size_t i, uint64_t k) { mask[i] = (k < threshold) ? 1.0f : 0.0f; });
+    mt_generate(st, n, [=](size_t i, uint64_t k) { mask[i] = (k < threshold) ? 1.0f : 0.0f; }, before);
 }
 
 // u[i] = next_double() for i in [0,n) (used by fill_gaussian, also to skip ahead).
@@ -244,11 +253,6 @@ __global__ void rng_copy_state_kernel(const RngState* src, RngState* dst) {
     if (threadIdx.x == 0) { dst->pos = src->pos; }
 }
 
-void rng_release() {
-    std::lock_guard<std::mutex> lock(g_rng_mutex);
-    if (g_state) { pool_free_raw(g_state); g_state = nullptr; }
-}
-
 static int rng_ensure_state() {
     if (g_state) return 0;
     void* p = nullptr;
@@ -256,6 +260,197 @@ static int rng_ensure_state() {
     if (st != 0) return st;
     g_state = static_cast<RngState*>(p);
     return 0;
+}
+
+// ------------------------------ mask prefetch ------------------------------
+// A mask costs a fixed sequential time on ONE compute unit and depends on
+// nothing but the stream position, while a training loop asks for the same
+// masks, in the same order, every step. Once the recent requests (n, p) repeat
+// with some period P, the next P masks are drawn ahead of time on a second
+// stream into staging buffers, overlapping the step's other kernels; a matching
+// request then is a wait on an event plus a device copy, and the entry is drawn
+// again for the step after. Each entry keeps the stream position from before
+// its draw, so any request that does not match the prediction (or any other use
+// of the generator) rewinds to exactly the position a purely sequential
+// generator would have, and results never depend on whether a prefetch hit.
+struct MaskPrefetch {
+    size_t n;
+    double p;
+    float* staging;
+    RngState* before;      // key and pos before this mask was drawn
+    hipEvent_t ready;      // second stream: the mask is in staging
+    hipEvent_t consumed;   // main stream: staging has been copied out
+};
+static std::deque<MaskPrefetch> g_fifo;
+static std::vector<std::pair<size_t, double>> g_history;
+static hipStream_t g_side = nullptr;
+static hipEvent_t g_join = nullptr;          // orders one stream behind the other
+constexpr size_t kMaxPeriod = 16;
+static size_t g_min_period = 1;              // raised after a wrong guess, see prefetch_flush()
+constexpr size_t kMaxPrefetchFloats = size_t(1) << 26;   // per period: 256 MiB of staging at most
+
+static bool prefetch_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("BSHIP_RNG_PREFETCH");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+static void free_entry(MaskPrefetch& e) {
+    if (e.staging) pool_free_raw(e.staging);
+    if (e.before) pool_free_raw(e.before);
+    if (e.ready) (void)hipEventDestroy(e.ready);
+    if (e.consumed) (void)hipEventDestroy(e.consumed);
+    e = MaskPrefetch();
+}
+
+// Makes `later` wait for everything enqueued on `earlier` so far.
+static int order_streams(hipStream_t earlier, hipStream_t later) {
+    if (!g_join) BSHIP_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    BSHIP_HIP(hipEventRecord(g_join, earlier));
+    BSHIP_HIP(hipStreamWaitEvent(later, g_join, 0));
+    return 0;
+}
+
+// Drops every prefetched mask and puts the generator back to the position before
+// the oldest of them. Afterwards the main stream owns the generator again.
+static int prefetch_flush(bool restore_position, bool wrong_guess = false) {
+    g_history.clear();
+    if (g_fifo.empty()) return 0;
+    // "A B B" looks like period 1 after its second B: when a guess turns out wrong, only
+    // longer periods are tried next (any multiple of the true period serves as well)
+    if (wrong_guess) g_min_period = g_fifo.size() + 1 > kMaxPeriod ? 1 : g_fifo.size() + 1;
+    int st = order_streams(g_side, ctx().stream);
+    if (st == 0 && restore_position) {
+        hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, ctx().stream,
+                           g_fifo.front().before, g_state);
+        st = check_launch("random stream rewind");
+    }
+    // the blocks go back to the pool; their next owners run on the main stream, which is
+    // ordered behind the second stream now
+    for (MaskPrefetch& e : g_fifo) free_entry(e);
+    g_fifo.clear();
+    return st;
+}
+
+// Enqueues the draw of one mask on the second stream and appends it to the queue.
+static int prefetch_schedule(MaskPrefetch e, bool wait_consumed) {
+    if (wait_consumed) BSHIP_HIP(hipStreamWaitEvent(g_side, e.consumed, 0));
+    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, g_side, g_state, e.staging, e.n, e.p,
+                       e.before);
+    int st = check_launch("mask prefetch");
+    if (st != 0) { free_entry(e); return st; }
+    BSHIP_HIP(hipEventRecord(e.ready, g_side));
+    g_fifo.push_back(e);
+    return 0;
+}
+
+// After a mask was drawn directly: if the recent requests repeat with period P,
+// draw the next P masks ahead. Failures here only mean "no prefetch".
+static void prefetch_maybe_start() {
+    const size_t h = g_history.size();
+    size_t period = 0;
+    for (size_t P = g_min_period; P <= kMaxPeriod && 2 * P <= h; ++P) {
+        bool same = true;
+        for (size_t k = 0; k < P && same; ++k) same = g_history[h - 1 - k] == g_history[h - 1 - k - P];
+        if (same) { period = P; break; }
+    }
+    if (h > 4 * kMaxPeriod) g_history.erase(g_history.begin(), g_history.begin() + (h - 2 * kMaxPeriod));
+    if (period == 0) return;
+    size_t total = 0;
+    for (size_t k = 0; k < period; ++k) total += g_history[g_history.size() - period + k].first;
+    if (total > kMaxPrefetchFloats) return;
+    if (!g_side && hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking) != hipSuccess) { g_side = nullptr; return; }
+    if (order_streams(ctx().stream, g_side) != 0) return;
+    const std::vector<std::pair<size_t, double>> next(g_history.end() - period, g_history.end());
+    for (const auto& req : next) {
+        MaskPrefetch e = MaskPrefetch();
+        e.n = req.first;
+        e.p = req.second;
+        void* a = nullptr;
+        void* b = nullptr;
+        bool ok = pool_alloc_raw(e.n * sizeof(float), &a) == 0;
+        e.staging = static_cast<float*>(a);
+        ok = ok && pool_alloc_raw(sizeof(RngState), &b) == 0;
+        e.before = static_cast<RngState*>(b);
+        ok = ok && hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) == hipSuccess;
+        ok = ok && hipEventCreateWithFlags(&e.consumed, hipEventDisableTiming) == hipSuccess;
+        if (!ok) { free_entry(e); break; }
+        // fresh pool blocks may still be in use by earlier main-stream work: already ordered above
+        if (prefetch_schedule(e, false) != 0) break;
+    }
+}
+
+// Serves a mask request: either hands back the queue's front entry (*is_hit; the caller reads
+// hit->staging on the main stream and then calls mask_end), or draws the mask into `mask` directly.
+static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* is_hit) {
+    *is_hit = false;
+    if (!g_fifo.empty()) {
+        const MaskPrefetch& e = g_fifo.front();
+        if (e.n == n && e.p == p) {
+            BSHIP_HIP(hipStreamWaitEvent(ctx().stream, e.ready, 0));
+            *hit = e;
+            *is_hit = true;
+            g_fifo.pop_front();
+            return 0;
+        }
+        int st = prefetch_flush(true, true);
+        if (st != 0) return st;
+    }
+    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, ctx().stream, g_state, mask, n, p,
+                       static_cast<RngState*>(nullptr));
+    int st = check_launch("generate_probability_mask");
+    if (st == 0 && prefetch_enabled()) {
+        g_history.emplace_back(n, p);
+        prefetch_maybe_start();
+    }
+    return st;
+}
+
+// The main stream has enqueued its read of the entry's staging buffer: draw the entry again
+// for the next round.
+static int mask_end(MaskPrefetch& e) {
+    hipError_t err = hipEventRecord(e.consumed, ctx().stream);
+    if (err != hipSuccess) { free_entry(e); return check_hip(err, "hipEventRecord"); }
+    return prefetch_schedule(e, true);
+}
+
+// Dropout forward (dropout_layer.py:41-45) behind the mask: mask = src (the mask as drawn),
+// out = in * mask, out = scale * out.
+template <bool AL>
+__global__ __launch_bounds__(kBlock) void dropout_apply_kernel(const float* src, float* mask, const float* in,
+                                                               float* out, float scale, size_t n) {
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {
+        const f4 m = vload<4, AL>(src + i);
+        const f4 x = vload<4, AL>(in + i);
+        if (src != mask) vstore<4, AL>(mask + i, m);
+        f4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { const float t = x[k] * m[k]; o[k] = scale * t; }
+        vstore<4, AL>(out + i, o);
+    } else {
+        for (size_t j = i; j < n; ++j) {
+            const float m = src[j];
+            const float t = in[j] * m;
+            mask[j] = m;
+            out[j] = scale * t;
+        }
+    }
+}
+
+void rng_release() {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (g_side) (void)hipStreamSynchronize(g_side);
+    for (MaskPrefetch& e : g_fifo) free_entry(e);
+    g_fifo.clear();
+    g_history.clear();
+    g_min_period = 1;
+    if (g_join) { (void)hipEventDestroy(g_join); g_join = nullptr; }
+    if (g_side) { (void)hipStreamDestroy(g_side); g_side = nullptr; }
+    if (g_state) { pool_free_raw(g_state); g_state = nullptr; }
 }
 
 }  // namespace bship
@@ -268,6 +463,7 @@ int bship_rng_seed(uint32_t seed) {
     BSHIP_REQUIRE_INIT();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     int st = rng_ensure_state();
+    if (st == 0) st = prefetch_flush(false);
     if (st != 0) return st;
     // init_genrand of the MT19937 reference code, as used by RandomState(int)
     RngState h;
@@ -285,7 +481,8 @@ int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, 
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_rng_get_state: bship_rng_seed() has not been called");
     RngState h;
-    int st = bship_d2h(&h, g_state, sizeof(RngState));
+    int st = prefetch_flush(true);
+    if (st == 0) st = bship_d2h(&h, g_state, sizeof(RngState));
     if (st != 0) return st;
     if (key_host) for (int i = 0; i < kMtN; ++i) key_host[i] = h.key[i];
     if (pos_host) *pos_host = h.pos;
@@ -301,8 +498,45 @@ int bship_prob_mask_f32(float* mask, size_t n, double p) {
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_prob_mask_f32: bship_rng_seed() has not been called");
-    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, ctx().stream, g_state, mask, n, p);
-    return check_launch("generate_probability_mask");
+    MaskPrefetch hit;
+    bool is_hit = false;
+    int st = mask_begin(mask, n, p, &hit, &is_hit);
+    if (st != 0 || !is_hit) return st;
+    st = bship_d2d(mask, hit.staging, n * sizeof(float));
+    if (st != 0) { free_entry(hit); return st; }
+    return mask_end(hit);
+}
+
+int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, double keep_probability,
+                          float scale) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_PTR(in);
+    BSHIP_REQUIRE_PTR(mask);
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(in);
+    BSHIP_REQUIRE_F32_ALIGNED(mask);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    const size_t tiles = (n + static_cast<size_t>(kBlock) * 4 - 1) / (static_cast<size_t>(kBlock) * 4);
+    if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", __func__, n);
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_dropout_fwd_f32: bship_rng_seed() has not been called");
+    MaskPrefetch hit;
+    bool is_hit = false;
+    int st = mask_begin(mask, n, keep_probability, &hit, &is_hit);
+    if (st != 0) return st;
+    const float* src = is_hit ? hit.staging : mask;
+    const dim3 grid(static_cast<unsigned>(tiles)), blk(kBlock);
+    if (aligned16(src) && aligned16(mask) && aligned16(in) && aligned16(out))
+        hipLaunchKernelGGL(dropout_apply_kernel<true>, grid, blk, 0, ctx().stream, src, mask, in, out, scale, n);
+    else
+        hipLaunchKernelGGL(dropout_apply_kernel<false>, grid, blk, 0, ctx().stream, src, mask, in, out, scale, n);
+    st = check_launch("dropout_forward");
+    if (is_hit) {
+        if (st != 0) { free_entry(hit); return st; }
+        st = mask_end(hit);
+    }
+    return st;
 }
 
 int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
@@ -313,9 +547,11 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_fill_gaussian_f32: bship_rng_seed() has not been called");
     hipStream_t s = ctx().stream;
+    int st = prefetch_flush(true);
+    if (st != 0) return st;
     // device scalars: [0] trials consumed, [1] outputs written, [2] outputs taken from the cache
     void* rp = nullptr;
-    int st = pool_alloc_raw(3 * sizeof(unsigned long long), &rp);
+    st = pool_alloc_raw(3 * sizeof(unsigned long long), &rp);
     if (st != 0) return st;
     unsigned long long* result = static_cast<unsigned long long*>(rp);
     void* snap_p = nullptr;

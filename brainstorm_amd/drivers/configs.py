@@ -48,18 +48,18 @@ def _finish(net, data, flat):
     return net, data
 
 
-def build_mlp(handler, seed=1, batch=100, in_size=784, hidden=1200, classes=10):
+def build_mlp(handler, seed=1, batch=100, in_size=784, hidden=1200, classes=10, fused=False):
     rng = np.random.RandomState(seed)
     data = {"default": rng.uniform(0, 1, (1, batch, in_size)).astype(F32),
             "targets": rng.randint(0, classes, (1, batch, 1)).astype(F32)}
     net = Net(handler, [
         ("Input", Input({"default": (in_size,), "targets": (1,)}), {}),
-        ("drop1", Dropout(0.2), {"default": "Input.default"}),
-        ("fc1", FullyConnected(hidden, "rel"), {"default": "drop1.default"}),
-        ("drop2", Dropout(0.5), {"default": "fc1.default"}),
-        ("fc2", FullyConnected(hidden, "rel"), {"default": "drop2.default"}),
-        ("drop3", Dropout(0.5), {"default": "fc2.default"}),
-        ("out", FullyConnected(classes, "linear"), {"default": "drop3.default"}),
+        ("drop1", Dropout(0.2, fused=fused), {"default": "Input.default"}),
+        ("fc1", FullyConnected(hidden, "rel", fused=fused), {"default": "drop1.default"}),
+        ("drop2", Dropout(0.5, fused=fused), {"default": "fc1.default"}),
+        ("fc2", FullyConnected(hidden, "rel", fused=fused), {"default": "drop2.default"}),
+        ("drop3", Dropout(0.5, fused=fused), {"default": "fc2.default"}),
+        ("out", FullyConnected(classes, "linear", fused=fused), {"default": "drop3.default"}),
         ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),
     ])

@@ -138,8 +138,9 @@ class FullyConnected(Layer):
 class Dropout(Layer):
     """layers/dropout_layer.py:36-52"""
 
-    def __init__(self, drop_prob=0.5):
+    def __init__(self, drop_prob=0.5, fused=False):
         self.drop_prob = drop_prob
+        self.fused = bool(fused)        # mask, product and scaling through handler.dropout_forward
 
     def setup(self, in_shapes):
         shape = in_shapes["default"].feature_shape
@@ -147,7 +148,10 @@ class Dropout(Layer):
 
     def forward_pass(self, buffers, training_pass=True):
         _h = self.handler
-        if training_pass:
+        if training_pass and self.fused and hasattr(_h, "dropout_forward"):
+            _h.dropout_forward(buffers.inputs["default"], 1 - self.drop_prob, 1 / (1 - self.drop_prob),
+                               buffers.internals["mask"], buffers.outputs["default"])
+        elif training_pass:
             _h.generate_probability_mask(buffers.internals["mask"], 1 - self.drop_prob)
             _h.mult_tt(buffers.inputs["default"], buffers.internals["mask"], out=buffers.outputs["default"])
             _h.mult_st(1 / (1 - self.drop_prob), buffers.outputs["default"], out=buffers.outputs["default"])

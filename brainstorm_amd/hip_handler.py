@@ -525,3 +525,11 @@ class HipHandler(Handler):
             raise ValueError("batchnorm_backward: inconsistent shapes")
         self._call(self._lib.bship_batchnorm_bwd_f32(out_deltas.ptr, x_hat.ptr, gamma.ptr, sigma_b.ptr,
                                                      dgamma.ptr, dbeta.ptr, in_deltas.ptr, rows, n))
+
+    def dropout_forward(self, inputs, keep_probability, scale, mask, out):
+        """generate_probability_mask(mask, keep_probability); out = inputs * mask;
+        out = scale * out (dropout_layer.py:41-45) with one pass behind the mask."""
+        if not (inputs.shape == mask.shape == out.shape):
+            raise ValueError("dropout_forward: inconsistent shapes")
+        self._call(self._lib.bship_dropout_fwd_f32(inputs.ptr, mask.ptr, out.ptr, out.size,
+                                                   float(keep_probability), float(scale)))

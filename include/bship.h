@@ -336,6 +336,12 @@ int bship_highway_bwd_f32(const float* H, const float* T, const float* x,
  * out (M,N), bias N elements, act one of BSHIP_ACT_*. out may be in. */
 int bship_bias_act_f32(int act, const float* in, const float* bias, float* out,
                        int64_t M, int64_t N);
+/* DropoutLayerImpl.forward_pass, training branch (dropout_layer.py 41-45) in
+ * one pass behind the mask: generate_probability_mask(mask, keep_probability);
+ * out = in * mask; out = scale * out. The mask comes from the same stream, at
+ * the same position, as bship_prob_mask_f32 would draw it. */
+int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n,
+                          double keep_probability, float scale);
 /* BatchNormLayerImpl.forward_pass (batch_normalization_layer.py 54-105) on
  * (M,N) matrices and N-element vectors. training != 0: batch statistics (the
  * negative batch mean and then the deviation go through sigma_b as in the

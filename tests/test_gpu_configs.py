@@ -199,3 +199,23 @@ def test_cnn_forward_backward(hip):
         worst = max(worst, err)
         assert err <= 5e-5, (name, err)
     print("cnn: worst gradient block %.2e" % worst)
+
+
+def test_device_resident_inputs(hip):
+    # provide_external_data takes arrays of the handler's own type (network.py:399-400): the one-hot
+    # input of the LSTM workload is built on the device from the 40 kB of symbol ids with binarize_v
+    # instead of uploading the 8 MB one-hot tensor every batch (data_iterators.py:222-231 does it on the host)
+    kw = dict(time_steps=100, batch=100, symbols=205, hidden=16)
+    net_a, data = configs.build_lstm(hip, **kw)
+    net_b, _ = configs.build_lstm(hip, **kw)
+    net_a.provide_external_data(data)
+    t, b, s = data["default"].shape
+    ids = hip.create_from_numpy(data["targets"].reshape(t * b, 1))
+    onehot = hip.allocate((t * b, s))
+    hip.binarize_v(ids, onehot)
+    net_b.provide_external_data({"default": onehot.reshape((t, b, s)), "targets": ids.reshape((t, b, 1))})
+    for key in ("default", "targets"):
+        assert_bit_equal(net_b.get("Input", "outputs", key), net_a.get("Input", "outputs", key), key)
+    net_a.forward_pass(training_pass=True)
+    net_b.forward_pass(training_pass=True)
+    assert_bit_equal(net_b.get("loss", "outputs", "loss"), net_a.get("loss", "outputs", "loss"), "loss")

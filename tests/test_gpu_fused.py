@@ -284,3 +284,43 @@ def test_fused_layer_argument_errors(hip):
     assert lib.bship_batchnorm_bwd_f32(a.ptr, a.ptr, v.ptr, v.ptr, v.ptr, v.ptr, a.ptr, 0, 8) == -3
     assert lib.bship_batchnorm_fwd_f32(1, a.ptr, v.ptr, v.ptr, v.ptr, v.ptr, 0.9, 1e-5, v.ptr, a.ptr,
                                        a.ptr, a.ptr, 4, 0) == 0
+
+
+def test_fused_mlp_training_is_bit_identical(hip):
+    # dropout (with masks served from the look-ahead queue once the pattern repeats) and
+    # bias+activation through the fused entry points: same masks, same parameters after 12 steps
+    from brainstorm_amd.drivers.net import MomentumStepper
+    results = []
+    for fused in (False, True):
+        hip.rnd.seed(31)
+        net, data = configs.build_mlp(hip, fused=fused, batch=37, in_size=50, hidden=129)
+        net.provide_external_data(data)
+        stepper = MomentumStepper(0.1, 0.9)
+        stepper.start(net)
+        for _ in range(12):
+            stepper.run()
+        results.append((hip.get_numpy_copy(net.parameters),
+                        [net.get(k, "internals", "mask") for k in ("drop1", "drop2", "drop3")],
+                        net.get("loss", "outputs", "loss"), hip.rnd.get_state()))
+    (p0, m0, l0, s0), (p1, m1, l1, s1) = results
+    assert_bit_equal(p1, p0, "parameters")
+    for a, b in zip(m1, m0):
+        assert_bit_equal(a, b, "mask")
+    assert_bit_equal(l1, l0, "loss")
+    assert s0[2] == s1[2] and np.array_equal(s0[1], s1[1])
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_dropout_forward_matches_single_operations(hip, n):
+    rng = np.random.RandomState(n)
+    x = hip.create_from_numpy(rng.standard_normal((n + 1,)).astype(F32))[1:]    # odd start address
+    for keep in (0.8, 0.5):
+        hip.rnd.seed(n)
+        rs = np.random.RandomState(n)
+        for rep in range(5):                       # repeats: later rounds come from the queue
+            mask, out = hip.allocate((n,)), hip.allocate((n,))
+            hip.dropout_forward(x, keep, 1 / keep, mask, out)
+            want_mask = (rs.uniform(size=(n,)) < keep).astype(F32)
+            assert_bit_equal(mask.get(), want_mask, "mask n=%d rep %d" % (n, rep))
+            want = (x.get() * want_mask) * F32(1 / keep)
+            assert_bit_equal(out.get(), want.astype(F32), "out n=%d rep %d" % (n, rep))

@@ -445,6 +445,50 @@ def test_generate_probability_mask_matches_randomstate(hip):
         np.testing.assert_array_equal(key, st[1])
 
 
+def test_mask_prefetch_never_changes_the_stream(hip):
+    # Repeating request patterns switch on the look-ahead generation on the second stream; whether a
+    # request is served from it, misses it, or another consumer of the generator cuts in, the masks
+    # and the generator state must be those of one sequential RandomState.
+    lib = hip._lib
+    hip.rnd.seed(11)
+    rs = np.random.RandomState(11)
+
+    def draw(shape, p, tag):
+        mask = hip.allocate(shape)
+        hip.generate_probability_mask(mask, p)
+        want = (rs.uniform(size=shape) < p).astype(F32)
+        assert_bit_equal(mask.get(), want, tag)
+
+    def check_state(tag):
+        _, key, pos, has_gauss, _ = hip.rnd.get_state()
+        st = rs.get_state()
+        assert (pos, has_gauss) == (st[2], st[3]), tag
+        np.testing.assert_array_equal(key, st[1], err_msg=tag)
+
+    pattern = [((100, 784), 0.8), ((100, 1200), 0.5), ((100, 1200), 0.5)]
+    for step in range(7):                      # period 3: served ahead of time from the third step on
+        for k, (shape, p) in enumerate(pattern):
+            draw(shape, p, "step %d mask %d" % (step, k))
+    draw((100, 1200), 0.5, "request out of turn")           # the queue expects (100, 784): rewind
+    check_state("after a miss")
+    for step in range(5):                      # period 1
+        draw((313,), 0.3, "period one, %d" % step)
+    check_state("reading the state while masks are queued")
+    for step in range(4):
+        draw((313,), 0.3, "period one again, %d" % step)
+    out = hip.allocate((1001,))                # the gaussian stream cuts in while masks are queued
+    hip.fill_gaussian(0.0, 1.0, out)
+    assert_max_ulp(out.get(), rs.standard_normal((1001,)).astype(F32), 1, "gaussian after prefetch")
+    for step in range(4):
+        draw((313,), 0.3, "after the gaussian, %d" % step)
+        draw((5, 7), 0.9, "after the gaussian, second mask %d" % step)
+    hip.rnd.seed(12)                           # reseeding with masks queued
+    rs = np.random.RandomState(12)
+    for step in range(4):
+        draw((64, 64), 0.5, "reseeded, %d" % step)
+    check_state("end")
+
+
 def test_fill_gaussian_matches_randomstate(hip):
     for seed in (0, 7):
         hip.rnd.seed(seed)
