@@ -5,27 +5,28 @@
 
 namespace bship {
 
-// out[i, j] = (j == (int)v[i]); a wavefront writes one row, 4 rows per workgroup.
-template <int W, bool AL>
+// out[i, j] = (j == (int)v[i]). Write-only: one workgroup per tile of kBlock*W
+// columns of one row, one store per lane (the shape of the fill kernel).
+// WT selects write-through stores (large outputs). KW = K / W.
+template <int W, bool AL, bool WT>
 __global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restrict__ v,
-                                                          float* __restrict__ out, int64_t M,
-                                                          int64_t K) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + threadIdx.x / kWave;
-    if (row >= M) return;
+                                                          float* __restrict__ out, int64_t KW,
+                                                          unsigned tiles_per_row) {
+    const int64_t row = blockIdx.x / tiles_per_row;
+    const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
+    if (c >= KW) return;
     const int64_t hot = static_cast<int64_t>(static_cast<int>(v[row]));
-    float* q = out + row * K;
-    const int64_t KW = K / W;
-    for (int64_t i = lane; i < KW; i += kWave) {
-        if constexpr (W == 4) {
-            const int64_t j = i * 4;
-            f4 r = {j == hot ? 1.0f : 0.0f, j + 1 == hot ? 1.0f : 0.0f,
-                    j + 2 == hot ? 1.0f : 0.0f, j + 3 == hot ? 1.0f : 0.0f};
-            vstore<4, AL>(q + j, r);
-        } else {
-            q[i] = (i == hot) ? 1.0f : 0.0f;
-        }
+    float* q = out + (row * KW + c) * W;
+    typename VecT<W>::type r;
+    if constexpr (W == 4) {
+        const int64_t j = c * 4;
+        r = f4{j == hot ? 1.0f : 0.0f, j + 1 == hot ? 1.0f : 0.0f, j + 2 == hot ? 1.0f : 0.0f,
+               j + 3 == hot ? 1.0f : 0.0f};
+    } else {
+        r = (c == hot) ? 1.0f : 0.0f;
     }
+    if constexpr (WT) vstore_writeonly<W>(q, r);
+    else vstore<W, AL>(q, r);
 }
 
 // out[i] = m[i, (int)v[i]]; labels outside [0,K) read as 0.
@@ -53,14 +54,19 @@ int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K) {
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(v);
     BSHIP_REQUIRE_F32_ALIGNED(out);
-    BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
-    dim3 grid(static_cast<unsigned>(ceil_div(M, kBlock / kWave)));
-    if (K % 4 == 0 && aligned16(out))
-        hipLaunchKernelGGL((binarize_kernel<4, true>), grid, dim3(kBlock), 0, ctx().stream, v, out, M, K);
-    else if (K % 4 == 0)
-        hipLaunchKernelGGL((binarize_kernel<4, false>), grid, dim3(kBlock), 0, ctx().stream, v, out, M, K);
-    else
-        hipLaunchKernelGGL((binarize_kernel<1, false>), grid, dim3(kBlock), 0, ctx().stream, v, out, M, K);
+    const bool vec = (K % 4 == 0);
+    const int64_t KW = vec ? K / 4 : K;
+    const int64_t tiles_per_row = ceil_div(KW, kBlock);
+    BSHIP_REQUIRE_DIM(tiles_per_row * M <= 0x7fffffff);
+    const dim3 grid(static_cast<unsigned>(tiles_per_row * M)), blk(kBlock);
+    const unsigned tpr = static_cast<unsigned>(tiles_per_row);
+    const bool wt = static_cast<size_t>(M) * static_cast<size_t>(K) >= kWriteThroughMin;
+    hipStream_t s = ctx().stream;
+    if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, out, KW, tpr);
+    else if (vec && aligned16(out))  hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, out, KW, tpr);
+    else if (vec)                    hipLaunchKernelGGL((binarize_kernel<4, false, false>), grid, blk, 0, s, v, out, KW, tpr);
+    else if (wt)                     hipLaunchKernelGGL((binarize_kernel<1, false, true>), grid, blk, 0, s, v, out, KW, tpr);
+    else                             hipLaunchKernelGGL((binarize_kernel<1, false, false>), grid, blk, 0, s, v, out, KW, tpr);
     return check_launch("binarize_v");
 }
 

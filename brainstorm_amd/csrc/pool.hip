@@ -108,12 +108,14 @@ void pool_release_all() {
 // One workgroup per tile of kBlock*4 floats, one 128-bit access per lane.
 constexpr size_t kCopyTile = static_cast<size_t>(kBlock) * 4;
 
-template <bool AL>
+// WT: write-through stores (large arrays); otherwise AL selects the aligned non-temporal store.
+template <bool AL, bool WT>
 __global__ __launch_bounds__(kBlock) void fill_kernel(float* __restrict__ p, float val, size_t n) {
     const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
     if (i + 4 <= n) {
         const f4 vv = {val, val, val, val};
-        vstore<4, AL>(p + i, vv);
+        if constexpr (WT) vstore_writeonly<4>(p + i, vv);
+        else vstore<4, AL>(p + i, vv);
     } else {
         for (size_t j = i; j < n; ++j) p[j] = val;
     }
@@ -135,10 +137,12 @@ int launch_fill(float* p, float val, size_t n) {
     const size_t tiles = (n + kCopyTile - 1) / kCopyTile;
     if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "fill: %zu elements exceed one launch", n);
     const dim3 grid(static_cast<unsigned>(tiles));
-    if (aligned16(p))
-        hipLaunchKernelGGL(fill_kernel<true>, grid, dim3(kBlock), 0, ctx().stream, p, val, n);
+    if (n >= kWriteThroughMin)
+        hipLaunchKernelGGL((fill_kernel<false, true>), grid, dim3(kBlock), 0, ctx().stream, p, val, n);
+    else if (aligned16(p))
+        hipLaunchKernelGGL((fill_kernel<true, false>), grid, dim3(kBlock), 0, ctx().stream, p, val, n);
     else
-        hipLaunchKernelGGL(fill_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, p, val, n);
+        hipLaunchKernelGGL((fill_kernel<false, false>), grid, dim3(kBlock), 0, ctx().stream, p, val, n);
     return check_launch("fill_kernel");
 }
 

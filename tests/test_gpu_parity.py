@@ -182,6 +182,18 @@ def test_fill_copy_allocate(hip, ref):
             assert_bit_equal(hip.get_numpy_copy(got), want, maker)
 
 
+def test_large_fill_uses_every_element(hip):
+    # arrays of 2^22 elements and more take the write-through store path
+    for n in ((1 << 22), (1 << 22) + 4099, 5000001):
+        base = hip.allocate((n + 2,))
+        hip.fill(base[1:n + 1], 2.5)                   # odd start address, untouched guards
+        got = base.get()
+        assert got[0] == 0.0 and got[-1] == 0.0
+        assert np.array_equal(got[1:n + 1], np.full(n, 2.5, F32))
+        big = hip.allocate((n,))                       # zero fill of the allocation itself
+        assert not big.get().any()
+
+
 def test_allocate_reuses_blocks_zeroed(hip):
     # a pool block that comes back must be handed out zero-filled again
     for _ in range(3):
@@ -411,7 +423,8 @@ def test_is_fully_finite(hip, ref):
 # -------------------------------------------------------------------- indexing
 def test_binarize_v_exact(hip, ref):
     rng = np.random.RandomState(21)
-    for rows, k in [(1, 1), (5, 3), (100, 10), (10000, 205), (64, 64), (300, 1031), (512, 4096)]:
+    for rows, k in [(1, 1), (5, 3), (100, 10), (10000, 205), (64, 64), (300, 1031), (512, 4096),
+                    (2048, 2048), (4100, 1031), (1025, 4100)]:      # the last three: 2^22 elements and more
         v = rng.randint(0, k, (rows, 1)).astype(F32)
         operation_check(hip, ref, "binarize_v", (v, np.full((rows, k), 7.0, F32)))
 
