@@ -27,7 +27,7 @@ template <bool ACC> struct MvSub { __device__ float apply(float m, float v, floa
 template <bool ACC> struct MvMul { __device__ float apply(float m, float v, float o) const { float r = m * v; return ACC ? o + r : r; } };
 template <bool ACC> struct MvDiv { __device__ float apply(float m, float v, float o) const { float r = m / v; return ACC ? o + r : r; } };
 
-// Row vector: a workgroup handles R consecutive rows of one tile of kBlock*W
+// Row vector: a workgroup handles R (= kMvRows) consecutive rows of one tile of kBlock*W
 // columns; each lane loads its slice of v once and applies it to R rows.
 // One workgroup per tile (see elementwise.hip for why). NW = N / W.
 template <int W, bool AL, bool ACC, int R, typename F>
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(kBlock) void mv_colvec_kernel(F f, const float* m, 
     vstore<W, AL>(out + e, vmap(f, a, splat(a, s), o));
 }
 
-constexpr int kMvRows = 4;
+// rows per workgroup; measured at 8192^2 / 16384^2: add_mv 0.79/0.76 of peak with 1 row,
+// 0.81/0.80 with 2, 0.75/0.79 with 4, 0.71/0.71 with 8
+constexpr int kMvRows = 2;
 
 template <bool ACC, typename F>
 int launch_mv(const char* name, F f, const float* m, const float* v, float* out, int64_t M,

@@ -24,6 +24,7 @@ struct Context {
     hipEvent_t events[BSHIP_MAX_EVENTS] = {nullptr};   // created on first use
     bool debug_sync = false;   // BSHIP_DEBUG_SYNC=1: sync + check after every launch
     int blocks_per_cu = 8;     // streaming kernels launch num_cus*blocks_per_cu blocks
+    int colsum_blocks_per_cu = 3;   // column sums: row bands are chosen to reach this many workgroups per CU (measured optimum)
     char name[256] = {0};
 };
 

@@ -73,6 +73,8 @@ int bship_init(int device) {
     g_ctx.debug_sync = dbg && dbg[0] && dbg[0] != '0';
     const char* bpc = getenv("BSHIP_BLOCKS_PER_CU");
     if (bpc && atoi(bpc) > 0 && atoi(bpc) <= 64) g_ctx.blocks_per_cu = atoi(bpc);
+    const char* cpc = getenv("BSHIP_COLSUM_BLOCKS_PER_CU");
+    if (cpc && atoi(cpc) > 0 && atoi(cpc) <= 64) g_ctx.colsum_blocks_per_cu = atoi(cpc);
     g_ctx.device = device;
     g_ctx.inited = true;
     return 0;

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
 // at this column, in = the matrix operands at this element, out = the results.
 // A body provides the pointer tables vecs[kVecs], ins[kIn], outs[kOut]; an output
 // may be the same array as an input (every lane loads all operands first).
-constexpr int kFusedRows = 4;
+constexpr int kFusedRows = 2;   // as kMvRows of the matrix-vector kernels
 
 template <int W, bool AL, typename Body>
 __global__ __launch_bounds__(kBlock) void rowvec_fused_kernel(Body b, int64_t M, int64_t NW,

@@ -156,58 +156,86 @@ static int launch_sumall(const float* a, float* out, int64_t n) {
 }
 
 // ================================ softmax ==================================
+// exp(x) for x <= 0 (softmax exponents are differences to the row maximum):
+// x*log2(e) split into an integer k and a remainder |r| <= 1/2 with the low part
+// of log2(e) carried along, 2^r from the hardware exp2 (1 ulp), scaled by 2^k.
+// About 2 ulp, a quarter of the instructions of the full-range expf; the softmax
+// bar is 1e-5 relative.
+__device__ __forceinline__ float exp_nonpositive(float x) {
+    const float kLog2eHi = 1.44269502162933349609375f;      // float32(log2 e)
+    const float kLog2eLo = 1.925963033500011e-8f;           // log2 e - float32(log2 e)
+    const float k = rintf(x * kLog2eHi);
+    float r = fmaf(x, kLog2eHi, -k);
+    r = fmaf(x, kLog2eLo, r);
+    const float e = ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(k));
+    return x < -104.0f ? 0.0f : e;                          // below 2^-150 (and -inf): zero
+}
+
 // One pass over HBM: THREADS lanes hold a whole row in registers (PER accesses
 // of W floats each), reduce max and sum across the lanes, then write e/sum.
+// THREADS is a wavefront (BLOCK/64 rows per workgroup) or the whole workgroup.
+// Long rows take workgroups of 1024 lanes: measured on MI355X at 16384 columns,
+// 4 vectors per lane x 1024 lanes reach 0.74 of peak where 16 x 256 reach 0.66.
 // out = exp(m - rowmax) / sum(exp(m - rowmax))      (numpy 292-295)
 // The launcher guarantees N % W == 0 and N / W <= THREADS * PER.
-template <int W, bool AL, int THREADS, int PER>
-__global__ __launch_bounds__(kBlock) void softmax_reg_kernel(const float* m, float* out, int64_t M,
-                                                             int64_t N) {
-    constexpr int ROWS = kBlock / THREADS;
+template <int W, bool AL, int BLOCK, int THREADS, int PER>
+__global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, float* out, int64_t M,
+                                                            int64_t N) {
+    constexpr int ROWS = BLOCK / THREADS;
+    constexpr int WAVES = BLOCK / kWave;
     typedef typename VecT<W>::type R;
-    __shared__ float lds[2][kBlock / kWave];
+    __shared__ float lds[2][WAVES];
     const int t = threadIdx.x % THREADS;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / THREADS;
     const bool live = row < M;
     const int64_t NW = N / W;
     const float* p = m + (live ? row : 0) * N;
     float* q = out + (live ? row : 0) * N;
+    // All loads are issued before anything depends on one of them: lanes beyond the row's
+    // end read element 0 instead (always valid) and are replaced by -inf afterwards, so
+    // the loads sit in no branch and the wavefront keeps PER of them in flight.
     R x[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int64_t i = t + static_cast<int64_t>(k) * THREADS;
+        x[k] = vload<W, AL>(p + ((live && i < NW) ? i : 0) * W);
+    }
     float mx = -INFINITY;
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int64_t i = t + static_cast<int64_t>(k) * THREADS;
-        if (live && i < NW) {
-            x[k] = vload<W, AL>(p + i * W);
-            mx = fmaxf(mx, hmax(x[k]));
-        }
+        if (!(live && i < NW)) x[k] = vzero<R>() - INFINITY;
+        mx = fmaxf(mx, hmax(x[k]));
     }
     mx = wave_max(mx);
     if (THREADS > kWave) {
         if ((threadIdx.x & (kWave - 1)) == 0) lds[0][threadIdx.x / kWave] = mx;
         __syncthreads();
-        mx = fmaxf(fmaxf(lds[0][0], lds[0][1]), fmaxf(lds[0][2], lds[0][3]));
+        mx = lds[0][0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) mx = fmaxf(mx, lds[0][w]);
     }
     float sum = 0.0f;
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int64_t i = t + static_cast<int64_t>(k) * THREADS;
-        if (live && i < NW) {
-            if constexpr (W == 4) {
+        if constexpr (W == 4) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) x[k][j] = expf(x[k][j] - mx);
-            } else {
-                x[k] = expf(x[k] - mx);
-            }
-            sum += hsum(x[k]);
+            for (int j = 0; j < 4; ++j) x[k][j] = exp_nonpositive(x[k][j] - mx);
+        } else {
+            x[k] = exp_nonpositive(x[k] - mx);
         }
+        if (live && i < NW) sum += hsum(x[k]);       // padding lanes hold exp(-inf - mx), not counted
     }
     sum = wave_sum(sum);
     if (THREADS > kWave) {
         if ((threadIdx.x & (kWave - 1)) == 0) lds[1][threadIdx.x / kWave] = sum;
         __syncthreads();
-        sum = (lds[1][0] + lds[1][1]) + (lds[1][2] + lds[1][3]);
+        sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w += 4) sum += (lds[1][w] + lds[1][w + 1]) + (lds[1][w + 2] + lds[1][w + 3]);
     }
+    const float inv = 1.0f / sum;        // one division per lane; e * inv is within 1 ulp of e / sum
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
         const int64_t i = t + static_cast<int64_t>(k) * THREADS;
@@ -215,9 +243,9 @@ __global__ __launch_bounds__(kBlock) void softmax_reg_kernel(const float* m, flo
             R r;
             if constexpr (W == 4) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) r[j] = x[k][j] / sum;
+                for (int j = 0; j < 4; ++j) r[j] = x[k][j] * inv;
             } else {
-                r = x[k] / sum;
+                r = x[k] * inv;
             }
             vstore<W, AL>(q + i * W, r);
         }
@@ -249,26 +277,28 @@ __global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, fl
     for (int64_t i = threadIdx.x; i < N; i += kBlock) q[i] = expf(p[i] - mx) / sum;
 }
 
-template <int W, bool AL, int THREADS>
+template <int W, bool AL, int BLOCK, int THREADS>
 static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N) {
     hipStream_t s = ctx().stream;
-    const dim3 b(kBlock);
+    const dim3 b(BLOCK);
     switch (per) {
-        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 1>), grid, b, 0, s, m, out, M, N); break;
-        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 2>), grid, b, 0, s, m, out, M, N); break;
-        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 4>), grid, b, 0, s, m, out, M, N); break;
-        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 8>), grid, b, 0, s, m, out, M, N); break;
-        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, THREADS, 16>), grid, b, 0, s, m, out, M, N); break;
+        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N); break;
+        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N); break;
+        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N); break;
+        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N); break;
+        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N); break;
     }
 }
 
-template <int THREADS>
+template <int BLOCK, int THREADS>
 static void launch_softmax_threads(bool vec, bool al, int per, dim3 grid, const float* m, float* out,
                                    int64_t M, int64_t N) {
-    if (vec && al) launch_softmax_per<4, true, THREADS>(per, grid, m, out, M, N);
-    else if (vec)  launch_softmax_per<4, false, THREADS>(per, grid, m, out, M, N);
-    else           launch_softmax_per<1, false, THREADS>(per, grid, m, out, M, N);
+    if (vec && al) launch_softmax_per<4, true, BLOCK, THREADS>(per, grid, m, out, M, N);
+    else if (vec)  launch_softmax_per<4, false, BLOCK, THREADS>(per, grid, m, out, M, N);
+    else           launch_softmax_per<1, false, BLOCK, THREADS>(per, grid, m, out, M, N);
 }
+
+constexpr int kWideBlock = 1024;
 
 static int launch_softmax(const float* m, float* out, int64_t M, int64_t N) {
     const bool vec = (N % 4 == 0);
@@ -281,10 +311,14 @@ static int launch_softmax(const float* m, float* out, int64_t M, int64_t N) {
         return per;
     };
     if (NW <= static_cast<int64_t>(kWave) * 16) {
-        launch_softmax_threads<kWave>(vec, al, per_for(kWave),
-                                      dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N);
-    } else if (NW <= static_cast<int64_t>(kBlock) * 16) {
-        launch_softmax_threads<kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N);
+        // a wavefront per row, 4 rows per workgroup
+        launch_softmax_threads<kBlock, kWave>(vec, al, per_for(kWave),
+                                              dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N);
+    } else if (NW <= static_cast<int64_t>(kBlock) * 4) {
+        launch_softmax_threads<kBlock, kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N);
+    } else if (NW <= static_cast<int64_t>(kWideBlock) * 16) {
+        launch_softmax_threads<kWideBlock, kWideBlock>(vec, al, per_for(kWideBlock),
+                                                       dim3(static_cast<unsigned>(M)), m, out, M, N);
     } else {
         hipLaunchKernelGGL(softmax_long_kernel, dim3(static_cast<unsigned>(M)), dim3(kBlock), 0,
                            ctx().stream, m, out, M, N);
