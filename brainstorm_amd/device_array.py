@@ -78,6 +78,53 @@ class DeviceArray:
         """NumPy copy of the contents (blocks until the device has caught up)."""
         return self._handler.get_numpy_copy(self)
 
+    # ------------------------------------------------------------ arithmetic
+    # brainstorm's ConstrainL2Norm writes `mat * mat` and `sq_norm ** 0.5` on handler arrays
+    # (value_modifiers.py:79-80). As with NumPy arrays each expression yields a NEW array;
+    # NumPy evaluates `x ** 0.5` as sqrt and `x ** 2` as x * x, so do these.
+    def _binary(self, other, tt, st):
+        h = self._handler
+        out = h.allocate(self.shape)
+        if isinstance(other, DeviceArray):
+            if other.shape != self.shape:
+                raise ValueError("operands have shapes %r and %r; broadcasting is not supported"
+                                 % (self.shape, other.shape))
+            getattr(h, tt)(self, other, out)
+        elif st is not None and isinstance(other, (int, float, np.integer, np.floating)):
+            getattr(h, st)(other, self, out)
+        else:
+            return NotImplemented
+        return out
+
+    def __mul__(self, other):
+        return self._binary(other, "mult_tt", "mult_st")
+
+    __rmul__ = __mul__
+
+    def __add__(self, other):
+        return self._binary(other, "add_tt", "add_st")
+
+    __radd__ = __add__
+
+    def __sub__(self, other):
+        return self._binary(other, "subtract_tt", None)
+
+    def __truediv__(self, other):
+        return self._binary(other, "divide_tt", None)
+
+    def __pow__(self, exponent):
+        h = self._handler
+        out = h.allocate(self.shape)
+        if exponent == 0.5:
+            h.sqrt_t(self, out)
+        elif exponent == 2:
+            h.mult_tt(self, self, out)
+        elif exponent == 1:
+            h.copy_to(self, out)
+        else:
+            raise NotImplementedError("DeviceArray ** %r: only the exponents 0.5, 1 and 2 are supported" % (exponent,))
+        return out
+
     # --------------------------------------------------------------- reshape
     def reshape(self, *new_shape):
         if len(new_shape) == 1 and not isinstance(new_shape[0], (int, np.integer)):

@@ -159,6 +159,23 @@ class Net:
             self.handler.fill(buf, 0.)
         for name, layer in reversed(list(self.layers.items())[1:]):
             layer.backward_pass(self.buffers[name])
+        self.apply_gradient_modifiers()                    # network.py:445
+
+    def apply_weight_modifiers(self):
+        """network.py:490-495; ``weight_modifiers`` maps (layer, parameter) to a list of modifiers."""
+        for (layer, view), mods in getattr(self, "weight_modifiers", {}).items():
+            for mod in mods:
+                mod(self.handler, self.buffers[layer].parameters[view])
+
+    def apply_gradient_modifiers(self):
+        """network.py:497-509: GradientModifiers get (parameters, gradients), others the gradients."""
+        from .modifiers import GradientModifier
+        for (layer, view), mods in getattr(self, "gradient_modifiers", {}).items():
+            for mod in mods:
+                if isinstance(mod, GradientModifier):
+                    mod(self.handler, self.buffers[layer].parameters[view], self.buffers[layer].gradients[view])
+                else:
+                    mod(self.handler, self.buffers[layer].gradients[view])
 
     def get(self, layer, group, name):
         return self.handler.get_numpy_copy(getattr(self.buffers[layer], group)[name])
@@ -201,3 +218,4 @@ class MomentumStepper:
         h.mult_st(momentum, self.velocity, out=self.velocity)
         h.mult_add_st(-learning_rate, self.net.gradients, out=self.velocity)
         h.add_tt(self.velocity, self.net.parameters, out=self.net.parameters)
+        self.net.apply_weight_modifiers()                  # the trainer does this after every update (trainer.py:101)

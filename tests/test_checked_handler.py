@@ -1,0 +1,165 @@
+"""CPU: the contract-checking wrapper and the value modifiers, on the float64/float32 oracle.
+
+The wrapper states the shape contracts of brainstorm's DebugHandler (debug_handler.py:61-548);
+running the op-trace drivers under it shows that the drivers only issue calls those contracts allow.
+"""
+import numpy as np
+import pytest
+
+from brainstorm_amd.checked_handler import CONTRACTS, CheckedHandler, ContractError
+from brainstorm_amd.drivers import configs, modifiers
+from brainstorm_amd.drivers.net import MomentumStepper
+from brainstorm_amd.handler_api import HANDLER_METHODS
+from oracle.numpy_ref_handler import NumpyRefHandler
+
+F32 = np.float32
+
+
+@pytest.fixture
+def checked():
+    return CheckedHandler(NumpyRefHandler(F32, seed=3), check_finite=True)
+
+
+def test_covers_the_whole_interface(checked):
+    assert set(HANDLER_METHODS) <= set(CONTRACTS)
+    for name in HANDLER_METHODS:
+        assert callable(getattr(checked, name))
+    assert checked.array_type is np.ndarray and checked.dtype == F32
+
+
+def test_valid_calls_reach_the_wrapped_handler(checked):
+    a = checked.create_from_numpy(np.arange(6, dtype=F32).reshape(2, 3))
+    out = checked.allocate((2, 3))
+    assert checked.add_tt(a, a, out) is None
+    assert np.array_equal(out, 2 * a)
+    checked.add_mv(a, checked.ones((1, 3)), out)
+    checked.mult_mv(a, a, out)                                   # mult_mv also takes a full matrix
+    checked.tanh_deriv(None, a, a, out)                          # x may be None
+    checked.dot_mm(a, a, checked.allocate((3, 3)), transa=True)
+    s = checked.allocate(())
+    checked.sum_t(a, None, s)
+    assert float(s) == 15.0
+    labels = checked.create_from_numpy(np.array([[2], [0]], F32))
+    checked.binarize_v(labels, out)
+    assert np.array_equal(out, [[0, 0, 1], [1, 0, 0]])
+    assert checked.is_fully_finite(out)
+    checked.act_func["sigmoid"](a, out)                          # the look-up tables go through the checks too
+
+
+@pytest.mark.parametrize("call", [
+    lambda h, a, b: h.add_tt(a, b, a),                           # shapes differ
+    lambda h, a, b: h.add_tt(a, [1.0], a),                       # not an array
+    lambda h, a, b: h.add_st(a, a, a),                           # s must be a number
+    lambda h, a, b: h.add_mv(a, h.ones((3, 1)), a),              # neither a row nor a column of a
+    lambda h, a, b: h.add_mv(a.reshape(6), h.ones((1, 3)), a.reshape(6)),     # m must be 2-D
+    lambda h, a, b: h.dot_mm(a, a, h.allocate((2, 2))),          # inner dimensions
+    lambda h, a, b: h.dot_mm(a, a, h.allocate((3, 2)), transa=True),          # out shape
+    lambda h, a, b: h.sum_t(a, 2, h.allocate((2,))),             # axis out of range
+    lambda h, a, b: h.clip_t(a, 1.0, -1.0, a),                   # a_min > a_max
+    lambda h, a, b: h.broadcast_t(a, 0, h.allocate((4, 3))),     # a.shape[axis] != 1
+    lambda h, a, b: h.binarize_v(h.create_from_numpy(np.array([[3], [0]], F32)), a),   # label out of range
+    lambda h, a, b: h.generate_probability_mask(a, 1.5),
+    lambda h, a, b: h.allocate([2, 3]),                          # shape must be a tuple
+    lambda h, a, b: h.maxpool2d_forward_batch(a, (2,), a, 0, (1, 1), a),      # window needs two entries
+    lambda h, a, b: h.set_from_numpy(a, np.zeros((3, 2), F32)),
+    lambda h, a, b: h.sigmoid_deriv(None, a, b, a),
+    lambda h, a, b: h.add_tt(a, a),                              # missing argument
+])
+def test_violations_are_reported(checked, call):
+    a = checked.create_from_numpy(np.ones((2, 3), F32))
+    b = checked.create_from_numpy(np.ones((3, 2), F32))
+    with pytest.raises(ContractError):
+        call(checked, a, b)
+
+
+def test_check_finite_names_the_operation(checked):
+    a = checked.create_from_numpy(np.array([[1.0, -1.0]], F32))
+    out = checked.allocate((1, 2))
+    with np.errstate(all="ignore"), pytest.raises(ValueError, match="log_t"):
+        checked.log_t(a, out)                                    # log(-1) = NaN
+    with pytest.raises(ValueError, match="mult_st"):
+        checked.mult_st(float("inf"), a, out)
+    quiet = CheckedHandler(NumpyRefHandler(F32, seed=3))         # without check_finite nothing is raised
+    with np.errstate(all="ignore"):
+        quiet.log_t(a, out)
+
+
+@pytest.mark.parametrize("builder,kw", [
+    (configs.build_mlp, dict(batch=5, in_size=7, hidden=6)),
+    (configs.build_lstm, dict(time_steps=4, batch=3, symbols=5, hidden=6)),
+    (configs.build_highway, dict(blocks=2, batch=6, width=5)),
+    (configs.build_cnn, dict(batch=2, size=8)),
+])
+def test_drivers_only_issue_calls_the_contracts_allow(builder, kw):
+    handler = CheckedHandler(NumpyRefHandler(np.float64, seed=5), check_finite=True)
+    net, data = builder(handler, **kw)
+    net.provide_external_data(data)
+    stepper = MomentumStepper(0.01, 0.9)
+    stepper.start(net)
+    for _ in range(2):
+        stepper.run()
+    assert np.isfinite(net.get("loss", "outputs", "loss")).all()
+
+
+def test_value_modifiers_closed_forms():
+    h = CheckedHandler(NumpyRefHandler(np.float64, seed=1))
+    rng = np.random.RandomState(0)
+    w = rng.standard_normal((5, 3, 4))
+    view = h.create_from_numpy(w.copy())
+    modifiers.ConstrainL2Norm(1.5)(h, view)
+    norms = np.sqrt((w.reshape(5, -1) ** 2).sum(axis=1))
+    want = w / np.maximum(norms / 1.5, 1.0)[:, None, None]
+    np.testing.assert_allclose(view, want, rtol=1e-12)
+    assert np.sqrt((view.reshape(5, -1) ** 2).sum(axis=1)).max() <= 1.5 * (1 + 1e-12)
+    vec = h.create_from_numpy(w[0, 0].copy())
+    modifiers.ConstrainL2Norm(0.1)(h, vec)                       # fewer than two dimensions: untouched
+    assert np.array_equal(vec, w[0, 0])
+
+    view = h.create_from_numpy(w.copy())
+    modifiers.ClipValues(-0.5, 0.25)(h, view)
+    assert np.array_equal(view, np.clip(w, -0.5, 0.25))
+
+    mask = (rng.uniform(size=w.shape) < 0.5).astype(np.float64)
+    view = h.create_from_numpy(w.copy())
+    mod = modifiers.MaskValues(mask)
+    mod(h, view)
+    mod(h, view)                                                 # the uploaded mask is reused
+    assert np.array_equal(view, w * mask)
+
+    view = h.create_from_numpy(w.copy())
+    freeze = modifiers.FreezeValues()
+    freeze(h, view)                                              # remembers what it saw first
+    view += 1.0
+    freeze(h, view)
+    assert np.array_equal(view, w)
+
+    g = rng.standard_normal(w.shape)
+    grad = h.create_from_numpy(g.copy())
+    modifiers.L1Decay(0.1)(h, h.create_from_numpy(w.copy()), grad)
+    np.testing.assert_array_equal(grad, g + 0.1 * np.sign(w))
+    grad = h.create_from_numpy(g.copy())
+    modifiers.L2Decay(0.1)(h, h.create_from_numpy(w.copy()), grad)
+    np.testing.assert_array_equal(grad, g + 0.1 * w)
+
+
+def test_net_applies_modifiers_where_the_reference_does():
+    h = NumpyRefHandler(np.float64, seed=2)
+    net, data = configs.build_mlp(h, batch=4, in_size=6, hidden=5)
+    net.provide_external_data(data)
+    net.weight_modifiers = {("fc1", "W"): [modifiers.ConstrainL2Norm(0.05)]}
+    net.gradient_modifiers = {("fc2", "W"): [modifiers.L2Decay(0.5)], ("fc1", "bias"): [modifiers.ClipValues(0, 0)]}
+    net.forward_pass(training_pass=True)
+    net.backward_pass()
+    assert not net.get("fc1", "gradients", "bias").any()         # a plain modifier sees the gradients only
+    plain, _ = configs.build_mlp(NumpyRefHandler(np.float64, seed=2), batch=4, in_size=6, hidden=5)
+    plain.provide_external_data(data)
+    plain.forward_pass(training_pass=True)
+    plain.backward_pass()
+    np.testing.assert_allclose(net.get("fc2", "gradients", "W"),
+                               plain.get("fc2", "gradients", "W") + 0.5 * plain.get("fc2", "parameters", "W"),
+                               rtol=1e-12)
+    stepper = MomentumStepper(0.1, 0.0)
+    stepper.start(net)
+    stepper.run()
+    w = net.get("fc1", "parameters", "W")
+    assert np.sqrt((w ** 2).sum(axis=1)).max() <= 0.05 * (1 + 1e-9)
