@@ -1,11 +1,16 @@
 // NHWC image kernels: im2col / col2im for the convolution GEMMs and max /
-// average pooling, forward and backward. One thread per output element with the
-// channel index fastest, so neighbouring lanes touch neighbouring addresses.
+// average pooling, forward and backward.
 //
-// The backward kernels are written in gather form (one thread per input
-// element, visiting the output positions that cover it in row-major order):
-// that is the order in which the reference's serial loops add their terms, so
-// results are deterministic and match the reference bit for bit.
+// Work is split per image (grid.y walks the images) and, inside an image, one
+// lane handles W consecutive channels of one position (W = 4 when the channel
+// count allows, so all accesses are 128-bit and neighbouring lanes touch
+// neighbouring addresses). Positions are decoded from the lane's index with
+// 32-bit multiply-shift divisions prepared on the host.
+//
+// The backward kernels are written in gather form (one lane per input position,
+// visiting the output positions that cover it in row-major order): that is the
+// order in which the reference's serial loops add their terms, so results are
+// deterministic and match the reference bit for bit.
 #pragma clang fp contract(off)
 
 #include <cfloat>
@@ -13,6 +18,12 @@
 #include "common.h"
 
 namespace bship {
+
+// A workgroup decodes its positions once and applies them to this many images.
+#ifndef BSHIP_IMAGES_PER_WG
+#define BSHIP_IMAGES_PER_WG 4
+#endif
+constexpr int kImagesPerWorkgroup = BSHIP_IMAGES_PER_WG;
 
 struct ImgGeom {
     int h, w, c;          // input image
@@ -24,174 +35,292 @@ struct ImgGeom {
 __host__ __device__ inline int imax(int a, int b) { return a > b ? a : b; }
 __host__ __device__ inline int imin(int a, int b) { return a < b ? a : b; }
 
+// n / d for 32-bit unsigned n by multiply and shift (Granlund-Montgomery, rounded-up
+// multiplier): with l = ceil(log2 d) and m = floor(2^32 (2^l - d) / d) + 1,
+// n / d = (mulhi(m, n) + n) >> l for every 32-bit n.
+struct FastDiv {
+    uint32_t d, magic, shift;
+    FastDiv() : d(1), magic(1), shift(0) {}
+    explicit FastDiv(uint32_t dd) : d(dd) {
+        shift = 0;
+        while ((uint64_t(1) << shift) < dd) ++shift;
+        magic = static_cast<uint32_t>(((uint64_t(1) << 32) * ((uint64_t(1) << shift) - dd)) / dd + 1);
+    }
+    __device__ __forceinline__ uint32_t div(uint32_t n) const {
+        return static_cast<uint32_t>((static_cast<uint64_t>(__umulhi(n, magic)) + n) >> shift);
+    }
+    __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
 // Range [lo, hi) of output positions o with  o*stride - pad <= p < o*stride - pad + k.
-__device__ __forceinline__ void cover_range(int p, int pad, int stride, int k, int n_out, int& lo,
-                                            int& hi) {
+__device__ __forceinline__ void cover_range(int p, int pad, const FastDiv& stride, int k, int n_out,
+                                            int& lo, int& hi) {
     const int q = p + pad;                       // o*stride <= q < o*stride + k
-    hi = imin(q / stride + 1, n_out);
+    hi = imin(static_cast<int>(stride.div(static_cast<uint32_t>(q))) + 1, n_out);
     const int t = q - k + 1;                     // o*stride >= t
-    lo = t <= 0 ? 0 : (t + stride - 1) / stride;
+    lo = t <= 0 ? 0 : static_cast<int>(stride.div(static_cast<uint32_t>(t) + stride.d - 1));
 }
 
+// Cached (not streaming) accesses: the images are re-read by overlapping windows.
+template <int W, bool AL>
+__device__ __forceinline__ typename VecT<W>::type img_load(const float* p) {
+    if constexpr (W == 1) return *p;
+    else if constexpr (AL) return *reinterpret_cast<const f4*>(p);
+    else return *reinterpret_cast<const f4u*>(p);
+}
+template <int W, bool AL>
+__device__ __forceinline__ void img_store(float* p, typename VecT<W>::type v) {
+    if constexpr (W == 1) *p = v;
+    else if constexpr (AL) *reinterpret_cast<f4*>(p) = v;
+    else *reinterpret_cast<f4u*>(p) = v;
+}
+template <int W> __device__ __forceinline__ float& comp(typename VecT<W>::type& v, int j) {
+    if constexpr (W == 1) return v;
+    else return reinterpret_cast<float*>(&v)[j];
+}
+template <int W> __device__ __forceinline__ typename VecT<W>::type vsplat(float s) {
+    if constexpr (W == 1) return s;
+    else return f4{s, s, s, s};
+}
+
+// What every kernel gets: the geometry, the number of W-wide lanes of one image and the
+// prepared divisors. cv = c / W channel vectors per position.
+struct ImgPlan {
+    ImgGeom g;
+    uint32_t lanes_per_image;
+    FastDiv d_cv, d_w, d_ow, d_kcv, d_kwcv, d_sh, d_sw;
+};
+
 // col[(img, oy, ox), (ky, kx, ch)] = in[img, oy*sh-pad+ky, ox*sw-pad+kx, ch] or 0   (_cpuop 264-277)
-__global__ __launch_bounds__(kBlock) void im2col_kernel(const float* __restrict__ in,
-                                                        float* __restrict__ col, int64_t total,
-                                                        ImgGeom g) {
-    const int64_t kc = static_cast<int64_t>(g.kh) * g.kw * g.c;
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int64_t row = e / kc;              // (img*oh + oy)*ow + ox
-        int r = static_cast<int>(e - row * kc);
-        const int ch = r % g.c; r /= g.c;
-        const int kx = r % g.kw;
-        const int ky = r / g.kw;
-        const int ox = static_cast<int>(row % g.ow);
-        const int64_t t = row / g.ow;
-        const int oy = static_cast<int>(t % g.oh);
-        const int64_t img = t / g.oh;
-        const int iy = oy * g.sh - g.pad + ky;
-        const int ix = ox * g.sw - g.pad + kx;
-        float v = 0.0f;
-        if (iy >= 0 && iy < g.h && ix >= 0 && ix < g.w)
-            v = in[((img * g.h + iy) * g.w + ix) * g.c + ch];
-        col[e] = v;
+// One lane per W channels of one (oy, ox, ky, kx); lanes_per_image = oh*ow*kh*kw*cv.
+// WT: write-through stores for a col matrix too large to stay in the caches.
+template <int W, bool AL, bool WT>
+__device__ __forceinline__ void im2col_body(const float* __restrict__ in, float* __restrict__ col,
+                                            int64_t n, const ImgPlan& pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t opix, r, oy, ox, ky, kxc, kx, chv;
+    pl.d_kcv.divmod(p, opix, r);
+    pl.d_ow.divmod(opix, oy, ox);
+    pl.d_kwcv.divmod(r, ky, kxc);
+    pl.d_cv.divmod(kxc, kx, chv);
+    const int iy = static_cast<int>(oy) * g.sh - g.pad + static_cast<int>(ky);
+    const int ix = static_cast<int>(ox) * g.sw - g.pad + static_cast<int>(kx);
+    const bool inside = iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+    const int64_t in_off = (static_cast<int64_t>(iy) * g.w + ix) * g.c + chv * W;
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    // kImagesPerWorkgroup images at a time: all loads first, then all stores
+    for (int64_t img0 = static_cast<int64_t>(blockIdx.y) * kImagesPerWorkgroup; img0 < n;
+         img0 += static_cast<int64_t>(gridDim.y) * kImagesPerWorkgroup) {
+        typename VecT<W>::type v[kImagesPerWorkgroup];
+#pragma unroll
+        for (int k = 0; k < kImagesPerWorkgroup; ++k) {
+            v[k] = vsplat<W>(0.0f);
+            if (inside && img0 + k < n) v[k] = img_load<W, AL>(in + (img0 + k) * in_img + in_off);
+        }
+#pragma unroll
+        for (int k = 0; k < kImagesPerWorkgroup; ++k) {
+            if (img0 + k < n) {
+                float* q = col + (img0 + k) * col_img + static_cast<int64_t>(p) * W;
+                if constexpr (WT) vstore_writeonly<W>(q, v[k]);
+                else img_store<W, AL>(q, v[k]);
+            }
+        }
     }
+}
+
+template <int W, bool AL>
+__global__ __launch_bounds__(kBlock) void im2col_cached(const float* __restrict__ in,
+                                                        float* __restrict__ col, int64_t n, ImgPlan pl) {
+    im2col_body<W, AL, false>(in, col, n, pl);
+}
+template <int W, bool AL>
+__global__ __launch_bounds__(kBlock) void im2col_wt(const float* __restrict__ in, float* __restrict__ col,
+                                                    int64_t n, ImgPlan pl) {
+    im2col_body<W, AL, true>(in, col, n, pl);
 }
 
 // in_deltas[img, y, x, ch] += sum over covering (oy, ox), in scan order, of
 // col[(img, oy, ox), (y - (oy*sh-pad), x - (ox*sw-pad), ch)]               (_cpuop 295-309)
+// One lane per W channels of one input pixel; lanes_per_image = h*w*cv.
+template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict__ col,
-                                                        float* __restrict__ in_deltas,
-                                                        int64_t total, ImgGeom g) {
+                                                        float* __restrict__ in_deltas, int64_t n,
+                                                        ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t pix, chv, yy, xx;
+    pl.d_cv.divmod(p, pix, chv);
+    pl.d_w.divmod(pix, yy, xx);
+    const int y = static_cast<int>(yy), x = static_cast<int>(xx);
+    int oy0, oy1, ox0, ox1;
+    cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
+    cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
     const int64_t kc = static_cast<int64_t>(g.kh) * g.kw * g.c;
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int ch = static_cast<int>(e % g.c);
-        int64_t t = e / g.c;
-        const int x = static_cast<int>(t % g.w); t /= g.w;
-        const int y = static_cast<int>(t % g.h);
-        const int64_t img = t / g.h;
-        int oy0, oy1, ox0, ox1;
-        cover_range(y, g.pad, g.sh, g.kh, g.oh, oy0, oy1);
-        cover_range(x, g.pad, g.sw, g.kw, g.ow, ox0, ox1);
-        float acc = in_deltas[e];
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t col_img = static_cast<int64_t>(g.oh) * g.ow * kc;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
+        typename VecT<W>::type acc = img_load<W, AL>(q);
+        const float* cimg = col + img * col_img + chv * W;
         for (int oy = oy0; oy < oy1; ++oy) {
             const int ky = y - (oy * g.sh - g.pad);
             for (int ox = ox0; ox < ox1; ++ox) {
                 const int kx = x - (ox * g.sw - g.pad);
-                const int64_t row = (img * g.oh + oy) * g.ow + ox;
-                acc += col[row * kc + (static_cast<int64_t>(ky) * g.kw + kx) * g.c + ch];
+                acc += img_load<W, AL>(cimg + (static_cast<int64_t>(oy) * g.ow + ox) * kc +
+                                       (ky * g.kw + kx) * g.c);
             }
         }
-        in_deltas[e] = acc;
+        img_store<W, AL>(q, acc);
     }
 }
 
 // _cpuop 57-80: strict '>' from -FLT_MAX, so the first maximum in (y, x) scan
 // order wins and NaN never does; empty windows give output 0 and argmax -1.
+// One lane per W channels of one output position; lanes_per_image = oh*ow*cv.
+template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void maxpool_fwd_kernel(const float* __restrict__ in,
                                                              float* __restrict__ out,
-                                                             float* __restrict__ argmax,
-                                                             int64_t total, ImgGeom g) {
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int ch = static_cast<int>(e % g.c);
-        int64_t t = e / g.c;
-        const int ox = static_cast<int>(t % g.ow); t /= g.ow;
-        const int oy = static_cast<int>(t % g.oh);
-        const int64_t img = t / g.oh;
-        const int y = oy * g.sh - g.pad, x = ox * g.sw - g.pad;
-        const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
-        const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
-        const float* base = in + img * g.h * g.w * g.c;
-        float best = -FLT_MAX;
-        int idx = -1;
+                                                             float* __restrict__ argmax, int64_t n,
+                                                             ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t opix, chv, oy, ox;
+    pl.d_cv.divmod(p, opix, chv);
+    pl.d_ow.divmod(opix, oy, ox);
+    const int y = static_cast<int>(oy) * g.sh - g.pad, x = static_cast<int>(ox) * g.sw - g.pad;
+    const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
+    const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    const int ch0 = static_cast<int>(chv) * W;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        const float* base = in + img * in_img + ch0;
+        typename VecT<W>::type best = vsplat<W>(-FLT_MAX), where = vsplat<W>(-1.0f);
         for (int iy = y0; iy < y1; ++iy)
             for (int ix = x0; ix < x1; ++ix) {
-                const int k = (iy * g.w + ix) * g.c + ch;
-                const float v = base[k];
-                if (v > best) { best = v; idx = k; }
+                const int k = (iy * g.w + ix) * g.c;
+                typename VecT<W>::type v = img_load<W, AL>(base + k);
+#pragma unroll
+                for (int j = 0; j < W; ++j)
+                    if (comp<W>(v, j) > comp<W>(best, j)) {
+                        comp<W>(best, j) = comp<W>(v, j);
+                        comp<W>(where, j) = static_cast<float>(k + ch0 + j);
+                    }
             }
-        out[e] = idx == -1 ? 0.0f : best;
-        argmax[e] = static_cast<float>(idx);
+#pragma unroll
+        for (int j = 0; j < W; ++j)
+            if (comp<W>(where, j) < 0.0f) comp<W>(best, j) = 0.0f;
+        img_store<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, best);
+        img_store<W, AL>(argmax + img * out_img + static_cast<int64_t>(p) * W, where);
     }
 }
 
-// _cpuop 103-115 in gather form.
+// _cpuop 103-115 in gather form. One lane per W channels of one input pixel.
+template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void maxpool_bwd_kernel(const float* __restrict__ argmax,
                                                              const float* __restrict__ out_deltas,
-                                                             float* __restrict__ in_deltas,
-                                                             int64_t total, ImgGeom g) {
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int ch = static_cast<int>(e % g.c);
-        int64_t t = e / g.c;
-        const int x = static_cast<int>(t % g.w); t /= g.w;
-        const int y = static_cast<int>(t % g.h);
-        const int64_t img = t / g.h;
-        const int self = (y * g.w + x) * g.c + ch;        // what argmax holds for this pixel
-        int oy0, oy1, ox0, ox1;
-        cover_range(y, g.pad, g.sh, g.kh, g.oh, oy0, oy1);
-        cover_range(x, g.pad, g.sw, g.kw, g.ow, ox0, ox1);
-        float acc = in_deltas[e];
+                                                             float* __restrict__ in_deltas, int64_t n,
+                                                             ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t pix, chv, yy, xx;
+    pl.d_cv.divmod(p, pix, chv);
+    pl.d_w.divmod(pix, yy, xx);
+    const int y = static_cast<int>(yy), x = static_cast<int>(xx);
+    const int ch0 = static_cast<int>(chv) * W;
+    const int self = (y * g.w + x) * g.c + ch0;        // what argmax holds for this pixel's first channel
+    int oy0, oy1, ox0, ox1;
+    cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
+    cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
+        typename VecT<W>::type acc = img_load<W, AL>(q);
         for (int oy = oy0; oy < oy1; ++oy)
             for (int ox = ox0; ox < ox1; ++ox) {
-                const int64_t o = ((img * g.oh + oy) * g.ow + ox) * g.c + ch;
-                if (static_cast<int>(argmax[o]) == self) acc += out_deltas[o];
+                const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
+                typename VecT<W>::type am = img_load<W, AL>(argmax + o);
+                typename VecT<W>::type d = img_load<W, AL>(out_deltas + o);
+#pragma unroll
+                for (int j = 0; j < W; ++j)
+                    if (static_cast<int>(comp<W>(am, j)) == self + j) comp<W>(acc, j) += comp<W>(d, j);
             }
-        in_deltas[e] = acc;
+        img_store<W, AL>(q, acc);
     }
 }
 
 // _cpuop 143-162: mean over the non-padding pixels of the window.
+template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void avgpool_fwd_kernel(const float* __restrict__ in,
-                                                             float* __restrict__ out, int64_t total,
-                                                             ImgGeom g) {
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int ch = static_cast<int>(e % g.c);
-        int64_t t = e / g.c;
-        const int ox = static_cast<int>(t % g.ow); t /= g.ow;
-        const int oy = static_cast<int>(t % g.oh);
-        const int64_t img = t / g.oh;
-        const int y = oy * g.sh - g.pad, x = ox * g.sw - g.pad;
-        const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
-        const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
-        const float* base = in + img * g.h * g.w * g.c;
-        float sum = 0.0f;
+                                                             float* __restrict__ out, int64_t n,
+                                                             ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t opix, chv, oy, ox;
+    pl.d_cv.divmod(p, opix, chv);
+    pl.d_ow.divmod(opix, oy, ox);
+    const int y = static_cast<int>(oy) * g.sh - g.pad, x = static_cast<int>(ox) * g.sw - g.pad;
+    const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
+    const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
+    const float size = static_cast<float>(imax((y1 - y0) * (x1 - x0), 1));
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        const float* base = in + img * in_img + chv * W;
+        typename VecT<W>::type sum = vsplat<W>(0.0f);
         for (int iy = y0; iy < y1; ++iy)
-            for (int ix = x0; ix < x1; ++ix) sum += base[(iy * g.w + ix) * g.c + ch];
-        const int size = imax((y1 - y0) * (x1 - x0), 1);
-        out[e] = sum / static_cast<float>(size);
+            for (int ix = x0; ix < x1; ++ix) sum += img_load<W, AL>(base + (iy * g.w + ix) * g.c);
+#pragma unroll
+        for (int j = 0; j < W; ++j) comp<W>(sum, j) = comp<W>(sum, j) / size;
+        img_store<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, sum);
     }
 }
 
 // _cpuop 187-202 in gather form.
+template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void avgpool_bwd_kernel(const float* __restrict__ out_deltas,
-                                                             float* __restrict__ in_deltas,
-                                                             int64_t total, ImgGeom g) {
-    for (int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; e < total;
-         e += static_cast<int64_t>(gridDim.x) * kBlock) {
-        const int ch = static_cast<int>(e % g.c);
-        int64_t t = e / g.c;
-        const int x = static_cast<int>(t % g.w); t /= g.w;
-        const int y = static_cast<int>(t % g.h);
-        const int64_t img = t / g.h;
-        int oy0, oy1, ox0, ox1;
-        cover_range(y, g.pad, g.sh, g.kh, g.oh, oy0, oy1);
-        cover_range(x, g.pad, g.sw, g.kw, g.ow, ox0, ox1);
-        float acc = in_deltas[e];
+                                                             float* __restrict__ in_deltas, int64_t n,
+                                                             ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t pix, chv, yy, xx;
+    pl.d_cv.divmod(p, pix, chv);
+    pl.d_w.divmod(pix, yy, xx);
+    const int y = static_cast<int>(yy), x = static_cast<int>(xx);
+    int oy0, oy1, ox0, ox1;
+    cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
+    cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
+        typename VecT<W>::type acc = img_load<W, AL>(q);
         for (int oy = oy0; oy < oy1; ++oy) {
             const int wy = oy * g.sh - g.pad;
             const int ny = imin(wy + g.kh, g.h) - imax(wy, 0);
             for (int ox = ox0; ox < ox1; ++ox) {
                 const int wx = ox * g.sw - g.pad;
                 const int nx = imin(wx + g.kw, g.w) - imax(wx, 0);
-                const int64_t o = ((img * g.oh + oy) * g.ow + ox) * g.c + ch;
-                acc += out_deltas[o] / static_cast<float>(ny * nx);
+                const float size = static_cast<float>(ny * nx);
+                typename VecT<W>::type d = img_load<W, AL>(
+                    out_deltas + img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + chv * W);
+#pragma unroll
+                for (int j = 0; j < W; ++j) comp<W>(acc, j) += comp<W>(d, j) / size;
             }
         }
-        in_deltas[e] = acc;
+        img_store<W, AL>(q, acc);
     }
 }
 
@@ -214,9 +343,36 @@ static inline int conv_out(int in, int k, int pad, int stride) { return (in + 2 
 
 using namespace bship;
 
-#define BSHIP_LAUNCH_IMG(kernel, total, ...)                                                  \
-    hipLaunchKernelGGL(kernel, dim3(stream_grid(ceil_div((total), kBlock))), dim3(kBlock), 0, \
-                       ctx().stream, __VA_ARGS__)
+// Launches kernel<W, AL> over lanes_per_image x n: W = 4 when the channels come in fours,
+// AL when additionally every pointer is 16-byte aligned.
+#define BSHIP_LAUNCH_IMG(kernel, name, positions, aligned, ...)                                         \
+    do {                                                                                                \
+        const bool vec4_ = (g.c % 4 == 0);                                                              \
+        const int cv_ = vec4_ ? g.c / 4 : g.c;                                                          \
+        const int64_t lanes_ = static_cast<int64_t>(positions) * cv_;                                   \
+        if (lanes_ > 0x7fffffff)                                                                        \
+            return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: one image exceeds 2^31 elements", name);     \
+        ImgPlan pl_;                                                                                    \
+        pl_.g = g;                                                                                      \
+        pl_.lanes_per_image = static_cast<uint32_t>(lanes_);                                            \
+        pl_.d_cv = FastDiv(static_cast<uint32_t>(imax(cv_, 1)));                                        \
+        pl_.d_w = FastDiv(static_cast<uint32_t>(imax(g.w, 1)));                                         \
+        pl_.d_ow = FastDiv(static_cast<uint32_t>(imax(g.ow, 1)));                                       \
+        pl_.d_kcv = FastDiv(static_cast<uint32_t>(imax(g.kh * g.kw * cv_, 1)));                         \
+        pl_.d_kwcv = FastDiv(static_cast<uint32_t>(imax(g.kw * cv_, 1)));                               \
+        pl_.d_sh = FastDiv(static_cast<uint32_t>(g.sh));                                                \
+        pl_.d_sw = FastDiv(static_cast<uint32_t>(g.sw));                                                \
+        const int64_t gy_ = ceil_div(n, kImagesPerWorkgroup);                                           \
+        const dim3 grid_(static_cast<unsigned>(ceil_div(lanes_, kBlock)),                               \
+                         static_cast<unsigned>(gy_ < 65535 ? gy_ : 65535));                             \
+        if (vec4_ && (aligned))                                                                         \
+            hipLaunchKernelGGL((kernel<4, true>), grid_, dim3(kBlock), 0, ctx().stream, __VA_ARGS__, n, pl_); \
+        else if (vec4_)                                                                                 \
+            hipLaunchKernelGGL((kernel<4, false>), grid_, dim3(kBlock), 0, ctx().stream, __VA_ARGS__, n, pl_); \
+        else                                                                                            \
+            hipLaunchKernelGGL((kernel<1, false>), grid_, dim3(kBlock), 0, ctx().stream, __VA_ARGS__, n, pl_); \
+        return check_launch(name);                                                                      \
+    } while (0)
 
 extern "C" {
 
@@ -232,8 +388,11 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(col);
-    BSHIP_LAUNCH_IMG(im2col_kernel, total, in, col, total, g);
-    return check_launch("im2col");
+    if (static_cast<size_t>(total) >= (size_t(1) << 26))      // 256 MiB: beyond the last-level cache
+        BSHIP_LAUNCH_IMG(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,
+                         aligned16(in) && aligned16(col), in, col);
+    BSHIP_LAUNCH_IMG(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,
+                     aligned16(in) && aligned16(col), in, col);
 }
 
 int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, int w, int c,
@@ -248,8 +407,8 @@ int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(col);
     BSHIP_REQUIRE_PTR(in_deltas);
-    BSHIP_LAUNCH_IMG(col2im_kernel, total, col, in_deltas, total, g);
-    return check_launch("col2im");
+    BSHIP_LAUNCH_IMG(col2im_kernel, "col2im", static_cast<int64_t>(h) * w,
+                     aligned16(col) && aligned16(in_deltas), col, in_deltas);
 }
 
 int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64_t n, int h, int w,
@@ -264,8 +423,8 @@ int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_PTR(argmax);
-    BSHIP_LAUNCH_IMG(maxpool_fwd_kernel, total, in, out, argmax, total, g);
-    return check_launch("maxpool2d_forward_batch");
+    BSHIP_LAUNCH_IMG(maxpool_fwd_kernel, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w,
+                     aligned16(in) && aligned16(out) && aligned16(argmax), in, out, argmax);
 }
 
 int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, float* in_deltas,
@@ -280,8 +439,9 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
     BSHIP_REQUIRE_PTR(argmax);
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
-    BSHIP_LAUNCH_IMG(maxpool_bwd_kernel, total, argmax, out_deltas, in_deltas, total, g);
-    return check_launch("maxpool2d_backward_batch");
+    BSHIP_LAUNCH_IMG(maxpool_bwd_kernel, "maxpool2d_backward_batch", static_cast<int64_t>(h) * w,
+                     aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas), argmax, out_deltas,
+                     in_deltas);
 }
 
 int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, int w, int c,
@@ -295,8 +455,8 @@ int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, in
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
-    BSHIP_LAUNCH_IMG(avgpool_fwd_kernel, total, in, out, total, g);
-    return check_launch("avgpool2d_forward_batch");
+    BSHIP_LAUNCH_IMG(avgpool_fwd_kernel, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w,
+                     aligned16(in) && aligned16(out), in, out);
 }
 
 int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_t n, int h, int w,
@@ -310,8 +470,8 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_
     if (total == 0 || out_h == 0 || out_w == 0) return 0;
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
-    BSHIP_LAUNCH_IMG(avgpool_bwd_kernel, total, out_deltas, in_deltas, total, g);
-    return check_launch("avgpool2d_backward_batch");
+    BSHIP_LAUNCH_IMG(avgpool_bwd_kernel, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w,
+                     aligned16(out_deltas) && aligned16(in_deltas), out_deltas, in_deltas);
 }
 
 }  // extern "C"
