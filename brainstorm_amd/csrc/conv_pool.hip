@@ -184,11 +184,11 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
 // _cpuop 57-80: strict '>' from -FLT_MAX, so the first maximum in (y, x) scan
 // order wins and NaN never does; empty windows give output 0 and argmax -1.
 // One lane per W channels of one output position; lanes_per_image = oh*ow*cv.
-template <int W, bool AL>
-__global__ __launch_bounds__(kBlock) void maxpool_fwd_kernel(const float* __restrict__ in,
-                                                             float* __restrict__ out,
-                                                             float* __restrict__ argmax, int64_t n,
-                                                             ImgPlan pl) {
+// K > 0: the window is K x K, known at compile time; all K*K loads are issued first
+// (positions outside the image read a clamped address and are skipped in the scan).
+template <int W, bool AL, int K>
+__device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, float* __restrict__ out,
+                                                 float* __restrict__ argmax, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
     const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
@@ -201,20 +201,40 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_kernel(const float* __rest
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
     const int ch0 = static_cast<int>(chv) * W;
+    typedef typename VecT<W>::type R;
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         const float* base = in + img * in_img + ch0;
-        typename VecT<W>::type best = vsplat<W>(-FLT_MAX), where = vsplat<W>(-1.0f);
-        for (int iy = y0; iy < y1; ++iy)
-            for (int ix = x0; ix < x1; ++ix) {
-                const int k = (iy * g.w + ix) * g.c;
-                typename VecT<W>::type v = img_load<W, AL>(base + k);
+        R best = vsplat<W>(-FLT_MAX), where = vsplat<W>(-1.0f);
+        auto take = [&](R v, int k) {
 #pragma unroll
-                for (int j = 0; j < W; ++j)
-                    if (comp<W>(v, j) > comp<W>(best, j)) {
-                        comp<W>(best, j) = comp<W>(v, j);
-                        comp<W>(where, j) = static_cast<float>(k + ch0 + j);
-                    }
-            }
+            for (int j = 0; j < W; ++j)
+                if (comp<W>(v, j) > comp<W>(best, j)) {
+                    comp<W>(best, j) = comp<W>(v, j);
+                    comp<W>(where, j) = static_cast<float>(k + ch0 + j);
+                }
+        };
+        if constexpr (K > 0) {
+            R v[K * K];
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b) {
+                    const int iy = imin(imax(y + a, 0), g.h - 1), ix = imin(imax(x + b, 0), g.w - 1);
+                    v[a * K + b] = img_load<W, AL>(base + (iy * g.w + ix) * g.c);
+                }
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b)
+                    if (y + a >= y0 && y + a < y1 && x + b >= x0 && x + b < x1)
+                        take(v[a * K + b], ((y + a) * g.w + (x + b)) * g.c);
+        } else {
+            for (int iy = y0; iy < y1; ++iy)
+                for (int ix = x0; ix < x1; ++ix) {
+                    const int k = (iy * g.w + ix) * g.c;
+                    take(img_load<W, AL>(base + k), k);
+                }
+        }
 #pragma unroll
         for (int j = 0; j < W; ++j)
             if (comp<W>(where, j) < 0.0f) comp<W>(best, j) = 0.0f;
@@ -222,13 +242,23 @@ __global__ __launch_bounds__(kBlock) void maxpool_fwd_kernel(const float* __rest
         img_store<W, AL>(argmax + img * out_img + static_cast<int64_t>(p) * W, where);
     }
 }
+#define BSHIP_POOL_FWD_KERNEL(name, K)                                                                   \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void name(const float* __restrict__ in, float* __restrict__ out, \
+                                                   float* __restrict__ argmax, int64_t n, ImgPlan pl) {  \
+        maxpool_fwd_body<W, AL, K>(in, out, argmax, n, pl);                                              \
+    }
+BSHIP_POOL_FWD_KERNEL(maxpool_fwd_kernel, 0)
+BSHIP_POOL_FWD_KERNEL(maxpool_fwd_kernel_2x2, 2)
+BSHIP_POOL_FWD_KERNEL(maxpool_fwd_kernel_3x3, 3)
 
 // _cpuop 103-115 in gather form. One lane per W channels of one input pixel.
-template <int W, bool AL>
-__global__ __launch_bounds__(kBlock) void maxpool_bwd_kernel(const float* __restrict__ argmax,
-                                                             const float* __restrict__ out_deltas,
-                                                             float* __restrict__ in_deltas, int64_t n,
-                                                             ImgPlan pl) {
+// C > 0: at most C x C output positions cover a pixel (C = ceil(window / stride), known at
+// compile time); their loads are issued first, positions beyond the cover read a clamped address.
+template <int W, bool AL, int C>
+__device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argmax,
+                                                 const float* __restrict__ out_deltas,
+                                                 float* __restrict__ in_deltas, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
     const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
@@ -243,27 +273,56 @@ __global__ __launch_bounds__(kBlock) void maxpool_bwd_kernel(const float* __rest
     cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    typedef typename VecT<W>::type R;
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
-        typename VecT<W>::type acc = img_load<W, AL>(q);
-        for (int oy = oy0; oy < oy1; ++oy)
-            for (int ox = ox0; ox < ox1; ++ox) {
-                const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
-                typename VecT<W>::type am = img_load<W, AL>(argmax + o);
-                typename VecT<W>::type d = img_load<W, AL>(out_deltas + o);
+        R acc = img_load<W, AL>(q);
+        auto take = [&](R am, R d) {
 #pragma unroll
-                for (int j = 0; j < W; ++j)
-                    if (static_cast<int>(comp<W>(am, j)) == self + j) comp<W>(acc, j) += comp<W>(d, j);
-            }
+            for (int j = 0; j < W; ++j)
+                if (static_cast<int>(comp<W>(am, j)) == self + j) comp<W>(acc, j) += comp<W>(d, j);
+        };
+        if constexpr (C > 0) {
+            R am[C * C], d[C * C];
+#pragma unroll
+            for (int a = 0; a < C; ++a)
+#pragma unroll
+                for (int b = 0; b < C; ++b) {
+                    const int oy = imin(oy0 + a, g.oh - 1), ox = imin(ox0 + b, g.ow - 1);
+                    const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
+                    am[a * C + b] = img_load<W, AL>(argmax + o);
+                    d[a * C + b] = img_load<W, AL>(out_deltas + o);
+                }
+#pragma unroll
+            for (int a = 0; a < C; ++a)
+#pragma unroll
+                for (int b = 0; b < C; ++b)
+                    if (oy0 + a < oy1 && ox0 + b < ox1) take(am[a * C + b], d[a * C + b]);
+        } else {
+            for (int oy = oy0; oy < oy1; ++oy)
+                for (int ox = ox0; ox < ox1; ++ox) {
+                    const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
+                    take(img_load<W, AL>(argmax + o), img_load<W, AL>(out_deltas + o));
+                }
+        }
         img_store<W, AL>(q, acc);
     }
 }
+#define BSHIP_POOL_BWD_KERNEL(name, C)                                                                   \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void name(const float* __restrict__ argmax,                     \
+                                                   const float* __restrict__ out_deltas,                 \
+                                                   float* __restrict__ in_deltas, int64_t n, ImgPlan pl) { \
+        maxpool_bwd_body<W, AL, C>(argmax, out_deltas, in_deltas, n, pl);                                \
+    }
+BSHIP_POOL_BWD_KERNEL(maxpool_bwd_kernel, 0)
+BSHIP_POOL_BWD_KERNEL(maxpool_bwd_kernel_c1, 1)
+BSHIP_POOL_BWD_KERNEL(maxpool_bwd_kernel_c2, 2)
 
-// _cpuop 143-162: mean over the non-padding pixels of the window.
-template <int W, bool AL>
-__global__ __launch_bounds__(kBlock) void avgpool_fwd_kernel(const float* __restrict__ in,
-                                                             float* __restrict__ out, int64_t n,
-                                                             ImgPlan pl) {
+// _cpuop 143-162: mean over the non-padding pixels of the window. K as for max pooling.
+template <int W, bool AL, int K>
+__device__ __forceinline__ void avgpool_fwd_body(const float* __restrict__ in, float* __restrict__ out,
+                                                 int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
     const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
@@ -276,22 +335,47 @@ __global__ __launch_bounds__(kBlock) void avgpool_fwd_kernel(const float* __rest
     const float size = static_cast<float>(imax((y1 - y0) * (x1 - x0), 1));
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    typedef typename VecT<W>::type R;
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         const float* base = in + img * in_img + chv * W;
-        typename VecT<W>::type sum = vsplat<W>(0.0f);
-        for (int iy = y0; iy < y1; ++iy)
-            for (int ix = x0; ix < x1; ++ix) sum += img_load<W, AL>(base + (iy * g.w + ix) * g.c);
+        R sum = vsplat<W>(0.0f);
+        if constexpr (K > 0) {
+            R v[K * K];
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b) {
+                    const int iy = imin(imax(y + a, 0), g.h - 1), ix = imin(imax(x + b, 0), g.w - 1);
+                    v[a * K + b] = img_load<W, AL>(base + (iy * g.w + ix) * g.c);
+                }
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b)
+                    if (y + a >= y0 && y + a < y1 && x + b >= x0 && x + b < x1) sum += v[a * K + b];
+        } else {
+            for (int iy = y0; iy < y1; ++iy)
+                for (int ix = x0; ix < x1; ++ix) sum += img_load<W, AL>(base + (iy * g.w + ix) * g.c);
+        }
 #pragma unroll
         for (int j = 0; j < W; ++j) comp<W>(sum, j) = comp<W>(sum, j) / size;
         img_store<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, sum);
     }
 }
+#define BSHIP_AVG_FWD_KERNEL(name, K)                                                                    \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void name(const float* __restrict__ in, float* __restrict__ out, \
+                                                   int64_t n, ImgPlan pl) {                              \
+        avgpool_fwd_body<W, AL, K>(in, out, n, pl);                                                      \
+    }
+BSHIP_AVG_FWD_KERNEL(avgpool_fwd_kernel, 0)
+BSHIP_AVG_FWD_KERNEL(avgpool_fwd_kernel_2x2, 2)
+BSHIP_AVG_FWD_KERNEL(avgpool_fwd_kernel_3x3, 3)
 
-// _cpuop 187-202 in gather form.
-template <int W, bool AL>
-__global__ __launch_bounds__(kBlock) void avgpool_bwd_kernel(const float* __restrict__ out_deltas,
-                                                             float* __restrict__ in_deltas, int64_t n,
-                                                             ImgPlan pl) {
+// _cpuop 187-202 in gather form. C as for max pooling.
+template <int W, bool AL, int C>
+__device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_deltas,
+                                                 float* __restrict__ in_deltas, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
     const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
@@ -304,25 +388,57 @@ __global__ __launch_bounds__(kBlock) void avgpool_bwd_kernel(const float* __rest
     cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    typedef typename VecT<W>::type R;
+    // number of image pixels under the window at output position (oy, ox)
+    auto window_size = [&](int oy, int ox) {
+        const int wy = oy * g.sh - g.pad, wx = ox * g.sw - g.pad;
+        const int ny = imin(wy + g.kh, g.h) - imax(wy, 0);
+        const int nx = imin(wx + g.kw, g.w) - imax(wx, 0);
+        return static_cast<float>(ny * nx);
+    };
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
-        typename VecT<W>::type acc = img_load<W, AL>(q);
-        for (int oy = oy0; oy < oy1; ++oy) {
-            const int wy = oy * g.sh - g.pad;
-            const int ny = imin(wy + g.kh, g.h) - imax(wy, 0);
-            for (int ox = ox0; ox < ox1; ++ox) {
-                const int wx = ox * g.sw - g.pad;
-                const int nx = imin(wx + g.kw, g.w) - imax(wx, 0);
-                const float size = static_cast<float>(ny * nx);
-                typename VecT<W>::type d = img_load<W, AL>(
-                    out_deltas + img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + chv * W);
+        R acc = img_load<W, AL>(q);
+        const float* dimg = out_deltas + img * out_img + chv * W;
+        if constexpr (C > 0) {
+            R d[C * C];
 #pragma unroll
-                for (int j = 0; j < W; ++j) comp<W>(acc, j) += comp<W>(d, j) / size;
-            }
+            for (int a = 0; a < C; ++a)
+#pragma unroll
+                for (int b = 0; b < C; ++b) {
+                    const int oy = imin(oy0 + a, g.oh - 1), ox = imin(ox0 + b, g.ow - 1);
+                    d[a * C + b] = img_load<W, AL>(dimg + (static_cast<int64_t>(oy) * g.ow + ox) * g.c);
+                }
+#pragma unroll
+            for (int a = 0; a < C; ++a)
+#pragma unroll
+                for (int b = 0; b < C; ++b)
+                    if (oy0 + a < oy1 && ox0 + b < ox1) {
+                        const float size = window_size(oy0 + a, ox0 + b);
+#pragma unroll
+                        for (int j = 0; j < W; ++j) comp<W>(acc, j) += comp<W>(d[a * C + b], j) / size;
+                    }
+        } else {
+            for (int oy = oy0; oy < oy1; ++oy)
+                for (int ox = ox0; ox < ox1; ++ox) {
+                    const float size = window_size(oy, ox);
+                    R d = img_load<W, AL>(dimg + (static_cast<int64_t>(oy) * g.ow + ox) * g.c);
+#pragma unroll
+                    for (int j = 0; j < W; ++j) comp<W>(acc, j) += comp<W>(d, j) / size;
+                }
         }
         img_store<W, AL>(q, acc);
     }
 }
+#define BSHIP_AVG_BWD_KERNEL(name, C)                                                                    \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void name(const float* __restrict__ out_deltas,                 \
+                                                   float* __restrict__ in_deltas, int64_t n, ImgPlan pl) { \
+        avgpool_bwd_body<W, AL, C>(out_deltas, in_deltas, n, pl);                                        \
+    }
+BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel, 0)
+BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel_c1, 1)
+BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel_c2, 2)
 
 static int check_geom(const char* fn, int64_t n, const ImgGeom& g) {
     if (n < 0 || g.h < 0 || g.w < 0 || g.c < 0 || g.oh < 0 || g.ow < 0 || g.kh < 1 || g.kw < 1 ||
@@ -423,8 +539,12 @@ int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_PTR(argmax);
-    BSHIP_LAUNCH_IMG(maxpool_fwd_kernel, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w,
-                     aligned16(in) && aligned16(out) && aligned16(argmax), in, out, argmax);
+    const bool al = aligned16(in) && aligned16(out) && aligned16(argmax);
+    if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
+        BSHIP_LAUNCH_IMG(maxpool_fwd_kernel_3x3, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out, argmax);
+    if (pool_h == 2 && pool_w == 2 && h >= 1 && w >= 1)
+        BSHIP_LAUNCH_IMG(maxpool_fwd_kernel_2x2, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out, argmax);
+    BSHIP_LAUNCH_IMG(maxpool_fwd_kernel, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out, argmax);
 }
 
 int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, float* in_deltas,
@@ -439,9 +559,14 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
     BSHIP_REQUIRE_PTR(argmax);
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
-    BSHIP_LAUNCH_IMG(maxpool_bwd_kernel, "maxpool2d_backward_batch", static_cast<int64_t>(h) * w,
-                     aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas), argmax, out_deltas,
-                     in_deltas);
+    const bool al = aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas);
+    // how many output positions can cover one pixel along each axis
+    const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
+    if (cover == 1)
+        BSHIP_LAUNCH_IMG(maxpool_bwd_kernel_c1, "maxpool2d_backward_batch", static_cast<int64_t>(h) * w, al, argmax, out_deltas, in_deltas);
+    if (cover == 2)
+        BSHIP_LAUNCH_IMG(maxpool_bwd_kernel_c2, "maxpool2d_backward_batch", static_cast<int64_t>(h) * w, al, argmax, out_deltas, in_deltas);
+    BSHIP_LAUNCH_IMG(maxpool_bwd_kernel, "maxpool2d_backward_batch", static_cast<int64_t>(h) * w, al, argmax, out_deltas, in_deltas);
 }
 
 int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, int w, int c,
@@ -455,8 +580,12 @@ int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, in
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
-    BSHIP_LAUNCH_IMG(avgpool_fwd_kernel, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w,
-                     aligned16(in) && aligned16(out), in, out);
+    const bool al = aligned16(in) && aligned16(out);
+    if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
+        BSHIP_LAUNCH_IMG(avgpool_fwd_kernel_3x3, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
+    if (pool_h == 2 && pool_w == 2 && h >= 1 && w >= 1)
+        BSHIP_LAUNCH_IMG(avgpool_fwd_kernel_2x2, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
+    BSHIP_LAUNCH_IMG(avgpool_fwd_kernel, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
 }
 
 int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_t n, int h, int w,
@@ -470,8 +599,13 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_
     if (total == 0 || out_h == 0 || out_w == 0) return 0;
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
-    BSHIP_LAUNCH_IMG(avgpool_bwd_kernel, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w,
-                     aligned16(out_deltas) && aligned16(in_deltas), out_deltas, in_deltas);
+    const bool al = aligned16(out_deltas) && aligned16(in_deltas);
+    const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
+    if (cover == 1)
+        BSHIP_LAUNCH_IMG(avgpool_bwd_kernel_c1, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w, al, out_deltas, in_deltas);
+    if (cover == 2)
+        BSHIP_LAUNCH_IMG(avgpool_bwd_kernel_c2, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w, al, out_deltas, in_deltas);
+    BSHIP_LAUNCH_IMG(avgpool_bwd_kernel, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w, al, out_deltas, in_deltas);
 }
 
 }  // extern "C"
