@@ -179,6 +179,61 @@ def run_gpu(size, steps, warmup):
     return hip, name, cus, elapsed, {n: float(np.mean(v)) for n, v in per_op_ms.items()}
 
 
+def run_image_ops(hip, n_img=2048, reps=10):
+    """The image operations (im2col/col2im of the convolutions, max/avg pooling) at the shapes of
+    the CNN workload with a batch large enough to leave the caches: us per launch and the fraction
+    of peak for the bytes each must move at least (inputs read once, outputs written once)."""
+    lib = hip._lib
+    ms = ctypes.c_float()
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        lib.bship_event_record(0)
+        for _ in range(reps):
+            fn()
+        lib.bship_event_record(1)
+        hip._call(lib.bship_event_elapsed_ms(0, 1, ctypes.byref(ms)))
+        return ms.value * 1e3 / reps
+
+    def filled(shape):
+        a = hip.allocate(shape)
+        hip.fill(a, 0.5)
+        return a
+
+    out = {}
+
+    def report(name, us, nbytes):
+        gbps = nbytes / us / 1e3
+        out[name] = {"us": round(us, 1), "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+
+    for h, w, c, k, pad, tag in ((32, 32, 3, 5, 2, "conv1_32x32x3_k5"), (15, 15, 32, 5, 2, "conv2_15x15x32_k5")):
+        x = filled((n_img, h, w, c))
+        oh, ow = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+        col = hip.allocate((n_img * oh * ow, k * k * c))
+        dx = hip.allocate((n_img, h, w, c))
+        report("im2col_" + tag, timed(lambda: hip._call(lib.bship_im2col_nhwc_f32(
+            x.ptr, col.ptr, n_img, h, w, c, k, k, pad, 1, 1))), 4 * (x.size + col.size))
+        report("col2im_" + tag, timed(lambda: hip._call(lib.bship_col2im_nhwc_f32(
+            col.ptr, dx.ptr, n_img, h, w, c, k, k, pad, 1, 1))), 4 * (2 * x.size + col.size))
+        del col, dx, x
+    for h, w, c, k, s, tag in ((32, 32, 32, 3, 2, "pool1_32x32x32_k3s2"), (15, 15, 64, 3, 2, "pool2_15x15x64_k3s2")):
+        x = filled((n_img, h, w, c))
+        oh, ow = (h - k) // s + 1, (w - k) // s + 1
+        o, am, do = hip.allocate((n_img, oh, ow, c)), hip.allocate((n_img, oh, ow, c)), filled((n_img, oh, ow, c))
+        dx = hip.allocate((n_img, h, w, c))
+        report("maxpool_fwd_" + tag, timed(lambda: hip.maxpool2d_forward_batch(x, (k, k), o, 0, (s, s), am)),
+               4 * (x.size + 2 * o.size))
+        report("maxpool_bwd_" + tag, timed(lambda: hip.maxpool2d_backward_batch(x, (k, k), o, 0, (s, s), am, dx, do)),
+               4 * (2 * x.size + 2 * o.size))
+        report("avgpool_fwd_" + tag, timed(lambda: hip.avgpool2d_forward_batch(x, (k, k), o, 0, (s, s))),
+               4 * (x.size + o.size))
+        report("avgpool_bwd_" + tag, timed(lambda: hip.avgpool2d_backward_batch(x, (k, k), o, 0, (s, s), dx, do)),
+               4 * (2 * x.size + o.size))
+        del x, o, am, do, dx
+    return out
+
+
 def time_net(handler, builder, steps, warmup, sync, **kw):
     """Training steps per second of one network workload (forward + backward + momentum update,
     inputs uploaded once; the per-step loss read-back of a Trainer is included)."""
@@ -257,6 +312,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-nets", action="store_true", help="skip the MLP/LSTM samples/s runs")
+    ap.add_argument("--no-image-ops", action="store_true", help="skip the im2col/col2im/pooling measurements")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the handler path has no multi-GPU part "
@@ -295,6 +351,8 @@ def main():
         "roofline": roofline,
         "ops": ops,
     }
+    if not args.no_image_ops:
+        out["image_ops"] = run_image_ops(hip)
     if not args.no_nets:
         # second part of the metric: training samples/s of the MLP and LSTM workloads
         out["nets"] = run_nets_gpu(hip)
