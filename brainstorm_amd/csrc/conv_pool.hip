@@ -134,6 +134,52 @@ __device__ __forceinline__ void im2col_body(const float* __restrict__ in, float*
     }
 }
 
+// Channel counts that are not a multiple of 4 (RGB input): a lane still writes 4 consecutive
+// col elements with one 128-bit store, gathering them with 4 scalar loads; each element is
+// decoded on its own (they may lie in different kernel positions or output pixels). Needs
+// oh*ow*kh*kw*c to be a multiple of 4; the plan's divisors are those of W = 1 and
+// lanes_per_image counts the groups of 4.
+template <bool WT>
+__global__ __launch_bounds__(kBlock) void im2col_gather4(const float* __restrict__ in,
+                                                         float* __restrict__ col, int64_t n, ImgPlan pl) {
+    const ImgGeom& g = pl.g;
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    int in_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t opix, r, oy, ox, ky, kxc, kx, ch;
+        pl.d_kcv.divmod(p * 4 + j, opix, r);
+        pl.d_ow.divmod(opix, oy, ox);
+        pl.d_kwcv.divmod(r, ky, kxc);
+        pl.d_cv.divmod(kxc, kx, ch);
+        const int iy = static_cast<int>(oy) * g.sh - g.pad + static_cast<int>(ky);
+        const int ix = static_cast<int>(ox) * g.sw - g.pad + static_cast<int>(kx);
+        const bool inside = iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+        in_off[j] = inside ? (iy * g.w + ix) * g.c + static_cast<int>(ch) : -1;
+    }
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * 4;
+    for (int64_t img0 = static_cast<int64_t>(blockIdx.y) * kImagesPerWorkgroup; img0 < n;
+         img0 += static_cast<int64_t>(gridDim.y) * kImagesPerWorkgroup) {
+        f4 v[kImagesPerWorkgroup];
+#pragma unroll
+        for (int k = 0; k < kImagesPerWorkgroup; ++k) {
+            const float* base = in + (img0 + k < n ? img0 + k : img0) * in_img;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[k][j] = in_off[j] >= 0 ? base[in_off[j]] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < kImagesPerWorkgroup; ++k) {
+            if (img0 + k < n) {
+                float* q = col + (img0 + k) * col_img + static_cast<int64_t>(p) * 4;
+                if constexpr (WT) vstore_writeonly<4>(q, v[k]);
+                else *reinterpret_cast<f4u*>(q) = v[k];
+            }
+        }
+    }
+}
+
 template <int W, bool AL>
 __global__ __launch_bounds__(kBlock) void im2col_cached(const float* __restrict__ in,
                                                         float* __restrict__ col, int64_t n, ImgPlan pl) {
@@ -504,7 +550,23 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(col);
-    if (static_cast<size_t>(total) >= (size_t(1) << 26))      // 256 MiB: beyond the last-level cache
+    const bool write_through = static_cast<size_t>(total) >= (size_t(1) << 26);   // 256 MiB: beyond the last-level cache
+    const int64_t per_image = static_cast<int64_t>(g.oh) * g.ow * kh * kw * c;
+    if (c % 4 != 0 && per_image % 4 == 0 && per_image <= 0x7fffffff) {
+        ImgPlan pl;
+        pl.g = g;
+        pl.lanes_per_image = static_cast<uint32_t>(per_image / 4);
+        pl.d_cv = FastDiv(static_cast<uint32_t>(c));
+        pl.d_ow = FastDiv(static_cast<uint32_t>(g.ow));
+        pl.d_kcv = FastDiv(static_cast<uint32_t>(kh * kw * c));
+        pl.d_kwcv = FastDiv(static_cast<uint32_t>(kw * c));
+        const int64_t gy = ceil_div(n, kImagesPerWorkgroup);
+        const dim3 grid(static_cast<unsigned>(ceil_div(per_image / 4, kBlock)), static_cast<unsigned>(gy < 65535 ? gy : 65535));
+        if (write_through) hipLaunchKernelGGL(im2col_gather4<true>, grid, dim3(kBlock), 0, ctx().stream, in, col, n, pl);
+        else               hipLaunchKernelGGL(im2col_gather4<false>, grid, dim3(kBlock), 0, ctx().stream, in, col, n, pl);
+        return check_launch("im2col");
+    }
+    if (write_through)
         BSHIP_LAUNCH_IMG(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,
                          aligned16(in) && aligned16(col), in, col);
     BSHIP_LAUNCH_IMG(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,

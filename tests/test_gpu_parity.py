@@ -601,7 +601,10 @@ def test_avgpool_forward_backward_exact(hip, ref):
 
 CONV_CASES = [(2, 5, 4, 3, 2, 3, 3, 0, (1, 1)), (2, 5, 4, 3, 2, 3, 3, 1, (2, 1)), (1, 3, 3, 1, 1, 1, 1, 0, (1, 1)),
               (4, 9, 9, 3, 4, 5, 5, 2, (1, 1)), (3, 9, 6, 1, 3, 3, 2, 1, (2, 3)),
-              (10, 32, 32, 3, 32, 5, 5, 2, (1, 1)), (10, 15, 15, 32, 64, 5, 5, 2, (1, 1))]
+              (10, 32, 32, 3, 32, 5, 5, 2, (1, 1)), (10, 15, 15, 32, 64, 5, 5, 2, (1, 1)),
+              # channel counts that are no multiple of 4 with a col matrix that is: groups of four
+              # col elements that straddle kernel positions and output pixels
+              (2, 6, 6, 3, 4, 2, 2, 1, (2, 2)), (5, 8, 4, 2, 3, 3, 3, 1, (1, 1)), (9, 6, 6, 1, 2, 3, 3, 1, (1, 1))]
 
 
 def test_conv2d_forward_backward(hip, ref):
