@@ -17,7 +17,7 @@ template <typename R> __device__ __forceinline__ R vzero();
 template <> __device__ __forceinline__ float vzero<float>() { return 0.0f; }
 template <> __device__ __forceinline__ f4 vzero<f4>() { f4 z = {0.0f, 0.0f, 0.0f, 0.0f}; return z; }
 
-// A workgroup is 64 column-lanes x 4 row-lanes (one wavefront per row-lane): each
+// A workgroup is (for wide matrices) 64 column-lanes x 4 row-lanes, one wavefront per row-lane: each
 // wavefront reads 64*W consecutive columns of one row per access, walks down the
 // rows of its band with 4 independent accumulators, and the 4 wavefronts are
 // combined through LDS. grid.x tiles the columns, grid.y splits the rows into bands;
@@ -40,50 +40,75 @@ struct PlainSrc {
     }
 };
 
-template <int W, bool AL, typename Src>
+// CL column-lanes x (kBlock / CL) row-lanes. CL = 64 for matrices at least 64 accesses wide;
+// narrower matrices (bias gradients of small layers, image channels) take CL = 8, 16 or 32 so
+// that the lanes that would have no column walk down more rows instead.
+template <int W, bool AL, int CL, typename Src>
 __global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int64_t M, int64_t NW) {
     typedef typename VecT<W>::type R;
+    constexpr int RL = kBlock / CL;                          // row-lanes
+    constexpr int GROUP = 4 * RL;                            // rows per group: 4 per row-lane
     __shared__ R lds[kBlock];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wv = threadIdx.x / kWave;                      // 0..3: row-lane
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * kWave + lane;
+    const int lane = threadIdx.x & (CL - 1);
+    const int rl = threadIdx.x / CL;
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * CL + lane;
     R acc0 = vzero<R>(), acc1 = vzero<R>(), acc2 = vzero<R>(), acc3 = vzero<R>();
     if (c < NW) {
         const int64_t col = c * W;
         const int64_t pitch = NW * W;
         const R cx = src.template prep<W, AL>(col);
-        // Groups of 16 rows are dealt round-robin to the row bands (blockIdx.y), so all
-        // bands together read one contiguous region that moves down the matrix. (Bands of
+        // Groups of rows are dealt round-robin to the row bands (blockIdx.y), so all bands
+        // together read one contiguous region that moves down the matrix. (Bands of
         // consecutive rows start a power-of-two number of bytes apart for the usual matrix
         // sizes and were measured 5-10 % slower.)
-        for (int64_t g = blockIdx.y; g * 16 < M; g += gridDim.y) {
-            int64_t r = g * 16 + wv;
-            if (r + 12 < M) {
+        for (int64_t g = blockIdx.y; g * GROUP < M; g += gridDim.y) {
+            int64_t r = g * GROUP + rl;
+            if (r + 3 * RL < M) {
                 R x0 = src.template load<W, AL>(col + r * pitch, cx);
-                R x1 = src.template load<W, AL>(col + (r + 4) * pitch, cx);
-                R x2 = src.template load<W, AL>(col + (r + 8) * pitch, cx);
-                R x3 = src.template load<W, AL>(col + (r + 12) * pitch, cx);
+                R x1 = src.template load<W, AL>(col + (r + RL) * pitch, cx);
+                R x2 = src.template load<W, AL>(col + (r + 2 * RL) * pitch, cx);
+                R x3 = src.template load<W, AL>(col + (r + 3 * RL) * pitch, cx);
                 acc0 += x0; acc1 += x1; acc2 += x2; acc3 += x3;
             } else {
-                for (; r < M; r += 4) acc0 += src.template load<W, AL>(col + r * pitch, cx);
+                for (; r < M; r += RL) acc0 += src.template load<W, AL>(col + r * pitch, cx);
             }
         }
     }
     lds[threadIdx.x] = (acc0 + acc1) + (acc2 + acc3);
     __syncthreads();
-    if (wv == 0 && c < NW) {
-        R t = (lds[lane] + lds[lane + kWave]) + (lds[lane + 2 * kWave] + lds[lane + 3 * kWave]);
+    if (rl == 0 && c < NW) {
+        R t;
+        if constexpr (RL == 4) {
+            t = (lds[lane] + lds[lane + CL]) + (lds[lane + 2 * CL] + lds[lane + 3 * CL]);
+        } else {
+            t = lds[lane];
+#pragma unroll
+            for (int k = 1; k < RL; ++k) t += lds[lane + k * CL];
+        }
         vstore<W, AL>(out + (static_cast<int64_t>(blockIdx.y) * NW + c) * W, t);
     }
 }
 
-template <typename Src>
-static void launch_colsum_kernel(bool vec, bool al, dim3 grid, Src src, float* dst, int64_t M,
-                                 int64_t NW) {
+// Column-lanes for a matrix of NW accesses per row.
+static inline int colsum_lanes(int64_t NW) { return NW > 32 ? 64 : NW > 16 ? 32 : NW > 8 ? 16 : 8; }
+
+template <int W, bool AL, typename Src>
+static void launch_colsum_lanes(int cl, dim3 grid, Src src, float* dst, int64_t M, int64_t NW) {
     hipStream_t s = ctx().stream;
-    if (vec && al) hipLaunchKernelGGL((colsum_kernel<4, true, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW);
-    else if (vec)  hipLaunchKernelGGL((colsum_kernel<4, false, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW);
-    else           hipLaunchKernelGGL((colsum_kernel<1, false, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW);
+    switch (cl) {
+        case 8:  hipLaunchKernelGGL((colsum_kernel<W, AL, 8, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
+        case 16: hipLaunchKernelGGL((colsum_kernel<W, AL, 16, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
+        case 32: hipLaunchKernelGGL((colsum_kernel<W, AL, 32, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
+        default: hipLaunchKernelGGL((colsum_kernel<W, AL, 64, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
+    }
+}
+
+template <typename Src>
+static void launch_colsum_kernel(bool vec, bool al, int cl, dim3 grid, Src src, float* dst, int64_t M,
+                                 int64_t NW) {
+    if (vec && al) launch_colsum_lanes<4, true, Src>(cl, grid, src, dst, M, NW);
+    else if (vec)  launch_colsum_lanes<4, false, Src>(cl, grid, src, dst, M, NW);
+    else           launch_colsum_lanes<1, false, Src>(cl, grid, src, dst, M, NW);
 }
 
 template <typename Src>
@@ -91,11 +116,12 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N) {
     const Context& c = ctx();
     const bool vec = (N % 4 == 0);
     const int64_t NW = vec ? N / 4 : N;
-    const int64_t gx = ceil_div(NW, kWave);
+    const int cl = colsum_lanes(NW);
+    const int64_t gx = ceil_div(NW, cl);
     const int64_t target = static_cast<int64_t>(c.num_cus) * c.colsum_blocks_per_cu;
     int64_t bands = target / gx;
     if (bands < 1) bands = 1;
-    const int64_t min_rows = 64;             // at least 4 unrolled steps per wavefront
+    const int64_t min_rows = 4 * (4 * kBlock / cl);      // at least 4 unrolled steps per lane
     if (bands > ceil_div(M, min_rows)) bands = ceil_div(M, min_rows);
     if (bands > 1024) bands = 1024;
     float* dst = out;
@@ -107,13 +133,13 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N) {
         partial = static_cast<float*>(p);
         dst = partial;
     }
-    launch_colsum_kernel(vec, src.aligned() && aligned16(dst),
+    launch_colsum_kernel(vec, src.aligned() && aligned16(dst), cl,
                          dim3(static_cast<unsigned>(gx), static_cast<unsigned>(bands)), src, dst, M, NW);
     int st = check_launch("sum over axis 0");
     if (partial) {
         if (st == 0) {
             // second stage: column sums of the (bands, N) partials in one band
-            launch_colsum_kernel(vec, aligned16(partial) && aligned16(out),
+            launch_colsum_kernel(vec, aligned16(partial) && aligned16(out), cl,
                                  dim3(static_cast<unsigned>(gx), 1), PlainSrc{partial}, out, bands, NW);
             st = check_launch("sum over axis 0, stage 2");
         }

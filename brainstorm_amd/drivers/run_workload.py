@@ -1,0 +1,34 @@
+"""Runs training steps of one network workload on HipHandler: the program to put under a profiler.
+
+    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused]
+
+``fused`` is passed to the workload's builder ("1" for the fused entry points, "packed" for the
+LSTM's stacked recurrent product). One step = forward + backward + momentum update.
+"""
+import sys
+
+from brainstorm_amd import HipHandler
+from brainstorm_amd.drivers import configs
+from brainstorm_amd.drivers.net import MomentumStepper
+
+
+def main(argv):
+    name = argv[1]
+    steps = int(argv[2]) if len(argv) > 2 else 3
+    fused = argv[3] if len(argv) > 3 else ""
+    kw = {}
+    if fused:
+        kw["fused"] = "packed" if fused == "packed" else True
+    handler = HipHandler(seed=0)
+    net, data = getattr(configs, "build_" + name)(handler, **kw)
+    net.provide_external_data(data)
+    stepper = MomentumStepper(0.1, 0.9)
+    stepper.start(net)
+    for _ in range(steps):
+        stepper.run()
+    handler.synchronize()
+    print("%s: %d steps done" % (name, steps))
+
+
+if __name__ == "__main__":
+    main(sys.argv)
