@@ -40,6 +40,7 @@ SIGNATURES = {
     "bship_h2d": [_P, c_void_p, c_size_t],
     "bship_d2h": [c_void_p, _P, c_size_t],
     "bship_d2d": [_P, _P, c_size_t],
+    "bship_copy2d_f32": [_P, _I64, _P, _I64, _I64, _I64],
     "bship_fill_f32": [_P, c_float, c_size_t],
     "bship_binary_f32": [c_int, _P, _P, _P, c_size_t],
     "bship_mult_add_tt_f32": [_P, _P, _P, c_size_t],

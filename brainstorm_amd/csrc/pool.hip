@@ -132,6 +132,16 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
     }
 }
 
+// dst(rows, cols) with row pitch ld_dst = src(rows, cols) with row pitch ld_src; pitches in
+// elements. One workgroup per tile of kBlock columns of one row.
+__global__ __launch_bounds__(kBlock) void copy2d_kernel(const float* __restrict__ src, int64_t ld_src,
+                                                        float* __restrict__ dst, int64_t ld_dst,
+                                                        int64_t cols, unsigned tiles_per_row) {
+    const int64_t row = blockIdx.x / tiles_per_row;
+    const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
+    if (c < cols) dst[row * ld_dst + c] = src[row * ld_src + c];
+}
+
 int launch_fill(float* p, float val, size_t n) {
     if (n == 0) return 0;
     const size_t tiles = (n + kCopyTile - 1) / kCopyTile;
@@ -223,6 +233,24 @@ int bship_d2d(void* dst, const void* src, size_t nbytes) {
     else
         hipLaunchKernelGGL(copy_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, s, d, n);
     return check_launch("copy_kernel");
+}
+
+int bship_copy2d_f32(float* dst, int64_t ld_dst, const float* src, int64_t ld_src, int64_t rows,
+                     int64_t cols) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(rows >= 0 && cols >= 0);
+    if (rows == 0 || cols == 0) return 0;
+    BSHIP_REQUIRE_PTR(dst);
+    BSHIP_REQUIRE_PTR(src);
+    BSHIP_REQUIRE_F32_ALIGNED(dst);
+    BSHIP_REQUIRE_F32_ALIGNED(src);
+    BSHIP_REQUIRE_DIM(ld_dst >= cols && ld_src >= cols);
+    if (ld_dst == cols && ld_src == cols) return bship_d2d(dst, src, static_cast<size_t>(rows * cols) * 4);
+    const int64_t tiles_per_row = ceil_div(cols, kBlock);
+    BSHIP_REQUIRE_DIM(tiles_per_row * rows <= 0x7fffffff);
+    hipLaunchKernelGGL(copy2d_kernel, dim3(static_cast<unsigned>(tiles_per_row * rows)), dim3(kBlock), 0,
+                       ctx().stream, src, ld_src, dst, ld_dst, cols, static_cast<unsigned>(tiles_per_row));
+    return check_launch("copy2d");
 }
 
 int bship_fill_f32(float* mem, float val, size_t n) {

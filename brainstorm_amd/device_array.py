@@ -10,8 +10,10 @@ integer / slice / tuple indexing (step 1 only), ``reshape``, zero-sized and
 0-d arrays -- all returning views that alias the parent. The minimal array
 contract is the one brainstorm's DebugArray states (debug_handler.py:12-35).
 
-Only views that stay dense are representable. A slice that would need a row
-pitch (e.g. ``a[:, 1:3]`` of a wider matrix) raises NotImplementedError.
+Views that stay dense are plain DeviceArrays. A slice that needs a row pitch
+(e.g. ``a[:, 1:3]`` of a wider matrix) raises NotImplementedError unless the
+handler was created with ``pitched_views=True``, in which case it becomes a
+PitchedDeviceArray (see there).
 """
 from __future__ import annotations
 
@@ -188,12 +190,7 @@ class DeviceArray:
             raise IndexError("too many indices for array: array is %d-dimensional, "
                              "but %d were indexed" % (len(shape), len(key)))
         key = key + (slice(None),) * (len(shape) - len(key))
-        # element strides of the dense parent
-        strides = [0] * len(shape)
-        acc = 1
-        for ax in range(len(shape) - 1, -1, -1):
-            strides[ax] = acc
-            acc *= shape[ax]
+        strides = self._strides()
         offset = 0
         new_shape, new_strides = [], []
         for ax, k in enumerate(key):
@@ -217,14 +214,123 @@ class DeviceArray:
             else:
                 raise IndexError("DeviceArray indices must be integers or slices, not %s"
                                  % type(k).__name__)
-        new_shape = tuple(new_shape)
-        if _prod(new_shape) != 0:
-            expect = 1
-            for n, st in zip(reversed(new_shape), reversed(new_strides)):
-                if n != 1 and st != expect:
-                    raise NotImplementedError(
-                        "slicing %r out of shape %r needs a row pitch; DeviceArray views "
-                        "must stay dense" % (key, shape))
-                expect *= n
-        return DeviceArray(self.ptr + offset * ITEMSIZE if self.ptr else 0, new_shape,
-                           self._owner, self._handler)
+        return _view(self, offset, tuple(new_shape), new_strides, key)
+
+    def _strides(self):
+        """Element strides (dense, C order)."""
+        strides = [0] * len(self.shape)
+        acc = 1
+        for ax in range(len(self.shape) - 1, -1, -1):
+            strides[ax] = acc
+            acc *= self.shape[ax]
+        return strides
+
+    def _address(self):
+        return self.ptr
+
+    pitch = None      # dense: rows follow each other without gaps
+
+
+class PitchedViewError(TypeError):
+    """A row-pitched view reached code that needs a dense array."""
+
+
+class PitchedDeviceArray(DeviceArray):
+    """A view whose rows (the last axis) are contiguous but lie ``pitch`` elements apart.
+
+    brainstorm lets several layers write side by side into one hub and hands each of
+    them the feature slice ``hub[:, :, a:b]`` (buffer_structure.py:232-245); NumPy
+    addresses such a slice with strides. The kernels of this library work on dense
+    arrays, so a handler created with ``pitched_views=True`` moves a pitched operand
+    into a dense temporary before an operation and moves written operands back
+    (``bship_copy2d_f32``): correct everywhere, two extra passes over the operand.
+    Reading ``ptr`` raises, so that no code path can mistake the view for a dense array.
+    """
+
+    __slots__ = ("_base", "pitch")
+
+    def __init__(self, base, shape, pitch, owner, handler):
+        # DeviceArray.__init__ would assign self.ptr, which is read-only here
+        self._base = base
+        self.shape = shape
+        self.size = _prod(shape)
+        self.pitch = pitch
+        self._owner = owner
+        self._handler = handler
+
+    @property
+    def ptr(self):
+        raise PitchedViewError(
+            "row-pitched view of shape %r (pitch %d) used where a dense array is needed"
+            % (self.shape, self.pitch))
+
+    @property
+    def rows(self):
+        return self.size // self.shape[-1] if self.shape[-1] else 0
+
+    def _address(self):
+        return self._base
+
+    def _strides(self):
+        strides = [1] * len(self.shape)
+        acc = self.pitch
+        for ax in range(len(self.shape) - 2, -1, -1):
+            strides[ax] = acc
+            acc *= self.shape[ax]
+        return strides
+
+    def __repr__(self):
+        return "PitchedDeviceArray(shape=%r, pitch=%d, ptr=0x%x)" % (self.shape, self.pitch, self._base)
+
+    def __getitem__(self, key):
+        return self._getitem_general(key)
+
+    def reshape(self, *new_shape):
+        if len(new_shape) == 1 and not isinstance(new_shape[0], (int, np.integer)):
+            new_shape = tuple(new_shape[0])
+        new_shape = tuple(int(s) for s in new_shape)
+        if -1 in new_shape:
+            known = _prod(s for s in new_shape if s != -1)
+            if new_shape.count(-1) > 1 or known == 0 or self.size % known:
+                raise ValueError("cannot reshape array of size %d into shape %r" % (self.size, new_shape))
+            new_shape = tuple(self.size // known if s == -1 else s for s in new_shape)
+        if any(s < 0 for s in new_shape) or _prod(new_shape) != self.size:
+            raise ValueError("cannot reshape array of size %d into shape %r" % (self.size, new_shape))
+        if not new_shape or new_shape[-1] != self.shape[-1]:
+            raise NotImplementedError("a row-pitched view can only be reshaped over its leading axes "
+                                      "(%r -> %r)" % (self.shape, new_shape))
+        return PitchedDeviceArray(self._base, new_shape, self.pitch, self._owner, self._handler)
+
+
+def _view(parent, offset, shape, strides, key):
+    """The view of `parent` at element `offset` with the given shape and element strides:
+    dense if it is, row-pitched if the parent's handler allows that, else an error."""
+    base = parent._address()
+    ptr = base + offset * ITEMSIZE if base else 0
+    owner, handler = parent._owner, parent._handler
+    if _prod(shape) == 0 or not shape:
+        return DeviceArray(ptr if _prod(shape) else 0, shape, owner, handler)
+    cols = shape[-1]
+    # the leading axes must advance like the rows of one matrix: stride = pitch * rows below
+    pitch = None
+    below = 1
+    ok = cols == 1 or strides[-1] == 1
+    for n, st in zip(reversed(shape[:-1]), reversed(strides[:-1])):
+        if n != 1:
+            if pitch is None:
+                if st % below:
+                    ok = False
+                pitch = st // below
+            elif st != pitch * below:
+                ok = False
+        below *= n
+    if not ok:
+        raise NotImplementedError("slicing %r out of shape %r leaves more than a row pitch; "
+                                  "such views are not supported" % (key, parent.shape))
+    if pitch is None or pitch == cols:
+        return DeviceArray(ptr, shape, owner, handler)
+    if not getattr(handler, "pitched_views", False):
+        raise NotImplementedError(
+            "slicing %r out of shape %r needs a row pitch; create the handler with "
+            "pitched_views=True to work on such views through dense temporaries" % (key, parent.shape))
+    return PitchedDeviceArray(ptr, shape, pitch, owner, handler)

@@ -20,7 +20,7 @@ from . import _lib
 from ._lib import (ABS, ADD, ADD_IF, ADD_ST, COPY_IF, DIV, EL, EL_DERIV, FILL_IF, FMOD, LOG, MUL,
                    MULT_ADD_ST, MULT_ST, REL, REL_DERIV, SIGMOID, SIGMOID_DERIV, SIGN, SQRT, SUB,
                    TANH, TANH_DERIV)
-from .device_array import DeviceArray, _Block, _prod
+from .device_array import DeviceArray, PitchedDeviceArray, _Block, _prod
 from .handler_api import Handler
 
 SEED_RANGE = (0, 1000000000)   # brainstorm/randomness.py:16
@@ -75,7 +75,14 @@ class HipHandler(Handler):
 
     array_type = DeviceArray
 
-    def __init__(self, seed=None, device=0):
+    def __init__(self, seed=None, device=0, pitched_views=False):
+        # pitched_views: let slices that need a row pitch (feature slices of a hub with several
+        # sources, buffer_structure.py:232-245) exist as PitchedDeviceArray and serve operations
+        # on them through dense temporaries. Off by default: it puts a Python-level argument
+        # check in front of every operation.
+        self.pitched_views = bool(pitched_views)
+        if self.pitched_views:
+            self._install_pitched_wrappers()        # before the activation tables bind the methods
         super(HipHandler, self).__init__()
         self._lib = _lib.load()
         self._call(self._lib.bship_init(int(device)))
@@ -93,6 +100,67 @@ class HipHandler(Handler):
         self.__init__()
 
     # ------------------------------------------------------------- plumbing
+    # parameters an operation writes (everything else is only read); operations that are not
+    # listed (the fused extensions) are assumed to write every array they get
+    _WRITTEN = {
+        "copy_to": ("dest",), "copy_to_if": ("dest",), "fill": ("mem",), "fill_if": ("mem",),
+        "set_from_numpy": ("mem",), "get_numpy_copy": (), "is_fully_finite": (),
+        "split_add_tt": ("out_a", "out_b"), "generate_probability_mask": ("mask",),
+        "conv2d_forward_batch": ("outputs",),
+        "conv2d_backward_batch": ("in_deltas", "weight_deltas", "bias_deltas"),
+        "maxpool2d_forward_batch": ("outputs", "argmax"), "maxpool2d_backward_batch": ("in_deltas",),
+        "avgpool2d_forward_batch": ("outputs",), "avgpool2d_backward_batch": ("in_deltas",),
+        "sigmoid": ("y",), "tanh": ("y",), "rel": ("y",), "el": ("y",),
+        "sigmoid_deriv": ("dx",), "tanh_deriv": ("dx",), "rel_deriv": ("dx",), "el_deriv": ("dx",),
+        "dropout_forward": ("mask", "out"),
+        "batchnorm_forward": ("mu", "sigma", "sigma_b", "centered", "x_hat", "out"),
+        "batchnorm_backward": ("dgamma", "dbeta", "in_deltas"),
+    }
+
+    def _install_pitched_wrappers(self):
+        import functools
+        import inspect
+        cls = type(self)
+        for name in dir(cls):
+            if name.startswith("_") or name in ("allocate", "zeros", "ones", "create_from_numpy",
+                                                "synchronize", "device_info", "stack_adjacent"):
+                continue
+            fn = getattr(cls, name)
+            if not inspect.isfunction(fn):
+                continue
+            sig = inspect.signature(fn)
+            written = self._WRITTEN.get(name, ("out",) if "out" in sig.parameters else None)
+            setattr(self, name, functools.partial(self._dense_call, fn, sig, written))
+
+    def _copy2d(self, pitched, dense, to_dense):
+        cols = pitched.shape[-1]
+        args = ((dense.ptr, cols, pitched._base, pitched.pitch) if to_dense
+                else (pitched._base, pitched.pitch, dense.ptr, cols))
+        self._call(self._lib.bship_copy2d_f32(*args, pitched.rows, cols))
+
+    def _dense_call(self, fn, sig, written, *args, **kwargs):
+        """Runs fn with every row-pitched operand replaced by a dense temporary."""
+        bound = sig.bind(self, *args, **kwargs)
+        pitched = [(k, a) for k, a in bound.arguments.items() if type(a) is PitchedDeviceArray]
+        if not pitched:
+            return fn(self, *args, **kwargs)
+        temps = {}
+        for name, a in pitched:
+            key = (a._base, a.shape, a.pitch)
+            if key not in temps:                 # the same view twice (out is an input): one temporary
+                t = self.allocate(a.shape)
+                self._copy2d(a, t, True)
+                temps[key] = t
+            bound.arguments[name] = temps[key]
+        result = fn(*bound.args, **bound.kwargs)
+        done = set()
+        for name, a in pitched:
+            key = (a._base, a.shape, a.pitch)
+            if (written is None or name in written) and key not in done:
+                self._copy2d(a, temps[key], False)
+                done.add(key)
+        return result
+
     def _call(self, status):
         if status:
             _lib.raise_for_status(self._lib, status)

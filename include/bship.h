@@ -90,6 +90,13 @@ int bship_h2d(void* dst, const void* src_host, size_t nbytes);
 int bship_d2h(void* dst_host, const void* src, size_t nbytes);
 /* copy_to (numpy 47-52, pycuda 83-85). */
 int bship_d2d(void* dst, const void* src, size_t nbytes);
+/* Copy between row-pitched matrices: dst(rows, cols) with ld_dst elements from one
+ * row to the next = src(rows, cols) with ld_src. This is how a feature slice of a
+ * hub that several layers write side by side (buffer_structure.py 232-245), which
+ * NumPy addresses with strides, is moved into and out of the dense form that the
+ * kernels work on. */
+int bship_copy2d_f32(float* dst, int64_t ld_dst, const float* src, int64_t ld_src,
+                     int64_t rows, int64_t cols);
 /* fill (numpy 57-58, pycuda 93-94). */
 int bship_fill_f32(float* mem, float val, size_t n);
 
