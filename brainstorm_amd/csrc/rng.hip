@@ -21,7 +21,11 @@
 // convert the words that became visible at the previous barrier. Measured on
 // MI355X: 1.5 ns per double (a 100x1200 dropout mask in 0.16 ms); a minimal
 // LDS-read / write / barrier step of a 1024-lane workgroup costs 0.13 us there,
-// which bounds this single-stream design at roughly 0.4 ns per double.
+// which bounds this single-stream design at roughly 0.4 ns per double. (A variant
+// in which ONE wavefront generates 10 words per lane without any barrier, with
+// the others converting behind it through counters in LDS, was measured at
+// 4.4 ns per double: the address and twist arithmetic of a whole step then runs
+// on a single SIMD.)
 #include <cstdlib>
 #include <deque>
 #include <mutex>
@@ -334,14 +338,20 @@ static int prefetch_flush(bool restore_position, bool wrong_guess = false) {
     return st;
 }
 
-// Enqueues the draw of one mask on the second stream and appends it to the queue.
+// Enqueues the draw of one mask on the second stream and appends it to the queue. Once the
+// draw is enqueued the entry is queued in every case: it records how far the generator has run.
 static int prefetch_schedule(MaskPrefetch e, bool wait_consumed) {
-    if (wait_consumed) BSHIP_HIP(hipStreamWaitEvent(g_side, e.consumed, 0));
+    if (wait_consumed && hipStreamWaitEvent(g_side, e.consumed, 0) != hipSuccess) {
+        // cannot order behind the reader of the staging buffer: wait for it on the host instead
+        int st = check_hip(hipStreamSynchronize(ctx().stream), "hipStreamSynchronize");
+        if (st != 0) { free_entry(e); return st; }
+    }
     hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, g_side, g_state, e.staging, e.n, e.p,
                        e.before);
     int st = check_launch("mask prefetch");
     if (st != 0) { free_entry(e); return st; }
-    BSHIP_HIP(hipEventRecord(e.ready, g_side));
+    if (hipEventRecord(e.ready, g_side) != hipSuccess)
+        (void)hipStreamSynchronize(g_side);      // no event to wait for later: finish the draw now
     g_fifo.push_back(e);
     return 0;
 }
