@@ -9,24 +9,30 @@
 // The generator is treated as one linear stream of raw words r[0], r[1], ...:
 // the 624 words of the current block are r[0..623] and every later word follows
 // from
-//     r[n] = r[n-227] ^ T(n-624),      T(m) = twist(r[m], r[m+1])
+//     r[n] = r[n-227] ^ T(r[n-624], r[n-623]),     T = the MT19937 twist
 // (the block-wise regeneration of the MT19937 reference code, unrolled). Words
 // closer than 227 apart are independent, so a step of 227 lanes would do; but
 // each step costs an LDS round trip and a workgroup barrier, which is what the
-// kernel's time consists of. Substituting the recurrence into itself twice,
-//     r[n] = r[n-681] ^ T(n-624) ^ T(n-851) ^ T(n-1078),
-// makes every operand at least 623 words old, so one step can produce 623
-// consecutive words (three twists per word instead of one, 2.7 times fewer
-// steps). While the generator lanes run a step, the remaining lanes temper and
-// convert the words that became visible at the previous barrier. Measured on
-// MI355X: 1.5 ns per double (a 100x1200 dropout mask in 0.16 ms); a minimal
-// LDS-read / write / barrier step of a 1024-lane workgroup costs 0.13 us there,
-// which bounds this single-stream design at roughly 0.4 ns per double. (A variant
-// in which ONE wavefront generates 10 words per lane without any barrier, with
-// the others converting behind it through counters in LDS, was measured at
-// 4.4 ns per double: the address and twist arithmetic of a whole step then runs
-// on a single SIMD.)
+// serial kernel's time consists of. Two properties shorten it:
+//  * T is linear over GF(2) (its OR joins disjoint bit fields), so substituting
+//    the recurrence into itself twice collapses into ONE twist,
+//        r[n] = r[n-681] ^ T(r[n-624]^r[n-851]^r[n-1078], r[n-623]^r[n-850]^r[n-1077]),
+//    in which every operand is at least 623 words old: one step produces 623
+//    consecutive words (2.7 times fewer steps) for the price of 4 more XORs;
+//  * the serial kernel only EXTENDS THE STREAM and stores raw words; tempering,
+//    pairing into 53-bit doubles and the compare with p run afterwards in an
+//    ordinary data-parallel kernel over the whole device.
+// Measured on MI355X: 0.72 ns per double (a 100x1200 dropout mask in 0.09 ms).
+// History of the serial part: block-wise three-phase twist 2.25 ns per double;
+// 227-word steps with the conversion in the same workgroup 1.48; 623-word steps
+// with register-cached operands and separate conversion wavefronts 1.31; raw
+// words only 1.15; all LDS reads of a step issued together 0.85; one twist 0.72.
+// A minimal LDS-read / write / barrier step of such a workgroup costs 0.13 us,
+// which bounds the single-stream design near 0.4 ns per double. (A variant in
+// which ONE wavefront generates 10 words per lane without any barrier was
+// measured at 4.4 ns per double: a whole step's arithmetic on a single SIMD.)
 #include <cstdlib>
+#include <type_traits>
 #include <deque>
 #include <mutex>
 #include <utility>
@@ -63,7 +69,7 @@ __device__ __forceinline__ uint32_t mt_temper(uint32_t y) {
 }
 
 // Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for
-// the wavefront's outstanding GLOBAL stores (the mask being written), which
+// the wavefront's outstanding GLOBAL stores (the raw words being written), which
 // would put a memory round trip into the serial chain.
 __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -72,103 +78,99 @@ __device__ __forceinline__ void lds_barrier() {
 constexpr int kLag = kMtN - kMtM;             // 227
 constexpr int kWide = kMtN - 1;               // 623 words per wide step
 constexpr int kWideHistory = kMtN + 2 * kLag; // 1078: oldest word a wide step reads is n-1078
-constexpr int kRing = 4096;                   // LDS ring of raw words (power of two)
-constexpr unsigned kRingMask = kRing - 1;
-constexpr int kRngThreads = 1024;
-constexpr int kGenLanes = 640;                // lanes 0..622 generate one word per step,
-                                              // lanes 640..1023 temper and convert
-constexpr int kConLanes = kRngThreads - kGenLanes;
-static_assert(kGenLanes >= kWide && kGenLanes % kWave == 0, "generator lanes cover a step");
-static_assert(kWideHistory + 2 * kWide + 2 <= kRing, "ring holds history, a step and the consumers' lag");
 
-// Draws n (> 0) 53-bit doubles from the stream, in order, and hands double number
-// i to sink(i, k) as the integer k = value * 2^53; leaves the state as numpy's
-// RandomState would have it (whole blocks regenerated, position inside the last
-// one). One workgroup of kRngThreads threads; every control decision is the same
-// in all threads, so the barriers are reached uniformly.
-// If `before` is not null it receives the stream position (key, pos) as found.
-template <typename Sink>
-__device__ __forceinline__ void mt_generate(RngState* st, size_t n, Sink sink, RngState* before = nullptr) {
-    __shared__ uint32_t ring[kRing];
+constexpr int kRawThreads = 640;              // lanes 0..622 generate one word per wide step
+static_assert(kRawThreads >= kWide && kRawThreads % kWave == 0, "generator lanes cover a step");
+
+// raw[0..nw) = the next nw words of the stream r[pos0 .. pos0+nw); state left as numpy leaves it.
+//
+// LDS holds the last kWin = 2048 words twice: word n lives in slots (n mod kWin) and
+// (n mod kWin) + kWin. A step reads words n-1078 .. n-623 relative to its own word; starting
+// from slot (have mod kWin) + kWin - 1078 + lane all of them sit at fixed positive distances,
+// never wrap, and are addressed by the constant offsets of the LDS instructions (no index
+// arithmetic per load). The 623 slots a step writes and the 1078 it reads are disjoint modulo
+// kWin (623 + 1078 <= 2048), so one barrier per step still suffices.
+constexpr int kWin = 2048;
+static_assert(kWide + kWideHistory <= kWin, "a step's reads and writes must not alias");
+
+__global__ __launch_bounds__(kRawThreads) void mt_raw_kernel(RngState* st, uint32_t* __restrict__ raw,
+                                                             size_t nw, RngState* before) {
+    __shared__ uint32_t win[2 * kWin];
     const unsigned t = threadIdx.x;
-    for (unsigned i = t; i < kMtN; i += kRngThreads) ring[i] = st->key[i];
-    const size_t pos0 = static_cast<size_t>(st->pos);        // 0..624, next unread word
+    for (unsigned i = t; i < kMtN; i += kRawThreads) {
+        const uint32_t v = st->key[i];
+        win[i] = v;
+        win[i + kWin] = v;
+    }
+    const size_t pos0 = static_cast<size_t>(st->pos);
     if (before != nullptr) {
-        for (unsigned i = t; i < kMtN; i += kRngThreads) before->key[i] = ring[i];
+        for (unsigned i = t; i < kMtN; i += kRawThreads) before->key[i] = st->key[i];
         if (t == 0) before->pos = static_cast<int32_t>(pos0);
     }
     __syncthreads();
-    const size_t end_word = pos0 + 2 * n;                     // first word NOT consumed
-    const size_t gen_end = (end_word + kMtN - 1) / kMtN * kMtN;   // whole blocks
-    size_t have = kMtN;                                       // words r[0..have) exist and are visible
-    size_t next_word = pos0;                                  // first unconsumed word
-    size_t done = 0;                                          // doubles emitted
-    const bool generator = t < kGenLanes;
-    // number of complete pairs of words below `limit` that are still wanted
-    auto pairs_below = [&](size_t limit) -> size_t {
-        size_t pairs = limit > next_word ? (limit - next_word) / 2 : 0;
-        return pairs < n - done ? pairs : n - done;
-    };
-    // lane `lane` of `lanes` converts its share of the next `pairs` pairs
-    auto convert = [&](size_t pairs, unsigned lane, unsigned lanes) {
-        for (size_t j = lane; j < pairs; j += lanes) {
-            const unsigned w = static_cast<unsigned>(next_word) + 2 * static_cast<unsigned>(j);
-            const uint32_t w0 = mt_temper(ring[w & kRingMask]);
-            const uint32_t w1 = mt_temper(ring[(w + 1) & kRingMask]);
-            sink(done + j, (static_cast<uint64_t>(w0 >> 5) << 26) | static_cast<uint64_t>(w1 >> 6));
-        }
-    };
-    while (have < gen_end) {
-        const unsigned h = static_cast<unsigned>(have);       // only used modulo the ring size
-        const bool wide = have >= kWideHistory;
-        const size_t pairs = pairs_below(have);
-        if (generator) {
-            const unsigned i = h + t;
-            if (wide) {
-                if (t < kWide) {
-                    // seven independent loads, three independent twists
-                    const uint32_t c = ring[(i - 3 * kLag) & kRingMask];
-                    const uint32_t a0 = ring[(i - kMtN) & kRingMask], b0 = ring[(i - kMtN + 1) & kRingMask];
-                    const uint32_t a1 = ring[(i - kMtN - kLag) & kRingMask], b1 = ring[(i - kMtN - kLag + 1) & kRingMask];
-                    const uint32_t a2 = ring[(i - kMtN - 2 * kLag) & kRingMask], b2 = ring[(i - kMtN - 2 * kLag + 1) & kRingMask];
-                    ring[i & kRingMask] = (c ^ mt_twist(a0, b0)) ^ (mt_twist(a1, b1) ^ mt_twist(a2, b2));
-                }
-            } else if (t < kLag) {                            // the first two steps: plain recurrence
-                ring[i & kRingMask] = ring[(i - kLag) & kRingMask] ^
-                                      mt_twist(ring[(i - kMtN) & kRingMask], ring[(i - kMtN + 1) & kRingMask]);
+    const size_t end_word = pos0 + nw;
+    const size_t gen_end = (end_word + kMtN - 1) / kMtN * kMtN;
+    for (size_t i = pos0 + t; i < kMtN && i < end_word; i += kRawThreads) raw[i - pos0] = win[i];
+    size_t have = kMtN;
+    unsigned hm = kMtN;                                   // have mod kWin
+    // raw slot of word `have` (uniform; lane t adds t); words at or beyond end_word are not stored
+    uint32_t* out = raw + (kMtN - pos0);
+    // One step: lanes below `step` compute word have + t (all LDS reads are issued together),
+    // store it twice into the window and once into raw, then everybody meets at the barrier.
+    auto advance = [&](auto wide_tag) {
+        constexpr bool wide = decltype(wide_tag)::value;
+        constexpr unsigned step = wide ? kWide : kLag;
+        if (t < step) {
+            // slot of word (have + t - kWideHistory), in the upper copy
+            const uint32_t* p = win + (hm + kWin - kWideHistory) + t;
+            uint32_t v;
+            if constexpr (wide) {
+                const uint32_t a2 = p[0], b2 = p[1];
+                const uint32_t a1 = p[kWideHistory - kMtN - kLag], b1 = p[kWideHistory - kMtN - kLag + 1];
+                const uint32_t c = p[kWideHistory - 3 * kLag];
+                const uint32_t a0 = p[kWideHistory - kMtN], b0 = p[kWideHistory - kMtN + 1];
+                // the twist is linear over GF(2) (its OR joins disjoint bit fields), so the three
+                // twists of the wide step are one twist of the XORed operands
+                v = c ^ mt_twist(a0 ^ a1 ^ a2, b0 ^ b1 ^ b2);
+            } else {
+                v = p[kWideHistory - kLag] ^ mt_twist(p[kWideHistory - kMtN], p[kWideHistory - kMtN + 1]);
             }
-        } else {
-            convert(pairs, t - kGenLanes, kConLanes);         // words below `have` are visible
+            const unsigned x = (hm + t) & (kWin - 1);
+            win[x] = v;
+            win[x + kWin] = v;
+            const size_t rest = end_word > have ? end_word - have : 0;       // uniform
+            if (t < (rest < step ? static_cast<unsigned>(rest) : step)) out[t] = v;
         }
-        next_word += 2 * pairs;
-        done += pairs;
-        have += wide ? kWide : kLag;
+        have += step;
+        hm = (hm + step) & (kWin - 1);
+        out += step;
         lds_barrier();
-    }
-    convert(pairs_below(have), t, kRngThreads);               // whatever is left, all lanes
+    };
+    while (have < gen_end && have < kWideHistory) advance(std::false_type());    // two plain steps
+    while (have < gen_end) advance(std::true_type());
     __syncthreads();
-    // numpy keeps the block that holds the last consumed word and the position inside it
-    const unsigned block0 = static_cast<unsigned>(gen_end - kMtN);
-    for (unsigned i = t; i < kMtN; i += kRngThreads) st->key[i] = ring[(block0 + i) & kRingMask];
-    if (t == 0) st->pos = static_cast<int32_t>(end_word - (gen_end - kMtN));
+    const size_t block0 = gen_end - kMtN;
+    for (unsigned i = t; i < kMtN; i += kRawThreads) st->key[i] = win[(block0 + i) & (kWin - 1)];
+    if (t == 0) st->pos = static_cast<int32_t>(end_word - block0);
 }
 
-// mask[i] = (next_double() < p) ? 1 : 0 for i in [0,n).
-__global__ __launch_bounds__(kRngThreads) void mt_mask_kernel(RngState* st, float* __restrict__ mask,
-                                                         size_t n, double p, RngState* before) {
-    // k / 2^53 < p  <=>  k < ceil(p * 2^53): p * 2^53 is exact in float64, so the reference's
-    // float64 compare of the stream's double with p becomes an integer compare.
+__device__ __forceinline__ uint64_t raw_to_k53(const uint32_t* __restrict__ raw, size_t i) {
+    const uint32_t w0 = mt_temper(raw[2 * i]), w1 = mt_temper(raw[2 * i + 1]);
+    return (static_cast<uint64_t>(w0 >> 5) << 26) | static_cast<uint64_t>(w1 >> 6);
+}
+__global__ __launch_bounds__(kBlock) void raw_to_mask_kernel(const uint32_t* __restrict__ raw,
+                                                             float* __restrict__ mask, size_t n, double p) {
     uint64_t threshold;
-    if (!(p > 0.0)) threshold = 0;                                   // p <= 0 or NaN: never
-    else if (p >= 1.0) threshold = ~static_cast<uint64_t>(0);        // every k is below 2^53
+    if (!(p > 0.0)) threshold = 0;
+    else if (p >= 1.0) threshold = ~static_cast<uint64_t>(0);
     else threshold = static_cast<uint64_t>(ceil(p * 9007199254740992.0));
-    mt_generate(st, n, [=](size_t i, uint64_t k) { mask[i] = (k < threshold) ? 1.0f : 0.0f; }, before);
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) mask[i] = raw_to_k53(raw, i) < threshold ? 1.0f : 0.0f;
 }
-
-// u[i] = next_double() for i in [0,n) (used by fill_gaussian, also to skip ahead).
-__global__ __launch_bounds__(kRngThreads) void mt_doubles_kernel(RngState* st, double* __restrict__ u,
-                                                            size_t n) {
-    mt_generate(st, n, [=](size_t i, uint64_t k) { u[i] = static_cast<double>(k) * (1.0 / 9007199254740992.0); });
+__global__ __launch_bounds__(kBlock) void raw_to_doubles_kernel(const uint32_t* __restrict__ raw,
+                                                                double* __restrict__ u, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) u[i] = static_cast<double>(raw_to_k53(raw, i)) * (1.0 / 9007199254740992.0);
 }
 
 // Legacy polar method (RandomState.standard_normal): trial t uses doubles
@@ -281,6 +283,7 @@ struct MaskPrefetch {
     size_t n;
     double p;
     float* staging;
+    uint32_t* raw;         // the 2n raw words of the draw (scratch of the entry's own)
     RngState* before;      // key and pos before this mask was drawn
     hipEvent_t ready;      // second stream: the mask is in staging
     hipEvent_t consumed;   // main stream: staging has been copied out
@@ -293,6 +296,21 @@ constexpr size_t kMaxPeriod = 16;
 static size_t g_min_period = 1;              // raised after a wrong guess, see prefetch_flush()
 constexpr size_t kMaxPrefetchFloats = size_t(1) << 26;   // per period: 256 MiB of staging at most
 
+// Enqueues mask[0..n) = (next n doubles of the stream < p) on `stream`; raw is scratch for 2n words.
+static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw) {
+    hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, stream, g_state, raw, 2 * n, before);
+    hipLaunchKernelGGL(raw_to_mask_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
+                       dim3(kBlock), 0, stream, raw, mask, n, p);
+}
+
+// Enqueues u[0..n) = the next n doubles of the stream on the main stream (raw: scratch for 2n words).
+static void launch_doubles(double* u, size_t n, uint32_t* raw) {
+    hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, ctx().stream, g_state, raw, 2 * n,
+                       static_cast<RngState*>(nullptr));
+    hipLaunchKernelGGL(raw_to_doubles_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
+                       dim3(kBlock), 0, ctx().stream, raw, u, n);
+}
+
 static bool prefetch_enabled() {
     static const bool on = [] {
         const char* e = getenv("BSHIP_RNG_PREFETCH");
@@ -303,6 +321,7 @@ static bool prefetch_enabled() {
 
 static void free_entry(MaskPrefetch& e) {
     if (e.staging) pool_free_raw(e.staging);
+    if (e.raw) pool_free_raw(e.raw);
     if (e.before) pool_free_raw(e.before);
     if (e.ready) (void)hipEventDestroy(e.ready);
     if (e.consumed) (void)hipEventDestroy(e.consumed);
@@ -346,8 +365,7 @@ static int prefetch_schedule(MaskPrefetch e, bool wait_consumed) {
         int st = check_hip(hipStreamSynchronize(ctx().stream), "hipStreamSynchronize");
         if (st != 0) { free_entry(e); return st; }
     }
-    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, g_side, g_state, e.staging, e.n, e.p,
-                       e.before);
+    launch_mask(g_side, e.staging, e.n, e.p, e.before, e.raw);
     int st = check_launch("mask prefetch");
     if (st != 0) { free_entry(e); return st; }
     if (hipEventRecord(e.ready, g_side) != hipSuccess)
@@ -380,8 +398,11 @@ static void prefetch_maybe_start() {
         e.p = req.second;
         void* a = nullptr;
         void* b = nullptr;
+        void* r = nullptr;
         bool ok = pool_alloc_raw(e.n * sizeof(float), &a) == 0;
         e.staging = static_cast<float*>(a);
+        ok = ok && pool_alloc_raw(2 * e.n * sizeof(uint32_t), &r) == 0;
+        e.raw = static_cast<uint32_t*>(r);
         ok = ok && pool_alloc_raw(sizeof(RngState), &b) == 0;
         e.before = static_cast<RngState*>(b);
         ok = ok && hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) == hipSuccess;
@@ -408,9 +429,12 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
         int st = prefetch_flush(true, true);
         if (st != 0) return st;
     }
-    hipLaunchKernelGGL(mt_mask_kernel, dim3(1), dim3(kRngThreads), 0, ctx().stream, g_state, mask, n, p,
-                       static_cast<RngState*>(nullptr));
-    int st = check_launch("generate_probability_mask");
+    void* raw = nullptr;
+    int st = pool_alloc_raw(2 * n * sizeof(uint32_t), &raw);
+    if (st != 0) return st;
+    launch_mask(ctx().stream, mask, n, p, nullptr, static_cast<uint32_t*>(raw));
+    st = check_launch("generate_probability_mask");
+    pool_free_raw(raw);               // its next owner runs on this stream, after the two kernels
     if (st == 0 && prefetch_enabled()) {
         g_history.emplace_back(n, p);
         prefetch_maybe_start();
@@ -583,8 +607,12 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
         st = pool_alloc_raw(2 * trials * sizeof(double), &up);
         if (st != 0) break;
         double* u = static_cast<double*>(up);
+        void* rawp = nullptr;
+        st = pool_alloc_raw(4 * trials * sizeof(uint32_t), &rawp);
+        if (st != 0) { pool_free_raw(up); break; }
+        uint32_t* raw = static_cast<uint32_t*>(rawp);
         hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, s, g_state, snap);
-        hipLaunchKernelGGL(mt_doubles_kernel, dim3(1), dim3(kRngThreads), 0, s, g_state, u, 2 * trials);
+        launch_doubles(u, 2 * trials, raw);
         hipLaunchKernelGGL(gauss_polar_kernel, dim3(1), dim3(kBlock), 0, s, g_state, u, trials, out, n,
                            produced, mean, stdv, result);
         st = check_launch("fill_gaussian");
@@ -595,11 +623,13 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
             if (used < trials) {
                 // rewind: restore the snapshot and skip exactly 2*used doubles
                 hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, s, snap, g_state);
-                if (used > 0)
-                    hipLaunchKernelGGL(mt_doubles_kernel, dim3(1), dim3(kRngThreads), 0, s, g_state, u, 2 * used);
+                if (used > 0)      // only the position matters: the words go to the scratch again
+                    hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, s, g_state, raw, 4 * used,
+                                       static_cast<RngState*>(nullptr));
                 st = check_launch("fill_gaussian rewind");
             }
         }
+        pool_free_raw(rawp);
         pool_free_raw(up);
     }
     pool_free_raw(snap_p);
