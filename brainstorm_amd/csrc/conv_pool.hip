@@ -14,6 +14,7 @@
 #pragma clang fp contract(off)
 
 #include <cfloat>
+#include <map>
 
 #include "common.h"
 
@@ -191,6 +192,87 @@ __global__ __launch_bounds__(kBlock) void im2col_wt(const float* __restrict__ in
     im2col_body<W, AL, true>(in, col, n, pl);
 }
 
+// im2col through LDS. A workgroup produces one band of an image's col matrix: `band` consecutive
+// floats (a multiple of 4), i.e. a few output rows. The image rows those output rows look at are
+// staged once in LDS, zero-padded on all sides, so that every col element is an unconditional
+// LDS read at (oy_rel*sh + ky) * wpc + ox*sw*c + (kx*c + ch); the band is then written with one
+// 128-bit store per lane and iteration. Each input element is read from global memory once per
+// band instead of once per col element, which leaves the vector memory path to the stores.
+// Two LDS tiles alternate, so consecutive images of a workgroup need one barrier each.
+struct BandPlan {
+    ImgGeom g;
+    uint32_t band;         // col floats per band
+    uint32_t per_image;    // oh*ow*kh*kw*c
+    int tile_rows;         // most image rows a band looks at
+    int wpc;               // (w + 2*pad) * c : LDS row pitch
+    FastDiv d_k, d_ow, d_kwc, d_wpc, d_owk;
+};
+
+template <int W, bool WT>
+__global__ __launch_bounds__(kBlock) void im2col_band(const float* __restrict__ in, float* __restrict__ col,
+                                                      int64_t n, BandPlan pl) {
+    extern __shared__ float band_tile[];
+    const ImgGeom& g = pl.g;
+    const int tid = static_cast<int>(threadIdx.x);
+    const uint32_t first = blockIdx.x * pl.band;
+    const uint32_t len = pl.per_image - first < pl.band ? pl.per_image - first : pl.band;
+    const int oy_first = static_cast<int>(pl.d_owk.div(first));
+    const int oy_last = static_cast<int>(pl.d_owk.div(first + len - 1));
+    const int iy0 = oy_first * g.sh - g.pad;
+    const int tile_len = ((oy_last - oy_first) * g.sh + g.kh) * pl.wpc;
+    const int tile_cap = pl.tile_rows * pl.wpc;
+    const int wc = g.w * g.c, padc = g.pad * g.c, swc = g.sw * g.c;
+    const uint32_t kwc = static_cast<uint32_t>(g.kw * g.c);
+    const int64_t in_img = static_cast<int64_t>(g.h) * wc;
+    int buf = 0;
+    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+        float* t = band_tile + buf * tile_cap;
+        const float* src = in + img * in_img;
+        for (int e = tid * W; e < tile_len; e += kBlock * W) {
+            uint32_t row, cx;
+            pl.d_wpc.divmod(static_cast<uint32_t>(e), row, cx);
+            const int iy = iy0 + static_cast<int>(row), xo = static_cast<int>(cx) - padc;
+            const bool inside = iy >= 0 && iy < g.h && xo >= 0 && xo < wc;
+            if constexpr (W == 4) {
+                f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (inside) v = *reinterpret_cast<const f4u*>(src + iy * wc + xo);
+                *reinterpret_cast<f4*>(t + e) = v;
+            } else {
+                t[e] = inside ? src[iy * wc + xo] : 0.0f;
+            }
+        }
+        __syncthreads();
+        float* dst = col + img * static_cast<int64_t>(pl.per_image) + first;
+        for (uint32_t s = static_cast<uint32_t>(tid) * 4; s < len; s += kBlock * 4) {
+            uint32_t opix, kk, oy, ox, ky, r;
+            pl.d_k.divmod(first + s, opix, kk);
+            pl.d_ow.divmod(opix, oy, ox);
+            pl.d_kwc.divmod(kk, ky, r);
+            uint32_t oyr = oy - static_cast<uint32_t>(oy_first);
+            f4 v;
+            if constexpr (W == 4) {
+                v = *reinterpret_cast<const f4*>(t + (oyr * g.sh + ky) * pl.wpc + ox * swc + r);
+            } else {
+                // the four elements may straddle kernel rows, output pixels and output rows
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[j] = t[(oyr * g.sh + ky) * pl.wpc + ox * swc + r];
+                    if (++r == kwc) {
+                        r = 0;
+                        if (++ky == static_cast<uint32_t>(g.kh)) {
+                            ky = 0;
+                            if (++ox == static_cast<uint32_t>(g.ow)) { ox = 0; ++oyr; }
+                        }
+                    }
+                }
+            }
+            if constexpr (WT) vstore_writeonly<4>(dst + s, v);
+            else *reinterpret_cast<f4u*>(dst + s) = v;
+        }
+        buf ^= 1;
+    }
+}
+
 // in_deltas[img, y, x, ch] += sum over covering (oy, ox), in scan order, of
 // col[(img, oy, ox), (y - (oy*sh-pad), x - (ox*sw-pad), ch)]               (_cpuop 295-309)
 // One lane per W channels of one input pixel; lanes_per_image = h*w*cv.
@@ -224,6 +306,204 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
             }
         }
         img_store<W, AL>(q, acc);
+    }
+}
+
+// col2im through LDS, for narrow channel counts: there a lane's 4*c-byte pieces of the col
+// matrix lie kh*kw*c floats apart and every cache line would be fetched several times.
+// A workgroup walks down a band of image rows, `rows` of them per phase. The col rows (oy) that
+// cover the rows of a phase are one contiguous range of the col matrix; they live in a ring of
+// `ring` col rows in LDS (col row oy in slot oy mod ring). While the lanes gather the terms of
+// the current phase from LDS (one lane per input element, same scan order as above), the col
+// rows that the next phase adds are already on their way into registers; they replace the
+// oldest slots after the phase. Inside a band every col element is therefore read once, with
+// coalesced 128-bit loads; bands of one image overlap by the col rows that cover both.
+// Bands of one image have the same workgroup index modulo 8 and follow each other, so with
+// workgroups dealt round-robin to the 8 XCDs they meet in one L2.
+// Needs ow*kh*kw*c (floats per col row) to be a multiple of 4.
+constexpr int kCol2imThreads = 512;  // few workgroups fit a compute unit's LDS: make them large
+constexpr int kCol2imPrefetch = 5;      // 128-bit loads in flight per lane
+constexpr int kCol2imOutsPerLane = 2;   // image elements of one phase per lane, at most
+constexpr uint32_t kXcds = 8;
+
+struct Col2imBandPlan {
+    ImgGeom g;
+    int rows;              // image rows per phase
+    int phases;            // phases per workgroup
+    int bands;             // workgroups per image
+    int ring;              // col rows held in LDS
+    uint32_t owk;          // ow*kh*kw*c : floats per col row
+    FastDiv d_bands, d_wc, d_w, d_sh, d_sw, d_ring, d_owk4;
+};
+
+// Copies col rows [lo, hi) of one image into their ring slots, kBatch loads in flight per lane.
+template <int kBatch>
+__device__ __forceinline__ void col2im_stage(const float* __restrict__ cimg, float* __restrict__ tile,
+                                             int lo, int hi, const Col2imBandPlan& pl) {
+    const int count4 = hi > lo ? (hi - lo) * static_cast<int>(pl.owk / 4) : 0;
+    const float* src = cimg + static_cast<int64_t>(lo) * pl.owk;
+    for (int q0 = static_cast<int>(threadIdx.x); q0 < count4; q0 += kCol2imThreads * kBatch) {
+        f4 v[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int q = q0 + u * kCol2imThreads;
+            if (q < count4) v[u] = *reinterpret_cast<const f4u*>(src + static_cast<int64_t>(q) * 4);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int q = q0 + u * kCol2imThreads;
+            if (q < count4) {
+                uint32_t row, within;
+                pl.d_owk4.divmod(static_cast<uint32_t>(q), row, within);
+                const uint32_t slot = pl.d_ring.div(static_cast<uint32_t>(lo) + row);
+                const uint32_t s = static_cast<uint32_t>(lo) + row - slot * pl.d_ring.d;
+                *reinterpret_cast<f4*>(tile + s * pl.owk + within * 4) = v[u];
+            }
+        }
+    }
+}
+
+// KS > 0: kh = kw = KS with stride 1, known at compile time: the KS*KS reads of an element are
+// issued together (terms outside the col matrix read a clamped address and are not added).
+template <int KS>
+__global__ __launch_bounds__(kCol2imThreads) void col2im_band(const float* __restrict__ col,
+                                                      float* __restrict__ in_deltas, int64_t n,
+                                                      Col2imBandPlan pl) {
+    extern __shared__ float band_tile[];
+    const ImgGeom& g = pl.g;
+    const uint32_t lane_group = blockIdx.x / kXcds, xcd = blockIdx.x % kXcds;
+    uint32_t img_group, band;
+    pl.d_bands.divmod(lane_group, img_group, band);
+    const int64_t img = static_cast<int64_t>(img_group) * kXcds + xcd;
+    if (img >= n) return;
+    const int ybeg = static_cast<int>(band) * pl.rows * pl.phases;
+    const int yend = imin(ybeg + pl.rows * pl.phases, g.h);
+    const int kc = g.kh * g.kw * g.c, wc = g.w * g.c;
+    const int pitch = static_cast<int>(pl.owk);
+    const float* cimg = col + img * (static_cast<int64_t>(g.oh) * pl.owk);
+    float* dimg = in_deltas + img * (static_cast<int64_t>(g.h) * wc);
+    // Lane index o of a phase -> image element: within an image row the lanes are ordered channel
+    // first, then x, so that neighbouring lanes read LDS words kh*kw*c apart (an odd stride for
+    // RGB images: no bank conflicts) rather than runs of c words with gaps.
+    auto element_of = [&](int o) {
+        uint32_t yr, rem, xx, ch;
+        pl.d_wc.divmod(static_cast<uint32_t>(o), yr, rem);
+        pl.d_w.divmod(rem, ch, xx);
+        return static_cast<int>(yr * wc + xx * g.c + ch);
+    };
+    auto ring_slot = [&](int oy) {
+        return static_cast<int>(static_cast<uint32_t>(oy) - pl.d_ring.div(static_cast<uint32_t>(oy)) * pl.d_ring.d);
+    };
+
+    // col rows of the first phase; a lane's image elements are o = lane + u*kCol2imThreads of the phase
+    int p_lo, p_hi, unused;
+    cover_range(ybeg, g.pad, pl.d_sh, g.kh, g.oh, p_lo, unused);
+    cover_range(imin(ybeg + pl.rows, yend) - 1, g.pad, pl.d_sh, g.kh, g.oh, unused, p_hi);
+    float init[kCol2imOutsPerLane];     // in_deltas before the update, loaded a phase ahead
+    {
+        const int outs = (imin(ybeg + pl.rows, yend) - ybeg) * wc;
+        const float* drow = dimg + static_cast<int64_t>(ybeg) * wc;
+#pragma unroll
+        for (int u = 0; u < kCol2imOutsPerLane; ++u) {
+            const int o = static_cast<int>(threadIdx.x) + u * kCol2imThreads;
+            init[u] = o < outs ? drow[element_of(o)] : 0.0f;
+        }
+    }
+    col2im_stage<8>(cimg, band_tile, p_lo, p_hi, pl);
+    int have_hi = imax(p_hi, p_lo);     // col rows below have_hi have been loaded
+    __syncthreads();
+
+    for (int ya = ybeg; ya < yend; ya += pl.rows) {
+        const int yb = imin(ya + pl.rows, yend);
+        // what the next phase adds, into registers: col rows and the image rows' old values
+        int n_lo = p_lo, n_hi = p_hi, new_lo = 0, count4 = 0;
+        f4 pre[kCol2imPrefetch];
+        float init_next[kCol2imOutsPerLane];
+        if (yb < yend) {
+            cover_range(yb, g.pad, pl.d_sh, g.kh, g.oh, n_lo, unused);
+            cover_range(imin(yb + pl.rows, yend) - 1, g.pad, pl.d_sh, g.kh, g.oh, unused, n_hi);
+            new_lo = imax(have_hi, n_lo);
+            count4 = n_hi > new_lo ? (n_hi - new_lo) * static_cast<int>(pl.owk / 4) : 0;
+            const float* src = cimg + static_cast<int64_t>(new_lo) * pl.owk;
+#pragma unroll
+            for (int u = 0; u < kCol2imPrefetch; ++u) {
+                const int q = static_cast<int>(threadIdx.x) + u * kCol2imThreads;
+                if (q < count4) pre[u] = *reinterpret_cast<const f4u*>(src + static_cast<int64_t>(q) * 4);
+            }
+            const int outs_next = (imin(yb + pl.rows, yend) - yb) * wc;
+            const float* drow_next = dimg + static_cast<int64_t>(yb) * wc;
+#pragma unroll
+            for (int u = 0; u < kCol2imOutsPerLane; ++u) {
+                const int o = static_cast<int>(threadIdx.x) + u * kCol2imThreads;
+                init_next[u] = o < outs_next ? drow_next[element_of(o)] : 0.0f;
+            }
+        }
+        // this phase's image rows from LDS
+        const int outs = (yb - ya) * wc;
+        float* drow = dimg + static_cast<int64_t>(ya) * wc;
+#pragma unroll
+        for (int u = 0; u < kCol2imOutsPerLane; ++u) {
+            const int o = static_cast<int>(threadIdx.x) + u * kCol2imThreads;
+            if (o >= outs) break;
+            uint32_t yr, rem, xx, ch;
+            pl.d_wc.divmod(static_cast<uint32_t>(o), yr, rem);
+            pl.d_w.divmod(rem, ch, xx);
+            const int y = ya + static_cast<int>(yr), x = static_cast<int>(xx);
+            float acc = init[u];
+            if constexpr (KS > 0) {
+                // oy = y + pad - ky ascends as ky descends; the same for ox
+                float v[KS * KS];
+#pragma unroll
+                for (int a = 0; a < KS; ++a) {
+                    const int ky = KS - 1 - a;
+                    const int oy = imin(imax(y + g.pad - ky, p_lo), p_hi - 1);
+                    const float* trow = band_tile + ring_slot(oy) * pitch + ky * KS * g.c + static_cast<int>(ch);
+#pragma unroll
+                    for (int b = 0; b < KS; ++b) {
+                        const int kx = KS - 1 - b;
+                        const int ox = imin(imax(x + g.pad - kx, 0), g.ow - 1);
+                        v[a * KS + b] = trow[ox * kc + kx * g.c];
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < KS; ++a)
+#pragma unroll
+                    for (int b = 0; b < KS; ++b) {
+                        const int oy = y + g.pad - (KS - 1 - a), ox = x + g.pad - (KS - 1 - b);
+                        if (oy >= 0 && oy < g.oh && ox >= 0 && ox < g.ow) acc += v[a * KS + b];
+                    }
+            } else {
+                int oy0, oy1, ox0, ox1;
+                cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
+                cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
+                for (int oy = oy0; oy < oy1; ++oy) {
+                    const int ky = y - (oy * g.sh - g.pad);
+                    const float* trow = band_tile + ring_slot(oy) * pitch + ky * g.kw * g.c + ch;
+                    for (int ox = ox0; ox < ox1; ++ox) {
+                        const int kx = x - (ox * g.sw - g.pad);
+                        acc += trow[ox * kc + kx * g.c];
+                    }
+                }
+            }
+            drow[yr * wc + xx * g.c + ch] = acc;
+        }
+        if (yb >= yend) break;
+        __syncthreads();                 // every lane is done with the slots that are replaced now
+#pragma unroll
+        for (int u = 0; u < kCol2imPrefetch; ++u) {
+            const int q = static_cast<int>(threadIdx.x) + u * kCol2imThreads;
+            if (q < count4) {
+                uint32_t row, within;
+                pl.d_owk4.divmod(static_cast<uint32_t>(q), row, within);
+                *reinterpret_cast<f4*>(band_tile + ring_slot(new_lo + static_cast<int>(row)) * pitch + within * 4) = pre[u];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCol2imOutsPerLane; ++u) init[u] = init_next[u];
+        have_hi = imax(have_hi, n_hi);
+        p_lo = n_lo;
+        p_hi = n_hi;
+        __syncthreads();
     }
 }
 
@@ -501,6 +781,133 @@ static int check_geom(const char* fn, int64_t n, const ImgGeom& g) {
 
 static inline int conv_out(int in, int k, int pad, int stride) { return (in + 2 * pad - k) / stride + 1; }
 
+// Band size of im2col_band: about kBandFloats col floats, whole output rows when a row is a
+// multiple of 4 floats, fewer when the batch is small (to keep every compute unit busy), and such
+// that the two LDS tiles fit. Returns false when the geometry does not suit the banded kernel
+// (col rows of an image not a multiple of 4 floats in total, or image rows too wide for LDS).
+constexpr int64_t kBandFloats = 8192;
+constexpr int64_t kBandMinWorkgroups = 1024;
+constexpr size_t kBandLdsBytes = 64 * 1024;
+
+static bool plan_im2col_band(const ImgGeom& g, int64_t n, int64_t per_image, BandPlan* out) {
+    if (per_image % 4 != 0 || per_image > 0x7fffffff || per_image == 0) return false;
+    const int64_t owk = static_cast<int64_t>(g.ow) * g.kh * g.kw * g.c;
+    const int64_t wpc = (static_cast<int64_t>(g.w) + 2 * g.pad) * g.c;
+    auto tile_rows_of = [&](int64_t band) {
+        // output rows that `band` consecutive floats can touch, wherever they start
+        const int64_t span = owk % 4 == 0 ? band / owk : (band >= 2 ? (band - 2) / owk + 2 : 1);
+        return (span - 1) * g.sh + g.kh;
+    };
+    auto fits = [&](int64_t band) {
+        return 2 * static_cast<size_t>(tile_rows_of(band) * wpc) * sizeof(float) <= kBandLdsBytes;
+    };
+    int64_t band;
+    if (owk % 4 == 0) {
+        int64_t rows = ceil_div(kBandFloats, owk);
+        if (rows > g.oh) rows = g.oh;
+        while (rows > 1 && (ceil_div(g.oh, rows) * n < kBandMinWorkgroups || !fits(rows * owk))) rows = (rows + 1) / 2;
+        band = rows * owk;
+    } else {
+        band = kBandFloats;
+        while (band > 1024 && (ceil_div(per_image, band) * n < kBandMinWorkgroups || !fits(band))) band /= 2;
+    }
+    if (!fits(band)) return false;
+    out->g = g;
+    out->band = static_cast<uint32_t>(band);
+    out->per_image = static_cast<uint32_t>(per_image);
+    out->tile_rows = static_cast<int>(tile_rows_of(band));
+    out->wpc = static_cast<int>(wpc);
+    out->d_k = FastDiv(static_cast<uint32_t>(g.kh * g.kw * g.c));
+    out->d_ow = FastDiv(static_cast<uint32_t>(g.ow));
+    out->d_kwc = FastDiv(static_cast<uint32_t>(g.kw * g.c));
+    out->d_wpc = FastDiv(static_cast<uint32_t>(wpc));
+    out->d_owk = FastDiv(static_cast<uint32_t>(owk));
+    return true;
+}
+
+// Host mirror of cover_range().
+static void cover_range_host(int p, int pad, int stride, int k, int n_out, int* lo, int* hi) {
+    const int q = p + pad;
+    *hi = imin(q / stride + 1, n_out);
+    const int t = q - k + 1;
+    *lo = t <= 0 ? 0 : (t + stride - 1) / stride;
+}
+
+// Phases of `rows` image rows: the most col rows one phase needs (`ring`) and the most col rows
+// a phase adds to those of the phase before (`fresh`).
+static void col2im_phase_extent(const ImgGeom& g, int rows, int* ring, int* fresh) {
+    *ring = 0;
+    *fresh = 0;
+    int have_hi = 0;
+    for (int y0 = 0; y0 < g.h; y0 += rows) {
+        int lo, hi, unused;
+        cover_range_host(y0, g.pad, g.sh, g.kh, g.oh, &lo, &unused);
+        cover_range_host(imin(y0 + rows, g.h) - 1, g.pad, g.sh, g.kh, g.oh, &unused, &hi);
+        *ring = imax(*ring, hi - lo);
+        if (y0 > 0) *fresh = imax(*fresh, hi - imax(have_hi, lo));
+        have_hi = imax(have_hi, imax(hi, lo));
+    }
+}
+
+// col2im_band is used for fewer than 16 channels when the col rows are multiples of 4 floats and
+// a ring for at least one image row per phase fits half of a compute unit's LDS. A workgroup gets
+// as many phases as leave about kCol2imMinWorkgroups workgroups in the launch.
+constexpr size_t kCol2imLdsBytes = 80 * 1024;
+constexpr int64_t kCol2imMinWorkgroups = 1024;
+
+static bool plan_col2im_band(const ImgGeom& g, int64_t n, Col2imBandPlan* out, size_t* lds_bytes) {
+    if (g.c >= 16 || g.h == 0 || g.w == 0 || g.c == 0 || g.oh == 0 || g.ow == 0 || n == 0) return false;
+    const int64_t owk = static_cast<int64_t>(g.ow) * g.kh * g.kw * g.c;
+    if (owk % 4 != 0 || owk * g.oh > 0x7fffffff) return false;
+    int rows = 0, ring = 0;
+    for (int r = 1; r <= g.h; ++r) {
+        int rg, fresh;
+        col2im_phase_extent(g, r, &rg, &fresh);
+        if (static_cast<size_t>(rg) * owk * sizeof(float) > kCol2imLdsBytes ||
+            static_cast<int64_t>(fresh) * (owk / 4) > static_cast<int64_t>(kCol2imPrefetch) * kCol2imThreads ||
+            static_cast<int64_t>(r) * g.w * g.c > static_cast<int64_t>(kCol2imOutsPerLane) * kCol2imThreads)
+            break;
+        rows = r;
+        ring = rg;
+    }
+    if (rows == 0 || ring == 0) return false;
+    const int64_t all_phases = ceil_div(g.h, rows);
+    int64_t phases = n * all_phases / kCol2imMinWorkgroups;
+    if (phases < 1) phases = 1;
+    if (phases > all_phases) phases = all_phases;
+    out->g = g;
+    out->rows = rows;
+    out->phases = static_cast<int>(phases);
+    out->bands = static_cast<int>(ceil_div(all_phases, phases));
+    out->ring = ring;
+    out->owk = static_cast<uint32_t>(owk);
+    out->d_bands = FastDiv(static_cast<uint32_t>(out->bands));
+    out->d_wc = FastDiv(static_cast<uint32_t>(g.w * g.c));
+    out->d_w = FastDiv(static_cast<uint32_t>(g.w));
+    out->d_sh = FastDiv(static_cast<uint32_t>(g.sh));
+    out->d_sw = FastDiv(static_cast<uint32_t>(g.sw));
+    out->d_ring = FastDiv(static_cast<uint32_t>(ring));
+    out->d_owk4 = FastDiv(static_cast<uint32_t>(owk / 4));
+    *lds_bytes = static_cast<size_t>(ring) * owk * sizeof(float);
+    return true;
+}
+
+// Lets `kernel` use `bytes` of dynamic LDS (more than the default limit has to be asked for);
+// remembers what each kernel was granted.
+static bool allow_dynamic_lds_impl(const void* kernel, size_t bytes) {
+    static std::map<const void*, size_t> granted;
+    auto it = granted.find(kernel);
+    if (it != granted.end() && it->second >= bytes) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) != hipSuccess)
+        return false;
+    granted[kernel] = bytes;
+    return true;
+}
+template <typename K>
+static bool allow_dynamic_lds(K kernel, size_t bytes) {
+    return allow_dynamic_lds_impl(reinterpret_cast<const void*>(kernel), bytes);
+}
+
 }  // namespace bship
 
 using namespace bship;
@@ -552,6 +959,19 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
     BSHIP_REQUIRE_PTR(col);
     const bool write_through = static_cast<size_t>(total) >= (size_t(1) << 26);   // 256 MiB: beyond the last-level cache
     const int64_t per_image = static_cast<int64_t>(g.oh) * g.ow * kh * kw * c;
+    BandPlan bp;
+    if (plan_im2col_band(g, n, per_image, &bp)) {
+        const size_t lds = 2 * static_cast<size_t>(bp.tile_rows) * bp.wpc * sizeof(float);
+        const dim3 grid(static_cast<unsigned>(ceil_div(per_image, bp.band)), static_cast<unsigned>(n < 65535 ? n : 65535));
+        if (c % 4 == 0) {
+            if (write_through) hipLaunchKernelGGL((im2col_band<4, true>), grid, dim3(kBlock), lds, ctx().stream, in, col, n, bp);
+            else               hipLaunchKernelGGL((im2col_band<4, false>), grid, dim3(kBlock), lds, ctx().stream, in, col, n, bp);
+        } else {
+            if (write_through) hipLaunchKernelGGL((im2col_band<1, true>), grid, dim3(kBlock), lds, ctx().stream, in, col, n, bp);
+            else               hipLaunchKernelGGL((im2col_band<1, false>), grid, dim3(kBlock), lds, ctx().stream, in, col, n, bp);
+        }
+        return check_launch("im2col");
+    }
     if (c % 4 != 0 && per_image % 4 == 0 && per_image <= 0x7fffffff) {
         ImgPlan pl;
         pl.g = g;
@@ -585,6 +1005,26 @@ int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(col);
     BSHIP_REQUIRE_PTR(in_deltas);
+    Col2imBandPlan bp;
+    size_t lds = 0;
+    if (plan_col2im_band(g, n, &bp, &lds)) {
+        const int ks = (kh == kw && stride_h == 1 && stride_w == 1 && (kh == 3 || kh == 5)) ? kh : 0;
+        const int64_t groups = ceil_div(n, kXcds) * bp.bands;
+        if (groups * kXcds <= 0x7fffffff) {
+            const dim3 grid(static_cast<unsigned>(groups * kXcds));
+#define BSHIP_COL2IM_BAND(KS_)                                                                          \
+            if (ks == KS_ && allow_dynamic_lds(col2im_band<KS_>, lds)) {                                \
+                hipLaunchKernelGGL(col2im_band<KS_>, grid, dim3(kCol2imThreads), lds, ctx().stream, col,        \
+                                   in_deltas, n, bp);                                                   \
+                return check_launch("col2im");                                                          \
+            }
+            BSHIP_COL2IM_BAND(5)
+            BSHIP_COL2IM_BAND(3)
+            BSHIP_COL2IM_BAND(0)
+#undef BSHIP_COL2IM_BAND
+        }
+        (void)hipGetLastError();   // the attribute was refused: use the kernel without LDS
+    }
     BSHIP_LAUNCH_IMG(col2im_kernel, "col2im", static_cast<int64_t>(h) * w,
                      aligned16(col) && aligned16(in_deltas), col, in_deltas);
 }

@@ -660,6 +660,41 @@ def test_im2col_col2im_exact(hip, ref):
         assert_bit_equal(dind.get(), want, "col2im")
 
 
+# Geometries for the LDS-banded kernels: several bands per image, several phases per workgroup
+# (enough images that a workgroup walks down more than one group of image rows), strides,
+# col rows that are and are not multiples of 4 floats, few images (single-phase bands).
+BAND_CASES = [(260, 40, 32, 3, 5, 5, 2, (1, 1)), (210, 40, 256, 3, 3, 3, 1, (2, 2)), (1030, 28, 28, 1, 5, 5, 2, (1, 1)),
+              (9, 40, 32, 3, 5, 5, 2, (1, 1)), (130, 17, 12, 8, 3, 3, 0, (1, 1)), (70, 30, 30, 6, 3, 3, 1, (3, 1)),
+              (300, 19, 16, 12, 2, 2, 0, (2, 2)), (33, 15, 15, 32, 5, 5, 2, (1, 1)), (40, 11, 9, 5, 3, 3, 1, (1, 1)),
+              (20, 10, 10, 3, 3, 3, 1, (1, 1)), (20, 12, 10, 3, 3, 3, 1, (2, 1))]
+
+
+def test_im2col_col2im_banded_exact(hip, ref):
+    rng = np.random.RandomState(127)
+    lib = hip._lib
+    for n, h, w, c, kh, kw, pad, stride in BAND_CASES:
+        oh, ow = _out_size(h, kh, pad, stride[0]), _out_size(w, kw, pad, stride[1])
+        x = rand(rng, (n, h, w, c))
+        col = np.zeros((n, oh * ow, kh * kw * c), F32)
+        for i in range(n):
+            ref._im2col(x[i], kh, kw, pad, stride, col[i])
+        xd = hip.create_from_numpy(x)
+        cold = hip.allocate(col.shape)
+        hip.fill(cold, 7.0)
+        hip._call(lib.bship_im2col_nhwc_f32(xd.ptr, cold.ptr, n, h, w, c, kh, kw, pad, stride[0], stride[1]))
+        assert_bit_equal(cold.get(), col, "im2col %r" % ((n, h, w, c, kh, kw, pad, stride),))
+        cols = rand(rng, col.shape)
+        din = rand(rng, x.shape)
+        want = din.copy()
+        for i in range(n):
+            ref._col2im(cols[i], kh, kw, pad, stride, want[i])
+        dind = hip.create_from_numpy(din)
+        colsd = hip.create_from_numpy(cols)
+        hip._call(lib.bship_col2im_nhwc_f32(colsd.ptr, dind.ptr, n, h, w, c, kh, kw, pad,
+                                            stride[0], stride[1]))
+        assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, kh, kw, pad, stride),))
+
+
 # ---------------------------------------------------------- views of one buffer
 def test_ops_on_unaligned_views(hip, ref):
     # Layer buffers are slices of one flat array (buffers.py:79-83) and may start at any element,
