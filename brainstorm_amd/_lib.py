@@ -33,6 +33,10 @@ SIGNATURES = {
     "bship_device_info": [ctypes.c_char_p, c_size_t, POINTER(c_int)],
     "bship_event_record": [c_int],
     "bship_event_elapsed_ms": [c_int, c_int, POINTER(c_float)],
+    "bship_graph_begin": [],
+    "bship_graph_end": [POINTER(c_int)],
+    "bship_graph_launch": [c_int],
+    "bship_graph_destroy": [c_int],
     "bship_malloc": [c_size_t, POINTER(c_void_p)],
     "bship_free": [_P],
     "bship_pool_trim": [],

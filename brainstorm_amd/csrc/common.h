@@ -131,6 +131,30 @@ static inline unsigned stream_grid(int64_t tiles) {
 // Scratch from the pool without zero-fill (internal partial-result buffers).
 int pool_alloc_raw(size_t nbytes, void** out);
 int pool_free_raw(void* p);
+
+// ---- recorded steps (graph.hip) ----
+// True while bship_graph_begin() ... bship_graph_end() records the library's stream. Calls that
+// wait for the device or move data to or from host memory are refused then (BSHIP_REQUIRE_EAGER).
+bool graph_recording();
+// Pool blocks handed out while graph `id` is recorded belong to it: when their owner frees them
+// they are parked, not reused, until the graph is destroyed (its kernels keep writing to them).
+void pool_graph_begin(int id);
+void pool_graph_end();
+void pool_graph_destroyed(int id);
+
+// rng.hip: dropout masks of a recorded step (see "masks of recorded steps" there)
+int rng_graph_begin(int id);
+int rng_graph_end(int id);
+int rng_graph_before_launch(int id);
+void rng_graph_destroyed(int id);
+
+#define BSHIP_REQUIRE_EAGER()                                                                    \
+    do {                                                                                         \
+        if (::bship::graph_recording())                                                          \
+            return ::bship::set_error(BSHIP_ERR_UNSUPPORTED,                                     \
+                                      "%s: not possible while a step is being recorded "         \
+                                      "(bship_graph_begin)", __func__);                          \
+    } while (0)
 // Enqueues mem[0:n] = val.
 int launch_fill(float* mem, float val, size_t n);
 

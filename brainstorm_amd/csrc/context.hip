@@ -31,10 +31,11 @@ int check_hip(hipError_t e, const char* what) {
 int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return check_hip(e, what);
-    if (g_ctx.debug_sync) return check_hip(hipStreamSynchronize(g_ctx.stream), what);
+    if (g_ctx.debug_sync && !graph_recording()) return check_hip(hipStreamSynchronize(g_ctx.stream), what);
     return 0;
 }
 
+void graph_release_all();  // graph.hip
 void pool_release_all();   // pool.hip
 void rng_release();        // rng.hip
 void gemm_release();       // gemm.hip
@@ -83,6 +84,7 @@ int bship_init(int device) {
 int bship_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_ctx_mutex);
     if (!g_ctx.inited) return 0;
+    graph_release_all();
     (void)hipStreamSynchronize(g_ctx.stream);
     gemm_release();
     rng_release();
@@ -96,6 +98,7 @@ int bship_shutdown(void) {
 
 int bship_sync(void) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
     BSHIP_HIP(hipStreamSynchronize(g_ctx.stream));
     return 0;
 }
@@ -113,6 +116,7 @@ int bship_device_info(char* name_host, size_t name_len, int* compute_units) {
 int bship_event_record(int slot) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(slot >= 0 && slot < BSHIP_MAX_EVENTS);
+    BSHIP_REQUIRE_EAGER();
     if (!g_ctx.events[slot]) BSHIP_HIP(hipEventCreate(&g_ctx.events[slot]));
     BSHIP_HIP(hipEventRecord(g_ctx.events[slot], g_ctx.stream));
     return 0;
@@ -121,6 +125,7 @@ int bship_event_record(int slot) {
 int bship_event_elapsed_ms(int start_slot, int stop_slot, float* ms_host) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_PTR(ms_host);
+    BSHIP_REQUIRE_EAGER();
     BSHIP_REQUIRE_DIM(start_slot >= 0 && start_slot < BSHIP_MAX_EVENTS);
     BSHIP_REQUIRE_DIM(stop_slot >= 0 && stop_slot < BSHIP_MAX_EVENTS);
     if (!g_ctx.events[start_slot] || !g_ctx.events[stop_slot])

@@ -19,6 +19,10 @@ std::mutex g_pool_mutex;
 std::map<size_t, std::vector<void*>> g_free;       // rounded size -> cached blocks
 std::unordered_map<void*, size_t> g_live;          // handed-out block -> rounded size
 size_t g_in_use = 0, g_cached = 0, g_device_allocs = 0;
+int g_recording_graph = 0;                          // graph whose step is being recorded, or 0
+std::unordered_map<void*, int> g_graph_owner;      // block handed out during a recording -> graph
+struct Parked { size_t size; int graph; };
+std::unordered_map<void*, Parked> g_parked;        // such blocks after their owner freed them
 
 size_t round_size(size_t n) {
     size_t q = n < (64u << 10) ? 256 : (n < (1u << 20) ? 4096 : (2u << 20));
@@ -50,6 +54,8 @@ int pool_alloc_raw(size_t nbytes, void** out) {
         g_cached -= sz;
     } else {
         size_t limit = pool_limit();
+        if (g_recording_graph && limit && g_in_use + g_cached + sz > limit)
+            return set_error(BSHIP_ERR_OUT_OF_MEMORY, "pool limit of %zu bytes reached while a step is being recorded", limit);
         if (limit && g_in_use + g_cached + sz > limit) {
             // Give cached blocks back before refusing.
             (void)hipStreamSynchronize(ctx().stream);
@@ -60,6 +66,12 @@ int pool_alloc_raw(size_t nbytes, void** out) {
                                  limit, g_in_use, sz);
         }
         hipError_t e = hipMalloc(out, sz);
+        if (e != hipSuccess && g_recording_graph) {
+            (void)hipGetLastError();
+            *out = nullptr;
+            return set_error(BSHIP_ERR_OUT_OF_MEMORY, "hipMalloc of %zu bytes failed while a step is being recorded: %s",
+                             sz, hipGetErrorString(e));
+        }
         if (e != hipSuccess) {
             (void)hipGetLastError();
             (void)hipStreamSynchronize(ctx().stream);
@@ -77,6 +89,7 @@ int pool_alloc_raw(size_t nbytes, void** out) {
     }
     g_live[*out] = sz;
     g_in_use += sz;
+    if (g_recording_graph) g_graph_owner[*out] = g_recording_graph;
     return 0;
 }
 
@@ -88,10 +101,43 @@ int pool_free_raw(void* p) {
         return set_error(BSHIP_ERR_BAD_POINTER, "bship_free: %p was not allocated by the pool", p);
     size_t sz = it->second;
     g_live.erase(it);
+    auto owner = g_graph_owner.find(p);
+    if (owner != g_graph_owner.end()) {
+        // a recorded step uses this block on every replay: keep it out of circulation
+        g_parked[p] = Parked{sz, owner->second};
+        g_graph_owner.erase(owner);
+        return 0;
+    }
     g_in_use -= sz;
     g_free[sz].push_back(p);
     g_cached += sz;
     return 0;
+}
+
+void pool_graph_begin(int id) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    g_recording_graph = id;
+}
+
+void pool_graph_end() {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    g_recording_graph = 0;
+}
+
+void pool_graph_destroyed(int id) {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    for (auto it = g_parked.begin(); it != g_parked.end();) {
+        if (it->second.graph == id) {
+            g_in_use -= it->second.size;
+            g_free[it->second.size].push_back(it->first);
+            g_cached += it->second.size;
+            it = g_parked.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    for (auto it = g_graph_owner.begin(); it != g_graph_owner.end();)
+        it = it->second == id ? g_graph_owner.erase(it) : std::next(it);
 }
 
 void pool_release_all() {
@@ -99,6 +145,10 @@ void pool_release_all() {
     trim_locked();
     for (auto& kv : g_live) (void)hipFree(kv.first);
     g_live.clear();
+    for (auto& kv : g_parked) (void)hipFree(kv.first);
+    g_parked.clear();
+    g_graph_owner.clear();
+    g_recording_graph = 0;
     g_in_use = 0;
     g_device_allocs = 0;
 }
@@ -178,6 +228,7 @@ int bship_free(void* p) {
 
 int bship_pool_trim(void) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
     BSHIP_HIP(hipStreamSynchronize(ctx().stream));
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     trim_locked();
@@ -197,6 +248,7 @@ int bship_h2d(void* dst, const void* src_host, size_t nbytes) {
     if (nbytes == 0) return 0;
     BSHIP_REQUIRE_PTR(dst);
     BSHIP_REQUIRE_PTR(src_host);
+    BSHIP_REQUIRE_EAGER();
     BSHIP_HIP(hipMemcpyAsync(dst, src_host, nbytes, hipMemcpyHostToDevice, ctx().stream));
     BSHIP_HIP(hipStreamSynchronize(ctx().stream));
     return 0;
@@ -207,6 +259,7 @@ int bship_d2h(void* dst_host, const void* src, size_t nbytes) {
     if (nbytes == 0) return 0;
     BSHIP_REQUIRE_PTR(dst_host);
     BSHIP_REQUIRE_PTR(src);
+    BSHIP_REQUIRE_EAGER();
     BSHIP_HIP(hipMemcpyAsync(dst_host, src, nbytes, hipMemcpyDeviceToHost, ctx().stream));
     BSHIP_HIP(hipStreamSynchronize(ctx().stream));
     return 0;

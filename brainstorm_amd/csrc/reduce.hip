@@ -377,6 +377,7 @@ int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N) {
 int bship_isfinite_f32(const float* a, size_t n, int* result_host) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_PTR(result_host);
+    BSHIP_REQUIRE_EAGER();
     *result_host = 1;
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(a);

@@ -34,6 +34,7 @@
 #include <cstdlib>
 #include <type_traits>
 #include <deque>
+#include <map>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -413,10 +414,127 @@ static void prefetch_maybe_start() {
     }
 }
 
+// --------------------------- masks of recorded steps ---------------------------
+// A recorded step (bship_graph_begin ... bship_graph_end) replays the same kernels with the same
+// arguments, so its masks cannot be served by the queue above, and drawing them inline would put
+// their sequential time on the step's critical path. Instead every mask request of the recording
+// gets a slot of its own (staging, raw words, generator snapshot). In the recorded graph the main
+// stream reads the slot's staging buffer, and a branch on the second stream, ordered behind that
+// read, draws the slot's next mask: replay r consumes what replay r-1 (or the priming below) drew,
+// in request order, so the random stream is used exactly as by eager execution. Before the first
+// replay, and after any other use of the generator, the slots are "primed": their masks are drawn
+// eagerly in order. Any eager use of the generator first "unprimes": it puts the generator back to
+// the snapshot taken before the pending, not yet consumed masks.
+struct GraphMasks {
+    std::vector<MaskPrefetch> slots;
+    bool primed = false;
+};
+static std::map<int, GraphMasks> g_graph_masks;
+static int g_recording_masks = 0;      // graph being recorded, or 0
+static int g_primed_graph = 0;         // graph whose slots hold drawn, unconsumed masks, or 0
+
+// The pending masks of the primed graph are given up: the generator returns to the position before them.
+static int graph_masks_unprime() {
+    if (g_primed_graph == 0) return 0;
+    GraphMasks& gm = g_graph_masks[g_primed_graph];
+    g_primed_graph = 0;
+    gm.primed = false;
+    if (gm.slots.empty()) return 0;
+    hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, ctx().stream, gm.slots.front().before, g_state);
+    return check_launch("random stream rewind");
+}
+
+static int ensure_side_stream() {
+    if (!g_side) BSHIP_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
+    if (!g_join) BSHIP_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    return 0;
+}
+
+// A mask request while recording: a new slot, handed back like a queue hit.
+static int graph_mask_slot(size_t n, double p, MaskPrefetch* hit) {
+    MaskPrefetch e = MaskPrefetch();
+    e.n = n;
+    e.p = p;
+    void* a = nullptr;
+    void* b = nullptr;
+    void* r = nullptr;
+    int st = pool_alloc_raw(n * sizeof(float), &a);
+    e.staging = static_cast<float*>(a);
+    if (st == 0) st = pool_alloc_raw(2 * n * sizeof(uint32_t), &r);
+    e.raw = static_cast<uint32_t*>(r);
+    if (st == 0) st = pool_alloc_raw(sizeof(RngState), &b);
+    e.before = static_cast<RngState*>(b);
+    if (st == 0) st = check_hip(hipEventCreateWithFlags(&e.consumed, hipEventDisableTiming), "hipEventCreate");
+    if (st != 0) { free_entry(e); return st; }
+    *hit = e;
+    return 0;
+}
+
+// The recorded main stream has read the slot's staging buffer: the second stream draws the next mask.
+static int graph_mask_redraw(MaskPrefetch& e) {
+    BSHIP_HIP(hipEventRecord(e.consumed, ctx().stream));
+    BSHIP_HIP(hipStreamWaitEvent(g_side, e.consumed, 0));
+    launch_mask(g_side, e.staging, e.n, e.p, e.before, e.raw);
+    int st = check_launch("recorded mask");
+    g_graph_masks[g_recording_masks].slots.push_back(e);
+    return st;
+}
+
+int rng_graph_begin(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    int st = ensure_side_stream();
+    if (st == 0 && g_state) st = prefetch_flush(true);
+    if (st == 0 && g_state) st = graph_masks_unprime();
+    if (st != 0) return st;
+    g_recording_masks = id;
+    g_graph_masks[id] = GraphMasks();
+    return 0;
+}
+
+// Joins the second stream's branch, if the recording made one, back into the main stream.
+int rng_graph_end(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    g_recording_masks = 0;
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    return order_streams(g_side, ctx().stream);
+}
+
+int rng_graph_before_launch(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    if (g_primed_graph == id) return 0;
+    int st = prefetch_flush(true);
+    if (st == 0) st = graph_masks_unprime();
+    if (st != 0) return st;
+    for (MaskPrefetch& e : it->second.slots) launch_mask(ctx().stream, e.staging, e.n, e.p, e.before, e.raw);
+    st = check_launch("recorded masks, first draw");
+    if (st != 0) return st;
+    it->second.primed = true;
+    g_primed_graph = id;
+    return 0;
+}
+
+void rng_graph_destroyed(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end()) return;
+    if (g_primed_graph == id) (void)graph_masks_unprime();
+    for (MaskPrefetch& e : it->second.slots) free_entry(e);
+    g_graph_masks.erase(it);
+}
+
 // Serves a mask request: either hands back the queue's front entry (*is_hit; the caller reads
 // hit->staging on the main stream and then calls mask_end), or draws the mask into `mask` directly.
 static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* is_hit) {
     *is_hit = false;
+    if (g_recording_masks) {
+        *is_hit = true;
+        return graph_mask_slot(n, p, hit);
+    }
+    int ust = graph_masks_unprime();
+    if (ust != 0) return ust;
     if (!g_fifo.empty()) {
         const MaskPrefetch& e = g_fifo.front();
         if (e.n == n && e.p == p) {
@@ -445,6 +563,7 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
 // The main stream has enqueued its read of the entry's staging buffer: draw the entry again
 // for the next round.
 static int mask_end(MaskPrefetch& e) {
+    if (g_recording_masks) return graph_mask_redraw(e);
     hipError_t err = hipEventRecord(e.consumed, ctx().stream);
     if (err != hipSuccess) { free_entry(e); return check_hip(err, "hipEventRecord"); }
     return prefetch_schedule(e, true);
@@ -480,6 +599,11 @@ void rng_release() {
     if (g_side) (void)hipStreamSynchronize(g_side);
     for (MaskPrefetch& e : g_fifo) free_entry(e);
     g_fifo.clear();
+    for (auto& kv : g_graph_masks)
+        for (MaskPrefetch& e : kv.second.slots) free_entry(e);
+    g_graph_masks.clear();
+    g_primed_graph = 0;
+    g_recording_masks = 0;
     g_history.clear();
     g_min_period = 1;
     if (g_join) { (void)hipEventDestroy(g_join); g_join = nullptr; }
@@ -495,9 +619,11 @@ extern "C" {
 
 int bship_rng_seed(uint32_t seed) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     int st = rng_ensure_state();
     if (st == 0) st = prefetch_flush(false);
+    if (st == 0) st = graph_masks_unprime();
     if (st != 0) return st;
     // init_genrand of the MT19937 reference code, as used by RandomState(int)
     RngState h;
@@ -512,10 +638,12 @@ int bship_rng_seed(uint32_t seed) {
 
 int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_rng_get_state: bship_rng_seed() has not been called");
     RngState h;
     int st = prefetch_flush(true);
+    if (st == 0) st = graph_masks_unprime();
     if (st == 0) st = bship_d2h(&h, g_state, sizeof(RngState));
     if (st != 0) return st;
     if (key_host) for (int i = 0; i < kMtN; ++i) key_host[i] = h.key[i];
@@ -575,6 +703,7 @@ int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, do
 
 int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(out);
@@ -582,6 +711,7 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_fill_gaussian_f32: bship_rng_seed() has not been called");
     hipStream_t s = ctx().stream;
     int st = prefetch_flush(true);
+    if (st == 0) st = graph_masks_unprime();
     if (st != 0) return st;
     // device scalars: [0] trials consumed, [1] outputs written, [2] outputs taken from the cache
     void* rp = nullptr;

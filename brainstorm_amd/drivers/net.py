@@ -219,3 +219,18 @@ class MomentumStepper:
         h.mult_add_st(-learning_rate, self.net.gradients, out=self.velocity)
         h.add_tt(self.velocity, self.net.parameters, out=self.net.parameters)
         self.net.apply_weight_modifiers()                  # the trainer does this after every update (trainer.py:101)
+
+    def run_recorded(self):
+        """The same step through a recording: the first call records ``run`` with the handler's
+        ``record`` (the network must have done at least one ordinary step before, so that nothing is
+        set up lazily inside the recording) and replays it; later calls only replay. Input data has
+        to be in place in the network's buffers (``provide_external_data``) before each call, and
+        the batch shape must not change."""
+        if getattr(self, "_recorded", None) is None:
+            self._recorded = self.net.handler.record(self.run)
+        self._recorded.replay()
+
+    def release_recorded(self):
+        if getattr(self, "_recorded", None) is not None:
+            self._recorded.release()
+            self._recorded = None

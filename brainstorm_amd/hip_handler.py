@@ -70,6 +70,32 @@ class HipRandomState:
                 has_gauss.value, gauss.value)
 
 
+class RecordedStep(object):
+    """A recorded sequence of handler calls (see :meth:`HipHandler.record`)."""
+
+    def __init__(self, handler, graph_id):
+        self._handler = handler
+        self._id = graph_id
+
+    def replay(self):
+        if self._id is None:
+            raise RuntimeError("this recorded step has been released")
+        self._handler._call(self._handler._lib.bship_graph_launch(self._id))
+
+    def release(self):
+        if self._id is not None:
+            gid, self._id = self._id, None
+            self._handler._call(self._handler._lib.bship_graph_destroy(gid))
+
+    def __del__(self):
+        try:
+            if self._id is not None and self._handler._lib is not None:
+                self._handler._lib.bship_graph_destroy(self._id)
+                self._id = None
+        except Exception:
+            pass
+
+
 class HipHandler(Handler):
     __undescribed__ = {'context', 'dtype', 'EMPTY', 'rnd'}
 
@@ -168,6 +194,29 @@ class HipHandler(Handler):
     def synchronize(self):
         """Waits until every operation issued so far has finished."""
         self._call(self._lib.bship_sync())
+
+    # --------------------------------------------------- recorded steps
+    def record(self, fn):
+        """Runs ``fn()`` once in recording mode and returns a :class:`RecordedStep`.
+
+        While recording, the handler calls made by ``fn`` are captured, not executed; the
+        returned object's ``replay()`` then issues all of them with one launch. ``fn`` must not
+        read results back or upload data (``get_numpy_copy``, ``set_from_numpy``,
+        ``is_fully_finite``, ``fill_gaussian``, ``synchronize`` raise while recording): place
+        those around the replay. Arrays that ``fn`` allocates keep their memory for as long
+        as the recording exists. Shapes and addresses are fixed at recording time.
+        """
+        self._call(self._lib.bship_graph_begin())
+        try:
+            fn()
+        except BaseException:
+            gid = ctypes.c_int()
+            if self._lib.bship_graph_end(ctypes.byref(gid)) == 0:
+                self._lib.bship_graph_destroy(gid.value)
+            raise
+        gid = ctypes.c_int()
+        self._call(self._lib.bship_graph_end(ctypes.byref(gid)))
+        return RecordedStep(self, gid.value)
 
     def device_info(self):
         name = ctypes.create_string_buffer(256)

@@ -69,6 +69,26 @@ int bship_device_info(char* name_host, size_t name_len, int* compute_units);
 int bship_event_record(int slot);
 int bship_event_elapsed_ms(int start_slot, int stop_slot, float* ms_host);
 
+/* Recorded steps. The reference's trainer issues every handler call of a
+ * training step one by one from Python (trainer.py 83-100, steppers.py 60-140,
+ * network.py 409-460); small networks are bound by that, not by the device.
+ * Between bship_graph_begin and bship_graph_end the calls of this library are
+ * recorded (HIP stream capture) instead of executed; bship_graph_launch then
+ * replays the whole recording with one launch, on the library's stream and in
+ * order with every other call. A recording may contain compute calls, device
+ * to device copies, bship_malloc and bship_free (blocks handed out while
+ * recording stay reserved for the graph until it is destroyed). Calls that wait
+ * for the device or touch host memory (bship_sync, bship_h2d, bship_d2h, timers,
+ * bship_isfinite_f32, bship_fill_gaussian_f32, bship_rng_seed,
+ * bship_rng_get_state, bship_pool_trim) return BSHIP_ERR_UNSUPPORTED while
+ * recording. Dropout masks of a recorded step continue the random stream
+ * exactly as eager calls would (replay r uses the draws that follow those of
+ * replay r-1; other uses of the generator between replays are allowed). */
+int bship_graph_begin(void);
+int bship_graph_end(int* graph_id);
+int bship_graph_launch(int graph_id);
+int bship_graph_destroy(int graph_id);
+
 /* ------------------------------- memory ---------------------------------- */
 
 /* allocate/zeros (numpy 36-43, pycuda 70-79): a block of at least `nbytes`
