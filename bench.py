@@ -234,24 +234,30 @@ def run_image_ops(hip, n_img=2048, reps=10):
     return out
 
 
-def time_net(handler, builder, steps, warmup, sync, **kw):
+def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
     """Training steps per second of one network workload (forward + backward + momentum update,
-    inputs uploaded once; the per-step loss read-back of a Trainer is included)."""
+    inputs uploaded once; the per-step loss read-back of a Trainer is included). recorded: the
+    step's handler calls are recorded once (after an ordinary step) and replayed with one launch."""
     from brainstorm_amd.drivers.net import MomentumStepper
     net, data = builder(handler, **kw)
     net.provide_external_data(data)
     stepper = MomentumStepper(0.1, 0.9)
     stepper.start(net)
-    for _ in range(warmup):
+    if recorded:
         stepper.run()
+    step = stepper.run_recorded if recorded else stepper.run
+    for _ in range(warmup):
+        step()
         net.get("loss", "outputs", "loss")
     sync()
     t0 = time.perf_counter()
     for _ in range(steps):
-        stepper.run()
+        step()
         net.get("loss", "outputs", "loss")      # device-to-host copy + wait, as trainer.py:100 does
     sync()
     dt = (time.perf_counter() - t0) / steps
+    if recorded:
+        stepper.release_recorded()
     samples = data["default"].shape[0] * data["default"].shape[1]
     return {"ms_per_step": round(dt * 1e3, 3), "samples_per_s": round(samples / dt, 1)}
 
@@ -263,6 +269,11 @@ def run_nets_gpu(hip):
         # same network, dropout and bias+activation through the fused entry points (same bits)
         "mlp_784-1200-1200-10_batch100_fused": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize,
                                                         fused=True),
+        # same network and bits, the step recorded into a HIP graph and replayed
+        "mlp_784-1200-1200-10_batch100_recorded": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize,
+                                                           recorded=True),
+        "mlp_784-1200-1200-10_batch100_fused_recorded": time_net(hip, configs.build_mlp, 600, 20,
+                                                                 hip.synchronize, recorded=True, fused=True),
         "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
         # same network, the elementwise part of each time step in one launch (same bits)
         "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,
