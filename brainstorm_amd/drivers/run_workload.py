@@ -1,9 +1,11 @@
 """Runs training steps of one network workload on HipHandler: the program to put under a profiler.
 
-    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused]
+    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded]
 
-``fused`` is passed to the workload's builder ("1" for the fused entry points, "packed" for the
-LSTM's stacked recurrent product). One step = forward + backward + momentum update.
+``fused`` is passed to the workload's builder ("0" for single handler operations, "1" for the fused
+entry points, "packed" for the LSTM's stacked recurrent product). With a fourth argument "recorded"
+the step is recorded after one ordinary step and replayed. One step = forward + backward + momentum
+update.
 """
 import sys
 
@@ -17,15 +19,21 @@ def main(argv):
     steps = int(argv[2]) if len(argv) > 2 else 3
     fused = argv[3] if len(argv) > 3 else ""
     kw = {}
-    if fused:
+    recorded = len(argv) > 4 and argv[4] == "recorded"
+    if fused and fused != "0":
         kw["fused"] = "packed" if fused == "packed" else True
     handler = HipHandler(seed=0)
     net, data = getattr(configs, "build_" + name)(handler, **kw)
     net.provide_external_data(data)
     stepper = MomentumStepper(0.1, 0.9)
     stepper.start(net)
-    for _ in range(steps):
+    if recorded:
         stepper.run()
+    for _ in range(steps):
+        if recorded:
+            stepper.run_recorded()
+        else:
+            stepper.run()
     handler.synchronize()
     print("%s: %d steps done" % (name, steps))
 
