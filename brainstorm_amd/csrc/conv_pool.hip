@@ -65,7 +65,9 @@ __device__ __forceinline__ void cover_range(int p, int pad, const FastDiv& strid
     lo = t <= 0 ? 0 : static_cast<int>(stride.div(static_cast<uint32_t>(t) + stride.d - 1));
 }
 
-// Cached (not streaming) accesses: the images are re-read by overlapping windows.
+// Cached (not streaming) accesses for what overlapping windows read again; operands that a kernel
+// touches once (pooling outputs, the in_deltas a backward kernel updates) go through the
+// non-temporal vload/vstore like the elementwise kernels' (max-pool backward 32x32x32: 149 -> 135 us).
 template <int W, bool AL>
 __device__ __forceinline__ typename VecT<W>::type img_load(const float* p) {
     if constexpr (W == 1) return *p;
@@ -564,8 +566,8 @@ __device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, f
 #pragma unroll
         for (int j = 0; j < W; ++j)
             if (comp<W>(where, j) < 0.0f) comp<W>(best, j) = 0.0f;
-        img_store<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, best);
-        img_store<W, AL>(argmax + img * out_img + static_cast<int64_t>(p) * W, where);
+        vstore<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, best);
+        vstore<W, AL>(argmax + img * out_img + static_cast<int64_t>(p) * W, where);
     }
 }
 #define BSHIP_POOL_FWD_KERNEL(name, K)                                                                   \
@@ -602,7 +604,7 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
     typedef typename VecT<W>::type R;
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
-        R acc = img_load<W, AL>(q);
+        R acc = vload<W, AL>(q);
         auto take = [&](R am, R d) {
 #pragma unroll
             for (int j = 0; j < W; ++j)
@@ -631,7 +633,7 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
                     take(img_load<W, AL>(argmax + o), img_load<W, AL>(out_deltas + o));
                 }
         }
-        img_store<W, AL>(q, acc);
+        vstore<W, AL>(q, acc);
     }
 }
 #define BSHIP_POOL_BWD_KERNEL(name, C)                                                                   \
@@ -685,7 +687,7 @@ __device__ __forceinline__ void avgpool_fwd_body(const float* __restrict__ in, f
         }
 #pragma unroll
         for (int j = 0; j < W; ++j) comp<W>(sum, j) = comp<W>(sum, j) / size;
-        img_store<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, sum);
+        vstore<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, sum);
     }
 }
 #define BSHIP_AVG_FWD_KERNEL(name, K)                                                                    \
@@ -724,7 +726,7 @@ __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_d
     };
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
-        R acc = img_load<W, AL>(q);
+        R acc = vload<W, AL>(q);
         const float* dimg = out_deltas + img * out_img + chv * W;
         if constexpr (C > 0) {
             R d[C * C];
@@ -753,7 +755,7 @@ __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_d
                     for (int j = 0; j < W; ++j) comp<W>(acc, j) += comp<W>(d, j) / size;
                 }
         }
-        img_store<W, AL>(q, acc);
+        vstore<W, AL>(q, acc);
     }
 }
 #define BSHIP_AVG_BWD_KERNEL(name, C)                                                                    \
