@@ -37,12 +37,26 @@ int check_hip(hipError_t e, const char* what);
 // To be called right after a kernel launch.
 int check_launch(const char* what);
 
-#define BSHIP_REQUIRE_INIT()                                                     \
+// Small fills are collected and enqueued together as one launch (pool.hip); every entry point
+// first enqueues what has been collected, so the order of effects is the order of the calls.
+int flush_deferred_fills();
+extern int g_deferred_fill_count;
+
+#define BSHIP_REQUIRE_INIT_NO_FLUSH()                                            \
     do {                                                                         \
         if (!::bship::ctx().inited)                                              \
             return ::bship::set_error(BSHIP_ERR_NOT_INITIALIZED,                 \
                                       "%s: bship_init() has not been called",    \
                                       __func__);                                 \
+    } while (0)
+
+#define BSHIP_REQUIRE_INIT()                                                     \
+    do {                                                                         \
+        BSHIP_REQUIRE_INIT_NO_FLUSH();                                           \
+        if (::bship::g_deferred_fill_count != 0) {                               \
+            int flush_st_ = ::bship::flush_deferred_fills();                     \
+            if (flush_st_ != 0) return flush_st_;                                \
+        }                                                                        \
     } while (0)
 
 #define BSHIP_REQUIRE_PTR(p)                                                     \

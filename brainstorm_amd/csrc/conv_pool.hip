@@ -15,6 +15,7 @@
 
 #include <cfloat>
 #include <map>
+#include <mutex>
 
 #include "common.h"
 
@@ -897,7 +898,9 @@ static bool plan_col2im_band(const ImgGeom& g, int64_t n, Col2imBandPlan* out, s
 // Lets `kernel` use `bytes` of dynamic LDS (more than the default limit has to be asked for);
 // remembers what each kernel was granted.
 static bool allow_dynamic_lds_impl(const void* kernel, size_t bytes) {
+    static std::mutex mutex;
     static std::map<const void*, size_t> granted;
+    std::lock_guard<std::mutex> lock(mutex);
     auto it = granted.find(kernel);
     if (it != granted.end() && it->second >= bytes) return true;
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) != hipSuccess)

@@ -206,6 +206,63 @@ int launch_fill(float* p, float val, size_t n) {
     return check_launch("fill_kernel");
 }
 
+// ------------------------------ deferred fills ------------------------------
+// A training step clears a dozen small buffers in a row (BufferManager.clear_backward_buffers,
+// buffers.py:147-150: one fill per backward-only hub), each a launch of a few microseconds that
+// costs more to issue than to run. Fills of up to kDeferredFillMax elements are therefore only
+// noted; the next entry point of any kind (BSHIP_REQUIRE_INIT), or a full list, enqueues all
+// noted fills as ONE launch (grid.y = fill). Fills that overlap a noted one are enqueued in
+// order: the noted ones go first.
+constexpr int kMaxDeferredFills = 16;
+constexpr size_t kDeferredFillMax = size_t(1) << 18;      // 1 MiB
+struct DeferredFill { float* p; size_t n; float val; };
+struct DeferredFills { DeferredFill f[kMaxDeferredFills]; };
+static DeferredFills g_deferred;
+int g_deferred_fill_count = 0;
+static std::mutex g_deferred_mutex;
+
+__global__ __launch_bounds__(kBlock) void multi_fill_kernel(DeferredFills d) {
+    const DeferredFill f = d.f[blockIdx.y];
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i >= f.n) return;
+    if (i + 4 <= f.n && (reinterpret_cast<uintptr_t>(f.p + i) & 15u) == 0) {
+        *reinterpret_cast<f4*>(f.p + i) = f4{f.val, f.val, f.val, f.val};
+    } else {
+        for (size_t j = i; j < f.n && j < i + 4; ++j) f.p[j] = f.val;
+    }
+}
+
+static int flush_deferred_locked() {
+    if (g_deferred_fill_count == 0) return 0;
+    size_t most = 0;
+    for (int k = 0; k < g_deferred_fill_count; ++k) most = g_deferred.f[k].n > most ? g_deferred.f[k].n : most;
+    const dim3 grid(static_cast<unsigned>((most + kCopyTile - 1) / kCopyTile), static_cast<unsigned>(g_deferred_fill_count));
+    g_deferred_fill_count = 0;
+    hipLaunchKernelGGL(multi_fill_kernel, grid, dim3(kBlock), 0, ctx().stream, g_deferred);
+    return check_launch("multi_fill_kernel");
+}
+
+int flush_deferred_fills() {
+    std::lock_guard<std::mutex> lock(g_deferred_mutex);
+    return flush_deferred_locked();
+}
+
+// Notes mem[0:n] = val for the next flush (n <= kDeferredFillMax).
+static int defer_fill(float* mem, float val, size_t n) {
+    std::lock_guard<std::mutex> lock(g_deferred_mutex);
+    bool overlaps = false;
+    for (int k = 0; k < g_deferred_fill_count; ++k) {
+        const DeferredFill& f = g_deferred.f[k];
+        overlaps = overlaps || (mem < f.p + f.n && f.p < mem + n);
+    }
+    if (overlaps || g_deferred_fill_count == kMaxDeferredFills) {
+        int st = flush_deferred_locked();
+        if (st != 0) return st;
+    }
+    g_deferred.f[g_deferred_fill_count++] = DeferredFill{mem, n, val};
+    return 0;
+}
+
 }  // namespace bship
 
 using namespace bship;
@@ -307,11 +364,13 @@ int bship_copy2d_f32(float* dst, int64_t ld_dst, const float* src, int64_t ld_sr
 }
 
 int bship_fill_f32(float* mem, float val, size_t n) {
-    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(mem);
     BSHIP_REQUIRE_F32_ALIGNED(mem);
-    return launch_fill(mem, val, n);
+    if (n <= kDeferredFillMax) return defer_fill(mem, val, n);
+    int st = flush_deferred_fills();
+    return st != 0 ? st : launch_fill(mem, val, n);
 }
 
 }  // extern "C"

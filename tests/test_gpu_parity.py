@@ -695,6 +695,36 @@ def test_im2col_col2im_banded_exact(hip, ref):
         assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, kh, kw, pad, stride),))
 
 
+def test_many_small_fills_keep_call_order(hip):
+    # small fills are collected and enqueued together: overlapping ones, more than fit one launch,
+    # fills of unaligned views, and fills followed directly by a reader must all act in call order
+    flat = hip.allocate((40000,))
+    want = np.zeros((40000,), F32)
+    hip.fill(flat, 1.0)
+    want[:] = 1.0
+    for k in range(40):                               # more fills than one collected launch holds
+        lo, hi = 37 * k + 1, 37 * k + 1 + 5 * (k % 7) + 1
+        hip.fill(flat[lo:hi], float(k + 2))
+        want[lo:hi] = k + 2
+    hip.fill(flat[3:30000], 5.0)                      # overlaps many of the above
+    want[3:30000] = 5.0
+    hip.fill(flat[10:20], 6.0)                        # overlaps the one just before
+    want[10:20] = 6.0
+    other = hip.allocate((7, 9))
+    hip.fill(other, 9.0)
+    hip.add_st(1.0, flat, flat)                       # a reader right behind the fills
+    want += 1.0
+    assert_bit_equal(flat.get(), want, "small fills in call order")
+    assert_bit_equal(other.get(), np.full((7, 9), 9.0, F32), "small fill of another array")
+    big = hip.allocate((1 << 19,))                    # a large fill between small ones
+    hip.fill(big[5:100], 3.0)
+    hip.fill(big, 2.0)
+    hip.fill(big[7:9], 4.0)
+    wb = np.full((1 << 19,), 2.0, F32)
+    wb[7:9] = 4.0
+    assert_bit_equal(big.get(), wb, "large fill between small ones")
+
+
 # ---------------------------------------------------------- views of one buffer
 def test_ops_on_unaligned_views(hip, ref):
     # Layer buffers are slices of one flat array (buffers.py:79-83) and may start at any element,
