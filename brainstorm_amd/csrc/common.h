@@ -172,16 +172,37 @@ void rng_graph_destroyed(int id);
 // Enqueues mem[0:n] = val.
 int launch_fill(float* mem, float val, size_t n);
 
-// ---- wavefront / workgroup reductions (device) ----
+// ---- wavefront reductions (device) ----
+// All 64 lanes must be active. Four DPP steps (lane^1, lane^2, mirror inside 8 lanes, mirror inside
+// a row of 16) leave every lane of a row with the row's result without touching LDS (a shuffle is a
+// ds_bpermute through the LDS crossbar, ~100 cycles each, six in a butterfly); the four row results
+// are read out as scalars and combined, so every lane returns the same value.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    const int x = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+constexpr int kDppXor1 = 0xB1;          // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;          // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;   // row_half_mirror
+constexpr int kDppMirror = 0x140;       // row_mirror
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    v += dpp_move<kDppMirror>(v);
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    v = fmaxf(v, dpp_move<kDppXor1>(v));
+    v = fmaxf(v, dpp_move<kDppXor2>(v));
+    v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kDppMirror>(v));
+    return fmaxf(fmaxf(read_lane(v, 0), read_lane(v, 16)), fmaxf(read_lane(v, 32), read_lane(v, 48)));
 }
 
 }  // namespace bship
