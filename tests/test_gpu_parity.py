@@ -695,6 +695,48 @@ def test_im2col_col2im_banded_exact(hip, ref):
         assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, kh, kw, pad, stride),))
 
 
+def test_im2col_col2im_random_geometries(hip, ref):
+    # the banded kernels choose band sizes, LDS rings and phases from the geometry: many random
+    # geometries (non-square kernels, strides up to 3, padding up to the kernel size minus one,
+    # 1-20 channels, few and many images) against the oracle, bit for bit
+    rng = np.random.RandomState(321)
+    lib = hip._lib
+    cases = []
+    while len(cases) < 70:
+        kh, kw = rng.randint(1, 6), rng.randint(1, 6)
+        pad = rng.randint(0, min(kh, kw))
+        sh, sw = rng.randint(1, 4), rng.randint(1, 4)
+        h, w = rng.randint(1, 41), rng.randint(1, 41)
+        if h + 2 * pad < kh or w + 2 * pad < kw:
+            continue
+        c = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 20]))
+        n = int(rng.choice([1, 2, 3, 9, 17, 40, 130, 600]))
+        oh, ow = _out_size(h, kh, pad, sh), _out_size(w, kw, pad, sw)
+        if n * oh * ow * kh * kw * c > 6_000_000:
+            continue
+        cases.append((n, h, w, c, kh, kw, pad, (sh, sw)))
+    for n, h, w, c, kh, kw, pad, stride in cases:
+        oh, ow = _out_size(h, kh, pad, stride[0]), _out_size(w, kw, pad, stride[1])
+        what = "%r" % ((n, h, w, c, kh, kw, pad, stride),)
+        x = rand(rng, (n, h, w, c))
+        col = np.zeros((n, oh * ow, kh * kw * c), F32)
+        for i in range(n):
+            ref._im2col(x[i], kh, kw, pad, stride, col[i])
+        xd = hip.create_from_numpy(x)
+        cold = hip.allocate(col.shape)
+        hip._call(lib.bship_im2col_nhwc_f32(xd.ptr, cold.ptr, n, h, w, c, kh, kw, pad, stride[0], stride[1]))
+        assert_bit_equal(cold.get(), col, "im2col " + what)
+        cols = rand(rng, col.shape)
+        din = rand(rng, x.shape)
+        want = din.copy()
+        for i in range(n):
+            ref._col2im(cols[i], kh, kw, pad, stride, want[i])
+        dind = hip.create_from_numpy(din)
+        colsd = hip.create_from_numpy(cols)
+        hip._call(lib.bship_col2im_nhwc_f32(colsd.ptr, dind.ptr, n, h, w, c, kh, kw, pad, stride[0], stride[1]))
+        assert_bit_equal(dind.get(), want, "col2im " + what)
+
+
 def test_many_small_fills_keep_call_order(hip):
     # small fills are collected and enqueued together: overlapping ones, more than fit one launch,
     # fills of unaligned views, and fills followed directly by a reader must all act in call order
