@@ -129,6 +129,20 @@ class DeviceArray:
 
     # --------------------------------------------------------------- reshape
     def reshape(self, *new_shape):
+        if len(new_shape) == 1 and type(new_shape[0]) is tuple:
+            new_shape = new_shape[0]
+        # fast path (the layers reshape their buffers on every call): plain non-negative ints
+        n = 1
+        for s in new_shape:
+            if type(s) is not int or s < 0:
+                break
+            n *= s
+        else:
+            if n != self.size:
+                raise ValueError("cannot reshape array of size %d into shape %r" % (self.size, new_shape))
+            out = DeviceArray.__new__(DeviceArray)
+            out.ptr, out.shape, out.size, out._owner, out._handler = self.ptr, new_shape, n, self._owner, self._handler
+            return out
         if len(new_shape) == 1 and not isinstance(new_shape[0], (int, np.integer)):
             new_shape = tuple(new_shape[0])
         new_shape = tuple(int(s) for s in new_shape)
