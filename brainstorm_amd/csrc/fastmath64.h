@@ -108,7 +108,8 @@ __device__ __forceinline__ float tanh_f32(float x) {
     const double s = pow2_f64(k);
     const double em = __builtin_fma(s, rq, s - 1.0);
     const float r = static_cast<float>(em * rcp64(em + 2.0));
-    return (x != x) ? x : r;
+    // tanh is odd: the sign is the argument's (for -0.0 the fma above has produced +0.0)
+    return (x != x) ? x : __builtin_copysignf(r, x);
 }
 
 // ln(x): x = m * 2^e with m in [sqrt(1/2), sqrt(2)); ln m = 2 atanh(s) = 2s (1 + z P(z)) with

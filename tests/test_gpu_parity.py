@@ -263,6 +263,26 @@ def test_transcendentals(hip, ref, shape):
     _check_transcendental(hip, ref, "log_t", (x + 10).astype(F32), np.log, "N(10,1)")
 
 
+def test_transcendentals_special_values(hip):
+    # signed zeros, infinities, NaN, denormals, the clamping thresholds and beyond: the bits of the
+    # float64 evaluation rounded to float32
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-40, -1e-40, 1.17549435e-38,
+                  -1.17549435e-38, 1e-30, -1e-30, 1e-10, -1e-10, 0.17, -0.17, 0.1733, -0.1733, 0.3466, -0.3466,
+                  8.9, 9.1, -9.1, 19.99, 20.0, 20.01, -20.01, 87.0, -87.0, 88.8, -88.8, 103.0, -103.0, 104.5,
+                  -104.5, 199.0, -199.0, 201.0, -201.0, 1e10, -1e10, 3.4e38, -3.4e38, 1.0, -1.0, 0.5, 2.0],
+                 dtype=F32)
+    xd = hip.create_from_numpy(x)
+    yd = hip.allocate(x.shape)
+    x64 = x.astype(np.float64)
+    with np.errstate(all="ignore"):
+        hip.tanh(xd, yd)
+        assert_bit_equal(yd.get(), np.tanh(x64).astype(F32), "tanh of special values")
+        hip.sigmoid(xd, yd)
+        assert_bit_equal(yd.get(), _sigmoid64(x64).astype(F32), "sigmoid of special values")
+        hip.log_t(xd, yd)
+        assert_bit_equal(yd.get(), np.log(x64).astype(F32), "log of special values")
+
+
 def test_el(hip, ref):
     # el = x*(x>=0) + (exp(x)-1)*(x<0) in float32 steps (numpy_handler.py:305). exp(x)-1 cancels,
     # so an ulp of exp(x) (<= 2^-24 for x<0) is an ABSOLUTE error of the result: the bound is
