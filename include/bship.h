@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define BSHIP_VERSION 100 /* major*10000 + minor*100 + patch */
+#define BSHIP_VERSION 200 /* major*10000 + minor*100 + patch */
 
 /* argument / state errors (negative so they never collide with hipError_t) */
 #define BSHIP_ERR_NOT_INITIALIZED (-1)
