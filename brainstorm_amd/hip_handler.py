@@ -149,8 +149,9 @@ class HipHandler(Handler):
         cls = type(self)
         for name in dir(cls):
             if name.startswith("_") or name in ("allocate", "zeros", "ones", "create_from_numpy",
-                                                "synchronize", "device_info", "stack_adjacent"):
-                continue
+                                                "synchronize", "device_info", "stack_adjacent",
+                                                "record", "dot_mm", "dot_add_mm"):
+                continue                          # matrix products take row pitches natively (_gemm)
             fn = getattr(cls, name)
             if not inspect.isfunction(fn):
                 continue
@@ -434,9 +435,13 @@ class HipHandler(Handler):
             raise ValueError("shapes %r%s . %r%s -> %r do not match"
                              % (a.shape, "^T" if transa else "", b.shape, "^T" if transb else "",
                                 out.shape))
+        # a row-pitched matrix (a feature slice of a hub) goes in as it is: its pitch is the
+        # leading dimension of the product
+        pa, lda = (a._base, a.pitch) if type(a) is PitchedDeviceArray else (a.ptr, a.shape[1])
+        pb, ldb = (b._base, b.pitch) if type(b) is PitchedDeviceArray else (b.ptr, b.shape[1])
+        pc, ldc = (out._base, out.pitch) if type(out) is PitchedDeviceArray else (out.ptr, n)
         self._call(self._lib.bship_gemm_f32(int(bool(transa)), int(bool(transb)), m, n, k, 1.0,
-                                            a.ptr, a.shape[1], b.ptr, b.shape[1], beta,
-                                            out.ptr, n))
+                                            pa, lda, pb, ldb, beta, pc, ldc))
 
     def dot_mm(self, a, b, out, transa=False, transb=False):
         self._gemm(a, b, out, transa, transb, 0.0)

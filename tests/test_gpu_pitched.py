@@ -92,6 +92,31 @@ def test_operations_on_pitched_slices(php, name, call):
             np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=name + ": " + tag)
 
 
+def test_matrix_products_take_pitched_operands_as_they_are(php):
+    # the pitch of a feature slice is the leading dimension of the product: no dense temporaries
+    rng = np.random.RandomState(11)
+    rows, width = 9, 40
+    hub = rng.standard_normal((rows, width)).astype(F32)
+    w = rng.standard_normal((7, 6)).astype(F32)
+    dev_hub, dev_w = php.create_from_numpy(hub), php.create_from_numpy(w)
+    allocations = []
+    real_allocate = php.allocate
+    php.allocate = lambda shape: allocations.append(shape) or real_allocate(shape)
+    try:
+        php.dot_mm(dev_hub[:, 3:9], dev_w, dev_hub[:, 20:27], transb=True)      # (9,6) . (7,6)^T -> (9,7)
+        php.dot_add_mm(dev_hub[:, 20:27], dev_w, dev_hub[:, 30:36])             # += (9,7) . (7,6)
+    finally:
+        php.allocate = real_allocate
+    assert allocations == [], allocations
+    want = hub.copy()
+    want[:, 20:27] = want[:, 3:9] @ w.T
+    want[:, 30:36] += want[:, 20:27] @ w
+    np.testing.assert_allclose(dev_hub.get(), want, rtol=1e-5, atol=1e-5)
+    untouched = np.ones(width, bool)
+    untouched[20:27] = untouched[30:36] = False
+    assert_bit_equal(dev_hub.get()[:, untouched], hub[:, untouched], "columns outside the written slices")
+
+
 def test_two_layers_writing_one_hub(php):
     # two fully connected layers put their outputs side by side into one hub, a third reads the whole
     # hub: the multi-source hub of buffer_structure.py:232-245, forward and backward
