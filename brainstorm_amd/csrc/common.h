@@ -3,6 +3,8 @@
 // streaming kernel. gfx950 only: wavefronts are 64 lanes wide.
 #pragma once
 
+#include <atomic>
+
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -40,7 +42,7 @@ int check_launch(const char* what);
 // Small fills are collected and enqueued together as one launch (pool.hip); every entry point
 // first enqueues what has been collected, so the order of effects is the order of the calls.
 int flush_deferred_fills();
-extern int g_deferred_fill_count;
+extern std::atomic<int> g_deferred_fill_count;   // read without the list's lock: 0 means nothing to do
 
 #define BSHIP_REQUIRE_INIT_NO_FLUSH()                                            \
     do {                                                                         \
@@ -53,7 +55,7 @@ extern int g_deferred_fill_count;
 #define BSHIP_REQUIRE_INIT()                                                     \
     do {                                                                         \
         BSHIP_REQUIRE_INIT_NO_FLUSH();                                           \
-        if (::bship::g_deferred_fill_count != 0) {                               \
+        if (::bship::g_deferred_fill_count.load(std::memory_order_relaxed) != 0) { \
             int flush_st_ = ::bship::flush_deferred_fills();                     \
             if (flush_st_ != 0) return flush_st_;                                \
         }                                                                        \

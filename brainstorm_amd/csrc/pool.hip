@@ -218,7 +218,7 @@ constexpr size_t kDeferredFillMax = size_t(1) << 18;      // 1 MiB
 struct DeferredFill { float* p; size_t n; float val; };
 struct DeferredFills { DeferredFill f[kMaxDeferredFills]; };
 static DeferredFills g_deferred;
-int g_deferred_fill_count = 0;
+std::atomic<int> g_deferred_fill_count{0};
 static std::mutex g_deferred_mutex;
 
 __global__ __launch_bounds__(kBlock) void multi_fill_kernel(DeferredFills d) {
@@ -235,8 +235,9 @@ __global__ __launch_bounds__(kBlock) void multi_fill_kernel(DeferredFills d) {
 static int flush_deferred_locked() {
     if (g_deferred_fill_count == 0) return 0;
     size_t most = 0;
-    for (int k = 0; k < g_deferred_fill_count; ++k) most = g_deferred.f[k].n > most ? g_deferred.f[k].n : most;
-    const dim3 grid(static_cast<unsigned>((most + kCopyTile - 1) / kCopyTile), static_cast<unsigned>(g_deferred_fill_count));
+    const int count = g_deferred_fill_count.load();
+    for (int k = 0; k < count; ++k) most = g_deferred.f[k].n > most ? g_deferred.f[k].n : most;
+    const dim3 grid(static_cast<unsigned>((most + kCopyTile - 1) / kCopyTile), static_cast<unsigned>(count));
     g_deferred_fill_count = 0;
     hipLaunchKernelGGL(multi_fill_kernel, grid, dim3(kBlock), 0, ctx().stream, g_deferred);
     return check_launch("multi_fill_kernel");
@@ -251,7 +252,7 @@ int flush_deferred_fills() {
 static int defer_fill(float* mem, float val, size_t n) {
     std::lock_guard<std::mutex> lock(g_deferred_mutex);
     bool overlaps = false;
-    for (int k = 0; k < g_deferred_fill_count; ++k) {
+    for (int k = 0, count = g_deferred_fill_count.load(); k < count; ++k) {
         const DeferredFill& f = g_deferred.f[k];
         overlaps = overlaps || (mem < f.p + f.n && f.p < mem + n);
     }
@@ -259,7 +260,9 @@ static int defer_fill(float* mem, float val, size_t n) {
         int st = flush_deferred_locked();
         if (st != 0) return st;
     }
-    g_deferred.f[g_deferred_fill_count++] = DeferredFill{mem, n, val};
+    const int slot = g_deferred_fill_count.load();
+    g_deferred.f[slot] = DeferredFill{mem, n, val};
+    g_deferred_fill_count = slot + 1;
     return 0;
 }
 
