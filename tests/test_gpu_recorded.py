@@ -185,3 +185,32 @@ def test_recorded_training_steps_equal_eager_ones():
         got_losses, got_params = train(True, fused)
         assert got_losses == want_losses, (fused, got_losses, want_losses)
         assert_bit_equal(got_params, want_params, "parameters after recorded steps (fused=%r)" % fused)
+
+
+def test_graph_entry_points_report_misuse(hip):
+    import ctypes
+    lib = hip._lib
+    gid = ctypes.c_int(-1)
+    assert lib.bship_graph_end(ctypes.byref(gid)) != 0              # nothing is being recorded
+    assert b"no step" in lib.bship_last_error()
+    assert lib.bship_graph_launch(12345) != 0                       # unknown recording
+    assert lib.bship_graph_destroy(12345) != 0
+    assert lib.bship_graph_begin() == 0
+    assert lib.bship_graph_begin() != 0                             # already recording
+    assert lib.bship_graph_launch(1) != 0                           # not while recording
+    a = hip.allocate((4, 4))
+    hip.add_st(1.0, a, a)
+    assert lib.bship_graph_end(ctypes.byref(gid)) == 0 and gid.value > 0
+    assert lib.bship_graph_launch(gid.value) == 0
+    assert lib.bship_graph_destroy(gid.value) == 0
+    assert lib.bship_graph_destroy(gid.value) != 0                  # already destroyed
+    assert lib.bship_graph_launch(gid.value) != 0
+    assert_bit_equal(hip.get_numpy_copy(a), np.full((4, 4), 1.0, F32), "one replay of add_st")
+    # an empty recording is refused, and the handler stays usable
+    assert lib.bship_graph_begin() == 0
+    status = lib.bship_graph_end(ctypes.byref(gid))
+    if status == 0:
+        assert lib.bship_graph_launch(gid.value) == 0
+        assert lib.bship_graph_destroy(gid.value) == 0
+    hip.add_st(1.0, a, a)
+    assert_bit_equal(hip.get_numpy_copy(a), np.full((4, 4), 2.0, F32), "eager call after the recordings")
