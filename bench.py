@@ -275,6 +275,9 @@ def run_nets_gpu(hip):
         "mlp_784-1200-1200-10_batch100_fused_recorded": time_net(hip, configs.build_mlp, 600, 20,
                                                                  hip.synchronize, recorded=True, fused=True),
         "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
+        # same network and bits, the ~4000 launches of a step recorded into a HIP graph and replayed
+        "lstm_205-1000-205_T100_batch100_recorded": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize,
+                                                             recorded=True),
         # same network, the elementwise part of each time step in one launch (same bits)
         "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,
                                                                hip.synchronize, fused=True),
