@@ -111,3 +111,73 @@ def test_zero_sized_and_zero_dimensional():
     dev, host = make((3, 4))
     check_same(dev[1:1], host[1:1], host)
     assert dev.nbytes == 48 and len(dev) == 3
+
+
+# ------------------------------------------------------------------ randomised against NumPy
+from hypothesis import given, settings, strategies as st
+
+
+class _PitchedHandler:
+    pitched_views = True
+
+
+def _index_strategy(ndim):
+    def one(n_axes):
+        item = st.one_of(st.integers(-7, 6),
+                         st.builds(slice, st.one_of(st.none(), st.integers(-7, 7)),
+                                   st.one_of(st.none(), st.integers(-7, 7))))
+        return st.lists(item, min_size=0, max_size=n_axes).map(tuple)
+    with_ellipsis = st.tuples(one(ndim), one(ndim)).map(lambda ab: ab[0] + (Ellipsis,) + ab[1])
+    return st.one_of(one(ndim), with_ellipsis, st.integers(-7, 6))
+
+
+@settings(max_examples=600, deadline=None)
+@given(st.data())
+def test_random_index_chains_match_numpy(data):
+    """Two index operations in a row on random shapes: NumPy decides what the view is (its
+    offset, shape and strides); DeviceArray must return the same dense view, or the same
+    row-pitched view when the handler allows those, or refuse exactly the views that are neither
+    (and raise IndexError exactly where NumPy does)."""
+    shape = tuple(data.draw(st.lists(st.integers(0, 5), min_size=1, max_size=4)))
+    pitched = data.draw(st.booleans())
+    host_base = np.arange(int(np.prod(shape)), dtype=np.float32).reshape(shape)
+    dev = DeviceArray(BASE_PTR, shape, None, _PitchedHandler() if pitched else None)
+    host = host_base
+    for _ in range(2):
+        key = data.draw(_index_strategy(host.ndim))
+        try:
+            want = npview(host, key)
+        except IndexError:
+            with pytest.raises(IndexError):
+                dev[key]
+            return
+        dense = want.size == 0 or want.ndim == 0 or want.flags["C_CONTIGUOUS"]
+        # a row-pitched view: last axis contiguous (or of length 1), leading axes like the rows of one matrix
+        representable = dense
+        if not dense and pitched and (want.shape[-1] == 1 or want.strides[-1] == 4):
+            pitch, below, ok = None, 1, True
+            for n, s in zip(reversed(want.shape[:-1]), reversed(want.strides[:-1])):
+                if n != 1:
+                    if pitch is None:
+                        ok = ok and (s // 4) % below == 0
+                        pitch = (s // 4) // below
+                    else:
+                        ok = ok and s // 4 == pitch * below
+                below *= n
+            representable = ok
+        if not representable:
+            with pytest.raises(NotImplementedError):
+                dev[key]
+            return
+        got = dev[key]
+        assert got.shape == want.shape and got.size == want.size
+        if want.size:
+            assert (got._address() - BASE_PTR) // 4 == int(want.reshape(-1)[0]) if dense else \
+                (got._address() - BASE_PTR) // 4 == int(want[(0,) * want.ndim])
+            if dense:
+                assert type(got) is DeviceArray
+            else:
+                assert got.pitch == [s // 4 for n, s in zip(want.shape[:-1], want.strides[:-1]) if n != 1][-1]
+        dev, host = got, want
+        if type(dev) is not DeviceArray:
+            return                                   # chains continue on dense views only here
