@@ -428,6 +428,32 @@ def test_softmax_m(hip, ref):
     np.testing.assert_allclose(md.get(), want, rtol=1e-5)
 
 
+def test_random_shapes_reductions_broadcasts_indexing(hip, ref):
+    # the launch plans of these kernels depend on the shape (column lanes, row bands, wavefront or
+    # workgroup per row, vector width by divisibility): 80 random shapes, log-uniform in both
+    # dimensions, each through sum_t on all axes, softmax_m, the mv operations with both vector
+    # shapes, binarize_v and index_m_by_v
+    rng = np.random.RandomState(4242)
+    for case in range(80):
+        rows = int(np.exp(rng.uniform(0, np.log(3000))))
+        cols = int(np.exp(rng.uniform(0, np.log(3000))))
+        a = rand(rng, (rows, cols))
+        _check_sum(hip, ref, a, 0, (1, cols))
+        _check_sum(hip, ref, a, 1, (rows, 1))
+        _check_sum(hip, ref, a, None, ())
+        pairs = operation_check(hip, ref, "softmax_m", (a, np.zeros_like(a)), compare="rel", rtol=1e-5, atol=1e-37)
+        np.testing.assert_allclose(pairs[1][1].astype(np.float64).sum(axis=1), 1.0, rtol=0, atol=1e-5)
+        row, col = rand(rng, (1, cols)), rand(rng, (rows, 1))
+        for op in ("add_mv", "mult_mv", "subtract_mv", "divide_mv"):
+            operation_check(hip, ref, op, (a, row, np.zeros_like(a)))
+            operation_check(hip, ref, op, (a, col, np.zeros_like(a)))
+        operation_check(hip, ref, "mult_add_mv", (a, row, rand(rng, (rows, cols))))
+        operation_check(hip, ref, "mult_add_mv", (a, col, rand(rng, (rows, cols))))
+        labels = rng.randint(0, cols, (rows, 1)).astype(F32)
+        operation_check(hip, ref, "binarize_v", (labels, np.full((rows, cols), 3.0, F32)))
+        operation_check(hip, ref, "index_m_by_v", (a, labels, np.zeros((rows, 1), F32)))
+
+
 def test_is_fully_finite(hip, ref):
     rng = np.random.RandomState(20)
     for shape in ((5, 5), (37, 1031), (1 << 20,)):
