@@ -54,20 +54,25 @@ struct LstmFwdArgs {
 // PACKED: the four recurrent products arrive as one (batch, 4n) matrix instead of
 // having been accumulated into Za, Ia, Fa, Oa; they are added first, which is what
 // the accumulating product does with its finished dot products.
+// Streaming accesses of the step kernels: what a time step reads and writes once should not push
+// the recurrent matrices, which the next step's product reads again, out of the L2 caches.
+__device__ __forceinline__ float ldg(const float* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void stg(float* p, float v) { __builtin_nontemporal_store(v, p); }
+
 template <bool PACKED>
 __global__ __launch_bounds__(kBlock) void lstm_fwd_step_kernel(LstmFwdArgs a, int act, int64_t total,
                                                                unsigned n) {
     const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (e >= total) return;
     const unsigned j = static_cast<unsigned>(e % n);       // column: index into the (1,n) parameters
-    const float c_prev = a.Ca_prev[e];
-    float za = a.Za[e], ia = a.Ia[e], fa = a.Fa[e], oa = a.Oa[e];
+    const float c_prev = ldg(a.Ca_prev + e);
+    float za = ldg(a.Za + e), ia = ldg(a.Ia + e), fa = ldg(a.Fa + e), oa = ldg(a.Oa + e);
     if (PACKED) {
         const float* r = a.rec + (e / n) * (4 * static_cast<int64_t>(n)) + j;
-        za = za + r[0];
-        ia = ia + r[n];
-        fa = fa + r[2 * static_cast<int64_t>(n)];
-        oa = oa + r[3 * static_cast<int64_t>(n)];
+        za = za + ldg(r);
+        ia = ia + ldg(r + n);
+        fa = fa + ldg(r + 2 * static_cast<int64_t>(n));
+        oa = oa + ldg(r + 3 * static_cast<int64_t>(n));
     }
     za = za + a.bz[j];
     const float zb = act_forward(act, za);
@@ -83,8 +88,8 @@ __global__ __launch_bounds__(kBlock) void lstm_fwd_step_kernel(LstmFwdArgs a, in
     oa = oa + a.bo[j];
     const float ob = SigmoidOp{}.apply(oa, 0.0f, 0.0f);
     const float cb = act_forward(act, ca);
-    a.Za[e] = za; a.Zb[e] = zb; a.Ia[e] = ia; a.Ib[e] = ib; a.Fa[e] = fa; a.Fb[e] = fb;
-    a.Ca[e] = ca; a.Oa[e] = oa; a.Ob[e] = ob; a.Cb[e] = cb;
+    stg(a.Za + e, za); stg(a.Zb + e, zb); stg(a.Ia + e, ia); stg(a.Ib + e, ib); stg(a.Fa + e, fa); stg(a.Fb + e, fb);
+    stg(a.Ca + e, ca); stg(a.Oa + e, oa); stg(a.Ob + e, ob); stg(a.Cb + e, cb);
     a.y[e] = ob * cb;
 }
 
@@ -113,31 +118,32 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
     const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (e >= total) return;
     const unsigned j = static_cast<unsigned>(e % n);
-    float dy = a.dy[e];
+    float dy = ldg(a.dy + e);
     if (PACKED) {
-        dy = a.deltas[e] + dy;
+        dy = ldg(a.deltas + e) + dy;
         a.dy_out[e] = dy;
     }
-    float dca = a.dCa[e];
-    { const float p = a.dIa_next[e] * a.pi[j]; dca = dca + p; }
-    { const float p = a.dFa_next[e] * a.pf[j]; dca = dca + p; }
-    const float ob = a.Ob[e], cb = a.Cb[e];
+    float dca = ldg(a.dCa + e);
+    { const float p = ldg(a.dIa_next + e) * a.pi[j]; dca = dca + p; }
+    { const float p = ldg(a.dFa_next + e) * a.pf[j]; dca = dca + p; }
+    const float ob = ldg(a.Ob + e), cb = ldg(a.Cb + e);
     const float dob = dy * cb;
     const float doa = SigmoidDerivOp{}.apply(ob, dob, 0.0f);
     { const float p = doa * a.po[j]; dca = dca + p; }
     float dcb = dy * ob;
     dcb = act_backward(act, cb, dcb);
     dca = dca + dcb;
-    { const float p = a.dCa_next[e] * a.Fb_next[e]; dca = dca + p; }
-    const float dfb = dca * a.Ca_prev[e];
-    const float dfa = SigmoidDerivOp{}.apply(a.Fb[e], dfb, 0.0f);
-    const float zb = a.Zb[e], ib = a.Ib[e];
+    { const float p = ldg(a.dCa_next + e) * ldg(a.Fb_next + e); dca = dca + p; }
+    const float dfb = dca * ldg(a.Ca_prev + e);
+    const float dfa = SigmoidDerivOp{}.apply(ldg(a.Fb + e), dfb, 0.0f);
+    const float zb = ldg(a.Zb + e), ib = ldg(a.Ib + e);
     const float dib = dca * zb;
     const float dia = SigmoidDerivOp{}.apply(ib, dib, 0.0f);
     const float dzb = dca * ib;
     const float dza = act_backward(act, zb, dzb);
-    a.dOb[e] = dob; a.dOa[e] = doa; a.dCb[e] = dcb; a.dCa[e] = dca; a.dFb[e] = dfb; a.dFa[e] = dfa;
-    a.dIb[e] = dib; a.dIa[e] = dia; a.dZb[e] = dzb; a.dZa[e] = dza;
+    // the gate deltas feed the matrix products that follow and dCa the next step: those stay cached
+    stg(a.dOb + e, dob); a.dOa[e] = doa; stg(a.dCb + e, dcb); a.dCa[e] = dca; stg(a.dFb + e, dfb); a.dFa[e] = dfa;
+    stg(a.dIb + e, dib); a.dIa[e] = dia; stg(a.dZb + e, dzb); a.dZa[e] = dza;
     if (PACKED) {
         float* q = a.packed_out + (e / n) * (4 * static_cast<int64_t>(n)) + j;
         q[0] = dza;
