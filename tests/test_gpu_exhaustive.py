@@ -69,3 +69,37 @@ def test_all_float32_inputs(op, exact_f64):
     assert worst <= 1, "%s: %d ulp at x=%r (got %r, float64 evaluation %r)" % ((op, worst) + tuple(example))
     assert differing <= 1000, "%s: %d inputs are not the rounded float64 evaluation" % (op, differing)
     assert wrong_zeros == 0
+
+
+def _exact_compare(got, x, op):
+    from oracle.numpy_ref_handler import NumpyRefHandler
+    ref = NumpyRefHandler(F32, seed=0)
+    want = np.zeros_like(x)
+    with np.errstate(all="ignore"):
+        getattr(ref, op)(x, want)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    bad = np.flatnonzero(~same)
+    return int(bad.size), (None if bad.size == 0 else (x[bad[0]], got[bad[0]], want[bad[0]]))
+
+
+@pytest.mark.parametrize("op", ["abs_t", "sign_t", "sqrt_t", "rel"])
+def test_all_float32_inputs_bit_exact(op):
+    """The operations that have one right answer in float32: the same bits as the oracle for every input."""
+    from brainstorm_amd import HipHandler
+    hip = HipHandler(seed=0)
+    xd, yd = hip.allocate((CHUNK,)), hip.allocate((CHUNK,))
+    differing, example = 0, None
+    with ThreadPoolExecutor(8) as pool:
+        pending = []
+        for c in range((1 << 32) // CHUNK):
+            x = (np.arange(CHUNK, dtype=np.uint64) + c * CHUNK).astype(np.uint32).view(F32)
+            hip.set_from_numpy(xd, x)
+            getattr(hip, op)(xd, yd)
+            pending.append(pool.submit(_exact_compare, hip.get_numpy_copy(yd), x, op))
+            if len(pending) == 8 or c == (1 << 32) // CHUNK - 1:
+                for p in pending:
+                    n, e = p.result()
+                    differing += n
+                    example = example or e
+                pending = []
+    assert differing == 0, "%s: %d of 2^32 inputs differ, e.g. x=%r got %r want %r" % ((op, differing) + tuple(example))
