@@ -262,6 +262,12 @@ def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
     return {"ms_per_step": round(dt * 1e3, 3), "samples_per_s": round(samples / dt, 1)}
 
 
+def time_net_fast_masks(builder, steps, warmup):
+    from brainstorm_amd import HipHandler
+    handler = HipHandler(seed=0, fast_masks=True)
+    return time_net(handler, builder, steps, warmup, handler.synchronize, recorded=True, fused=True)
+
+
 def run_nets_gpu(hip):
     from brainstorm_amd.drivers import configs
     return {
@@ -274,6 +280,9 @@ def run_nets_gpu(hip):
                                                            recorded=True),
         "mlp_784-1200-1200-10_batch100_fused_recorded": time_net(hip, configs.build_mlp, 600, 20,
                                                                  hip.synchronize, recorded=True, fused=True),
+        # NOT the reference's masks: dropout masks from the optional counter-based generator
+        # (HipHandler(fast_masks=True)), one parallel launch per mask instead of the MT19937 walk
+        "mlp_784-1200-1200-10_batch100_fused_recorded_fast_masks": time_net_fast_masks(configs.build_mlp, 600, 20),
         "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
         # same network and bits, the ~4000 launches of a step recorded into a HIP graph and replayed
         "lstm_205-1000-205_T100_batch100_recorded": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize,

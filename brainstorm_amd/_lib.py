@@ -65,6 +65,10 @@ SIGNATURES = {
     "bship_rng_seed": [c_uint32],
     "bship_prob_mask_f32": [_P, c_size_t, c_double],
     "bship_fill_gaussian_f32": [_P, c_size_t, c_double, c_double],
+    "bship_fast_rng_seed": [ctypes.c_ulonglong],
+    "bship_fast_rng_get_state": [POINTER(ctypes.c_ulonglong), POINTER(ctypes.c_ulonglong)],
+    "bship_prob_mask_fast_f32": [_P, c_size_t, c_double],
+    "bship_dropout_fwd_fast_f32": [_P, _P, _P, c_size_t, c_double, c_float],
     "bship_rng_get_state": [POINTER(c_uint32), POINTER(c_int), POINTER(c_int), POINTER(c_double)],
     "bship_gemm_f32": [c_int, c_int, _I64, _I64, _I64, c_float, _P, _I64, _P, _I64, c_float, _P, _I64],
     "bship_im2col_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,

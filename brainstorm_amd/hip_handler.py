@@ -101,7 +101,11 @@ class HipHandler(Handler):
 
     array_type = DeviceArray
 
-    def __init__(self, seed=None, device=0, pitched_views=False):
+    def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False):
+        # fast_masks: dropout masks from a counter-based generator (Philox4x32-10) instead of
+        # NumPy's MT19937 stream. One parallel launch per mask instead of a sequential walk, but
+        # NOT the masks NumpyHandler draws for the same seed (the reference's own GPU handler does
+        # not match NumPy either, pycuda_handler.py:37-39). fill_gaussian keeps NumPy's stream.
         # pitched_views: let slices that need a row pitch (feature slices of a hub with several
         # sources, buffer_structure.py:232-245) exist as PitchedDeviceArray and serve operations
         # on them through dense temporaries. Off by default: it puts a Python-level argument
@@ -118,6 +122,9 @@ class HipHandler(Handler):
         self._free = self._lib.bship_free
         self.EMPTY = DeviceArray(0, (0,), None, self)
         self.rnd = HipRandomState(self, seed)
+        self.fast_masks = bool(fast_masks)
+        if self.fast_masks:
+            self._call(self._lib.bship_fast_rng_seed(int(self.rnd.get_seed())))
 
     def __describe__(self):
         return {'@type': self.__class__.__name__}
@@ -425,7 +432,16 @@ class HipHandler(Handler):
         self._call(self._lib.bship_fill_gaussian_f32(out.ptr, out.size, mean, std))
 
     def generate_probability_mask(self, mask, probability):
-        self._call(self._lib.bship_prob_mask_f32(mask.ptr, mask.size, probability))
+        if self.fast_masks:
+            self._call(self._lib.bship_prob_mask_fast_f32(mask.ptr, mask.size, probability))
+        else:
+            self._call(self._lib.bship_prob_mask_f32(mask.ptr, mask.size, probability))
+
+    def fast_mask_state(self):
+        """(seed, next block) of the fast mask generator (fast_masks=True)."""
+        seed, block = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        self._call(self._lib.bship_fast_rng_get_state(ctypes.byref(seed), ctypes.byref(block)))
+        return seed.value, block.value
 
     # ------------------------------------------------------- dense products
     def _gemm(self, a, b, out, transa, transb, beta):
@@ -653,5 +669,5 @@ class HipHandler(Handler):
         out = scale * out (dropout_layer.py:41-45) with one pass behind the mask."""
         if not (inputs.shape == mask.shape == out.shape):
             raise ValueError("dropout_forward: inconsistent shapes")
-        self._call(self._lib.bship_dropout_fwd_f32(inputs.ptr, mask.ptr, out.ptr, out.size,
-                                                   float(keep_probability), float(scale)))
+        fn = self._lib.bship_dropout_fwd_fast_f32 if self.fast_masks else self._lib.bship_dropout_fwd_f32
+        self._call(fn(inputs.ptr, mask.ptr, out.ptr, out.size, float(keep_probability), float(scale)))

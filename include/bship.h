@@ -369,6 +369,21 @@ int bship_bias_act_f32(int act, const float* in, const float* bias, float* out,
  * the same position, as bship_prob_mask_f32 would draw it. */
 int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n,
                           double keep_probability, float scale);
+/* Optional fast mask stream. No counterpart in NumpyHandler: masks come from
+ * the counter-based Philox4x32-10 generator (four mask elements per block, a
+ * pure function of a 64-bit key and a 64-bit block number kept in device
+ * memory), one parallel launch per mask instead of the sequential MT19937 walk.
+ * For callers that want dropout at memory speed and do not need the masks
+ * NumpyHandler would draw; the reference's GPU handler is in the same position
+ * (cuRAND XORWOW, pycuda_handler.py 37-39 and 191-193). element i of a mask is
+ * 1.0 when word i%4 of block next_block + i/4 is below floor(p * 2^32); every
+ * call advances next_block by ceil(n/4), also inside recorded steps.
+ * bship_dropout_fwd_fast_f32 is bship_dropout_fwd_f32 on this stream. */
+int bship_fast_rng_seed(unsigned long long seed);
+int bship_fast_rng_get_state(unsigned long long* seed_host, unsigned long long* next_block_host);
+int bship_prob_mask_fast_f32(float* mask, size_t n, double p);
+int bship_dropout_fwd_fast_f32(const float* in, float* mask, float* out, size_t n,
+                               double keep_probability, float scale);
 /* BatchNormLayerImpl.forward_pass (batch_normalization_layer.py 54-105) on
  * (M,N) matrices and N-element vectors. training != 0: batch statistics (the
  * negative batch mean and then the deviation go through sigma_b as in the

@@ -505,3 +505,32 @@ def test_conv_forward_brute_force_and_backward_finite_differences(ref64):
         np.testing.assert_allclose(dw, num_grad(wts, "w"), rtol=1e-5, atol=1e-6)
         np.testing.assert_allclose(db, num_grad(bias, "b"), rtol=1e-5, atol=1e-6)
         np.testing.assert_allclose(din - din0, num_grad(x, "x"), rtol=1e-5, atol=1e-6)   # in_deltas are ADDED to
+
+
+def test_philox_known_answers_and_mask_rule():
+    """oracle/philox.py against the generator's published known-answer vectors (Random123's
+    kat_vectors for philox4x32 with 10 rounds) and the mask rule against a direct restatement."""
+    from oracle import philox
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+            (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        got = philox.philox4x32_10(np.array([ctr], np.uint32), key)[0]
+        assert tuple(int(x) for x in got) == want
+    # several counters at once give what each gives alone
+    ctrs = np.array([[5, 0, 0, 0], [6, 0, 0, 0], [0xffffffff, 7, 0, 0]], np.uint32)
+    many = philox.philox4x32_10(ctrs, (11, 22))
+    for i in range(3):
+        assert np.array_equal(many[i], philox.philox4x32_10(ctrs[i:i + 1], (11, 22))[0])
+    # the mask: block offset+b serves elements 4b..4b+3; 64-bit offsets carry into the second counter word
+    seed, offset, n, p = (3 << 32) | 9, (1 << 32) - 2, 19, 0.3
+    mask, blocks = philox.probability_mask(n, p, seed, offset)
+    assert blocks == 5 and mask.shape == (n,)
+    for i in range(n):
+        b = offset + i // 4
+        words = philox.philox4x32_10(np.array([[b & 0xffffffff, b >> 32, 0, 0]], np.uint32), (9, 3))[0]
+        assert mask[i] == (1.0 if int(words[i % 4]) < int(np.floor(0.3 * 2 ** 32)) else 0.0)
+    assert philox.mask_threshold(1.0) == 2 ** 32 and philox.mask_threshold(0.0) == 0 and philox.mask_threshold(-1.0) == 0
+    big, _ = philox.probability_mask(400000, 0.8, 1234, 0)
+    assert abs(float(big.mean()) - 0.8) < 0.005
