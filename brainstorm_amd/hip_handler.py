@@ -174,10 +174,17 @@ class HipHandler(Handler):
 
     def _dense_call(self, fn, sig, written, *args, **kwargs):
         """Runs fn with every row-pitched operand replaced by a dense temporary."""
+        for a in args:
+            if type(a) is PitchedDeviceArray:
+                break
+        else:
+            for a in kwargs.values():
+                if type(a) is PitchedDeviceArray:
+                    break
+            else:
+                return fn(self, *args, **kwargs)         # the usual case: nothing to do
         bound = sig.bind(self, *args, **kwargs)
         pitched = [(k, a) for k, a in bound.arguments.items() if type(a) is PitchedDeviceArray]
-        if not pitched:
-            return fn(self, *args, **kwargs)
         temps = {}
         for name, a in pitched:
             key = (a._base, a.shape, a.pitch)
