@@ -38,6 +38,7 @@ SIGNATURES = {
     "bship_graph_launch": [c_int],
     "bship_graph_destroy": [c_int],
     "bship_malloc": [c_size_t, POINTER(c_void_p)],
+    "bship_malloc_scratch": [c_size_t, POINTER(c_void_p)],
     "bship_free": [_P],
     "bship_pool_trim": [],
     "bship_pool_stats": [POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)],
@@ -71,6 +72,7 @@ SIGNATURES = {
     "bship_dropout_fwd_fast_f32": [_P, _P, _P, c_size_t, c_double, c_float],
     "bship_rng_get_state": [POINTER(c_uint32), POINTER(c_int), POINTER(c_int), POINTER(c_double)],
     "bship_gemm_f32": [c_int, c_int, _I64, _I64, _I64, c_float, _P, _I64, _P, _I64, c_float, _P, _I64],
+    "bship_gemm_bias_f32": [c_int, c_int, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P, _I64],
     "bship_im2col_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
     "bship_col2im_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
     "bship_maxpool_fwd_nhwc_f32": [_P, _P, _P, _I64] + [c_int] * 10,

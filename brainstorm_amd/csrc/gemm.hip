@@ -22,7 +22,7 @@ struct GemmPlan {
     size_t workspace = 0;
 };
 
-typedef std::tuple<int, int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t> GemmKey;
+typedef std::tuple<int, int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int> GemmKey;   // ..., with bias
 
 std::mutex g_gemm_mutex;
 hipblasLtHandle_t g_handle = nullptr;
@@ -49,9 +49,16 @@ void destroy_plan(GemmPlan& p) {
 }
 
 // Column-major problem: D(m x n) = opA(A) opB(B), leading dimensions lda/ldb/ldc.
+// with_bias: the epilogue adds a vector of m elements to every column of D (the pointer is set per call).
 int make_plan(GemmPlan& p, hipblasOperation_t opa, hipblasOperation_t opb, int64_t m, int64_t n,
-              int64_t k, int64_t lda, int64_t ldb, int64_t ldc) {
+              int64_t k, int64_t lda, int64_t ldb, int64_t ldc, bool with_bias) {
     BSHIP_BLAS(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+    if (with_bias) {
+        const uint32_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+        const int32_t bias_type = HIP_R_32F;
+        BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)));
+        BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)));
+    }
     int32_t ta = static_cast<int32_t>(opa), tb = static_cast<int32_t>(opb);
     BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)));
     BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)));
@@ -93,6 +100,36 @@ void gemm_release() {
 
 using namespace bship;
 
+static int gemm_impl(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha, const float* A,
+                     int64_t lda, const float* B, int64_t ldb, float beta, const float* bias, float* C,
+                     int64_t ldc) {
+    std::lock_guard<std::mutex> lock(g_gemm_mutex);
+    if (!g_handle) BSHIP_BLAS(hipblasLtCreate(&g_handle));
+    if (!g_workspace) {
+        int st = pool_alloc_raw(kWorkspaceBytes, &g_workspace);
+        if (st != 0) return st;
+    }
+    // Row-major C(MxN) = op(A) op(B)  <=>  column-major C^T(NxM) = op(B)^T op(A)^T.
+    // A row-major matrix read as column-major is its transpose, so the first
+    // column-major operand is B with opB, the second is A with opA. A bias per column of the
+    // row-major C is a bias per row of C^T, which is what the library's epilogue adds.
+    const GemmKey key(transa != 0, transb != 0, M, N, K, lda, ldb, ldc, bias != nullptr);
+    auto it = g_plans.find(key);
+    if (it == g_plans.end()) {
+        GemmPlan plan;
+        int st = make_plan(plan, transb ? HIPBLAS_OP_T : HIPBLAS_OP_N, transa ? HIPBLAS_OP_T : HIPBLAS_OP_N,
+                           N, M, K, ldb, lda, ldc, bias != nullptr);
+        if (st != 0) { destroy_plan(plan); return st; }
+        it = g_plans.emplace(key, plan).first;
+    }
+    const GemmPlan& p = it->second;
+    if (bias)
+        BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
+    BSHIP_BLAS(hipblasLtMatmul(g_handle, p.desc, &alpha, B, p.la, A, p.lb, &beta, C, p.lc, C, p.lc,
+                               &p.algo, g_workspace, kWorkspaceBytes, ctx().stream));
+    return check_launch("gemm");
+}
+
 extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
                               const float* A, int64_t lda, const float* B, int64_t ldb, float beta,
                               float* C, int64_t ldc) {
@@ -112,26 +149,21 @@ extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int6
     BSHIP_REQUIRE_PTR(B);
     BSHIP_REQUIRE_DIM(lda >= (transa ? M : K));
     BSHIP_REQUIRE_DIM(ldb >= (transb ? K : N));
-    std::lock_guard<std::mutex> lock(g_gemm_mutex);
-    if (!g_handle) BSHIP_BLAS(hipblasLtCreate(&g_handle));
-    if (!g_workspace) {
-        int st = pool_alloc_raw(kWorkspaceBytes, &g_workspace);
-        if (st != 0) return st;
-    }
-    // Row-major C(MxN) = op(A) op(B)  <=>  column-major C^T(NxM) = op(B)^T op(A)^T.
-    // A row-major matrix read as column-major is its transpose, so the first
-    // column-major operand is B with opB, the second is A with opA.
-    const GemmKey key(transa != 0, transb != 0, M, N, K, lda, ldb, ldc);
-    auto it = g_plans.find(key);
-    if (it == g_plans.end()) {
-        GemmPlan plan;
-        int st = make_plan(plan, transb ? HIPBLAS_OP_T : HIPBLAS_OP_N, transa ? HIPBLAS_OP_T : HIPBLAS_OP_N,
-                           N, M, K, ldb, lda, ldc);
-        if (st != 0) { destroy_plan(plan); return st; }
-        it = g_plans.emplace(key, plan).first;
-    }
-    const GemmPlan& p = it->second;
-    BSHIP_BLAS(hipblasLtMatmul(g_handle, p.desc, &alpha, B, p.la, A, p.lb, &beta, C, p.lc, C, p.lc,
-                               &p.algo, g_workspace, kWorkspaceBytes, ctx().stream));
-    return check_launch("gemm");
+    return gemm_impl(transa, transb, M, N, K, alpha, A, lda, B, ldb, beta, nullptr, C, ldc);
+}
+
+extern "C" int bship_gemm_bias_f32(int transa, int transb, int64_t M, int64_t N, int64_t K, const float* A,
+                                   int64_t lda, const float* B, int64_t ldb, const float* bias, float* C,
+                                   int64_t ldc) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0 && K >= 1);
+    if (M == 0 || N == 0) return 0;
+    BSHIP_REQUIRE_PTR(A);
+    BSHIP_REQUIRE_PTR(B);
+    BSHIP_REQUIRE_PTR(bias);
+    BSHIP_REQUIRE_PTR(C);
+    BSHIP_REQUIRE_DIM(ldc >= N);
+    BSHIP_REQUIRE_DIM(lda >= (transa ? M : K));
+    BSHIP_REQUIRE_DIM(ldb >= (transb ? K : N));
+    return gemm_impl(transa, transb, M, N, K, 1.0f, A, lda, B, ldb, 0.0f, bias, C, ldc);
 }

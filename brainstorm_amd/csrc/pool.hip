@@ -281,6 +281,12 @@ int bship_malloc(size_t nbytes, void** out) {
     return launch_fill(static_cast<float*>(*out), 0.0f, (nbytes + 3) / 4);
 }
 
+int bship_malloc_scratch(size_t nbytes, void** out) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(out);
+    return pool_alloc_raw(nbytes, out);
+}
+
 int bship_free(void* p) {
     BSHIP_REQUIRE_INIT();
     return pool_free_raw(p);

@@ -189,7 +189,7 @@ class HipHandler(Handler):
         for name, a in pitched:
             key = (a._base, a.shape, a.pitch)
             if key not in temps:                 # the same view twice (out is an input): one temporary
-                t = self.allocate(a.shape)
+                t = self._scratch(a.shape)
                 self._copy2d(a, t, True)
                 temps[key] = t
             bound.arguments[name] = temps[key]
@@ -252,11 +252,22 @@ class HipHandler(Handler):
         self._call(self._lib.bship_malloc(n * 4, ctypes.byref(p)))
         return DeviceArray(p.value, shape, _Block(p.value, self._free), self)
 
+    def _scratch(self, shape):
+        """An array with arbitrary content, for buffers that are overwritten completely before use."""
+        n = _prod(shape)
+        if n == 0:
+            return DeviceArray(0, tuple(shape), None, self)
+        p = ctypes.c_void_p()
+        self._call(self._lib.bship_malloc_scratch(n * 4, ctypes.byref(p)))
+        return DeviceArray(p.value, tuple(shape), _Block(p.value, self._free), self)
+
     def zeros(self, shape):
         return self.allocate(shape)
 
     def ones(self, shape):
-        a = self.allocate(shape)
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        a = self._scratch(tuple(int(s) for s in shape))
         self.fill(a, 1.0)
         return a
 
@@ -272,7 +283,7 @@ class HipHandler(Handler):
 
     def create_from_numpy(self, arr):
         arr = np.asarray(arr, dtype=np.float32, order='C')    # keeps 0-d arrays 0-d
-        out = self.allocate(arr.shape)
+        out = self._scratch(arr.shape)
         if out.size:
             self._call(self._lib.bship_h2d(out.ptr, arr.ctypes.data, arr.nbytes))
         return out
@@ -480,12 +491,12 @@ class HipHandler(Handler):
         oh, ow = outputs.shape[1], outputs.shape[2]
         kc = kh * kw * c
         rows = n * oh * ow
-        col = self.allocate((rows, kc))
+        col = self._scratch((rows, kc))       # im2col writes every element
         self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
                                                    padding, stride[0], stride[1]))
-        out2d = outputs.reshape((rows, f))
-        self._gemm(col, weights.reshape((f, kc)), out2d, False, True, 0.0)
-        self._mv(ADD, out2d, bias.reshape((1, f)), out2d, 0)
+        # product and bias in one call (the bias goes into the product's epilogue)
+        self._call(self._lib.bship_gemm_bias_f32(0, 1, rows, f, kc, col.ptr, kc, weights.ptr, kc,
+                                                 bias.ptr, outputs.ptr, f))
 
     def conv2d_backward_batch(self, inputs, weights, padding, stride, in_deltas, out_deltas,
                               weight_deltas, bias_deltas):
@@ -495,7 +506,7 @@ class HipHandler(Handler):
         oh, ow = out_deltas.shape[1], out_deltas.shape[2]
         kc = kh * kw * c
         rows = n * oh * ow
-        col = self.allocate((rows, kc))
+        col = self._scratch((rows, kc))       # im2col writes every element
         self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
                                                    padding, stride[0], stride[1]))
         dy = out_deltas.reshape((rows, f))

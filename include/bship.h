@@ -96,6 +96,11 @@ int bship_graph_destroy(int graph_id);
  * handlers return zeros from allocate, and lstm_layer.py 167/258 depends on
  * it). nbytes == 0 yields *out = NULL and status 0. */
 int bship_malloc(size_t nbytes, void** out);
+/* The same without the zero fill, for buffers that their owner overwrites
+ * completely before reading them (the col matrix of conv2d_*_batch, numpy 122
+ * and 156-157, which the reference allocates once per image; upload targets).
+ * The content is whatever the block's previous owner left. */
+int bship_malloc_scratch(size_t nbytes, void** out);
 /* Returns a block to the pool cache (no hipFree). NULL is a no-op. */
 int bship_free(void* p);
 /* hipFree()s every cached (unused) block. Blocks. */
@@ -244,6 +249,13 @@ int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host,
 int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int64_t K,
                    float alpha, const float* A, int64_t lda, const float* B,
                    int64_t ldb, float beta, float* C, int64_t ldc);
+/* The product and bias of conv2d_forward_batch (numpy 149-171: out[i] = col . W^T,
+ * then outputs += bias) in one call: C(M,N) = op(A) op(B) + bias, bias N elements,
+ * one per column of C, added to the float32 accumulator in the product's epilogue
+ * (the same single rounding as a separate add_mv over the stored product). */
+int bship_gemm_bias_f32(int transa, int transb, int64_t M, int64_t N, int64_t K,
+                        const float* A, int64_t lda, const float* B, int64_t ldb,
+                        const float* bias, float* C, int64_t ldc);
 
 /* im2col of a whole NHWC batch (_cpuop 251-277 applied per image by numpy
  * 158-166): col is (n*out_h*out_w, kh*kw*c). */

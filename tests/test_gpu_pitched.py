@@ -100,13 +100,14 @@ def test_matrix_products_take_pitched_operands_as_they_are(php):
     w = rng.standard_normal((7, 6)).astype(F32)
     dev_hub, dev_w = php.create_from_numpy(hub), php.create_from_numpy(w)
     allocations = []
-    real_allocate = php.allocate
+    real_allocate, real_scratch = php.allocate, php._scratch
     php.allocate = lambda shape: allocations.append(shape) or real_allocate(shape)
+    php._scratch = lambda shape: allocations.append(shape) or real_scratch(shape)
     try:
         php.dot_mm(dev_hub[:, 3:9], dev_w, dev_hub[:, 20:27], transb=True)      # (9,6) . (7,6)^T -> (9,7)
         php.dot_add_mm(dev_hub[:, 20:27], dev_w, dev_hub[:, 30:36])             # += (9,7) . (7,6)
     finally:
-        php.allocate = real_allocate
+        php.allocate, php._scratch = real_allocate, real_scratch
     assert allocations == [], allocations
     want = hub.copy()
     want[:, 20:27] = want[:, 3:9] @ w.T
