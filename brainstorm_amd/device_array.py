@@ -86,7 +86,7 @@ class DeviceArray:
     # NumPy evaluates `x ** 0.5` as sqrt and `x ** 2` as x * x, so do these.
     def _binary(self, other, tt, st):
         h = self._handler
-        out = h.allocate(self.shape)
+        out = h._scratch(self.shape)         # every element is written by the operation below
         if isinstance(other, DeviceArray):
             if other.shape != self.shape:
                 raise ValueError("operands have shapes %r and %r; broadcasting is not supported"
@@ -116,7 +116,7 @@ class DeviceArray:
 
     def __pow__(self, exponent):
         h = self._handler
-        out = h.allocate(self.shape)
+        out = h._scratch(self.shape)         # every element is written by the operation below
         if exponent == 0.5:
             h.sqrt_t(self, out)
         elif exponent == 2:
