@@ -234,6 +234,45 @@ def run_image_ops(hip, n_img=2048, reps=10):
     return out
 
 
+def run_pitched_ops(rows=8192, cols=8192, reps=10):
+    """Operations on row-pitched views: three (rows, cols) feature slices of one (rows, 3*cols) hub,
+    as the layers writing side by side into a hub see them (buffer_structure.py:232-245). For each
+    operation the fraction of peak with the row-pitched kernels and with the dense-temporaries path."""
+    from brainstorm_amd import HipHandler
+    hip = HipHandler(seed=0, pitched_views=True)
+    lib = hip._lib
+    ms = ctypes.c_float()
+    hub = hip.allocate((rows, 3 * cols))
+    hip.fill(hub, 0.25)
+    a, b, o = hub[:, :cols], hub[:, cols:2 * cols], hub[:, 2 * cols:]
+    row, col = hip.allocate((1, cols)), hip.allocate((rows, 1))
+    n = rows * cols
+    cases = [("add_tt", 12 * n, lambda: hip.add_tt(a, b, o)),
+             ("tanh", 8 * n, lambda: hip.tanh(a, o)),
+             ("mult_add_st", 12 * n, lambda: hip.mult_add_st(0.5, a, o)),
+             ("add_mv_row", 8 * n, lambda: hip.add_mv(a, row, o)),
+             ("mult_mv_col", 8 * n, lambda: hip.mult_mv(a, col, o)),
+             ("sum_t_axis0", 4 * n, lambda: hip.sum_t(a, 0, row)),
+             ("sum_t_axis1", 4 * n, lambda: hip.sum_t(a, 1, col)),
+             ("copy_to", 8 * n, lambda: hip.copy_to(a, o))]
+    out = {}
+    for native in (True, False):
+        hip.native_pitched = native
+        for name, nbytes, fn in cases:
+            for _ in range(2):
+                fn()
+            lib.bship_event_record(0)
+            for _ in range(reps):
+                fn()
+            lib.bship_event_record(1)
+            hip._call(lib.bship_event_elapsed_ms(0, 1, ctypes.byref(ms)))
+            gbps = nbytes / (ms.value / reps * 1e-3) / 1e9
+            out.setdefault(name, {})["row_pitched_kernels" if native else "dense_temporaries"] = {
+                "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    hip.native_pitched = True
+    return out
+
+
 def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
     """Training steps per second of one network workload (forward + backward + momentum update,
     inputs uploaded once; the per-step loss read-back of a Trainer is included). recorded: the
@@ -336,6 +375,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-nets", action="store_true", help="skip the MLP/LSTM samples/s runs")
     ap.add_argument("--no-image-ops", action="store_true", help="skip the im2col/col2im/pooling measurements")
+    ap.add_argument("--no-pitched", action="store_true", help="skip the operations on row-pitched views")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the handler path has no multi-GPU part "
@@ -380,6 +420,8 @@ def main():
     }
     if not args.no_image_ops:
         out["image_ops"] = run_image_ops(hip)
+    if not args.no_pitched:
+        out["pitched_ops"] = run_pitched_ops()
     if not args.no_nets:
         # second part of the metric: training samples/s of the MLP and LSTM workloads
         out["nets"] = run_nets_gpu(hip)

@@ -19,6 +19,8 @@ ADD_ST, MULT_ST, MULT_ADD_ST = 0, 1, 2
 ABS, SIGN, SQRT, LOG, SIGMOID, TANH, REL, EL = 0, 1, 2, 3, 4, 5, 6, 7
 SIGMOID_DERIV, TANH_DERIV, REL_DERIV, EL_DERIV = 0, 1, 2, 3
 COPY_IF, FILL_IF, ADD_IF = 0, 1, 2
+(PITCHED_BINARY, PITCHED_MULT_ADD, PITCHED_SCALAR, PITCHED_UNARY, PITCHED_DERIV, PITCHED_CLIP, PITCHED_COND,
+ PITCHED_FILL) = range(8)
 
 ERR_OUT_OF_MEMORY = -5
 
@@ -55,10 +57,13 @@ SIGNATURES = {
     "bship_clip_f32": [_P, c_float, c_float, _P, c_size_t],
     "bship_cond_f32": [c_int, _P, c_float, _P, _P, c_size_t],
     "bship_mv_f32": [c_int, _P, _P, _P, _I64, _I64, c_int, c_int],
+    "bship_elementwise_pitched_f32": [c_int, c_int, c_float, c_float, _P, _I64, c_int, _P, _I64, c_int,
+                                      _P, _I64, _I64, _I64],
     "bship_broadcast_f32": [_P, _P, _I64, _I64, _I64],
     "bship_merge_f32": [_P, _P, _P, _I64, _I64, _I64],
     "bship_split_add_f32": [_P, _P, _P, _I64, _I64, _I64],
     "bship_sum_f32": [_P, _P, _I64, _I64, c_int],
+    "bship_sum_pitched_f32": [_P, _I64, _P, _I64, _I64, c_int],
     "bship_softmax_rows_f32": [_P, _P, _I64, _I64],
     "bship_isfinite_f32": [_P, c_size_t, POINTER(c_int)],
     "bship_binarize_f32": [_P, _P, _I64, _I64],

@@ -44,7 +44,7 @@ struct PlainSrc {
 // narrower matrices (bias gradients of small layers, image channels) take CL = 8, 16 or 32 so
 // that the lanes that would have no column walk down more rows instead.
 template <int W, bool AL, int CL, typename Src>
-__global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int64_t M, int64_t NW) {
+__global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int64_t M, int64_t NW, int64_t ld) {
     typedef typename VecT<W>::type R;
     constexpr int RL = kBlock / CL;                          // row-lanes
     constexpr int GROUP = 4 * RL;                            // rows per group: 4 per row-lane
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int
     R acc0 = vzero<R>(), acc1 = vzero<R>(), acc2 = vzero<R>(), acc3 = vzero<R>();
     if (c < NW) {
         const int64_t col = c * W;
-        const int64_t pitch = NW * W;
+        const int64_t pitch = ld;                 // elements from one row of the source to the next
         const R cx = src.template prep<W, AL>(col);
         // Groups of rows are dealt round-robin to the row bands (blockIdx.y), so all bands
         // together read one contiguous region that moves down the matrix. (Bands of
@@ -93,27 +93,29 @@ __global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int
 static inline int colsum_lanes(int64_t NW) { return NW > 32 ? 64 : NW > 16 ? 32 : NW > 8 ? 16 : 8; }
 
 template <int W, bool AL, typename Src>
-static void launch_colsum_lanes(int cl, dim3 grid, Src src, float* dst, int64_t M, int64_t NW) {
+static void launch_colsum_lanes(int cl, dim3 grid, Src src, float* dst, int64_t M, int64_t NW, int64_t ld) {
     hipStream_t s = ctx().stream;
     switch (cl) {
-        case 8:  hipLaunchKernelGGL((colsum_kernel<W, AL, 8, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
-        case 16: hipLaunchKernelGGL((colsum_kernel<W, AL, 16, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
-        case 32: hipLaunchKernelGGL((colsum_kernel<W, AL, 32, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
-        default: hipLaunchKernelGGL((colsum_kernel<W, AL, 64, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW); break;
+        case 8:  hipLaunchKernelGGL((colsum_kernel<W, AL, 8, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW, ld); break;
+        case 16: hipLaunchKernelGGL((colsum_kernel<W, AL, 16, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW, ld); break;
+        case 32: hipLaunchKernelGGL((colsum_kernel<W, AL, 32, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW, ld); break;
+        default: hipLaunchKernelGGL((colsum_kernel<W, AL, 64, Src>), grid, dim3(kBlock), 0, s, src, dst, M, NW, ld); break;
     }
 }
 
 template <typename Src>
 static void launch_colsum_kernel(bool vec, bool al, int cl, dim3 grid, Src src, float* dst, int64_t M,
-                                 int64_t NW) {
-    if (vec && al) launch_colsum_lanes<4, true, Src>(cl, grid, src, dst, M, NW);
-    else if (vec)  launch_colsum_lanes<4, false, Src>(cl, grid, src, dst, M, NW);
-    else           launch_colsum_lanes<1, false, Src>(cl, grid, src, dst, M, NW);
+                                 int64_t NW, int64_t ld) {
+    if (vec && al) launch_colsum_lanes<4, true, Src>(cl, grid, src, dst, M, NW, ld);
+    else if (vec)  launch_colsum_lanes<4, false, Src>(cl, grid, src, dst, M, NW, ld);
+    else           launch_colsum_lanes<1, false, Src>(cl, grid, src, dst, M, NW, ld);
 }
 
+// ld: elements from one row of the source matrices to the next (0: dense, ld = N).
 template <typename Src>
-static int launch_colsum(Src src, float* out, int64_t M, int64_t N) {
+static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld = 0) {
     const Context& c = ctx();
+    if (ld == 0) ld = N;
     const bool vec = (N % 4 == 0);
     const int64_t NW = vec ? N / 4 : N;
     const int cl = colsum_lanes(NW);
@@ -133,14 +135,15 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N) {
         partial = static_cast<float*>(p);
         dst = partial;
     }
-    launch_colsum_kernel(vec, src.aligned() && aligned16(dst), cl,
-                         dim3(static_cast<unsigned>(gx), static_cast<unsigned>(bands)), src, dst, M, NW);
+    // 16-byte accesses need every row start aligned: the base, and a pitch of whole vectors
+    launch_colsum_kernel(vec, src.aligned() && aligned16(dst) && ld % 4 == 0, cl,
+                         dim3(static_cast<unsigned>(gx), static_cast<unsigned>(bands)), src, dst, M, NW, ld);
     int st = check_launch("sum over axis 0");
     if (partial) {
         if (st == 0) {
             // second stage: column sums of the (bands, N) partials in one band
             launch_colsum_kernel(vec, aligned16(partial) && aligned16(out), cl,
-                                 dim3(static_cast<unsigned>(gx), 1), PlainSrc{partial}, out, bands, NW);
+                                 dim3(static_cast<unsigned>(gx), 1), PlainSrc{partial}, out, bands, NW, N);
             st = check_launch("sum over axis 0, stage 2");
         }
         pool_free_raw(partial);   // a later owner of the block runs after this launch

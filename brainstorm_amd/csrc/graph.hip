@@ -28,7 +28,7 @@ struct GraphRec {
 std::mutex g_graph_mutex;
 std::map<int, GraphRec> g_graphs;
 int g_next_graph = 1;
-int g_recording = 0;
+std::atomic<int> g_recording{0};   // read by every entry point without the mutex
 
 void destroy_rec(int id, GraphRec& rec) {
     if (rec.exec) (void)hipGraphExecDestroy(rec.exec);
@@ -81,7 +81,7 @@ int bship_graph_end(int* graph_id) {
     std::lock_guard<std::mutex> lock(g_graph_mutex);
     if (!g_recording)
         return set_error(BSHIP_ERR_UNSUPPORTED, "bship_graph_end: no step is being recorded");
-    const int id = g_recording;
+    const int id = g_recording.load();
     GraphRec rec;
     int st = rng_graph_end(id);
     const hipError_t e = hipStreamEndCapture(ctx().stream, &rec.graph);

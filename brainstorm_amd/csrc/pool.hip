@@ -183,13 +183,22 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
 }
 
 // dst(rows, cols) with row pitch ld_dst = src(rows, cols) with row pitch ld_src; pitches in
-// elements. One workgroup per tile of kBlock columns of one row.
+// elements. 2^L lanes share a row (the power of two that covers its 128-bit accesses, 256 at
+// most), so a workgroup covers 2^(8-L) rows x one tile of 2^L accesses. Rows of a pitched view
+// start anywhere: the accesses promise 4-byte alignment only.
 __global__ __launch_bounds__(kBlock) void copy2d_kernel(const float* __restrict__ src, int64_t ld_src,
-                                                        float* __restrict__ dst, int64_t ld_dst,
-                                                        int64_t cols, unsigned tiles_per_row) {
-    const int64_t row = blockIdx.x / tiles_per_row;
-    const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
-    if (c < cols) dst[row * ld_dst + c] = src[row * ld_src + c];
+                                                        float* __restrict__ dst, int64_t ld_dst, int64_t rows,
+                                                        int64_t cols, unsigned tiles_per_row, int L) {
+    const int64_t row = (static_cast<int64_t>(blockIdx.x / tiles_per_row) << (8 - L)) + (threadIdx.x >> L);
+    const int64_t c = ((static_cast<int64_t>(blockIdx.x % tiles_per_row) << L) + (threadIdx.x & ((1u << L) - 1))) * 4;
+    if (row >= rows || c >= cols) return;
+    const float* s = src + row * ld_src + c;
+    float* d = dst + row * ld_dst + c;
+    if (c + 4 <= cols) {
+        vstore<4, false>(d, vload<4, false>(s));
+    } else {
+        for (int64_t j = 0; c + j < cols; ++j) d[j] = s[j];
+    }
 }
 
 int launch_fill(float* p, float val, size_t n) {
@@ -365,10 +374,13 @@ int bship_copy2d_f32(float* dst, int64_t ld_dst, const float* src, int64_t ld_sr
     BSHIP_REQUIRE_F32_ALIGNED(src);
     BSHIP_REQUIRE_DIM(ld_dst >= cols && ld_src >= cols);
     if (ld_dst == cols && ld_src == cols) return bship_d2d(dst, src, static_cast<size_t>(rows * cols) * 4);
-    const int64_t tiles_per_row = ceil_div(cols, kBlock);
-    BSHIP_REQUIRE_DIM(tiles_per_row * rows <= 0x7fffffff);
-    hipLaunchKernelGGL(copy2d_kernel, dim3(static_cast<unsigned>(tiles_per_row * rows)), dim3(kBlock), 0,
-                       ctx().stream, src, ld_src, dst, ld_dst, cols, static_cast<unsigned>(tiles_per_row));
+    int L = 0;
+    while (L < 8 && (int64_t(4) << L) < cols) ++L;
+    const int64_t tiles_per_row = ceil_div(cols, int64_t(4) << L);
+    const int64_t row_groups = ceil_div(rows, int64_t(1) << (8 - L));
+    BSHIP_REQUIRE_DIM(tiles_per_row * row_groups <= 0x7fffffff);
+    hipLaunchKernelGGL(copy2d_kernel, dim3(static_cast<unsigned>(tiles_per_row * row_groups)), dim3(kBlock), 0,
+                       ctx().stream, src, ld_src, dst, ld_dst, rows, cols, static_cast<unsigned>(tiles_per_row), L);
     return check_launch("copy2d");
 }
 

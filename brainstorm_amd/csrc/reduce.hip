@@ -16,7 +16,7 @@ namespace bship {
 template <int W, bool AL, int THREADS>
 __global__ __launch_bounds__(kBlock) void rowsum_kernel(const float* __restrict__ a,
                                                         float* __restrict__ out, int64_t M,
-                                                        int64_t N) {
+                                                        int64_t N, int64_t ld) {
     constexpr int ROWS = kBlock / THREADS;
     typedef typename VecT<W>::type R;
     __shared__ float lds[kBlock / kWave];
@@ -25,7 +25,7 @@ __global__ __launch_bounds__(kBlock) void rowsum_kernel(const float* __restrict_
     float total = 0.0f;
     if (row < M) {
         const int64_t NW = N / W;
-        const float* p = a + row * N;
+        const float* p = a + row * ld;
         R acc0 = vzero<R>(), acc1 = vzero<R>(), acc2 = vzero<R>(), acc3 = vzero<R>();
         int64_t i = t;
         for (; i + 3 * THREADS < NW; i += 4 * THREADS) {
@@ -53,36 +53,37 @@ __global__ __launch_bounds__(kBlock) void rowsum_kernel(const float* __restrict_
 // One thread per row, for very short rows.
 __global__ __launch_bounds__(kBlock) void rowsum_small_kernel(const float* __restrict__ a,
                                                               float* __restrict__ out, int64_t M,
-                                                              int64_t N) {
+                                                              int64_t N, int64_t ld) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (row >= M) return;
     float s = 0.0f;
-    for (int64_t j = 0; j < N; ++j) s += a[row * N + j];
+    for (int64_t j = 0; j < N; ++j) s += a[row * ld + j];
     out[row] = s;
 }
 
 template <int THREADS>
 static void launch_rowsum_kernel(bool vec, bool al, dim3 grid, const float* a, float* out,
-                                 int64_t M, int64_t N) {
+                                 int64_t M, int64_t N, int64_t ld) {
     hipStream_t s = ctx().stream;
-    if (vec && al) hipLaunchKernelGGL((rowsum_kernel<4, true, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
-    else if (vec)  hipLaunchKernelGGL((rowsum_kernel<4, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
-    else           hipLaunchKernelGGL((rowsum_kernel<1, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N);
+    if (vec && al) hipLaunchKernelGGL((rowsum_kernel<4, true, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N, ld);
+    else if (vec)  hipLaunchKernelGGL((rowsum_kernel<4, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N, ld);
+    else           hipLaunchKernelGGL((rowsum_kernel<1, false, THREADS>), grid, dim3(kBlock), 0, s, a, out, M, N, ld);
 }
 
-static int launch_rowsum(const float* a, float* out, int64_t M, int64_t N) {
+// ld: elements from one row of a to the next (N for a dense matrix)
+static int launch_rowsum(const float* a, float* out, int64_t M, int64_t N, int64_t ld) {
     if (N <= 16) {
         hipLaunchKernelGGL(rowsum_small_kernel, dim3(static_cast<unsigned>(ceil_div(M, kBlock))),
-                           dim3(kBlock), 0, ctx().stream, a, out, M, N);
+                           dim3(kBlock), 0, ctx().stream, a, out, M, N, ld);
         return check_launch("sum_t(axis=1) small");
     }
-    // every row starts on a 16-byte boundary only if N % 4 == 0 and the base does
+    // every row starts on a 16-byte boundary only if the pitch is a whole number of vectors and the base does
     const bool vec = (N % 4 == 0);
-    const bool al = aligned16(a);
+    const bool al = aligned16(a) && ld % 4 == 0;
     if (N <= 2048)
-        launch_rowsum_kernel<kWave>(vec, al, dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), a, out, M, N);
+        launch_rowsum_kernel<kWave>(vec, al, dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), a, out, M, N, ld);
     else
-        launch_rowsum_kernel<kBlock>(vec, al, dim3(static_cast<unsigned>(M)), a, out, M, N);
+        launch_rowsum_kernel<kBlock>(vec, al, dim3(static_cast<unsigned>(M)), a, out, M, N, ld);
     return check_launch("sum_t(axis=1)");
 }
 
@@ -147,7 +148,7 @@ static int launch_sumall(const float* a, float* out, int64_t n) {
     int st = check_launch("sum_t(axis=None) stage 1");
     if (partial) {
         if (st == 0) {
-            launch_rowsum_kernel<kBlock>(false, false, dim3(1), partial, out, 1, chunks);
+            launch_rowsum_kernel<kBlock>(false, false, dim3(1), partial, out, 1, chunks, chunks);
             st = check_launch("sum_t(axis=None) stage 2");
         }
         pool_free_raw(partial);
@@ -345,8 +346,13 @@ using namespace bship;
 extern "C" {
 
 int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
+    return bship_sum_pitched_f32(a, N, out, M, N, axis);
+}
+
+int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, int64_t N, int axis) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    BSHIP_REQUIRE_DIM(ld_a >= N);
     BSHIP_REQUIRE_DIM(axis == 0 || axis == 1 || axis == -1);
     const int64_t out_n = axis == 0 ? N : (axis == 1 ? M : 1);
     if (out_n == 0) return 0;
@@ -357,9 +363,17 @@ int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
     BSHIP_REQUIRE_F32_ALIGNED(a);
     BSHIP_REQUIRE_DIM(a != out);
     BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
-    if (axis == 0) return M == 1 ? bship_d2d(out, a, static_cast<size_t>(N) * 4) : launch_colsum(PlainSrc{a}, out, M, N);
-    if (axis == 1) return N == 1 ? bship_d2d(out, a, static_cast<size_t>(M) * 4) : launch_rowsum(a, out, M, N);
-    return launch_sumall(a, out, M * N);
+    if (axis == 0) return M == 1 ? bship_d2d(out, a, static_cast<size_t>(N) * 4) : launch_colsum(PlainSrc{a}, out, M, N, ld_a);
+    if (axis == 1) return N == 1 && ld_a == 1 ? bship_d2d(out, a, static_cast<size_t>(M) * 4) : launch_rowsum(a, out, M, N, ld_a);
+    if (ld_a == N || M == 1) return launch_sumall(a, out, M * N);
+    // everything, row-pitched: row sums, then their sum
+    void* rows = nullptr;
+    int st = pool_alloc_raw(static_cast<size_t>(M) * sizeof(float), &rows);
+    if (st != 0) return st;
+    st = launch_rowsum(a, static_cast<float*>(rows), M, N, ld_a);
+    if (st == 0) st = launch_sumall(static_cast<const float*>(rows), out, M);
+    pool_free_raw(rows);
+    return st;
 }
 
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N) {

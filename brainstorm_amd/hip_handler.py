@@ -18,8 +18,9 @@ import numpy as np
 
 from . import _lib
 from ._lib import (ABS, ADD, ADD_IF, ADD_ST, COPY_IF, DIV, EL, EL_DERIV, FILL_IF, FMOD, LOG, MUL,
-                   MULT_ADD_ST, MULT_ST, REL, REL_DERIV, SIGMOID, SIGMOID_DERIV, SIGN, SQRT, SUB,
-                   TANH, TANH_DERIV)
+                   MULT_ADD_ST, MULT_ST, PITCHED_BINARY, PITCHED_CLIP, PITCHED_COND, PITCHED_DERIV,
+                   PITCHED_FILL, PITCHED_MULT_ADD, PITCHED_SCALAR, PITCHED_UNARY, REL, REL_DERIV, SIGMOID,
+                   SIGMOID_DERIV, SIGN, SQRT, SUB, TANH, TANH_DERIV)
 from .device_array import DeviceArray, PitchedDeviceArray, _Block, _prod
 from .handler_api import Handler
 
@@ -48,6 +49,8 @@ class HipRandomState:
         if not 0 <= seed < 2 ** 32:
             raise ValueError("seed must be between 0 and 2**32 - 1")
         self._handler._call(self._handler._lib.bship_rng_seed(seed))
+        if self._handler.fast_masks:               # the optional mask stream restarts with it
+            self._handler._call(self._handler._lib.bship_fast_rng_seed(seed))
         self._seed = seed
 
     def get_seed(self):
@@ -96,6 +99,48 @@ class RecordedStep(object):
             pass
 
 
+class _NoNativePath(Exception):
+    """The operands of a call on row-pitched views do not fit the row-pitched kernels."""
+
+
+def _native_pitched_table():
+    """Handler operation -> function(handler, arguments) that runs it on row-pitched operands as they
+    are (bship_elementwise_pitched_f32, bship_sum_pitched_f32, bship_copy2d_f32)."""
+    def ew(family, op, out, a=None, b=None, s0=None, s1=None):
+        def run(h, A):
+            h._pitched_elementwise(family, op, A[out], A[a] if a else None, A[b] if b else None,
+                                   A[s0] if s0 else 0.0, A[s1] if s1 else 0.0)
+        return run
+
+    def mv(family, op):
+        def run(h, A):
+            h._pitched_elementwise(family, op, A["out"], A["m"], A["v"], 0.0, 0.0, b_is_vector=True)
+        return run
+
+    table = {"mult_add_tt": ew(PITCHED_MULT_ADD, 0, "out", "a", "b"),
+             "clip_t": ew(PITCHED_CLIP, 0, "out", "a", None, "a_min", "a_max"),
+             "fill": ew(PITCHED_FILL, 0, "mem", None, None, "val"),
+             "copy_to_if": ew(PITCHED_COND, COPY_IF, "dest", "src", "cond"),
+             "fill_if": ew(PITCHED_COND, FILL_IF, "mem", None, "cond", "val"),
+             "add_into_if": ew(PITCHED_COND, ADD_IF, "out", "a", "cond"),
+             "mult_add_mv": mv(PITCHED_MULT_ADD, 0),
+             "copy_to": lambda h, A: h._pitched_copy(A["src"], A["dest"]),
+             "sum_t": lambda h, A: h._pitched_sum(A["a"], A["axis"], A["out"])}
+    for name, op in (("add", ADD), ("subtract", SUB), ("mult", MUL), ("divide", DIV)):
+        table[name + "_tt"] = ew(PITCHED_BINARY, op, "out", "a", "b")
+        table[name + "_mv"] = mv(PITCHED_BINARY, op)
+    table["modulo_tt"] = ew(PITCHED_BINARY, FMOD, "out", "a", "b")
+    for name, op in (("add_st", ADD_ST), ("mult_st", MULT_ST), ("mult_add_st", MULT_ADD_ST)):
+        table[name] = ew(PITCHED_SCALAR, op, "out", "t", None, "s")
+    for name, op in (("abs_t", ABS), ("sign_t", SIGN), ("sqrt_t", SQRT), ("log_t", LOG)):
+        table[name] = ew(PITCHED_UNARY, op, "out", "a")
+    for name, op, dop in (("sigmoid", SIGMOID, SIGMOID_DERIV), ("tanh", TANH, TANH_DERIV),
+                          ("rel", REL, REL_DERIV), ("el", EL, EL_DERIV)):
+        table[name] = ew(PITCHED_UNARY, op, "y", "x")
+        table[name + "_deriv"] = ew(PITCHED_DERIV, dop, "dx", "y", "dy")
+    return table
+
+
 class HipHandler(Handler):
     __undescribed__ = {'context', 'dtype', 'EMPTY', 'rnd'}
 
@@ -111,6 +156,7 @@ class HipHandler(Handler):
         # on them through dense temporaries. Off by default: it puts a Python-level argument
         # check in front of every operation.
         self.pitched_views = bool(pitched_views)
+        self.native_pitched = True      # False: every call on a pitched view goes through dense temporaries
         if self.pitched_views:
             self._install_pitched_wrappers()        # before the activation tables bind the methods
         super(HipHandler, self).__init__()
@@ -121,10 +167,8 @@ class HipHandler(Handler):
         self.context = self._lib
         self._free = self._lib.bship_free
         self.EMPTY = DeviceArray(0, (0,), None, self)
-        self.rnd = HipRandomState(self, seed)
         self.fast_masks = bool(fast_masks)
-        if self.fast_masks:
-            self._call(self._lib.bship_fast_rng_seed(int(self.rnd.get_seed())))
+        self.rnd = HipRandomState(self, seed)
 
     def __describe__(self):
         return {'@type': self.__class__.__name__}
@@ -172,8 +216,56 @@ class HipHandler(Handler):
                 else (pitched._base, pitched.pitch, dense.ptr, cols))
         self._call(self._lib.bship_copy2d_f32(*args, pitched.rows, cols))
 
+    _NATIVE_PITCHED = _native_pitched_table()
+
+    def _as_matrix(self, a, rows, cols):
+        """(address, elements from row to row) of `a` read as a (rows, cols) matrix."""
+        if type(a) is PitchedDeviceArray:
+            if a.shape[-1] != cols or a.rows != rows:
+                raise _NoNativePath()
+            return a._base, a.pitch
+        if a.size != rows * cols:
+            raise _NoNativePath()
+        return a.ptr, cols
+
+    def _pitched_elementwise(self, family, op, out, a, b, s0, s1, b_is_vector=False):
+        cols = out.shape[-1] if out.shape else 1
+        rows = out.size // cols if cols else 0
+        po, ldo = self._as_matrix(out, rows, cols)
+        pa, lda = self._as_matrix(a, rows, cols) if a is not None else (None, 0)
+        pb, rsb, csb = None, 0, 1
+        if b is not None and b_is_vector and b.shape != a.shape:
+            vs = b.shape
+            pitched = type(b) is PitchedDeviceArray
+            if b.size == cols and (len(vs) == 1 or vs[0] == 1 or rows == 1) and not (pitched and b.rows != 1):
+                pb, rsb, csb = b._address(), 0, 1                      # row vector
+            elif b.size == rows and vs[-1] == 1:
+                pb, rsb, csb = b._address(), (b.pitch if pitched else 1), 0     # column vector
+            else:
+                raise _NoNativePath()
+        elif b is not None:
+            pb, rsb = self._as_matrix(b, rows, cols)
+        self._call(self._lib.bship_elementwise_pitched_f32(family, op, s0, s1, pa, lda, 1, pb, rsb, csb,
+                                                           po, ldo, rows, cols))
+
+    def _pitched_copy(self, src, dest):
+        cols = dest.shape[-1] if dest.shape else 1
+        rows = dest.size // cols if cols else 0
+        pd, ldd = self._as_matrix(dest, rows, cols)
+        ps, lds = self._as_matrix(src, rows, cols)
+        self._call(self._lib.bship_copy2d_f32(pd, ldd, ps, lds, rows, cols))
+
+    def _pitched_sum(self, a, axis, out):
+        if (type(a) is not PitchedDeviceArray or type(out) is PitchedDeviceArray
+                or (axis is not None and (a.ndim != 2 or axis not in (0, 1)))):
+            raise _NoNativePath()
+        cols = a.shape[-1]
+        self._call(self._lib.bship_sum_pitched_f32(a._base, a.pitch, out.ptr, a.rows, cols,
+                                                   -1 if axis is None else axis))
+
     def _dense_call(self, fn, sig, written, *args, **kwargs):
-        """Runs fn with every row-pitched operand replaced by a dense temporary."""
+        """Runs fn on row-pitched operands: with the row-pitched kernels where they cover the call,
+        else with every such operand replaced by a dense temporary."""
         for a in args:
             if type(a) is PitchedDeviceArray:
                 break
@@ -184,6 +276,12 @@ class HipHandler(Handler):
             else:
                 return fn(self, *args, **kwargs)         # the usual case: nothing to do
         bound = sig.bind(self, *args, **kwargs)
+        native = self._NATIVE_PITCHED.get(fn.__name__) if self.native_pitched else None
+        if native is not None:
+            try:
+                return native(self, bound.arguments)
+            except _NoNativePath:
+                pass                                 # e.g. operands of different row lengths
         pitched = [(k, a) for k, a in bound.arguments.items() if type(a) is PitchedDeviceArray]
         temps = {}
         for name, a in pitched:

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define BSHIP_VERSION 200 /* major*10000 + minor*100 + patch */
+#define BSHIP_VERSION 300 /* major*10000 + minor*100 + patch */
 
 /* argument / state errors (negative so they never collide with hipError_t) */
 #define BSHIP_ERR_NOT_INITIALIZED (-1)
@@ -204,11 +204,52 @@ int bship_merge_f32(const float* a, const float* b, float* out, int64_t rows,
 int bship_split_add_f32(const float* x, float* oa, float* ob, int64_t rows,
                         int64_t na, int64_t nb);
 
+/* ------------------------- row-pitched operands -------------------------- */
+
+/* Every elementwise operation above, and the matrix (op) vector operations, on
+ * (rows, cols) operands whose rows lie a pitch apart: the feature slices
+ * hub[:, :, a:b] of a hub that several layers write side by side
+ * (buffer_structure.py 232-245), which NumpyHandler reaches through NumPy's
+ * strides (numpy_handler.py: the same lines as the dense forms).
+ * `family` selects the dense entry point whose arithmetic is applied and `op`
+ * its operation code; the results equal the dense ones bit for bit.
+ *   family                 op codes of            inputs                 scalars
+ *   BSHIP_PITCHED_BINARY   bship_binary_f32       a, b                   -
+ *   BSHIP_PITCHED_MULT_ADD -                      a, b   (out += a*b)    -
+ *   BSHIP_PITCHED_SCALAR   bship_scalar_f32       a = t                  s0 = s
+ *   BSHIP_PITCHED_UNARY    bship_unary_f32        a = x                  -
+ *   BSHIP_PITCHED_DERIV    bship_deriv_f32        a = y, b = dy          -
+ *   BSHIP_PITCHED_CLIP     -                      a                      s0 = lo, s1 = hi
+ *   BSHIP_PITCHED_COND     bship_cond_f32         a (not FILL_IF), b = cond   s0 = val
+ *   BSHIP_PITCHED_FILL     -                      -                      s0 = val
+ * An input is a matrix (row stride = its pitch in elements, column stride 1),
+ * a row vector (row stride 0, column stride 1) or a column vector (row stride
+ * 1, column stride 0): with a vector for b, BINARY is add_mv / subtract_mv /
+ * mult_mv / divide_mv and MULT_ADD is mult_add_mv. out is (rows, cols) with
+ * ld_out elements from one row to the next and may be one of the inputs. */
+enum {
+    BSHIP_PITCHED_BINARY = 0,
+    BSHIP_PITCHED_MULT_ADD = 1,
+    BSHIP_PITCHED_SCALAR = 2,
+    BSHIP_PITCHED_UNARY = 3,
+    BSHIP_PITCHED_DERIV = 4,
+    BSHIP_PITCHED_CLIP = 5,
+    BSHIP_PITCHED_COND = 6,
+    BSHIP_PITCHED_FILL = 7
+};
+int bship_elementwise_pitched_f32(int family, int op, float s0, float s1,
+                                  const float* a, int64_t a_row_stride, int a_col_stride,
+                                  const float* b, int64_t b_row_stride, int b_col_stride,
+                                  float* out, int64_t ld_out, int64_t rows, int64_t cols);
+
 /* ------------------------------ reductions ------------------------------- */
 
 /* sum_t (numpy 268-273, pycuda 375-381) of a (M,N): axis 0 -> out[N],
  * axis 1 -> out[M], axis -1 (None) -> out[1]. Deterministic (no float atomics). */
 int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis);
+/* The same for a row-pitched a: ld_a elements from one row to the next (>= N).
+ * out is dense. With ld_a == N this is bship_sum_f32. */
+int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, int64_t N, int axis);
 /* softmax_m (numpy 292-295, pycuda 403-408): row-wise, one pass over HBM. */
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N);
 /* is_fully_finite (numpy 69-70, pycuda 111-114). *result_host = 1 if every

@@ -61,6 +61,12 @@ def test_fast_masks_match_the_oracle_generator():
     g = hip.allocate((33,))
     hip.fill_gaussian(0.0, 1.0, g)
     assert_bit_equal(hip.get_numpy_copy(g), np.random.RandomState(4711).standard_normal(33).astype(F32), "fill_gaussian")
+    # re-seeding the handler's random state restarts the mask stream too
+    hip.rnd.seed(99)
+    assert hip.fast_mask_state() == (99, 0)
+    hip.generate_probability_mask(a, 0.5)
+    wa, _ = philox.probability_mask(a.size, 0.5, 99, 0)
+    assert_bit_equal(hip.get_numpy_copy(a), wa.reshape(a.shape), "mask after re-seeding")
 
 
 def test_default_handler_keeps_numpys_stream():

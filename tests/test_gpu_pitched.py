@@ -92,6 +92,92 @@ def test_operations_on_pitched_slices(php, name, call):
             np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=name + ": " + tag)
 
 
+NATIVE_OPS = [
+    ("add_tt", lambda h, a, b, o, r, c: h.add_tt(a, b, o)),
+    ("subtract_tt in place", lambda h, a, b, o, r, c: h.subtract_tt(a, b, a)),
+    ("mult_tt", lambda h, a, b, o, r, c: h.mult_tt(a, b, o)),
+    ("divide_tt", lambda h, a, b, o, r, c: h.divide_tt(a, b, o)),
+    ("modulo_tt", lambda h, a, b, o, r, c: h.modulo_tt(a, b, o)),
+    ("mult_add_tt", lambda h, a, b, o, r, c: h.mult_add_tt(a, b, o)),
+    ("add_st", lambda h, a, b, o, r, c: h.add_st(1.5, a, o)),
+    ("mult_st in place", lambda h, a, b, o, r, c: h.mult_st(-0.7, a, a)),
+    ("mult_add_st", lambda h, a, b, o, r, c: h.mult_add_st(0.3, a, o)),
+    ("abs_t", lambda h, a, b, o, r, c: h.abs_t(a, o)),
+    ("sign_t", lambda h, a, b, o, r, c: h.sign_t(a, o)),
+    ("sqrt_t of abs", lambda h, a, b, o, r, c: (h.abs_t(a, o), h.sqrt_t(o, o))),
+    ("sigmoid", lambda h, a, b, o, r, c: h.sigmoid(a, o)),
+    ("rel in place", lambda h, a, b, o, r, c: h.rel(a, a)),
+    ("el", lambda h, a, b, o, r, c: h.el(a, o)),
+    ("sigmoid_deriv", lambda h, a, b, o, r, c: h.sigmoid_deriv(None, a, b, o)),
+    ("tanh_deriv in place", lambda h, a, b, o, r, c: h.tanh_deriv(None, a, b, b)),
+    ("rel_deriv", lambda h, a, b, o, r, c: h.rel_deriv(None, a, b, o)),
+    ("el_deriv", lambda h, a, b, o, r, c: h.el_deriv(None, a, b, o)),
+    ("clip_t", lambda h, a, b, o, r, c: h.clip_t(a, -0.5, 0.5, o)),
+    ("fill", lambda h, a, b, o, r, c: h.fill(o, 2.5)),
+    ("copy_to", lambda h, a, b, o, r, c: h.copy_to(a, o)),
+    ("copy_to_if", lambda h, a, b, o, r, c: (h.rel(b, b), h.copy_to_if(a, o, b))),
+    ("fill_if", lambda h, a, b, o, r, c: (h.rel(b, b), h.fill_if(o, 7.0, b))),
+    ("add_into_if", lambda h, a, b, o, r, c: (h.rel(b, b), h.add_into_if(a, o, b))),
+    ("add_mv row", lambda h, a, b, o, r, c: h.add_mv(a, r, o)),
+    ("subtract_mv col", lambda h, a, b, o, r, c: h.subtract_mv(a, c, o)),
+    ("mult_mv with a matrix", lambda h, a, b, o, r, c: h.mult_mv(a, b, o)),
+    ("divide_mv row in place", lambda h, a, b, o, r, c: h.divide_mv(a, r, a)),
+    ("mult_add_mv col", lambda h, a, b, o, r, c: h.mult_add_mv(a, c, o)),
+    ("mult_mv with a column of the hub", lambda h, a, b, o, r, c: h.mult_mv(a, b[:, 4:5], o)),
+    ("sum_t axis 0", lambda h, a, b, o, r, c: h.sum_t(a, 0, r)),
+    ("sum_t axis 1", lambda h, a, b, o, r, c: h.sum_t(a, 1, c)),
+    ("sum_t of all", lambda h, a, b, o, r, c: h.sum_t(a, None, c[0:1].reshape(()))),
+]
+
+
+@pytest.mark.parametrize("rows,width,cuts", [(37, 790, (3, 260, 517, 774)), (5, 40, (1, 8, 15, 22)),
+                                             (300, 4100, (4, 1028, 2052, 3076))],
+                         ids=["257 columns at odd offsets", "7 columns", "1024 columns, aligned"])
+@pytest.mark.parametrize("name,call", NATIVE_OPS, ids=[n for n, _ in NATIVE_OPS])
+def test_row_pitched_kernels(php, name, call, rows, width, cuts):
+    # the kernels that take row-pitched operands as they are: same bits as NumPy on strided views,
+    # nothing outside the slice changes, and no dense temporaries are made
+    rng = np.random.RandomState(8)
+    hub = rng.standard_normal((rows, width)).astype(F32)
+    cols = cuts[1] - cuts[0]
+    r = rng.uniform(0.5, 2.0, (1, cols)).astype(F32)
+    c = rng.uniform(0.5, 2.0, (rows, 1)).astype(F32)
+    ref = NumpyRefHandler(F32, seed=3)
+    want_hub, want_r, want_c = hub.copy(), r.copy(), c.copy()
+    call(ref, want_hub[:, cuts[0]:cuts[1]], want_hub[:, cuts[1]:cuts[2]], want_hub[:, cuts[2]:cuts[3]], want_r, want_c)
+    dev_hub, dev_r, dev_c = php.create_from_numpy(hub), php.create_from_numpy(r), php.create_from_numpy(c)
+    temporaries = []
+    real_scratch = php._scratch
+    php._scratch = lambda shape: temporaries.append(shape) or real_scratch(shape)
+    try:
+        call(php, dev_hub[:, cuts[0]:cuts[1]], dev_hub[:, cuts[1]:cuts[2]], dev_hub[:, cuts[2]:cuts[3]], dev_r, dev_c)
+    finally:
+        php._scratch = real_scratch
+    assert temporaries == [], temporaries
+    for got, want, tag in ((dev_hub.get(), want_hub, "hub"), (dev_r.get(), want_r, "row vector"),
+                           (dev_c.get(), want_c, "column vector")):
+        if name.startswith("sum_t"):
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=name + ": " + tag)
+        elif name == "sigmoid":
+            # NumPy's float32 formula and the device result are each within 2 units in the last place
+            # of the exact value (test_gpu_parity.py); the dense kernel's bits are checked below
+            np.testing.assert_array_max_ulp(got, want, maxulp=4)
+        elif name == "el":
+            # exp(x) - 1 cancels near 0, so one unit of exp is many units of the result
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-7, err_msg=name + ": " + tag)
+        else:
+            assert_bit_equal(got, want, name + ": " + tag)
+    # the path through dense temporaries gives the same bits
+    php.native_pitched = False
+    try:
+        dev_hub2, dev_r2, dev_c2 = php.create_from_numpy(hub), php.create_from_numpy(r), php.create_from_numpy(c)
+        call(php, dev_hub2[:, cuts[0]:cuts[1]], dev_hub2[:, cuts[1]:cuts[2]], dev_hub2[:, cuts[2]:cuts[3]], dev_r2, dev_c2)
+    finally:
+        php.native_pitched = True
+    if not name.startswith("sum_t"):
+        assert_bit_equal(dev_hub2.get(), dev_hub.get(), name + ": temporaries vs row-pitched kernels")
+
+
 def test_matrix_products_take_pitched_operands_as_they_are(php):
     # the pitch of a feature slice is the leading dimension of the product: no dense temporaries
     rng = np.random.RandomState(11)
