@@ -27,6 +27,7 @@ struct Context {
     bool debug_sync = false;   // BSHIP_DEBUG_SYNC=1: sync + check after every launch
     int blocks_per_cu = 8;     // streaming kernels launch num_cus*blocks_per_cu blocks
     int colsum_blocks_per_cu = 3;   // column sums: row bands are chosen to reach this many workgroups per CU (measured optimum)
+    size_t write_through_min = size_t(1) << 22;   // elements from which write-only kernels store write-through
     char name[256] = {0};
 };
 
@@ -126,9 +127,8 @@ __device__ __forceinline__ void vstore_writeonly(float* p, typename VecT<W>::typ
     if constexpr (W == 1) asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
     else asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
 }
-// Element count from which write-only kernels use it: below, the data is likely
-// to be read again soon and is better left to the default cache policy.
-constexpr size_t kWriteThroughMin = size_t(1) << 22;
+// Context::write_through_min is the element count from which write-only kernels use it: below,
+// the data is likely to be read again soon and is better left to the default cache policy.
 
 static inline bool aligned16(const void* p) {
     return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
@@ -162,6 +162,7 @@ void pool_graph_destroyed(int id);
 int rng_graph_begin(int id);
 int rng_graph_end(int id);
 int rng_graph_before_launch(int id);
+int rng_graph_after_launch(int id);
 void rng_graph_destroyed(int id);
 
 #define BSHIP_REQUIRE_EAGER()                                                                    \

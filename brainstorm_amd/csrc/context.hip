@@ -76,6 +76,8 @@ int bship_init(int device) {
     if (bpc && atoi(bpc) > 0 && atoi(bpc) <= 64) g_ctx.blocks_per_cu = atoi(bpc);
     const char* cpc = getenv("BSHIP_COLSUM_BLOCKS_PER_CU");
     if (cpc && atoi(cpc) > 0 && atoi(cpc) <= 64) g_ctx.colsum_blocks_per_cu = atoi(cpc);
+    const char* wtm = getenv("BSHIP_WRITE_THROUGH_MIN");
+    if (wtm && wtm[0]) g_ctx.write_through_min = static_cast<size_t>(strtoull(wtm, nullptr, 10));
     g_ctx.device = device;
     g_ctx.inited = true;
     return 0;

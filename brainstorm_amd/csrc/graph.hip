@@ -109,7 +109,8 @@ int bship_graph_launch(int graph_id) {
         return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_graph_launch: no recorded step %d", graph_id);
     int st = rng_graph_before_launch(graph_id);
     if (st != 0) return st;
-    return check_hip(hipGraphLaunch(it->second.exec, ctx().stream), "hipGraphLaunch");
+    st = check_hip(hipGraphLaunch(it->second.exec, ctx().stream), "hipGraphLaunch");
+    return st != 0 ? st : rng_graph_after_launch(graph_id);
 }
 
 int bship_graph_destroy(int graph_id) {

@@ -60,7 +60,7 @@ int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K) {
     BSHIP_REQUIRE_DIM(tiles_per_row * M <= 0x7fffffff);
     const dim3 grid(static_cast<unsigned>(tiles_per_row * M)), blk(kBlock);
     const unsigned tpr = static_cast<unsigned>(tiles_per_row);
-    const bool wt = static_cast<size_t>(M) * static_cast<size_t>(K) >= kWriteThroughMin;
+    const bool wt = static_cast<size_t>(M) * static_cast<size_t>(K) >= ctx().write_through_min;
     hipStream_t s = ctx().stream;
     if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, out, KW, tpr);
     else if (vec && aligned16(out))  hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, out, KW, tpr);

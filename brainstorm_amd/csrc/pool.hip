@@ -206,7 +206,7 @@ int launch_fill(float* p, float val, size_t n) {
     const size_t tiles = (n + kCopyTile - 1) / kCopyTile;
     if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "fill: %zu elements exceed one launch", n);
     const dim3 grid(static_cast<unsigned>(tiles));
-    if (n >= kWriteThroughMin)
+    if (n >= ctx().write_through_min)
         hipLaunchKernelGGL((fill_kernel<false, true>), grid, dim3(kBlock), 0, ctx().stream, p, val, n);
     else if (aligned16(p))
         hipLaunchKernelGGL((fill_kernel<true, false>), grid, dim3(kBlock), 0, ctx().stream, p, val, n);

@@ -40,6 +40,7 @@
 #include <vector>
 
 #include "common.h"
+#include "mt_jump.h"
 
 namespace bship {
 
@@ -94,19 +95,15 @@ static_assert(kRawThreads >= kWide && kRawThreads % kWave == 0, "generator lanes
 constexpr int kWin = 2048;
 static_assert(kWide + kWideHistory <= kWin, "a step's reads and writes must not alias");
 
-__global__ __launch_bounds__(kRawThreads) void mt_raw_kernel(RngState* st, uint32_t* __restrict__ raw,
-                                                             size_t nw, RngState* before) {
-    __shared__ uint32_t win[2 * kWin];
+// `win` is the workgroup's LDS window (2 * kWin words), `key` the 624-word block to start from (position
+// pos0 in it is the first word wanted), `st_out` (may be null) receives the state afterwards.
+__device__ __forceinline__ void mt_generate(uint32_t* win, const uint32_t* key, size_t pos0, size_t nw,
+                                            uint32_t* __restrict__ raw, RngState* st_out) {
     const unsigned t = threadIdx.x;
     for (unsigned i = t; i < kMtN; i += kRawThreads) {
-        const uint32_t v = st->key[i];
+        const uint32_t v = key[i];
         win[i] = v;
         win[i + kWin] = v;
-    }
-    const size_t pos0 = static_cast<size_t>(st->pos);
-    if (before != nullptr) {
-        for (unsigned i = t; i < kMtN; i += kRawThreads) before->key[i] = st->key[i];
-        if (t == 0) before->pos = static_cast<int32_t>(pos0);
     }
     __syncthreads();
     const size_t end_word = pos0 + nw;
@@ -150,9 +147,90 @@ __global__ __launch_bounds__(kRawThreads) void mt_raw_kernel(RngState* st, uint3
     while (have < gen_end && have < kWideHistory) advance(std::false_type());    // two plain steps
     while (have < gen_end) advance(std::true_type());
     __syncthreads();
-    const size_t block0 = gen_end - kMtN;
-    for (unsigned i = t; i < kMtN; i += kRawThreads) st->key[i] = win[(block0 + i) & (kWin - 1)];
-    if (t == 0) st->pos = static_cast<int32_t>(end_word - block0);
+    if (st_out != nullptr) {
+        const size_t block0 = gen_end - kMtN;
+        for (unsigned i = t; i < kMtN; i += kRawThreads) st_out->key[i] = win[(block0 + i) & (kWin - 1)];
+        if (t == 0) st_out->pos = static_cast<int32_t>(end_word - block0);
+    }
+}
+
+__global__ __launch_bounds__(kRawThreads) void mt_raw_kernel(RngState* st, uint32_t* __restrict__ raw,
+                                                             size_t nw, RngState* before) {
+    __shared__ uint32_t win[2 * kWin];
+    const unsigned t = threadIdx.x;
+    const size_t pos0 = static_cast<size_t>(st->pos);
+    if (before != nullptr) {
+        for (unsigned i = t; i < kMtN; i += kRawThreads) before->key[i] = st->key[i];
+        if (t == 0) before->pos = static_cast<int32_t>(pos0);
+    }
+    mt_generate(win, st->key, pos0, nw, raw, st);
+}
+
+// ------------------------------ parallel draws ------------------------------
+// A long draw is cut into segments of a whole number of 624-word blocks. The key block each segment
+// starts from is computed from the current one by jump-ahead (mt_jump.h): with w[0..] the stream
+// that starts at the current key block and g the polynomial of the distance d,
+//     block d words ahead [j] = XOR over { i : g_i = 1 } of w[i + j],     j = 0 .. 623,
+// so one workgroup first writes the "history" w[0 .. 19938 + 624), a grid then forms all the
+// segments' blocks from it (each workgroup a slice of the coefficients, combined with atomic XOR:
+// exact and order-free), and the segments are generated side by side, one workgroup each. The last
+// segment leaves the state exactly as the sequential generator would.
+constexpr int kJumpBits = 19938;                      // coefficients of a jump polynomial (mtjump::kPolyBits)
+constexpr int kHistWords = kJumpBits + kMtN;          // stream words the combination reads
+constexpr int kJumpChunk = 256;                       // coefficients per workgroup
+constexpr int kJumpChunks = (kJumpBits + kJumpChunk - 1) / kJumpChunk;
+static_assert(kJumpChunks * kJumpChunk == kMtN * 32, "a polynomial is stored as 624 words");
+
+// hist[0 .. kHistWords) = the stream from the start of the current key block; seeds[0] = the
+// current state, seeds[1 .. nseg) cleared for the combination; *before = the current key and pos.
+__global__ __launch_bounds__(kRawThreads) void mt_history_kernel(const RngState* st, uint32_t* __restrict__ hist,
+                                                                 RngState* seeds, int nseg, RngState* before) {
+    __shared__ uint32_t win[2 * kWin];
+    const unsigned t = threadIdx.x;
+    for (unsigned i = t; i < kMtN; i += kRawThreads) {
+        const uint32_t v = st->key[i];
+        seeds[0].key[i] = v;
+        if (before != nullptr) before->key[i] = v;
+        for (int s = 1; s < nseg; ++s) seeds[s].key[i] = 0u;
+    }
+    if (t == 0) {
+        seeds[0].pos = st->pos;
+        if (before != nullptr) before->pos = st->pos;
+    }
+    mt_generate(win, st->key, 0, kHistWords, hist, nullptr);
+}
+
+// seeds[blockIdx.y + 1].key ^= the part of the combination that coefficients
+// [blockIdx.x * kJumpChunk, +kJumpChunk) of polynomial blockIdx.y contribute.
+__global__ __launch_bounds__(kRawThreads) void mt_jump_kernel(const uint32_t* __restrict__ polys,
+                                                              const uint32_t* __restrict__ hist, RngState* seeds) {
+    __shared__ uint32_t h[kJumpChunk + kMtN];
+    const unsigned t = threadIdx.x;
+    const int i0 = blockIdx.x * kJumpChunk;
+    for (int i = t; i < kJumpChunk + kMtN; i += kRawThreads) h[i] = i0 + i < kHistWords ? hist[i0 + i] : 0u;
+    __syncthreads();
+    if (t >= kMtN) return;
+    const uint32_t* g = polys + static_cast<size_t>(blockIdx.y) * kMtN + i0 / 32;
+    uint32_t acc = 0;
+#pragma unroll
+    for (int wd = 0; wd < kJumpChunk / 32; ++wd) {
+        const uint32_t bits = g[wd];                      // the same for every lane
+#pragma unroll
+        for (int b = 0; b < 32; ++b) acc ^= h[wd * 32 + b + t] & (0u - ((bits >> b) & 1u));
+    }
+    if (acc != 0u) atomicXor(&seeds[blockIdx.y + 1].key[t], acc);
+}
+
+// Segment blockIdx.x: seg_words words (the last one: what is left of nw) from seeds[blockIdx.x], all
+// starting at position seeds[0].pos of their block; the last segment writes the state to *st.
+__global__ __launch_bounds__(kRawThreads) void mt_segments_kernel(const RngState* seeds, RngState* st,
+                                                                  uint32_t* __restrict__ raw, size_t nw,
+                                                                  size_t seg_words) {
+    __shared__ uint32_t win[2 * kWin];
+    const size_t first = static_cast<size_t>(blockIdx.x) * seg_words;
+    const bool last = blockIdx.x + 1 == gridDim.x;
+    mt_generate(win, seeds[blockIdx.x].key, static_cast<size_t>(seeds[0].pos), last ? nw - first : seg_words,
+                raw + first, last ? st : nullptr);
 }
 
 __device__ __forceinline__ uint64_t raw_to_k53(const uint32_t* __restrict__ raw, size_t i) {
@@ -284,6 +362,7 @@ struct MaskPrefetch {
     size_t n;
     double p;
     float* staging;
+    float* next;           // slots of a recorded step: the mask after the one in staging
     uint32_t* raw;         // the 2n raw words of the draw (scratch of the entry's own)
     RngState* before;      // key and pos before this mask was drawn
     hipEvent_t ready;      // second stream: the mask is in staging
@@ -297,17 +376,116 @@ constexpr size_t kMaxPeriod = 16;
 static size_t g_min_period = 1;              // raised after a wrong guess, see prefetch_flush()
 constexpr size_t kMaxPrefetchFloats = size_t(1) << 26;   // per period: 256 MiB of staging at most
 
+// ---- plan of a parallel draw ----
+// Cost model (measured): forming one segment's start block costs about 1 us of the whole device
+// (19938 x 624 AND-XOR pairs), generating a segment 0.13 us per 623 words on one compute unit, so
+// the time 1.05 P + 0.13 nw / (623 P) is least for P = sqrt(nw / 5000) segments.
+constexpr int kMaxSegments = 64;
+constexpr int kMinSegments = 4;                 // below (61 000 words), the sequential kernel is as fast
+constexpr size_t kEagerJumpMinWords = size_t(1) << 20;
+struct JumpPolys { uint32_t* dev; int count; };
+static std::vector<uint32_t*> g_jump_retired;          // replaced tables, freed at shutdown
+static std::map<size_t, JumpPolys> g_jump_polys;      // words per segment -> polynomials of 1, 2, ... segments ahead
+static uint32_t* g_hist = nullptr;                    // kHistWords words
+static RngState* g_seeds = nullptr;                   // kMaxSegments states
+// The generator's scratch (g_hist, g_seeds) is used like g_state itself: by one stream at a time,
+// in an order fixed by events; the polynomials are written once and then only read.
+
+static bool jump_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("BSHIP_RNG_JUMP");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+struct JumpPlan { int segments; size_t seg_words; const uint32_t* polys; };
+
+// Segments and words per segment for a draw of nw words, or false for "draw sequentially".
+static bool jump_shape(size_t nw, bool for_replay, int* segments, size_t* seg_words) {
+    if (!jump_enabled()) return false;
+    // A training step of small layers that is issued call by call is paced by the host: there the
+    // two extra launches cost more than the shorter draw saves (MLP 784-1200-1200-10: 0.35 -> 0.45 ms
+    // per step), so only long draws are cut up. Next to the replay of a recorded step the host is
+    // idle and the draw is what the step waits for: there every draw long enough is cut up.
+    if (!for_replay && nw < kEagerJumpMinWords) return false;
+    int target = static_cast<int>(sqrt(static_cast<double>(nw) / 5000.0) + 0.5);
+    if (target < kMinSegments) return false;
+    if (target > kMaxSegments) target = kMaxSegments;
+    const size_t blocks = static_cast<size_t>(ceil_div(static_cast<int64_t>(nw), static_cast<int64_t>(kMtN) * target));
+    *seg_words = blocks * kMtN;
+    *segments = static_cast<int>((nw + *seg_words - 1) / *seg_words);
+    return *segments >= 2;
+}
+
+// The polynomials of 1 ... count segments of seg_words ahead, on the device; computed (tens of
+// milliseconds on the host) and uploaded on first use. Not while a step is being recorded: the
+// upload is a blocking copy, which invalidates a recording. Null: not available.
+static const uint32_t* jump_polys(size_t seg_words, int count) {
+    auto it = g_jump_polys.find(seg_words);
+    if (it != g_jump_polys.end() && it->second.count >= count) return it->second.dev;
+    if (graph_recording()) return nullptr;
+    if (!g_hist && hipMalloc(reinterpret_cast<void**>(&g_hist), kHistWords * sizeof(uint32_t)) != hipSuccess) {
+        (void)hipGetLastError(); g_hist = nullptr; return nullptr;
+    }
+    if (!g_seeds && hipMalloc(reinterpret_cast<void**>(&g_seeds), kMaxSegments * sizeof(RngState)) != hipSuccess) {
+        (void)hipGetLastError(); g_seeds = nullptr; return nullptr;
+    }
+    std::vector<uint32_t> host;
+    if (!mtjump::jump_polynomials(seg_words, count, host)) return nullptr;
+    uint32_t* dev = nullptr;
+    // memory of its own, not a pool block: a pool block may still be read by kernels in flight,
+    // and this copy does not wait for the library's streams
+    if (hipMalloc(reinterpret_cast<void**>(&dev), host.size() * sizeof(uint32_t)) != hipSuccess) {
+        (void)hipGetLastError(); return nullptr;
+    }
+    if (hipMemcpy(dev, host.data(), host.size() * sizeof(uint32_t), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError(); (void)hipFree(dev); return nullptr;
+    }
+    if (it != g_jump_polys.end()) {
+        // a shorter table of the same length may be in use by kernels in flight or recorded steps: keep it
+        g_jump_retired.push_back(it->second.dev);
+        it->second = JumpPolys{dev, count};
+    } else {
+        g_jump_polys.emplace(seg_words, JumpPolys{dev, count});
+    }
+    return dev;
+}
+
+// Decides whether a draw of nw words is cut into segments. Any failure means "draw sequentially".
+static bool jump_plan(size_t nw, bool for_replay, JumpPlan* plan) {
+    if (!jump_shape(nw, for_replay, &plan->segments, &plan->seg_words)) return false;
+    plan->polys = jump_polys(plan->seg_words, plan->segments - 1);
+    return plan->polys != nullptr;
+}
+
+// Enqueues raw[0 .. nw) = the next nw words of the stream on `stream`, *before = the state before.
+static void launch_raw_words(hipStream_t stream, uint32_t* raw, size_t nw, RngState* before, bool for_replay = false) {
+    JumpPlan plan;
+    if (!jump_plan(nw, for_replay, &plan)) {
+        hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, stream, g_state, raw, nw, before);
+        return;
+    }
+    hipLaunchKernelGGL(mt_history_kernel, dim3(1), dim3(kRawThreads), 0, stream, g_state, g_hist, g_seeds,
+                       plan.segments, before);
+    hipLaunchKernelGGL(mt_jump_kernel, dim3(kJumpChunks, plan.segments - 1), dim3(kRawThreads), 0, stream,
+                       plan.polys, g_hist, g_seeds);
+    hipLaunchKernelGGL(mt_segments_kernel, dim3(plan.segments), dim3(kRawThreads), 0, stream, g_seeds, g_state, raw,
+                       nw, plan.seg_words);
+}
+
 // Enqueues mask[0..n) = (next n doubles of the stream < p) on `stream`; raw is scratch for 2n words.
-static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw) {
-    hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, stream, g_state, raw, 2 * n, before);
+// for_replay: the mask belongs to a recorded step (its draw overlaps the replay: see jump_shape).
+static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw,
+                        bool for_replay = false) {
+    launch_raw_words(stream, raw, 2 * n, before, for_replay);
     hipLaunchKernelGGL(raw_to_mask_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
                        dim3(kBlock), 0, stream, raw, mask, n, p);
 }
 
 // Enqueues u[0..n) = the next n doubles of the stream on the main stream (raw: scratch for 2n words).
 static void launch_doubles(double* u, size_t n, uint32_t* raw) {
-    hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, ctx().stream, g_state, raw, 2 * n,
-                       static_cast<RngState*>(nullptr));
+    launch_raw_words(ctx().stream, raw, 2 * n, nullptr);
     hipLaunchKernelGGL(raw_to_doubles_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
                        dim3(kBlock), 0, ctx().stream, raw, u, n);
 }
@@ -322,6 +500,7 @@ static bool prefetch_enabled() {
 
 static void free_entry(MaskPrefetch& e) {
     if (e.staging) pool_free_raw(e.staging);
+    if (e.next) pool_free_raw(e.next);
     if (e.raw) pool_free_raw(e.raw);
     if (e.before) pool_free_raw(e.before);
     if (e.ready) (void)hipEventDestroy(e.ready);
@@ -417,14 +596,19 @@ static void prefetch_maybe_start() {
 // --------------------------- masks of recorded steps ---------------------------
 // A recorded step (bship_graph_begin ... bship_graph_end) replays the same kernels with the same
 // arguments, so its masks cannot be served by the queue above, and drawing them inline would put
-// their sequential time on the step's critical path. Instead every mask request of the recording
-// gets a slot of its own (staging, raw words, generator snapshot). In the recorded graph the main
-// stream reads the slot's staging buffer, and a branch on the second stream, ordered behind that
-// read, draws the slot's next mask: replay r consumes what replay r-1 (or the priming below) drew,
-// in request order, so the random stream is used exactly as by eager execution. Before the first
-// replay, and after any other use of the generator, the slots are "primed": their masks are drawn
-// eagerly in order. Any eager use of the generator first "unprimes": it puts the generator back to
-// the snapshot taken before the pending, not yet consumed masks.
+// their time on the step's critical path. Instead every mask request of the recording gets a slot
+// of its own (two mask buffers, raw words, generator snapshot), and the recorded graph only READS
+// the slots' `staging` buffers: it contains no generator kernel at all. Each replay
+// (bship_graph_launch) then issues, next to the graph and on the second stream, the draws of every
+// slot's following mask into its `next` buffer, in request order, and behind the graph one kernel
+// that copies next -> staging. So replay r consumes what replay r-1 (or the priming below) drew, the
+// random stream is used exactly as by eager execution, and the draws overlap the whole step as
+// ordinary work of a second stream. (Drawing inside the graph, on a captured branch, was measured
+// first: the graph executor ran a branch forked where the mask is consumed partly, and a branch
+// forked at the root entirely, in series with the main chain.) Before the first replay, and after
+// any other use of the generator, the slots are "primed": their masks are drawn eagerly in order.
+// Any eager use of the generator first "unprimes": it puts the generator back to the snapshot taken
+// before the pending, not yet consumed masks.
 struct GraphMasks {
     std::vector<MaskPrefetch> slots;
     bool primed = false;
@@ -432,6 +616,7 @@ struct GraphMasks {
 static std::map<int, GraphMasks> g_graph_masks;
 static int g_recording_masks = 0;      // graph being recorded, or 0
 static int g_primed_graph = 0;         // graph whose slots hold drawn, unconsumed masks, or 0
+static hipEvent_t g_before_graph = nullptr;   // main stream, right before a replay's graph
 
 // The pending masks of the primed graph are given up: the generator returns to the position before them.
 static int graph_masks_unprime() {
@@ -447,6 +632,7 @@ static int graph_masks_unprime() {
 static int ensure_side_stream() {
     if (!g_side) BSHIP_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
     if (!g_join) BSHIP_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    if (!g_before_graph) BSHIP_HIP(hipEventCreateWithFlags(&g_before_graph, hipEventDisableTiming));
     return 0;
 }
 
@@ -456,28 +642,42 @@ static int graph_mask_slot(size_t n, double p, MaskPrefetch* hit) {
     e.n = n;
     e.p = p;
     void* a = nullptr;
+    void* a2 = nullptr;
     void* b = nullptr;
     void* r = nullptr;
     int st = pool_alloc_raw(n * sizeof(float), &a);
     e.staging = static_cast<float*>(a);
+    if (st == 0) st = pool_alloc_raw(n * sizeof(float), &a2);
+    e.next = static_cast<float*>(a2);
     if (st == 0) st = pool_alloc_raw(2 * n * sizeof(uint32_t), &r);
     e.raw = static_cast<uint32_t*>(r);
     if (st == 0) st = pool_alloc_raw(sizeof(RngState), &b);
     e.before = static_cast<RngState*>(b);
-    if (st == 0) st = check_hip(hipEventCreateWithFlags(&e.consumed, hipEventDisableTiming), "hipEventCreate");
     if (st != 0) { free_entry(e); return st; }
     *hit = e;
     return 0;
 }
 
-// The recorded main stream has read the slot's staging buffer: the second stream draws the next mask.
+// The recorded main stream has enqueued its read of the slot's staging buffer: the slot joins the recording.
 static int graph_mask_redraw(MaskPrefetch& e) {
-    BSHIP_HIP(hipEventRecord(e.consumed, ctx().stream));
-    BSHIP_HIP(hipStreamWaitEvent(g_side, e.consumed, 0));
-    launch_mask(g_side, e.staging, e.n, e.p, e.before, e.raw);
-    int st = check_launch("recorded mask");
     g_graph_masks[g_recording_masks].slots.push_back(e);
-    return st;
+    return 0;
+}
+
+// next -> staging for up to kMaxSlotCopies slots in one launch (grid.y = slot)
+constexpr int kMaxSlotCopies = 16;
+struct SlotCopies { const float* src[kMaxSlotCopies]; float* dst[kMaxSlotCopies]; size_t n[kMaxSlotCopies]; };
+__global__ __launch_bounds__(kBlock) void slot_copy_kernel(SlotCopies c) {
+    const float* src = c.src[blockIdx.y];
+    float* dst = c.dst[blockIdx.y];
+    const size_t n = c.n[blockIdx.y];
+    const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {                              // pool blocks: 256-byte aligned
+        *reinterpret_cast<f4*>(dst + i) = *reinterpret_cast<const f4*>(src + i);
+    } else {
+        for (size_t j = i; j < n; ++j) dst[j] = src[j];
+    }
 }
 
 int rng_graph_begin(int id) {
@@ -491,29 +691,60 @@ int rng_graph_begin(int id) {
     return 0;
 }
 
-// Joins the second stream's branch, if the recording made one, back into the main stream.
 int rng_graph_end(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    (void)id;
     g_recording_masks = 0;
-    auto it = g_graph_masks.find(id);
-    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
-    return order_streams(g_side, ctx().stream);
+    return 0;
 }
 
 int rng_graph_before_launch(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
-    if (g_primed_graph == id) return 0;
-    int st = prefetch_flush(true);
-    if (st == 0) st = graph_masks_unprime();
+    if (g_primed_graph != id) {
+        int st = prefetch_flush(true);
+        if (st == 0) st = graph_masks_unprime();
+        if (st != 0) return st;
+        for (MaskPrefetch& e : it->second.slots) launch_mask(ctx().stream, e.staging, e.n, e.p, e.before, e.raw, true);
+        st = check_launch("recorded masks, first draw");
+        if (st != 0) return st;
+        it->second.primed = true;
+        g_primed_graph = id;
+    }
+    return check_hip(hipEventRecord(g_before_graph, ctx().stream), "hipEventRecord");
+}
+
+// The graph of recording `id` has just been enqueued on the main stream: next to it, the second
+// stream draws the masks of the replay after this one; behind it, they move into place.
+int rng_graph_after_launch(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    std::vector<MaskPrefetch>& slots = it->second.slots;
+    // the second stream starts behind everything that preceded the graph on the main stream: the
+    // priming draws, or the previous replay's copy out of the `next` buffers
+    BSHIP_HIP(hipStreamWaitEvent(g_side, g_before_graph, 0));
+    for (MaskPrefetch& e : slots) launch_mask(g_side, e.next, e.n, e.p, e.before, e.raw, true);
+    int st = check_launch("masks of the next replay");
     if (st != 0) return st;
-    for (MaskPrefetch& e : it->second.slots) launch_mask(ctx().stream, e.staging, e.n, e.p, e.before, e.raw);
-    st = check_launch("recorded masks, first draw");
-    if (st != 0) return st;
-    it->second.primed = true;
-    g_primed_graph = id;
-    return 0;
+    st = order_streams(g_side, ctx().stream);
+    for (size_t first = 0; st == 0 && first < slots.size(); first += kMaxSlotCopies) {
+        SlotCopies c = SlotCopies();
+        size_t most = 0;
+        const size_t count = slots.size() - first < static_cast<size_t>(kMaxSlotCopies) ? slots.size() - first : kMaxSlotCopies;
+        for (size_t k = 0; k < count; ++k) {
+            c.src[k] = slots[first + k].next;
+            c.dst[k] = slots[first + k].staging;
+            c.n[k] = slots[first + k].n;
+            most = c.n[k] > most ? c.n[k] : most;
+        }
+        const size_t tiles = (most + static_cast<size_t>(kBlock) * 4 - 1) / (static_cast<size_t>(kBlock) * 4);
+        hipLaunchKernelGGL(slot_copy_kernel, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(count)),
+                           dim3(kBlock), 0, ctx().stream, c);
+        st = check_launch("masks of the next replay, move into place");
+    }
+    return st;
 }
 
 void rng_graph_destroyed(int id) {
@@ -694,8 +925,16 @@ void rng_release() {
     g_history.clear();
     g_min_period = 1;
     if (g_join) { (void)hipEventDestroy(g_join); g_join = nullptr; }
+    if (g_before_graph) { (void)hipEventDestroy(g_before_graph); g_before_graph = nullptr; }
+
     if (g_side) { (void)hipStreamDestroy(g_side); g_side = nullptr; }
     if (g_state) { pool_free_raw(g_state); g_state = nullptr; }
+    for (auto& kv : g_jump_polys) (void)hipFree(kv.second.dev);
+    g_jump_polys.clear();
+    for (uint32_t* p : g_jump_retired) (void)hipFree(p);
+    g_jump_retired.clear();
+    if (g_hist) { (void)hipFree(g_hist); g_hist = nullptr; }
+    if (g_seeds) { (void)hipFree(g_seeds); g_seeds = nullptr; }
     if (g_fast_state) { pool_free_raw(g_fast_state); g_fast_state = nullptr; }
 }
 

@@ -504,6 +504,34 @@ def test_generate_probability_mask_matches_randomstate(hip):
         np.testing.assert_array_equal(key, st[1])
 
 
+def test_long_masks_drawn_in_parallel_segments_match_randomstate(hip):
+    # Long draws (2^20 words = 524 288 doubles or more; inside recorded steps from about 61 000 words) are cut
+    # into 4 ... 64 segments of whole 624-word blocks by jump-ahead and generated side by side: masks and
+    # the state afterwards must still be those of one sequential RandomState, wherever in its block a draw
+    # starts and ends.
+    for seed in (3, 2718281828):
+        hip.rnd.seed(seed)
+        rs = np.random.RandomState(seed)
+        for n, p in [(524287, 0.5), (524288, 0.5), (5, 0.5), (524289, 0.3), (311, 0.5), (624 * 900, 0.9),
+                     (1000003, 0.2), (4096 * 1024, 0.65), (1, 0.5), (64 * 624 * 50, 0.5), (64 * 624 * 50 + 1, 0.5)]:
+            mask = hip.allocate((n,))
+            hip.generate_probability_mask(mask, p)
+            want = (rs.uniform(size=(n,)) < p).astype(F32)
+            assert_bit_equal(mask.get(), want, "mask seed %d, %d elements" % (seed, n))
+            _, key, pos, _, _ = hip.rnd.get_state()
+            st = rs.get_state()
+            assert pos == st[2], "position after %d elements" % n
+            np.testing.assert_array_equal(key, st[1], err_msg="key after %d elements" % n)
+    # the gaussian stream takes its uniform numbers the same way
+    out = hip.allocate((700000,))
+    hip.fill_gaussian(0.5, 2.0, out)
+    assert_max_ulp(out.get(), (2.0 * rs.standard_normal((700000,)) + 0.5).astype(F32), 1, "long fill_gaussian")
+    _, key, pos, has_gauss, _ = hip.rnd.get_state()
+    st = rs.get_state()
+    assert (pos, has_gauss) == (st[2], st[3])
+    np.testing.assert_array_equal(key, st[1])
+
+
 def test_mask_prefetch_never_changes_the_stream(hip):
     # Repeating request patterns switch on the look-ahead generation on the second stream; whether a
     # request is served from it, misses it, or another consumer of the generator cuts in, the masks
