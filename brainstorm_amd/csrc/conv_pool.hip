@@ -962,6 +962,8 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(col);
+    BSHIP_REQUIRE_F32_ALIGNED(in);
+    BSHIP_REQUIRE_F32_ALIGNED(col);
     const bool write_through = static_cast<size_t>(total) >= (size_t(1) << 26);   // 256 MiB: beyond the last-level cache
     const int64_t per_image = static_cast<int64_t>(g.oh) * g.ow * kh * kw * c;
     BandPlan bp;
@@ -1010,6 +1012,8 @@ int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, 
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(col);
     BSHIP_REQUIRE_PTR(in_deltas);
+    BSHIP_REQUIRE_F32_ALIGNED(col);
+    BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     Col2imBandPlan bp;
     size_t lds = 0;
     if (plan_col2im_band(g, n, &bp, &lds)) {
@@ -1046,6 +1050,9 @@ int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_PTR(argmax);
+    BSHIP_REQUIRE_F32_ALIGNED(in);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    BSHIP_REQUIRE_F32_ALIGNED(argmax);
     const bool al = aligned16(in) && aligned16(out) && aligned16(argmax);
     if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
         BSHIP_LAUNCH_IMG(maxpool_fwd_kernel_3x3, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out, argmax);
@@ -1066,6 +1073,9 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
     BSHIP_REQUIRE_PTR(argmax);
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
+    BSHIP_REQUIRE_F32_ALIGNED(argmax);
+    BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
+    BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     const bool al = aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas);
     // how many output positions can cover one pixel along each axis
     const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
@@ -1087,6 +1097,8 @@ int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, in
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(in);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
     const bool al = aligned16(in) && aligned16(out);
     if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
         BSHIP_LAUNCH_IMG(avgpool_fwd_kernel_3x3, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
@@ -1106,6 +1118,8 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_
     if (total == 0 || out_h == 0 || out_w == 0) return 0;
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
+    BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
+    BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     const bool al = aligned16(out_deltas) && aligned16(in_deltas);
     const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
     if (cover == 1)
