@@ -280,7 +280,7 @@ def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
     from brainstorm_amd.drivers.net import MomentumStepper
     net, data = builder(handler, **kw)
     net.provide_external_data(data)
-    stepper = MomentumStepper(0.1, 0.9)
+    stepper = MomentumStepper(0.1, 0.9, fused=bool(kw.get("fused")))
     stepper.start(net)
     if recorded:
         stepper.run()

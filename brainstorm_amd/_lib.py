@@ -88,6 +88,9 @@ SIGNATURES = {
     "bship_lstm_bwd_step_f32": [c_int, _I64, _I64] + [_P] * 24,
     "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,
     "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
+    "bship_softmax_ce_fwd_f32": [_P, _P, _P, _P, _I64, _I64],
+    "bship_softmax_ce_bwd_f32": [_P, _P, _P, _P, _P, _I64, _I64],
+    "bship_momentum_update_f32": [c_float, c_float, _P, _P, _P, c_size_t],
     "bship_highway_fwd_f32": [_P, _P, _P, _P, c_size_t],
     "bship_highway_bwd_f32": [_P] * 7 + [c_size_t],
     "bship_dropout_fwd_f32": [_P, _P, _P, c_size_t, c_double, c_float],

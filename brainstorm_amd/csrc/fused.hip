@@ -313,6 +313,54 @@ struct HighwayBwdBody {
     }
 };
 
+// ---- momentum update (steppers.py:104-114) ----
+// velocity = momentum * velocity; velocity += (-learning_rate) * gradients; parameters = velocity + parameters
+struct MomentumBody {
+    static constexpr int kVecs = 0, kIn = 3, kOut = 2;
+    const float* ins[3];   // gradients, velocity, parameters
+    float* outs[2];        // velocity, parameters
+    float momentum, neg_learning_rate;
+    __device__ void apply(const float*, const float* in, float* o) const {
+        float v = MultStOp{momentum}.apply(in[1], 0.0f, 0.0f);
+        v = MultAddStOp{neg_learning_rate}.apply(in[0], v, 0.0f);
+        o[0] = v;
+        o[1] = AddOp{}.apply(v, in[2], 0.0f);
+    }
+};
+
+// ---- softmax cross entropy (softmax_ce_layer.py:65-114) ----
+// forward, behind softmax_m: loss[i] = -1 * log(clip(probs[i, int(targets[i])], 1e-6, 1))
+// (index_m_by_v, clip_t, log_t, mult_st; the layer's fill(loss, 0) is overwritten by them)
+__global__ __launch_bounds__(kBlock) void softmax_ce_loss_kernel(const float* __restrict__ probs,
+                                                                 const float* __restrict__ targets,
+                                                                 float* __restrict__ loss, int64_t M, int64_t K) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (row >= M) return;
+    const int64_t j = static_cast<int64_t>(static_cast<int>(targets[row]));
+    float p = (j >= 0 && j < K) ? probs[row * K + j] : 0.0f;
+    p = ClipOp{1e-6f, 1.0f}.apply(p, 0.0f, 0.0f);
+    p = LogOp{}.apply(p, 0.0f, 0.0f);
+    loss[row] = MultStOp{-1.0f}.apply(p, 0.0f, 0.0f);
+}
+// backward: t = onehot(targets); t = -1 * t; t = t + probs; t = t * dloss[row]; t_bin = t;
+// dinputs = t + dinputs   (binarize_v, mult_st, add_tt, mult_mv, add_tt)
+__global__ __launch_bounds__(kBlock) void softmax_ce_bwd_kernel(const float* __restrict__ probs,
+                                                                const float* __restrict__ targets,
+                                                                const float* __restrict__ dloss,
+                                                                float* __restrict__ t_bin, float* dinputs,
+                                                                int64_t total, int64_t K) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int64_t row = i / K;
+    const int64_t j = i - row * K;
+    float t = (j == static_cast<int64_t>(static_cast<int>(targets[row]))) ? 1.0f : 0.0f;
+    t = MultStOp{-1.0f}.apply(t, 0.0f, 0.0f);
+    t = AddOp{}.apply(t, probs[i], 0.0f);
+    t = MulOp{}.apply(t, dloss[row], 0.0f);
+    t_bin[i] = t;
+    dinputs[i] = AddOp{}.apply(t, dinputs[i], 0.0f);
+}
+
 // ---- bias + activation of a fully connected layer (fully_connected_layer.py:62-64) ----
 template <typename Act>
 struct BiasActBody {
@@ -582,6 +630,48 @@ int bship_highway_bwd_f32(const float* H, const float* T, const float* x, const 
     if (st != 0) return st;
     HighwayBwdBody b{{H, T, x, dy, dx, dH, dT}, {dx, dH, dT}};
     return launch_flat_fused("highway_backward", b, n);
+}
+
+int bship_momentum_update_f32(float momentum, float neg_learning_rate, const float* gradients, float* velocity,
+                              float* parameters, size_t n) {
+    BSHIP_REQUIRE_INIT();
+    if (n == 0) return 0;
+    const void* ptrs[] = {gradients, velocity, parameters};
+    int st = check_pointers(__func__, ptrs, 3);
+    if (st != 0) return st;
+    MomentumBody b{{gradients, velocity, parameters}, {velocity, parameters}, momentum, neg_learning_rate};
+    return launch_flat_fused("momentum_update", b, n);
+}
+
+int bship_softmax_ce_fwd_f32(const float* inputs, const float* targets, float* probs, float* loss, int64_t M,
+                             int64_t K) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && K >= 0);
+    if (M == 0) return 0;
+    const void* ptrs[] = {inputs, targets, probs, loss};
+    int st = check_pointers(__func__, ptrs, 4);
+    if (st != 0) return st;
+    BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
+    st = bship_softmax_rows_f32(inputs, probs, M, K);
+    if (st != 0) return st;
+    hipLaunchKernelGGL(softmax_ce_loss_kernel, dim3(static_cast<unsigned>(ceil_div(M, kBlock))), dim3(kBlock), 0,
+                       ctx().stream, probs, targets, loss, M, K);
+    return check_launch("softmax_ce_forward");
+}
+
+int bship_softmax_ce_bwd_f32(const float* probs, const float* targets, const float* dloss, float* t_bin,
+                             float* dinputs, int64_t M, int64_t K) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && K >= 0);
+    if (M == 0 || K == 0) return 0;
+    const void* ptrs[] = {probs, targets, dloss, t_bin, dinputs};
+    int st = check_pointers(__func__, ptrs, 5);
+    if (st != 0) return st;
+    const int64_t total = M * K;
+    BSHIP_REQUIRE_DIM(ceil_div(total, kBlock) <= 0x7fffffff);
+    hipLaunchKernelGGL(softmax_ce_bwd_kernel, dim3(static_cast<unsigned>(ceil_div(total, kBlock))), dim3(kBlock), 0,
+                       ctx().stream, probs, targets, dloss, t_bin, dinputs, total, K);
+    return check_launch("softmax_ce_backward");
 }
 
 int bship_bias_act_f32(int act, const float* in, const float* bias, float* out, int64_t M, int64_t N) {

@@ -60,7 +60,7 @@ def build_mlp(handler, seed=1, batch=100, in_size=784, hidden=1200, classes=10, 
         ("fc2", FullyConnected(hidden, "rel", fused=fused), {"default": "drop2.default"}),
         ("drop3", Dropout(0.5, fused=fused), {"default": "fc2.default"}),
         ("out", FullyConnected(classes, "linear", fused=fused), {"default": "drop3.default"}),
-        ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
+        ("ce", SoftmaxCE(fused=fused), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),
     ])
     return _finish(net, data, _init_parameters(net, rng, 0.01))
@@ -75,8 +75,8 @@ def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1
     net = Net(handler, [
         ("Input", Input({"default": (symbols,), "targets": (1,)}), {}),
         ("lstm", Lstm(hidden, "tanh", fused=fused), {"default": "Input.default"}),
-        ("out", FullyConnected(symbols, "linear"), {"default": "lstm.default"}),
-        ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
+        ("out", FullyConnected(symbols, "linear", fused=bool(fused)), {"default": "lstm.default"}),
+        ("ce", SoftmaxCE(fused=bool(fused)), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),
     ])
     return _finish(net, data, _init_parameters(net, rng, 0.05))
@@ -98,8 +98,8 @@ def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10
         ]
         prev = "hw%d.default" % k
     layers += [
-        ("out", FullyConnected(classes, "linear"), {"default": prev}),
-        ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
+        ("out", FullyConnected(classes, "linear", fused=fused), {"default": prev}),
+        ("ce", SoftmaxCE(fused=fused), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),
     ]
     net = Net(handler, layers)

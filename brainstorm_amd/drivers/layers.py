@@ -166,6 +166,10 @@ class Dropout(Layer):
 class SoftmaxCE(Layer):
     """layers/softmax_ce_layer.py:65-114; inputs 'default' and integer 'targets' (..., 1)."""
 
+    def __init__(self, fused=False):
+        # fused: use the handler's softmax_ce_forward / softmax_ce_backward when it has them (same bits)
+        self.fused = bool(fused)
+
     def setup(self, in_shapes):
         in_shape = in_shapes["default"].feature_shape
         tar_shape = in_shapes["targets"].feature_shape
@@ -181,6 +185,9 @@ class SoftmaxCE(Layer):
         flat_probs = flatten_all_but_last(buffers.outputs["predictions"])
         flat_loss = flatten_all_but_last(loss)
         flat_targets = flatten_all_but_last(buffers.inputs["targets"])
+        if self.fused and hasattr(_h, "softmax_ce_forward"):
+            _h.softmax_ce_forward(flat_inputs, flat_targets, flat_probs, flat_loss)
+            return
         _h.softmax_m(flat_inputs, flat_probs)
         # cross entropy with index targets: -ln(p[target])
         _h.fill(loss, 0.)
@@ -197,6 +204,9 @@ class SoftmaxCE(Layer):
         flat_dloss = flatten_all_but_last(buffers.output_deltas["loss"])
         flat_dinputs = flatten_all_but_last(buffers.input_deltas["default"])
         # d loss / d input = (softmax - onehot) * dloss
+        if self.fused and hasattr(_h, "softmax_ce_backward"):
+            _h.softmax_ce_backward(flat_probs, flat_targets, flat_dloss, flat_t_bin, flat_dinputs)
+            return
         _h.binarize_v(flat_targets, flat_t_bin)
         _h.mult_st(-1, flat_t_bin, flat_t_bin)
         _h.add_tt(flat_t_bin, flat_probs, flat_t_bin)

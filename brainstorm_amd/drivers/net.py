@@ -196,10 +196,11 @@ class Net:
 class MomentumStepper:
     """training/steppers.py:83-114"""
 
-    def __init__(self, learning_rate=0.1, momentum=0.0, scale_learning_rate=True):
+    def __init__(self, learning_rate=0.1, momentum=0.0, scale_learning_rate=True, fused=False):
         self.learning_rate = learning_rate
         self.momentum = momentum
         self.scale_learning_rate = scale_learning_rate
+        self.fused = bool(fused)      # the three update operations through the handler's momentum_update (same bits)
         self.net = None
         self.velocity = None
 
@@ -215,9 +216,12 @@ class MomentumStepper:
         self.net.forward_pass(training_pass=True)
         self.net.backward_pass()
         h = self.net.handler
-        h.mult_st(momentum, self.velocity, out=self.velocity)
-        h.mult_add_st(-learning_rate, self.net.gradients, out=self.velocity)
-        h.add_tt(self.velocity, self.net.parameters, out=self.net.parameters)
+        if self.fused and hasattr(h, "momentum_update"):
+            h.momentum_update(momentum, -learning_rate, self.net.gradients, self.velocity, self.net.parameters)
+        else:
+            h.mult_st(momentum, self.velocity, out=self.velocity)
+            h.mult_add_st(-learning_rate, self.net.gradients, out=self.velocity)
+            h.add_tt(self.velocity, self.net.parameters, out=self.net.parameters)
         self.net.apply_weight_modifiers()                  # the trainer does this after every update (trainer.py:101)
 
     def run_recorded(self):

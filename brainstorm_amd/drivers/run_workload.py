@@ -25,7 +25,7 @@ def main(argv):
     handler = HipHandler(seed=0)
     net, data = getattr(configs, "build_" + name)(handler, **kw)
     net.provide_external_data(data)
-    stepper = MomentumStepper(0.1, 0.9)
+    stepper = MomentumStepper(0.1, 0.9, fused=bool(kw.get("fused")))
     stepper.start(net)
     if recorded:
         stepper.run()

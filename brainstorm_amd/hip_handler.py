@@ -190,6 +190,8 @@ class HipHandler(Handler):
         "sigmoid": ("y",), "tanh": ("y",), "rel": ("y",), "el": ("y",),
         "sigmoid_deriv": ("dx",), "tanh_deriv": ("dx",), "rel_deriv": ("dx",), "el_deriv": ("dx",),
         "dropout_forward": ("mask", "out"),
+        "softmax_ce_forward": ("probs", "loss"), "softmax_ce_backward": ("t_bin", "dinputs"),
+        "momentum_update": ("velocity", "parameters"),
         "batchnorm_forward": ("mu", "sigma", "sigma_b", "centered", "x_hat", "out"),
         "batchnorm_backward": ("dgamma", "dbeta", "in_deltas"),
     }
@@ -737,6 +739,31 @@ class HipHandler(Handler):
         self._call(self._lib.bship_lstm_bwd_step_packed_f32(
             self._ACT_CODES[activation], batch, n, deltas.ptr, dy.ptr, packed_out.ptr,
             *[a.ptr for a in mats[2:] + vecs]))
+
+    def softmax_ce_forward(self, inputs, targets, probs, loss):
+        """softmax_m(inputs, probs) and loss = -log(clip(probs[i, targets[i]], 1e-6, 1)) with the roundings of
+        softmax_ce_layer.py:79-89 (index_m_by_v, clip_t, log_t, mult_st) in two launches instead of six."""
+        rows, k = inputs.shape
+        if probs.shape != (rows, k) or targets.size != rows or loss.size != rows:
+            raise ValueError("softmax_ce_forward: inconsistent shapes")
+        self._call(self._lib.bship_softmax_ce_fwd_f32(inputs.ptr, targets.ptr, probs.ptr, loss.ptr, rows, k))
+
+    def softmax_ce_backward(self, probs, targets, dloss, t_bin, dinputs):
+        """softmax_ce_layer.py:108-112 (binarize_v, mult_st, add_tt, mult_mv, add_tt) in one pass."""
+        rows, k = probs.shape
+        if (t_bin.shape != (rows, k) or dinputs.shape != (rows, k) or targets.size != rows
+                or dloss.size != rows):
+            raise ValueError("softmax_ce_backward: inconsistent shapes")
+        self._call(self._lib.bship_softmax_ce_bwd_f32(probs.ptr, targets.ptr, dloss.ptr, t_bin.ptr,
+                                                      dinputs.ptr, rows, k))
+
+    def momentum_update(self, momentum, neg_learning_rate, gradients, velocity, parameters):
+        """mult_st(momentum, velocity, velocity); mult_add_st(neg_learning_rate, gradients, velocity);
+        add_tt(velocity, parameters, parameters) (steppers.py:104-112) in one pass."""
+        if not (gradients.size == velocity.size == parameters.size):
+            raise ValueError("momentum_update: inconsistent sizes")
+        self._call(self._lib.bship_momentum_update_f32(momentum, neg_learning_rate, gradients.ptr, velocity.ptr,
+                                                       parameters.ptr, parameters.size))
 
     def highway_forward(self, H, T, x, y):
         """y = T * (H - x) + x with the roundings of highway_layer.py:48-51, one pass."""

@@ -402,6 +402,20 @@ int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n,
                                    float* dCa, float* dCb, const float* pi,
                                    const float* pf, const float* po);
 
+/* SoftmaxCELayerImpl.forward_pass (softmax_ce_layer.py 79-89): softmax_m(inputs, probs), then in one
+ * launch loss[i] = -log(clip(probs[i, int(targets[i])], 1e-6, 1)) (index_m_by_v, clip_t, log_t,
+ * mult_st with the same roundings). inputs, probs are (M, K); targets, loss (M, 1). */
+int bship_softmax_ce_fwd_f32(const float* inputs, const float* targets, float* probs, float* loss,
+                             int64_t M, int64_t K);
+/* SoftmaxCELayerImpl.backward_pass (softmax_ce_layer.py 108-112) in one pass: t_bin = onehot(targets);
+ * t_bin = -1 * t_bin; t_bin += probs; t_bin *= dloss (a column); dinputs = t_bin + dinputs. */
+int bship_softmax_ce_bwd_f32(const float* probs, const float* targets, const float* dloss, float* t_bin,
+                             float* dinputs, int64_t M, int64_t K);
+/* MomentumStepper.run after the passes (steppers.py 104-112) in one pass: velocity = momentum * velocity;
+ * velocity += neg_learning_rate * gradients; parameters = velocity + parameters. */
+int bship_momentum_update_f32(float momentum, float neg_learning_rate, const float* gradients,
+                              float* velocity, float* parameters, size_t n);
+
 /* HighwayLayerImpl.forward_pass (highway_layer.py 48-51) in one pass:
  * tmp = H - x; tmp = T * tmp; y = tmp + x. */
 int bship_highway_fwd_f32(const float* H, const float* T, const float* x,

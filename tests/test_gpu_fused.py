@@ -287,15 +287,15 @@ def test_fused_layer_argument_errors(hip):
 
 
 def test_fused_mlp_training_is_bit_identical(hip):
-    # dropout (with masks served from the look-ahead queue once the pattern repeats) and
-    # bias+activation through the fused entry points: same masks, same parameters after 12 steps
+    # dropout (with masks served from the look-ahead queue once the pattern repeats), bias+activation,
+    # softmax cross entropy and the momentum update through the fused entry points: same masks, same parameters after 12 steps
     from brainstorm_amd.drivers.net import MomentumStepper
     results = []
     for fused in (False, True):
         hip.rnd.seed(31)
         net, data = configs.build_mlp(hip, fused=fused, batch=37, in_size=50, hidden=129)
         net.provide_external_data(data)
-        stepper = MomentumStepper(0.1, 0.9)
+        stepper = MomentumStepper(0.1, 0.9, fused=fused)
         stepper.start(net)
         for _ in range(12):
             stepper.run()
@@ -324,3 +324,69 @@ def test_dropout_forward_matches_single_operations(hip, n):
             assert_bit_equal(mask.get(), want_mask, "mask n=%d rep %d" % (n, rep))
             want = (x.get() * want_mask) * F32(1 / keep)
             assert_bit_equal(out.get(), want.astype(F32), "out n=%d rep %d" % (n, rep))
+
+
+@pytest.mark.parametrize("rows,k", [(1, 1), (100, 10), (37, 205), (10000, 205), (513, 4096)])
+def test_softmax_ce_fused_matches_single_operations(hip, rows, k):
+    # softmax_ce_layer.py:79-89 and 108-112 through the single operations and through the fused entry points
+    rng = np.random.RandomState(rows + k)
+    x = (rng.standard_normal((rows, k)) * 3).astype(F32)
+    tg = rng.randint(0, k, (rows, 1)).astype(F32)
+    dl = rng.standard_normal((rows, 1)).astype(F32)
+    di = rng.standard_normal((rows, k)).astype(F32)
+    up = hip.create_from_numpy
+    res = []
+    for fused in (False, True):
+        xd, td, dld, did = up(x), up(tg), up(dl), up(di)
+        probs, loss, t_bin = hip.allocate((rows, k)), hip.allocate((rows, 1)), hip.allocate((rows, k))
+        if fused:
+            hip.softmax_ce_forward(xd, td, probs, loss)
+            hip.softmax_ce_backward(probs, td, dld, t_bin, did)
+        else:
+            hip.softmax_m(xd, probs)
+            hip.fill(loss, 0.)
+            hip.index_m_by_v(probs, td, loss)
+            hip.clip_t(loss, 1e-6, 1.0, loss)
+            hip.log_t(loss, loss)
+            hip.mult_st(-1, loss, loss)
+            hip.binarize_v(td, t_bin)
+            hip.mult_st(-1, t_bin, t_bin)
+            hip.add_tt(t_bin, probs, t_bin)
+            hip.mult_mv(t_bin, dld, t_bin)
+            hip.add_tt(t_bin, did, did)
+        res.append([a.get() for a in (probs, loss, t_bin, did)])
+    for name, a, b in zip(("probs", "loss", "t_bin", "dinputs"), res[0], res[1]):
+        assert_bit_equal(b, a, "%s (%d, %d)" % (name, rows, k))
+    # and what it means: loss = -log(p[target]) clipped, dinputs += (p - onehot) * dloss
+    p = res[1][0].astype(np.float64)
+    want_loss = -np.log(np.clip(p[np.arange(rows), tg[:, 0].astype(int)], 1e-6, 1.0))
+    np.testing.assert_allclose(res[1][1][:, 0], want_loss, rtol=2e-6, atol=1e-7)
+    onehot = np.zeros((rows, k)); onehot[np.arange(rows), tg[:, 0].astype(int)] = 1
+    np.testing.assert_allclose(res[1][3], di + (p - onehot) * dl, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("n", [1, 5, 4099, 2395210])
+def test_momentum_update_matches_single_operations(hip, n):
+    rng = np.random.RandomState(n)
+    g, v, p = (rng.standard_normal((n + 1,)).astype(F32) for _ in range(3))
+    res = []
+    for fused in (False, True):
+        gd, vd, pd = (hip.create_from_numpy(a)[1:] for a in (g, v, p))       # odd start addresses
+        for _ in range(3):
+            if fused:
+                hip.momentum_update(0.9, -0.01, gd, vd, pd)
+            else:
+                hip.mult_st(0.9, vd, out=vd)
+                hip.mult_add_st(-0.01, gd, out=vd)
+                hip.add_tt(vd, pd, out=pd)
+        res.append((vd.get(), pd.get()))
+    assert_bit_equal(res[1][0], res[0][0], "velocity")
+    assert_bit_equal(res[1][1], res[0][1], "parameters")
+    m, lr = F32(0.9), F32(-0.01)
+    vv, pp = v[1:].copy(), p[1:].copy()
+    for _ in range(3):
+        vv = m * vv
+        vv = vv + lr * g[1:]
+        pp = vv + pp
+    assert_bit_equal(res[1][0], vv, "velocity against NumPy float32")
+    assert_bit_equal(res[1][1], pp, "parameters against NumPy float32")

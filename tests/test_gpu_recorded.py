@@ -166,7 +166,7 @@ def test_recorded_training_steps_equal_eager_ones():
         h = HipHandler(seed=77)
         net, data = configs.build_mlp(h, fused=fused)
         net.provide_external_data(data)
-        stepper = MomentumStepper(0.1, 0.9)
+        stepper = MomentumStepper(0.1, 0.9, fused=fused)
         stepper.start(net)
         stepper.run()
         losses = []
