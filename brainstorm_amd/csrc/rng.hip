@@ -460,6 +460,7 @@ static bool jump_plan(size_t nw, bool for_replay, JumpPlan* plan) {
 }
 
 // Enqueues raw[0 .. nw) = the next nw words of the stream on `stream`, *before = the state before.
+// for_replay: the words are masks of a recorded step (the draw overlaps the replay: see jump_shape).
 static void launch_raw_words(hipStream_t stream, uint32_t* raw, size_t nw, RngState* before, bool for_replay = false) {
     JumpPlan plan;
     if (!jump_plan(nw, for_replay, &plan)) {
@@ -475,10 +476,8 @@ static void launch_raw_words(hipStream_t stream, uint32_t* raw, size_t nw, RngSt
 }
 
 // Enqueues mask[0..n) = (next n doubles of the stream < p) on `stream`; raw is scratch for 2n words.
-// for_replay: the mask belongs to a recorded step (its draw overlaps the replay: see jump_shape).
-static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw,
-                        bool for_replay = false) {
-    launch_raw_words(stream, raw, 2 * n, before, for_replay);
+static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw) {
+    launch_raw_words(stream, raw, 2 * n, before);
     hipLaunchKernelGGL(raw_to_mask_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
                        dim3(kBlock), 0, stream, raw, mask, n, p);
 }
@@ -597,11 +596,12 @@ static void prefetch_maybe_start() {
 // A recorded step (bship_graph_begin ... bship_graph_end) replays the same kernels with the same
 // arguments, so its masks cannot be served by the queue above, and drawing them inline would put
 // their time on the step's critical path. Instead every mask request of the recording gets a slot
-// of its own (two mask buffers, raw words, generator snapshot), and the recorded graph only READS
-// the slots' `staging` buffers: it contains no generator kernel at all. Each replay
-// (bship_graph_launch) then issues, next to the graph and on the second stream, the draws of every
-// slot's following mask into its `next` buffer, in request order, and behind the graph one kernel
-// that copies next -> staging. So replay r consumes what replay r-1 (or the priming below) drew, the
+// of its own (two mask buffers, generator snapshot), and the recorded graph only READS the slots'
+// `staging` buffers: it contains no generator kernel at all. Each replay (bship_graph_launch) then
+// issues, next to the graph and on the second stream, ONE draw of the raw words of all slots'
+// following masks (they are consecutive in the stream; long enough, the draw is cut into parallel
+// segments) and one kernel that turns them into the slots' `next` buffers, and behind the graph one
+// kernel that copies next -> staging. So replay r consumes what replay r-1 (or the priming below) drew, the
 // random stream is used exactly as by eager execution, and the draws overlap the whole step as
 // ordinary work of a second stream. (Drawing inside the graph, on a captured branch, was measured
 // first: the graph executor ran a branch forked where the mask is consumed partly, and a branch
@@ -611,6 +611,8 @@ static void prefetch_maybe_start() {
 // before the pending, not yet consumed masks.
 struct GraphMasks {
     std::vector<MaskPrefetch> slots;
+    uint32_t* raw = nullptr;       // the raw words of one round of all slots' masks: they are consecutive in the
+    size_t words = 0;              // stream, so a round is ONE draw (a parallel one, if long enough)
     bool primed = false;
 };
 static std::map<int, GraphMasks> g_graph_masks;
@@ -644,13 +646,10 @@ static int graph_mask_slot(size_t n, double p, MaskPrefetch* hit) {
     void* a = nullptr;
     void* a2 = nullptr;
     void* b = nullptr;
-    void* r = nullptr;
     int st = pool_alloc_raw(n * sizeof(float), &a);
     e.staging = static_cast<float*>(a);
     if (st == 0) st = pool_alloc_raw(n * sizeof(float), &a2);
     e.next = static_cast<float*>(a2);
-    if (st == 0) st = pool_alloc_raw(2 * n * sizeof(uint32_t), &r);
-    e.raw = static_cast<uint32_t*>(r);
     if (st == 0) st = pool_alloc_raw(sizeof(RngState), &b);
     e.before = static_cast<RngState*>(b);
     if (st != 0) { free_entry(e); return st; }
@@ -664,8 +663,46 @@ static int graph_mask_redraw(MaskPrefetch& e) {
     return 0;
 }
 
-// next -> staging for up to kMaxSlotCopies slots in one launch (grid.y = slot)
+// masks of up to kMaxSlotCopies slots from their parts of one raw draw, in one launch (grid.y = slot)
 constexpr int kMaxSlotCopies = 16;
+struct SlotMasks { const uint32_t* raw[kMaxSlotCopies]; float* mask[kMaxSlotCopies]; size_t n[kMaxSlotCopies]; double p[kMaxSlotCopies]; };
+__global__ __launch_bounds__(kBlock) void raw_to_masks_kernel(SlotMasks c) {
+    const size_t n = c.n[blockIdx.y];
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const double p = c.p[blockIdx.y];
+    uint64_t threshold;
+    if (!(p > 0.0)) threshold = 0;
+    else if (p >= 1.0) threshold = ~static_cast<uint64_t>(0);
+    else threshold = static_cast<uint64_t>(ceil(p * 9007199254740992.0));
+    c.mask[blockIdx.y][i] = raw_to_k53(c.raw[blockIdx.y], i) < threshold ? 1.0f : 0.0f;
+}
+
+// One round of the slots' masks, drawn on `stream` into their `next` (or `staging`) buffers; the first
+// slot's snapshot receives the generator state from before the round.
+static int launch_graph_masks(hipStream_t stream, GraphMasks& gm, bool into_next) {
+    launch_raw_words(stream, gm.raw, gm.words, gm.slots.front().before, true);
+    size_t offset = 0;
+    for (size_t first = 0; first < gm.slots.size(); first += kMaxSlotCopies) {
+        SlotMasks c = SlotMasks();
+        size_t most = 0;
+        const size_t count = gm.slots.size() - first < static_cast<size_t>(kMaxSlotCopies) ? gm.slots.size() - first : kMaxSlotCopies;
+        for (size_t k = 0; k < count; ++k) {
+            const MaskPrefetch& e = gm.slots[first + k];
+            c.raw[k] = gm.raw + offset;
+            c.mask[k] = into_next ? e.next : e.staging;
+            c.n[k] = e.n;
+            c.p[k] = e.p;
+            offset += 2 * e.n;
+            most = e.n > most ? e.n : most;
+        }
+        hipLaunchKernelGGL(raw_to_masks_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(most), kBlock)),
+                                                     static_cast<unsigned>(count)), dim3(kBlock), 0, stream, c);
+    }
+    return check_launch("masks of a recorded step");
+}
+
+// next -> staging for up to kMaxSlotCopies slots in one launch (grid.y = slot)
 struct SlotCopies { const float* src[kMaxSlotCopies]; float* dst[kMaxSlotCopies]; size_t n[kMaxSlotCopies]; };
 __global__ __launch_bounds__(kBlock) void slot_copy_kernel(SlotCopies c) {
     const float* src = c.src[blockIdx.y];
@@ -691,11 +728,19 @@ int rng_graph_begin(int id) {
     return 0;
 }
 
+// The recording is complete: one buffer for the raw words of a round of its masks (a block of the recording's own).
 int rng_graph_end(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
-    (void)id;
     g_recording_masks = 0;
-    return 0;
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    GraphMasks& gm = it->second;
+    gm.words = 0;
+    for (const MaskPrefetch& e : gm.slots) gm.words += 2 * e.n;
+    void* r = nullptr;
+    int st = pool_alloc_raw(gm.words * sizeof(uint32_t), &r);
+    gm.raw = static_cast<uint32_t*>(r);
+    return st;
 }
 
 int rng_graph_before_launch(int id) {
@@ -706,8 +751,7 @@ int rng_graph_before_launch(int id) {
         int st = prefetch_flush(true);
         if (st == 0) st = graph_masks_unprime();
         if (st != 0) return st;
-        for (MaskPrefetch& e : it->second.slots) launch_mask(ctx().stream, e.staging, e.n, e.p, e.before, e.raw, true);
-        st = check_launch("recorded masks, first draw");
+        st = launch_graph_masks(ctx().stream, it->second, false);
         if (st != 0) return st;
         it->second.primed = true;
         g_primed_graph = id;
@@ -725,8 +769,7 @@ int rng_graph_after_launch(int id) {
     // the second stream starts behind everything that preceded the graph on the main stream: the
     // priming draws, or the previous replay's copy out of the `next` buffers
     BSHIP_HIP(hipStreamWaitEvent(g_side, g_before_graph, 0));
-    for (MaskPrefetch& e : slots) launch_mask(g_side, e.next, e.n, e.p, e.before, e.raw, true);
-    int st = check_launch("masks of the next replay");
+    int st = launch_graph_masks(g_side, it->second, true);
     if (st != 0) return st;
     st = order_streams(g_side, ctx().stream);
     for (size_t first = 0; st == 0 && first < slots.size(); first += kMaxSlotCopies) {
@@ -753,6 +796,7 @@ void rng_graph_destroyed(int id) {
     if (it == g_graph_masks.end()) return;
     if (g_primed_graph == id) (void)graph_masks_unprime();
     for (MaskPrefetch& e : it->second.slots) free_entry(e);
+    if (it->second.raw) pool_free_raw(it->second.raw);
     g_graph_masks.erase(it);
 }
 
@@ -917,8 +961,10 @@ void rng_release() {
     if (g_side) (void)hipStreamSynchronize(g_side);
     for (MaskPrefetch& e : g_fifo) free_entry(e);
     g_fifo.clear();
-    for (auto& kv : g_graph_masks)
+    for (auto& kv : g_graph_masks) {
         for (MaskPrefetch& e : kv.second.slots) free_entry(e);
+        if (kv.second.raw) pool_free_raw(kv.second.raw);
+    }
     g_graph_masks.clear();
     g_primed_graph = 0;
     g_recording_masks = 0;
