@@ -89,6 +89,9 @@ __global__ __launch_bounds__(kBlock) void colsum_kernel(Src src, float* out, int
     }
 }
 
+// Matrices of up to this many rows are summed by one band of workgroups (one launch).
+constexpr int64_t kColsumSingleBandRows = 256;
+
 // Column-lanes for a matrix of NW accesses per row.
 static inline int colsum_lanes(int64_t NW) { return NW > 32 ? 64 : NW > 16 ? 32 : NW > 8 ? 16 : 8; }
 
@@ -126,6 +129,9 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld =
     const int64_t min_rows = 4 * (4 * kBlock / cl);      // at least 4 unrolled steps per lane
     if (bands > ceil_div(M, min_rows)) bands = ceil_div(M, min_rows);
     if (bands > 1024) bands = 1024;
+    // few rows (bias gradients at small batch): a second launch costs more than one band loses
+    // (100 x 1200: 3.6 us against 7; 1000 x 200 would take 20 against 7)
+    if (M <= kColsumSingleBandRows) bands = 1;
     float* dst = out;
     float* partial = nullptr;
     if (bands > 1) {
