@@ -836,7 +836,7 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
 }
 
 // The main stream has enqueued its read of the entry's staging buffer: draw the entry again
-// for the next round.
+// for the step after.
 static int mask_end(MaskPrefetch& e) {
     if (g_recording_masks) return graph_mask_redraw(e);
     hipError_t err = hipEventRecord(e.consumed, ctx().stream);
