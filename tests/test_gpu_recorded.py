@@ -157,6 +157,52 @@ def test_masks_of_recorded_steps_continue_the_random_stream(hip, ref):
     check("eager step after release")
 
 
+def test_two_recordings_with_masks_share_the_random_stream(hip, ref):
+    # two recorded steps that both draw masks, replayed in turn: each replay takes the next numbers of the one
+    # stream (the pending masks of the other recording are given up, nothing is skipped or used twice)
+    sa, sb, sc = (100, 784), (64, 1200), (3, 7)
+    ma, mb, mc = hip.allocate(sa), hip.allocate(sb), hip.allocate(sc)
+    ra, rb, rc = np.zeros(sa, F32), np.zeros(sb, F32), np.zeros(sc, F32)
+
+    def step_a():
+        hip.generate_probability_mask(ma, 0.8)
+        hip.generate_probability_mask(mc, 0.5)
+
+    def step_b():
+        hip.generate_probability_mask(mb, 0.3)
+
+    def ref_a():
+        ref.generate_probability_mask(ra, 0.8)
+        ref.generate_probability_mask(rc, 0.5)
+
+    def ref_b():
+        ref.generate_probability_mask(rb, 0.3)
+
+    rec_a, rec_b = hip.record(step_a), hip.record(step_b)
+    for k, which in enumerate("aabababbba"):
+        if which == "a":
+            rec_a.replay()
+            ref_a()
+            assert_bit_equal(hip.get_numpy_copy(ma), ra, "replay %d (a): first mask" % k)
+            assert_bit_equal(hip.get_numpy_copy(mc), rc, "replay %d (a): second mask" % k)
+        else:
+            rec_b.replay()
+            ref_b()
+            assert_bit_equal(hip.get_numpy_copy(mb), rb, "replay %d (b)" % k)
+    rec_a.release()
+    step_b()
+    ref_b()
+    assert_bit_equal(hip.get_numpy_copy(mb), rb, "eager step after one recording was released")
+    rec_b.replay()
+    ref_b()
+    assert_bit_equal(hip.get_numpy_copy(mb), rb, "replay of the other recording afterwards")
+    rec_b.release()
+    _, key, pos, _, _ = hip.rnd.get_state()
+    st = ref.rnd.get_state()
+    assert pos == st[2]
+    np.testing.assert_array_equal(key, st[1])
+
+
 def test_recorded_training_steps_equal_eager_ones():
     from brainstorm_amd import HipHandler
     from brainstorm_amd.drivers import configs
