@@ -49,44 +49,71 @@ static inline int row_lanes_log2(int64_t cols) {
 }
 
 // out[row, c] = f(in0, in1, in2)[row, c]; an input may be `out` itself (a lane reads all of
-// its operands before it writes). A workgroup covers 2^(8-L) rows x one tile of 2^L accesses.
-template <int NIN, typename F>
+// its operands before it writes). A workgroup covers 2^(8-L) rows x one tile of VPL * 2^L accesses
+// (VPL = 2 for the float64 transcendentals, as in the dense kernels: more loads in flight per
+// wavefront to cover the long arithmetic phase).
+template <int NIN, int VPL, typename F>
 __global__ __launch_bounds__(kBlock) void map2d_kernel(F f, Operand2d in0, Operand2d in1, Operand2d in2,
                                                        float* out, int64_t ldo, int64_t rows, int64_t cols,
                                                        unsigned tiles_per_row, int L) {
     const int64_t row = (static_cast<int64_t>(blockIdx.x / tiles_per_row) << (8 - L)) + (threadIdx.x >> L);
-    const int64_t c = ((static_cast<int64_t>(blockIdx.x % tiles_per_row) << L) + (threadIdx.x & ((1u << L) - 1))) * 4;
-    if (row >= rows || c >= cols) return;
-    float* q = out + row * ldo + c;
-    if (c + 4 <= cols) {
-        const f4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-        const f4 v0 = NIN > 0 ? load4(in0, row, c) : zero;
-        const f4 v1 = NIN > 1 ? load4(in1, row, c) : zero;
-        const f4 v2 = NIN > 2 ? load4(in2, row, c) : zero;
-        f4 o;
+    const int64_t c0 = ((static_cast<int64_t>(blockIdx.x % tiles_per_row) * VPL << L) + (threadIdx.x & ((1u << L) - 1))) * 4;
+    if (row >= rows) return;
+    const f4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    f4 v0[VPL], v1[VPL], v2[VPL];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = f.apply(v0[k], v1[k], v2[k]);
-        vstore<4, false>(q, o);
-    } else {
-        for (int64_t j = 0; c + j < cols; ++j)
-            q[j] = f.apply(NIN > 0 ? load1(in0, row, c + j) : 0.0f, NIN > 1 ? load1(in1, row, c + j) : 0.0f,
-                           NIN > 2 ? load1(in2, row, c + j) : 0.0f);
+    for (int u = 0; u < VPL; ++u) {
+        const int64_t c = c0 + (static_cast<int64_t>(u) << (L + 2));
+        if (c + 4 <= cols) {
+            v0[u] = NIN > 0 ? load4(in0, row, c) : zero;
+            v1[u] = NIN > 1 ? load4(in1, row, c) : zero;
+            v2[u] = NIN > 2 ? load4(in2, row, c) : zero;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+        const int64_t c = c0 + (static_cast<int64_t>(u) << (L + 2));
+        if (c >= cols) continue;
+        float* q = out + row * ldo + c;
+        if (c + 4 <= cols) {
+            f4 o;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) o[k] = f.apply(v0[u][k], v1[u][k], v2[u][k]);
+            vstore<4, false>(q, o);
+        } else {
+            for (int64_t j = 0; c + j < cols; ++j)
+                q[j] = f.apply(NIN > 0 ? load1(in0, row, c + j) : 0.0f, NIN > 1 ? load1(in1, row, c + j) : 0.0f,
+                               NIN > 2 ? load1(in2, row, c + j) : 0.0f);
+        }
     }
 }
 
 struct FillOp { float val; __device__ float apply(float, float, float) const { return val; } };
 
+template <typename F, typename = void> struct VectorsPerLane2d { static constexpr int value = 1; };
+template <typename F> struct VectorsPerLane2d<F, std::void_t<decltype(F::kVectorsPerLane)>> {
+    static constexpr int value = F::kVectorsPerLane;
+};
+
 template <int NIN, typename F>
 static int launch_map2d(const char* name, F f, Operand2d in0, Operand2d in1, Operand2d in2, float* out,
                         int64_t ldo, int64_t rows, int64_t cols) {
+    constexpr int VPL = VectorsPerLane2d<F>::value;
     const int L = row_lanes_log2(cols);
-    const int64_t tiles_per_row = ceil_div(cols, int64_t(4) << L);
+    const bool wide = VPL > 1 && L == 8 && cols > (int64_t(4) << 8);      // rows longer than one tile
+    const int vpl = wide ? VPL : 1;
+    const int64_t tiles_per_row = ceil_div(cols, (int64_t(4) << L) * vpl);
     const int64_t row_groups = ceil_div(rows, int64_t(1) << (8 - L));
     if (tiles_per_row * row_groups > 0x7fffffff)
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %lld x %lld elements exceed one launch", name,
                          static_cast<long long>(rows), static_cast<long long>(cols));
-    hipLaunchKernelGGL((map2d_kernel<NIN, F>), dim3(static_cast<unsigned>(tiles_per_row * row_groups)), dim3(kBlock),
-                       0, ctx().stream, f, in0, in1, in2, out, ldo, rows, cols, static_cast<unsigned>(tiles_per_row), L);
+    const dim3 grid(static_cast<unsigned>(tiles_per_row * row_groups));
+    if (wide)
+        hipLaunchKernelGGL((map2d_kernel<NIN, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f, in0, in1, in2, out, ldo,
+                           rows, cols, static_cast<unsigned>(tiles_per_row), L);
+    else
+        hipLaunchKernelGGL((map2d_kernel<NIN, 1, F>), grid, dim3(kBlock), 0, ctx().stream, f, in0, in1, in2, out, ldo,
+                           rows, cols, static_cast<unsigned>(tiles_per_row), L);
     return check_launch(name);
 }
 

@@ -106,6 +106,8 @@ NATIVE_OPS = [
     ("sign_t", lambda h, a, b, o, r, c: h.sign_t(a, o)),
     ("sqrt_t of abs", lambda h, a, b, o, r, c: (h.abs_t(a, o), h.sqrt_t(o, o))),
     ("sigmoid", lambda h, a, b, o, r, c: h.sigmoid(a, o)),
+    ("tanh", lambda h, a, b, o, r, c: h.tanh(a, o)),
+    ("log_t of abs", lambda h, a, b, o, r, c: (h.abs_t(a, o), h.log_t(o, o))),
     ("rel in place", lambda h, a, b, o, r, c: h.rel(a, a)),
     ("el", lambda h, a, b, o, r, c: h.el(a, o)),
     ("sigmoid_deriv", lambda h, a, b, o, r, c: h.sigmoid_deriv(None, a, b, o)),
@@ -131,8 +133,8 @@ NATIVE_OPS = [
 
 
 @pytest.mark.parametrize("rows,width,cuts", [(37, 790, (3, 260, 517, 774)), (5, 40, (1, 8, 15, 22)),
-                                             (300, 4100, (4, 1028, 2052, 3076))],
-                         ids=["257 columns at odd offsets", "7 columns", "1024 columns, aligned"])
+                                             (300, 4100, (4, 1028, 2052, 3076)), (9, 7600, (5, 2530, 5055, 7580))],
+                         ids=["257 columns at odd offsets", "7 columns", "1024 columns, aligned", "2525 columns"])
 @pytest.mark.parametrize("name,call", NATIVE_OPS, ids=[n for n, _ in NATIVE_OPS])
 def test_row_pitched_kernels(php, name, call, rows, width, cuts):
     # the kernels that take row-pitched operands as they are: same bits as NumPy on strided views,
@@ -158,7 +160,7 @@ def test_row_pitched_kernels(php, name, call, rows, width, cuts):
                            (dev_c.get(), want_c, "column vector")):
         if name.startswith("sum_t"):
             np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=name + ": " + tag)
-        elif name == "sigmoid":
+        elif name in ("sigmoid", "tanh", "log_t of abs"):
             # NumPy's float32 formula and the device result are each within 2 units in the last place
             # of the exact value (test_gpu_parity.py); the dense kernel's bits are checked below
             np.testing.assert_array_max_ulp(got, want, maxulp=4)
