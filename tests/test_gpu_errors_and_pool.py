@@ -29,6 +29,17 @@ def test_bad_arguments_return_errors_not_crashes(hip):
     assert lib.bship_fill_f32(x.ptr + 2, 1.0, 1) == -7                      # not 4-byte aligned
     assert lib.bship_free(x.ptr + 4) == -7                                  # not a pool block
     assert lib.bship_maxpool_fwd_nhwc_f32(x.ptr, x.ptr, x.ptr, 1, 2, 2, 1, 1, 1, 0, 2, 0, 1, 1) == -3
+    # row-pitched forms: family / operation codes, pitches and strides are checked before any launch
+    pitched = lib.bship_elementwise_pitched_f32
+    assert pitched(99, 0, 0.0, 0.0, x.ptr, 4, 1, x.ptr, 4, 1, x.ptr, 4, 2, 4) == -4         # unknown family
+    assert pitched(0, 99, 0.0, 0.0, x.ptr, 4, 1, x.ptr, 4, 1, x.ptr, 4, 2, 4) == -4         # unknown operation
+    assert pitched(0, 0, 0.0, 0.0, x.ptr, 4, 1, x.ptr, 4, 1, x.ptr, 3, 2, 4) == -3          # pitch below the row length
+    assert pitched(0, 0, 0.0, 0.0, x.ptr, 4, 2, x.ptr, 4, 1, x.ptr, 4, 2, 4) == -3          # column stride not 0 or 1
+    assert pitched(0, 0, 0.0, 0.0, None, 4, 1, x.ptr, 4, 1, x.ptr, 4, 2, 4) == -2           # missing operand
+    assert pitched(0, 0, 0.0, 0.0, x.ptr, 4, 1, x.ptr, 4, 1, x.ptr, 4, 0, 4) == 0           # no rows: nothing to do
+    assert lib.bship_sum_pitched_f32(x.ptr, 3, x.ptr, 2, 4, 0) == -3                        # pitch below the row length
+    assert lib.bship_softmax_ce_bwd_f32(x.ptr, None, x.ptr, x.ptr, x.ptr, 2, 4) == -2
+    assert lib.bship_momentum_update_f32(0.9, -0.1, x.ptr, x.ptr + 2, x.ptr, 8) == -7
     assert lib.bship_init(hip.device) == 0                                   # idempotent
     assert lib.bship_init(hip.device + 1000) != 0                            # another device: refused
     with pytest.raises(_lib.BshipError):
