@@ -9,14 +9,14 @@ namespace bship {
 // columns of one row, one store per lane (the shape of the fill kernel).
 // WT selects write-through stores (large outputs). KW = K / W.
 template <int W, bool AL, bool WT>
-__global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restrict__ v,
-                                                          float* __restrict__ out, int64_t KW,
+__global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restrict__ v, int64_t ldv,
+                                                          float* __restrict__ out, int64_t ldo, int64_t KW,
                                                           unsigned tiles_per_row) {
     const int64_t row = blockIdx.x / tiles_per_row;
     const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
     if (c >= KW) return;
-    const int64_t hot = static_cast<int64_t>(static_cast<int>(v[row]));
-    float* q = out + (row * KW + c) * W;
+    const int64_t hot = static_cast<int64_t>(static_cast<int>(v[row * ldv]));
+    float* q = out + row * ldo + c * W;         // ldv, ldo: elements from one row to the next
     typename VecT<W>::type r;
     if constexpr (W == 4) {
         const int64_t j = c * 4;
@@ -30,14 +30,14 @@ __global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restric
 }
 
 // out[i] = m[i, (int)v[i]]; labels outside [0,K) read as 0.
-__global__ __launch_bounds__(kBlock) void index_m_by_v_kernel(const float* __restrict__ m,
-                                                              const float* __restrict__ v,
-                                                              float* __restrict__ out, int64_t M,
+__global__ __launch_bounds__(kBlock) void index_m_by_v_kernel(const float* __restrict__ m, int64_t ldm,
+                                                              const float* __restrict__ v, int64_t ldv,
+                                                              float* __restrict__ out, int64_t ldo, int64_t M,
                                                               int64_t K) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (row >= M) return;
-    const int64_t j = static_cast<int64_t>(static_cast<int>(v[row]));
-    out[row] = (j >= 0 && j < K) ? m[row * K + j] : 0.0f;
+    const int64_t j = static_cast<int64_t>(static_cast<int>(v[row * ldv]));
+    out[row * ldo] = (j >= 0 && j < K) ? m[row * ldm + j] : 0.0f;
 }
 
 }  // namespace bship
@@ -47,8 +47,13 @@ using namespace bship;
 extern "C" {
 
 int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K) {
+    return bship_binarize_pitched_f32(v, 1, out, K, M, K);
+}
+
+int bship_binarize_pitched_f32(const float* v, int64_t ld_v, float* out, int64_t ld_out, int64_t M, int64_t K) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(M >= 0 && K >= 0);
+    BSHIP_REQUIRE_DIM(ld_v >= 1 && ld_out >= K);
     if (M == 0 || K == 0) return 0;
     BSHIP_REQUIRE_PTR(v);
     BSHIP_REQUIRE_PTR(out);
@@ -56,29 +61,36 @@ int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K) {
     BSHIP_REQUIRE_F32_ALIGNED(out);
     const bool vec = (K % 4 == 0);
     const int64_t KW = vec ? K / 4 : K;
+    const bool al = aligned16(out) && ld_out % 4 == 0;
     const int64_t tiles_per_row = ceil_div(KW, kBlock);
     BSHIP_REQUIRE_DIM(tiles_per_row * M <= 0x7fffffff);
     const dim3 grid(static_cast<unsigned>(tiles_per_row * M)), blk(kBlock);
     const unsigned tpr = static_cast<unsigned>(tiles_per_row);
     const bool wt = static_cast<size_t>(M) * static_cast<size_t>(K) >= ctx().write_through_min;
     hipStream_t s = ctx().stream;
-    if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, out, KW, tpr);
-    else if (vec && aligned16(out))  hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, out, KW, tpr);
-    else if (vec)                    hipLaunchKernelGGL((binarize_kernel<4, false, false>), grid, blk, 0, s, v, out, KW, tpr);
-    else if (wt)                     hipLaunchKernelGGL((binarize_kernel<1, false, true>), grid, blk, 0, s, v, out, KW, tpr);
-    else                             hipLaunchKernelGGL((binarize_kernel<1, false, false>), grid, blk, 0, s, v, out, KW, tpr);
+    if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
+    else if (vec && al)              hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
+    else if (vec)                    hipLaunchKernelGGL((binarize_kernel<4, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
+    else if (wt)                     hipLaunchKernelGGL((binarize_kernel<1, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
+    else                             hipLaunchKernelGGL((binarize_kernel<1, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
     return check_launch("binarize_v");
 }
 
 int bship_index_m_by_v_f32(const float* m, const float* v, float* out, int64_t M, int64_t K) {
+    return bship_index_m_by_v_pitched_f32(m, K, v, 1, out, 1, M, K);
+}
+
+int bship_index_m_by_v_pitched_f32(const float* m, int64_t ld_m, const float* v, int64_t ld_v, float* out,
+                                   int64_t ld_out, int64_t M, int64_t K) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(M >= 0 && K >= 0);
+    BSHIP_REQUIRE_DIM(ld_m >= K && ld_v >= 1 && ld_out >= 1);
     if (M == 0) return 0;
     BSHIP_REQUIRE_PTR(m);
     BSHIP_REQUIRE_PTR(v);
     BSHIP_REQUIRE_PTR(out);
     hipLaunchKernelGGL(index_m_by_v_kernel, dim3(static_cast<unsigned>(ceil_div(M, kBlock))),
-                       dim3(kBlock), 0, ctx().stream, m, v, out, M, K);
+                       dim3(kBlock), 0, ctx().stream, m, ld_m, v, ld_v, out, ld_out, M, K);
     return check_launch("index_m_by_v");
 }
 

@@ -181,7 +181,7 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
 // The launcher guarantees N % W == 0 and N / W <= THREADS * PER.
 template <int W, bool AL, int BLOCK, int THREADS, int PER>
 __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, float* out, int64_t M,
-                                                            int64_t N) {
+                                                            int64_t N, int64_t ldm, int64_t ldo) {
     constexpr int ROWS = BLOCK / THREADS;
     constexpr int WAVES = BLOCK / kWave;
     typedef typename VecT<W>::type R;
@@ -190,8 +190,8 @@ __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, floa
     const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / THREADS;
     const bool live = row < M;
     const int64_t NW = N / W;
-    const float* p = m + (live ? row : 0) * N;
-    float* q = out + (live ? row : 0) * N;
+    const float* p = m + (live ? row : 0) * ldm;       // ldm, ldo: elements from one row to the next
+    float* q = out + (live ? row : 0) * ldo;
     // All loads are issued before anything depends on one of them: lanes beyond the row's
     // end read element 0 instead (always valid) and are replaced by -inf afterwards, so
     // the loads sit in no branch and the wavefront keeps PER of them in flight.
@@ -256,12 +256,12 @@ __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, floa
 // Rows too long for registers: a workgroup per row, three sweeps (max, sum of
 // exponentials, normalise); the second and third sweeps mostly hit the caches.
 __global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, float* out, int64_t M,
-                                                              int64_t N) {
+                                                              int64_t N, int64_t ldm, int64_t ldo) {
     __shared__ float lds[kBlock / kWave];
     const int wv = threadIdx.x / kWave;
     const int64_t row = blockIdx.x;
-    const float* p = m + row * N;
-    float* q = out + row * N;
+    const float* p = m + row * ldm;
+    float* q = out + row * ldo;
     float mx = -INFINITY;
     for (int64_t i = threadIdx.x; i < N; i += kBlock) mx = fmaxf(mx, p[i]);
     mx = wave_max(mx);
@@ -279,31 +279,32 @@ __global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, fl
 }
 
 template <int W, bool AL, int BLOCK, int THREADS>
-static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N) {
+static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N, int64_t ldm,
+                               int64_t ldo) {
     hipStream_t s = ctx().stream;
     const dim3 b(BLOCK);
     switch (per) {
-        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N); break;
-        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N); break;
-        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N); break;
-        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N); break;
-        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N); break;
+        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
+        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
+        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
+        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
+        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
     }
 }
 
 template <int BLOCK, int THREADS>
 static void launch_softmax_threads(bool vec, bool al, int per, dim3 grid, const float* m, float* out,
-                                   int64_t M, int64_t N) {
-    if (vec && al) launch_softmax_per<4, true, BLOCK, THREADS>(per, grid, m, out, M, N);
-    else if (vec)  launch_softmax_per<4, false, BLOCK, THREADS>(per, grid, m, out, M, N);
-    else           launch_softmax_per<1, false, BLOCK, THREADS>(per, grid, m, out, M, N);
+                                   int64_t M, int64_t N, int64_t ldm, int64_t ldo) {
+    if (vec && al) launch_softmax_per<4, true, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
+    else if (vec)  launch_softmax_per<4, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
+    else           launch_softmax_per<1, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
 }
 
 constexpr int kWideBlock = 1024;
 
-static int launch_softmax(const float* m, float* out, int64_t M, int64_t N) {
+static int launch_softmax(const float* m, float* out, int64_t M, int64_t N, int64_t ldm, int64_t ldo) {
     const bool vec = (N % 4 == 0);
-    const bool al = aligned16(m) && aligned16(out);
+    const bool al = aligned16(m) && aligned16(out) && ldm % 4 == 0 && ldo % 4 == 0;
     const int64_t NW = vec ? N / 4 : N;
     // smallest power-of-two number of accesses per lane that covers the row
     auto per_for = [&](int threads) {
@@ -314,15 +315,15 @@ static int launch_softmax(const float* m, float* out, int64_t M, int64_t N) {
     if (NW <= static_cast<int64_t>(kWave) * 16) {
         // a wavefront per row, 4 rows per workgroup
         launch_softmax_threads<kBlock, kWave>(vec, al, per_for(kWave),
-                                              dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N);
+                                              dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N, ldm, ldo);
     } else if (NW <= static_cast<int64_t>(kBlock) * 4) {
-        launch_softmax_threads<kBlock, kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N);
+        launch_softmax_threads<kBlock, kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo);
     } else if (NW <= static_cast<int64_t>(kWideBlock) * 16) {
         launch_softmax_threads<kWideBlock, kWideBlock>(vec, al, per_for(kWideBlock),
-                                                       dim3(static_cast<unsigned>(M)), m, out, M, N);
+                                                       dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo);
     } else {
         hipLaunchKernelGGL(softmax_long_kernel, dim3(static_cast<unsigned>(M)), dim3(kBlock), 0,
-                           ctx().stream, m, out, M, N);
+                           ctx().stream, m, out, M, N, ldm, ldo);
     }
     return check_launch("softmax_m");
 }
@@ -377,15 +378,20 @@ int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, i
 }
 
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N) {
+    return bship_softmax_rows_pitched_f32(m, N, out, N, M, N);
+}
+
+int bship_softmax_rows_pitched_f32(const float* m, int64_t ld_m, float* out, int64_t ld_out, int64_t M, int64_t N) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    BSHIP_REQUIRE_DIM(ld_m >= N && ld_out >= N);
     if (M == 0 || N == 0) return 0;
     BSHIP_REQUIRE_PTR(m);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(m);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
-    return launch_softmax(m, out, M, N);
+    return launch_softmax(m, out, M, N, ld_m, ld_out);
 }
 
 int bship_isfinite_f32(const float* a, size_t n, int* result_host) {

@@ -125,6 +125,9 @@ def _native_pitched_table():
              "add_into_if": ew(PITCHED_COND, ADD_IF, "out", "a", "cond"),
              "mult_add_mv": mv(PITCHED_MULT_ADD, 0),
              "copy_to": lambda h, A: h._pitched_copy(A["src"], A["dest"]),
+             "softmax_m": lambda h, A: h._pitched_softmax(A["m"], A["out"]),
+             "binarize_v": lambda h, A: h._pitched_binarize(A["v"], A["out"]),
+             "index_m_by_v": lambda h, A: h._pitched_index(A["m"], A["v"], A["out"]),
              "sum_t": lambda h, A: h._pitched_sum(A["a"], A["axis"], A["out"])}
     for name, op in (("add", ADD), ("subtract", SUB), ("mult", MUL), ("divide", DIV)):
         table[name + "_tt"] = ew(PITCHED_BINARY, op, "out", "a", "b")
@@ -256,6 +259,41 @@ class HipHandler(Handler):
         pd, ldd = self._as_matrix(dest, rows, cols)
         ps, lds = self._as_matrix(src, rows, cols)
         self._call(self._lib.bship_copy2d_f32(pd, ldd, ps, lds, rows, cols))
+
+    def _as_column(self, v, rows):
+        """(address, elements from entry to entry) of `v` read as a column of `rows` entries."""
+        if v.size != rows:
+            raise _NoNativePath()
+        if type(v) is PitchedDeviceArray:
+            if v.shape[-1] != 1:
+                raise _NoNativePath()
+            return v._base, v.pitch
+        return v.ptr, 1
+
+    def _pitched_softmax(self, m, out):
+        if m.ndim != 2 or out.shape != m.shape:
+            raise _NoNativePath()
+        rows, cols = m.shape
+        pm, ldm = self._as_matrix(m, rows, cols)
+        po, ldo = self._as_matrix(out, rows, cols)
+        self._call(self._lib.bship_softmax_rows_pitched_f32(pm, ldm, po, ldo, rows, cols))
+
+    def _pitched_binarize(self, v, out):
+        if out.ndim != 2:
+            raise _NoNativePath()
+        rows, k = out.shape
+        pv, ldv = self._as_column(v, rows)
+        po, ldo = self._as_matrix(out, rows, k)
+        self._call(self._lib.bship_binarize_pitched_f32(pv, ldv, po, ldo, rows, k))
+
+    def _pitched_index(self, m, v, out):
+        if m.ndim != 2:
+            raise _NoNativePath()
+        rows, k = m.shape
+        pm, ldm = self._as_matrix(m, rows, k)
+        pv, ldv = self._as_column(v, rows)
+        po, ldo = self._as_column(out, rows)
+        self._call(self._lib.bship_index_m_by_v_pitched_f32(pm, ldm, pv, ldv, po, ldo, rows, k))
 
     def _pitched_sum(self, a, axis, out):
         if (type(a) is not PitchedDeviceArray or type(out) is PitchedDeviceArray

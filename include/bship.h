@@ -252,6 +252,9 @@ int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis);
 int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, int64_t N, int axis);
 /* softmax_m (numpy 292-295, pycuda 403-408): row-wise, one pass over HBM. */
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N);
+/* The same for row-pitched m and out (ld_m, ld_out elements from one row to the next, >= N). */
+int bship_softmax_rows_pitched_f32(const float* m, int64_t ld_m, float* out, int64_t ld_out,
+                                   int64_t M, int64_t N);
 /* is_fully_finite (numpy 69-70, pycuda 111-114). *result_host = 1 if every
  * element is finite. Blocks. */
 int bship_isfinite_f32(const float* a, size_t n, int* result_host);
@@ -260,10 +263,16 @@ int bship_isfinite_f32(const float* a, size_t n, int* result_host);
 
 /* binarize_v (numpy 99-101, pycuda 163-164): out[i,j] = (j == (int)v[i]) */
 int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K);
+/* The same with the labels ld_v elements apart (a column of a wider matrix) and a row-pitched out. */
+int bship_binarize_pitched_f32(const float* v, int64_t ld_v, float* out, int64_t ld_out, int64_t M, int64_t K);
 /* index_m_by_v (numpy 202-203, pycuda 284-285): out[i] = m[i, (int)v[i]].
  * Labels outside [0,K) are undefined in the reference; here they read as 0. */
 int bship_index_m_by_v_f32(const float* m, const float* v, float* out,
                            int64_t M, int64_t K);
+/* The same for a row-pitched m, and labels / results that are columns of wider matrices
+ * (ld_v, ld_out elements from one row to the next). */
+int bship_index_m_by_v_pitched_f32(const float* m, int64_t ld_m, const float* v, int64_t ld_v,
+                                   float* out, int64_t ld_out, int64_t M, int64_t K);
 
 /* --------------------------------- RNG ----------------------------------- */
 

@@ -129,6 +129,12 @@ NATIVE_OPS = [
     ("sum_t axis 0", lambda h, a, b, o, r, c: h.sum_t(a, 0, r)),
     ("sum_t axis 1", lambda h, a, b, o, r, c: h.sum_t(a, 1, c)),
     ("sum_t of all", lambda h, a, b, o, r, c: h.sum_t(a, None, c[0:1].reshape(()))),
+    ("softmax_m", lambda h, a, b, o, r, c: h.softmax_m(a, o)),
+    ("softmax_m in place", lambda h, a, b, o, r, c: h.softmax_m(a, a)),
+    ("binarize_v", lambda h, a, b, o, r, c: (h.fill(c, 3.0), h.binarize_v(c, o))),
+    ("binarize_v by a column of the hub", lambda h, a, b, o, r, c: (h.fill(a[:, 2:3], 1.0), h.binarize_v(a[:, 2:3], o))),
+    ("index_m_by_v", lambda h, a, b, o, r, c: (h.fill(c, 2.0), h.index_m_by_v(a, c, c))),
+    ("index_m_by_v into a column of the hub", lambda h, a, b, o, r, c: (h.fill(c, 4.0), h.index_m_by_v(a, c, o[:, 1:2]))),
 ]
 
 
@@ -158,7 +164,7 @@ def test_row_pitched_kernels(php, name, call, rows, width, cuts):
     assert temporaries == [], temporaries
     for got, want, tag in ((dev_hub.get(), want_hub, "hub"), (dev_r.get(), want_r, "row vector"),
                            (dev_c.get(), want_c, "column vector")):
-        if name.startswith("sum_t"):
+        if name.startswith("sum_t") or name.startswith("softmax_m"):
             np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5, err_msg=name + ": " + tag)
         elif name in ("sigmoid", "tanh", "log_t of abs"):
             # NumPy's float32 formula and the device result are each within 2 units in the last place
