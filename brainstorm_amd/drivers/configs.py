@@ -107,7 +107,7 @@ def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10
     return _finish(net, data, flat)
 
 
-def build_cnn(handler, seed=4, batch=100, size=32, classes=10):
+def build_cnn(handler, seed=4, batch=100, size=32, classes=10, fused=False):
     rng = np.random.RandomState(seed)
     data = {"default": rng.standard_normal((1, batch, size, size, 3)).astype(F32),
             "targets": rng.randint(0, classes, (1, batch, 1)).astype(F32)}
@@ -117,9 +117,9 @@ def build_cnn(handler, seed=4, batch=100, size=32, classes=10):
         ("pool1", Pooling2D("max", (3, 3), stride=(2, 2)), {"default": "conv1.default"}),
         ("conv2", Convolution2D(64, (5, 5), padding=2, activation="rel"), {"default": "pool1.default"}),
         ("pool2", Pooling2D("max", (3, 3), stride=(2, 2)), {"default": "conv2.default"}),
-        ("fc", FullyConnected(1000, "rel"), {"default": "pool2.default"}),
-        ("out", FullyConnected(classes, "linear"), {"default": "fc.default"}),
-        ("ce", SoftmaxCE(), {"default": "out.default", "targets": "Input.targets"}),
+        ("fc", FullyConnected(1000, "rel", fused=fused), {"default": "pool2.default"}),
+        ("out", FullyConnected(classes, "linear", fused=fused), {"default": "fc.default"}),
+        ("ce", SoftmaxCE(fused=fused), {"default": "out.default", "targets": "Input.targets"}),
         ("loss", Loss(), {"default": "ce.loss"}),
     ])
     return _finish(net, data, _init_parameters(net, rng, 0.05))
