@@ -384,6 +384,7 @@ constexpr int kMaxSegments = 64;
 constexpr int kMinSegments = 4;                 // below (61 000 words), the sequential kernel is as fast
 constexpr size_t kEagerJumpMinWords = size_t(1) << 20;
 struct JumpPolys { uint32_t* dev; int count; };
+constexpr size_t kMaxJumpTables = 256;          // distinct segment lengths kept (up to 160 KB of device memory each)
 static std::vector<uint32_t*> g_jump_retired;          // replaced tables, freed at shutdown
 static std::map<size_t, JumpPolys> g_jump_polys;      // words per segment -> polynomials of 1, 2, ... segments ahead
 static uint32_t* g_hist = nullptr;                    // kHistWords words
@@ -425,6 +426,7 @@ static const uint32_t* jump_polys(size_t seg_words, int count) {
     auto it = g_jump_polys.find(seg_words);
     if (it != g_jump_polys.end() && it->second.count >= count) return it->second.dev;
     if (graph_recording()) return nullptr;
+    if (it == g_jump_polys.end() && g_jump_polys.size() >= kMaxJumpTables) return nullptr;   // draw sequentially
     if (!g_hist && hipMalloc(reinterpret_cast<void**>(&g_hist), kHistWords * sizeof(uint32_t)) != hipSuccess) {
         (void)hipGetLastError(); g_hist = nullptr; return nullptr;
     }
