@@ -832,13 +832,16 @@ def test_many_small_fills_keep_call_order(hip):
     want += 1.0
     assert_bit_equal(flat.get(), want, "small fills in call order")
     assert_bit_equal(other.get(), np.full((7, 9), 9.0, F32), "small fill of another array")
-    big = hip.allocate((1 << 19,))                    # a large fill between small ones
-    hip.fill(big[5:100], 3.0)
-    hip.fill(big, 2.0)
-    hip.fill(big[7:9], 4.0)
-    wb = np.full((1 << 19,), 2.0, F32)
-    wb[7:9] = 4.0
-    assert_bit_equal(big.get(), wb, "large fill between small ones")
+    for n in (1 << 19, 1 << 23):                      # a collected and an immediate large fill between small ones
+        big = hip.allocate((n,))
+        hip.fill(big[5:100], 3.0)
+        hip.fill(big, 2.0)
+        hip.fill(big[7:9], 4.0)
+        hip.fill(big[n - 3:], 8.0)
+        wb = np.full((n,), 2.0, F32)
+        wb[7:9] = 4.0
+        wb[n - 3:] = 8.0
+        assert_bit_equal(big.get(), wb, "large fill (%d elements) between small ones" % n)
 
 
 # ---------------------------------------------------------- views of one buffer
