@@ -763,15 +763,12 @@ int rng_graph_before_launch(int id) {
 
 // The graph of recording `id` has just been enqueued on the main stream: next to it, the second
 // stream draws the masks of the replay after this one; behind it, they move into place.
-int rng_graph_after_launch(int id) {
-    std::lock_guard<std::mutex> lock(g_rng_mutex);
-    auto it = g_graph_masks.find(id);
-    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
-    std::vector<MaskPrefetch>& slots = it->second.slots;
+static int draw_next_round(GraphMasks& gm) {
+    std::vector<MaskPrefetch>& slots = gm.slots;
     // the second stream starts behind everything that preceded the graph on the main stream: the
     // priming draws, or the previous replay's copy out of the `next` buffers
     BSHIP_HIP(hipStreamWaitEvent(g_side, g_before_graph, 0));
-    int st = launch_graph_masks(g_side, it->second, true);
+    int st = launch_graph_masks(g_side, gm, true);
     if (st != 0) return st;
     st = order_streams(g_side, ctx().stream);
     for (size_t first = 0; st == 0 && first < slots.size(); first += kMaxSlotCopies) {
@@ -788,6 +785,19 @@ int rng_graph_after_launch(int id) {
         hipLaunchKernelGGL(slot_copy_kernel, dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(count)),
                            dim3(kBlock), 0, ctx().stream, c);
         st = check_launch("masks of the next replay, move into place");
+    }
+    return st;
+}
+
+int rng_graph_after_launch(int id) {
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    auto it = g_graph_masks.find(id);
+    if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    const int st = draw_next_round(it->second);
+    if (st != 0) {
+        // the staging buffers were not refilled: the next replay must not consume them again
+        it->second.primed = false;
+        if (g_primed_graph == id) g_primed_graph = 0;
     }
     return st;
 }
