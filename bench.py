@@ -196,10 +196,16 @@ def run_image_ops(hip, n_img=2048, reps=10):
         hip._call(lib.bship_event_elapsed_ms(0, 1, ctypes.byref(ms)))
         return ms.value * 1e3 / reps
 
-    def filled(shape):
-        a = hip.allocate(shape)
-        hip.fill(a, 0.5)
-        return a
+    def filled(shape, seed=[0]):
+        # N(0,1) data (a seeded 4 MiB block repeated on the device): which pixel of a window is the
+        # largest decides what the pooling kernels touch, so constant inputs would not be representative
+        seed[0] += 1
+        n, base = int(np.prod(shape)), 1 << 20
+        src = hip.create_from_numpy(np.random.RandomState(seed[0]).standard_normal((1, base)).astype(F32))
+        reps = (n + base - 1) // base
+        big = hip.allocate((reps, base))
+        hip.broadcast_t(src, 0, big)
+        return big.reshape((reps * base,))[:n].reshape(shape)
 
     out = {}
 
