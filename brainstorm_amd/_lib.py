@@ -64,6 +64,7 @@ SIGNATURES = {
     "bship_split_add_f32": [_P, _P, _P, _I64, _I64, _I64],
     "bship_sum_f32": [_P, _P, _I64, _I64, c_int],
     "bship_sum_pitched_f32": [_P, _I64, _P, _I64, _I64, c_int],
+    "bship_sum_noalloc_f32": [_P, _P, _I64, _I64, c_int],
     "bship_softmax_rows_pitched_f32": [_P, _I64, _P, _I64, _I64, _I64],
     "bship_binarize_pitched_f32": [_P, _I64, _P, _I64, _I64, _I64],
     "bship_index_m_by_v_pitched_f32": [_P, _I64, _P, _I64, _P, _I64, _I64, _I64],

@@ -114,9 +114,17 @@ static void launch_colsum_kernel(bool vec, bool al, int cl, dim3 grid, Src src, 
     else           launch_colsum_lanes<1, false, Src>(cl, grid, src, dst, M, NW, ld);
 }
 
+// Where the partial sums of a multi-band launch go: a block of the pool (ptr == nullptr), or a
+// buffer the caller owns that holds `floats` floats (callers that must not allocate).
+struct PartialsBuffer {
+    float* ptr = nullptr;
+    size_t floats = 0;
+};
+
 // ld: elements from one row of the source matrices to the next (0: dense, ld = N).
 template <typename Src>
-static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld = 0) {
+static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld = 0,
+                         PartialsBuffer ws = PartialsBuffer()) {
     const Context& c = ctx();
     if (ld == 0) ld = N;
     const bool vec = (N % 4 == 0);
@@ -134,7 +142,14 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld =
     if (M <= kColsumSingleBandRows) bands = 1;
     float* dst = out;
     float* partial = nullptr;
-    if (bands > 1) {
+    if (bands > 1 && ws.ptr) {
+        if (static_cast<size_t>(bands) * N > ws.floats)
+            return set_error(BSHIP_ERR_BAD_DIMENSION,
+                             "sum over axis 0 of a (%lld, %lld) matrix needs %lld floats of partial sums, "
+                             "the buffer given holds %zu", static_cast<long long>(M), static_cast<long long>(N),
+                             static_cast<long long>(bands * N), ws.floats);
+        dst = ws.ptr;
+    } else if (bands > 1) {
         void* p = nullptr;
         int st = pool_alloc_raw(static_cast<size_t>(bands) * N * sizeof(float), &p);
         if (st != 0) return st;
@@ -145,14 +160,14 @@ static int launch_colsum(Src src, float* out, int64_t M, int64_t N, int64_t ld =
     launch_colsum_kernel(vec, src.aligned() && aligned16(dst) && ld % 4 == 0, cl,
                          dim3(static_cast<unsigned>(gx), static_cast<unsigned>(bands)), src, dst, M, NW, ld);
     int st = check_launch("sum over axis 0");
-    if (partial) {
+    if (dst != out) {
         if (st == 0) {
             // second stage: column sums of the (bands, N) partials in one band
-            launch_colsum_kernel(vec, aligned16(partial) && aligned16(out), cl,
-                                 dim3(static_cast<unsigned>(gx), 1), PlainSrc{partial}, out, bands, NW, N);
+            launch_colsum_kernel(vec, aligned16(dst) && aligned16(out), cl,
+                                 dim3(static_cast<unsigned>(gx), 1), PlainSrc{dst}, out, bands, NW, N);
             st = check_launch("sum over axis 0, stage 2");
         }
-        pool_free_raw(partial);   // a later owner of the block runs after this launch
+        if (partial) pool_free_raw(partial);   // a later owner of the block runs after this launch
     }
     return st;
 }

@@ -39,6 +39,7 @@ void graph_release_all();  // graph.hip
 void pool_release_all();   // pool.hip
 void rng_release();        // rng.hip
 void gemm_release();       // gemm.hip
+int reduce_scratch_init(int device);   // reduce.hip
 
 }  // namespace bship
 
@@ -70,6 +71,15 @@ int bship_init(int device) {
     snprintf(g_ctx.name, sizeof(g_ctx.name), "%s (%s)", prop.name, prop.gcnArchName);
     // One stream at the default priority; every kernel and copy goes here in call order.
     BSHIP_HIP(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking));
+    {
+        // device address of the static partial-sum buffer of bship_sum_noalloc_f32, once per device
+        int st = reduce_scratch_init(device);
+        if (st != 0) {
+            (void)hipStreamDestroy(g_ctx.stream);
+            g_ctx.stream = nullptr;
+            return st;
+        }
+    }
     const char* dbg = getenv("BSHIP_DEBUG_SYNC");
     g_ctx.debug_sync = dbg && dbg[0] && dbg[0] != '0';
     const char* bpc = getenv("BSHIP_BLOCKS_PER_CU");

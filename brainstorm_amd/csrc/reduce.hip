@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void sumchunk_kernel(const float* __restric
     if (threadIdx.x == 0) partial[blockIdx.x] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
 }
 
-static int launch_sumall(const float* a, float* out, int64_t n) {
+static int launch_sumall(const float* a, float* out, int64_t n, PartialsBuffer ws = PartialsBuffer()) {
     const Context& c = ctx();
     const int64_t min_chunk = 16384;
     int64_t chunks = static_cast<int64_t>(c.num_cus) * 8;
@@ -131,7 +131,13 @@ static int launch_sumall(const float* a, float* out, int64_t n) {
     chunks = ceil_div(n, len);
     float* dst = out;
     float* partial = nullptr;
-    if (chunks > 1) {
+    if (chunks > 1 && ws.ptr) {
+        if (static_cast<size_t>(chunks) > ws.floats)
+            return set_error(BSHIP_ERR_BAD_DIMENSION,
+                             "sum of %lld elements needs %lld floats of partial sums, the buffer given holds %zu",
+                             static_cast<long long>(n), static_cast<long long>(chunks), ws.floats);
+        dst = ws.ptr;
+    } else if (chunks > 1) {
         void* p = nullptr;
         int st = pool_alloc_raw(static_cast<size_t>(chunks) * sizeof(float), &p);
         if (st != 0) return st;
@@ -146,12 +152,12 @@ static int launch_sumall(const float* a, float* out, int64_t n) {
         hipLaunchKernelGGL(sumchunk_kernel<false>, grid, dim3(kBlock), 0, c.stream, a, dst,
                            static_cast<size_t>(n), static_cast<size_t>(len));
     int st = check_launch("sum_t(axis=None) stage 1");
-    if (partial) {
+    if (dst != out) {
         if (st == 0) {
-            launch_rowsum_kernel<kBlock>(false, false, dim3(1), partial, out, 1, chunks, chunks);
+            launch_rowsum_kernel<kBlock>(false, false, dim3(1), dst, out, 1, chunks, chunks);
             st = check_launch("sum_t(axis=None) stage 2");
         }
-        pool_free_raw(partial);
+        if (partial) pool_free_raw(partial);
     }
     return st;
 }
@@ -340,11 +346,56 @@ __global__ __launch_bounds__(kBlock) void nonfinite_kernel(const float* __restri
     if (bad) *flag = 1;    // every writer stores the same value
 }
 
+// ===================== partial sums without the pool ======================
+// bship_sum_noalloc_f32 keeps the partial sums of its first stage here instead of in a pool
+// block. 1 MiB per device, held until the process ends. In host code the array's name is only
+// a stand-in for the symbol: the device address is looked up once per device
+// (reduce_scratch_init) and every launch gets that pointer.
+constexpr size_t kScratchFloats = size_t(1) << 18;
+static __device__ __align__(256) float scratch[kScratchFloats];
+constexpr int kMaxScratchDevices = 64;
+static float* g_scratch_ptr[kMaxScratchDevices] = {nullptr};
+
+// Called by bship_init with `device` current.
+int reduce_scratch_init(int device) {
+    if (device < 0 || device >= kMaxScratchDevices)
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "device %d: no static partial-sum buffer beyond device %d",
+                         device, kMaxScratchDevices - 1);
+    if (g_scratch_ptr[device]) return 0;
+    void* p = nullptr;
+    int st = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(partial-sum buffer)");
+    if (st != 0) return st;
+    g_scratch_ptr[device] = static_cast<float*>(p);
+    return 0;
+}
+
 }  // namespace bship
 
 using namespace bship;
 
 extern "C" {
+
+int bship_sum_noalloc_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
+    BSHIP_REQUIRE_DIM(axis == 0 || axis == 1 || axis == -1);
+    const int64_t out_n = axis == 0 ? N : (axis == 1 ? M : 1);
+    if (out_n == 0) return 0;
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    if (M == 0 || N == 0) return launch_fill(out, 0.0f, static_cast<size_t>(out_n));  // empty sum
+    BSHIP_REQUIRE_PTR(a);
+    BSHIP_REQUIRE_F32_ALIGNED(a);
+    BSHIP_REQUIRE_DIM(a != out);
+    BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
+    const int device = ctx().device;
+    float* ws = device >= 0 && device < kMaxScratchDevices ? g_scratch_ptr[device] : nullptr;
+    if (!ws) return set_error(BSHIP_ERR_NOT_INITIALIZED, "%s: no partial-sum buffer on device %d", __func__, device);
+    const PartialsBuffer buf{ws, kScratchFloats};
+    if (axis == 0) return M == 1 ? bship_d2d(out, a, static_cast<size_t>(N) * 4) : launch_colsum(PlainSrc{a}, out, M, N, N, buf);
+    if (axis == 1) return N == 1 ? bship_d2d(out, a, static_cast<size_t>(M) * 4) : launch_rowsum(a, out, M, N, N);
+    return launch_sumall(a, out, M * N, buf);
+}
 
 int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
     return bship_sum_pitched_f32(a, N, out, M, N, axis);

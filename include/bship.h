@@ -250,6 +250,18 @@ int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis);
 /* The same for a row-pitched a: ld_a elements from one row to the next (>= N).
  * out is dense. With ld_a == N this is bship_sum_f32. */
 int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, int64_t N, int axis);
+/* bship_sum_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart
+ * in the reference. Same kernels and the same bits as bship_sum_f32, but the partial
+ * sums of the first stage go to a static 1 MiB device buffer (262144 floats, one per
+ * device, held until the process ends) instead of a pool block, and the call makes no
+ * hipMalloc/hipFree. A shape whose partial sums do not fit is refused with
+ * BSHIP_ERR_BAD_DIMENSION; with the default launch shapes a dense matrix needs at most
+ * 196608 floats (axis 0) or 2048 (axis -1), axis 1 needs none. All calls on a device
+ * share the buffer: calls that overlap on one device (several streams, several host
+ * threads) race; nothing in it needs clearing between calls (every partial sum read by
+ * the second stage was written by the first stage of the same call). */
+int bship_sum_noalloc_f32(const float* a, float* out, int64_t M, int64_t N, int axis);
 /* softmax_m (numpy 292-295, pycuda 403-408): row-wise, one pass over HBM. */
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N);
 /* The same for row-pitched m and out (ld_m, ld_out elements from one row to the next, >= N). */
