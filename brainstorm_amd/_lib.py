@@ -72,6 +72,9 @@ SIGNATURES = {
     "bship_isfinite_f32": [_P, c_size_t, POINTER(c_int)],
     "bship_binarize_f32": [_P, _P, _I64, _I64],
     "bship_index_m_by_v_f32": [_P, _P, _P, _I64, _I64],
+    "bship_rng_create": [POINTER(c_int)],
+    "bship_rng_select": [c_int],
+    "bship_rng_destroy": [c_int],
     "bship_rng_seed": [c_uint32],
     "bship_prob_mask_f32": [_P, c_size_t, c_double],
     "bship_fill_gaussian_f32": [_P, c_size_t, c_double, c_double],

@@ -54,8 +54,17 @@ struct RngState {
     double gauss;         // cached second variate of the polar method
 };
 
-static RngState* g_state = nullptr;   // device memory
+// Generators. Every handler object has its own random stream (numpy_handler.py:21: `self.rnd`), so
+// the library keeps any number of generators (MT19937 state + the optional fast stream's state, in
+// device memory) and ONE of them selected: g_state / g_fast_state below are the selected generator's,
+// and the look-ahead queue, the mask slots of a primed recorded step and the pattern history always
+// belong to it. Selecting another generator (bship_rng_select, a cheap no-op when it is selected
+// already) first gives up what was drawn ahead, so each generator's stream is exactly the
+// sequential one whatever the interleaving. Generator 0 exists from the start.
+static RngState* g_state = nullptr;   // device memory; the selected generator's
 static std::mutex g_rng_mutex;
+static int g_current_generator = 0;
+static int select_generator_locked(int id);      // caller holds g_rng_mutex
 
 __device__ __forceinline__ uint32_t mt_twist(uint32_t u, uint32_t v) {
     const uint32_t y = (u & 0x80000000u) | (v & 0x7fffffffu);
@@ -612,6 +621,7 @@ static void prefetch_maybe_start() {
 // Any eager use of the generator first "unprimes": it puts the generator back to the snapshot taken
 // before the pending, not yet consumed masks.
 struct GraphMasks {
+    int generator = 0;             // the generator selected while the step was recorded: its replays draw from it
     std::vector<MaskPrefetch> slots;
     uint32_t* raw = nullptr;       // the raw words of one round of all slots' masks: they are consecutive in the
     size_t words = 0;              // stream, so a round is ONE draw (a parallel one, if long enough)
@@ -727,6 +737,7 @@ int rng_graph_begin(int id) {
     if (st != 0) return st;
     g_recording_masks = id;
     g_graph_masks[id] = GraphMasks();
+    g_graph_masks[id].generator = g_current_generator;
     return 0;
 }
 
@@ -749,6 +760,10 @@ int rng_graph_before_launch(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
+    {
+        int st = select_generator_locked(it->second.generator);
+        if (st != 0) return st;
+    }
     if (g_primed_graph != id) {
         int st = prefetch_flush(true);
         if (st == 0) st = graph_masks_unprime();
@@ -892,7 +907,29 @@ struct FastRngState {
     unsigned long long key;
     unsigned long long next_block;
 };
-static FastRngState* g_fast_state = nullptr;
+static FastRngState* g_fast_state = nullptr;      // the selected generator's
+
+struct Generator { RngState* state = nullptr; FastRngState* fast = nullptr; };
+static std::map<int, Generator> g_generators = {{0, Generator()}};   // states of the generators NOT selected are kept here
+static int g_next_generator = 1;
+
+static int select_generator_locked(int id) {
+    if (id == g_current_generator) return 0;
+    if (g_generators.find(id) == g_generators.end())
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "random generator %d does not exist", id);
+    if (g_recording_masks)
+        return set_error(BSHIP_ERR_UNSUPPORTED, "another random generator cannot be selected while a step is being recorded");
+    // what was drawn ahead belongs to the generator selected so far: back to its sequential position
+    int st = g_state ? prefetch_flush(true) : 0;
+    if (st == 0) st = graph_masks_unprime();
+    if (st != 0) return st;
+    g_min_period = 1;
+    g_generators[g_current_generator] = Generator{g_state, g_fast_state};
+    g_state = g_generators[id].state;
+    g_fast_state = g_generators[id].fast;
+    g_current_generator = id;
+    return 0;
+}
 
 __device__ __forceinline__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
 #pragma unroll
@@ -986,14 +1023,23 @@ void rng_release() {
     if (g_before_graph) { (void)hipEventDestroy(g_before_graph); g_before_graph = nullptr; }
 
     if (g_side) { (void)hipStreamDestroy(g_side); g_side = nullptr; }
-    if (g_state) { pool_free_raw(g_state); g_state = nullptr; }
+    g_generators[g_current_generator] = Generator{g_state, g_fast_state};
+    for (auto& kv : g_generators) {
+        if (kv.second.state) pool_free_raw(kv.second.state);
+        if (kv.second.fast) pool_free_raw(kv.second.fast);
+    }
+    g_generators.clear();
+    g_generators[0] = Generator();
+    g_current_generator = 0;
+    g_next_generator = 1;
+    g_state = nullptr;
+    g_fast_state = nullptr;
     for (auto& kv : g_jump_polys) (void)hipFree(kv.second.dev);
     g_jump_polys.clear();
     for (uint32_t* p : g_jump_retired) (void)hipFree(p);
     g_jump_retired.clear();
     if (g_hist) { (void)hipFree(g_hist); g_hist = nullptr; }
     if (g_seeds) { (void)hipFree(g_seeds); g_seeds = nullptr; }
-    if (g_fast_state) { pool_free_raw(g_fast_state); g_fast_state = nullptr; }
 }
 
 }  // namespace bship
@@ -1001,6 +1047,39 @@ void rng_release() {
 using namespace bship;
 
 extern "C" {
+
+int bship_rng_create(int* generator_id) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(generator_id);
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    *generator_id = g_next_generator++;
+    g_generators[*generator_id] = Generator();
+    return 0;
+}
+
+int bship_rng_select(int generator_id) {
+    BSHIP_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    return select_generator_locked(generator_id);
+}
+
+int bship_rng_destroy(int generator_id) {
+    BSHIP_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator_id == 0) return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator 0 is the library's own");
+    if (g_generators.find(generator_id) == g_generators.end())
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator %d does not exist", generator_id);
+    if (generator_id == g_current_generator) {
+        int st = select_generator_locked(0);
+        if (st != 0) return st;
+    }
+    // the blocks' next owners run on the library's stream, behind every kernel that used them
+    const Generator g = g_generators[generator_id];
+    if (g.state) pool_free_raw(g.state);
+    if (g.fast) pool_free_raw(g.fast);
+    g_generators.erase(generator_id);
+    return 0;
+}
 
 int bship_rng_seed(uint32_t seed) {
     BSHIP_REQUIRE_INIT();

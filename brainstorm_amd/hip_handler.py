@@ -34,13 +34,35 @@ class HipRandomState:
     (randomness.py:10-64): it remembers its seed, can be re-seeded and reset.
     The stream equals numpy.random.RandomState(seed)'s, so masks drawn here
     equal the ones NumpyHandler draws from the same seed.
+
+    Every instance is a generator of its own in the library (bship_rng_create), as every
+    reference handler has its own ``self.rnd`` (numpy_handler.py:21): handlers that are alive
+    together do not disturb each other's streams. ``select()`` makes this generator the one the
+    library's random calls use; the handler calls it in front of each of them.
     """
 
     def __init__(self, handler, seed=None):
         self._handler = handler
+        self._lib = handler._lib
+        gid = ctypes.c_int()
+        handler._call(self._lib.bship_rng_create(ctypes.byref(gid)))
+        self._id = gid.value
         if seed is None:
             seed = int(np.random.randint(*SEED_RANGE))
         self.seed(seed)
+
+    def select(self):
+        st = self._lib.bship_rng_select(self._id)
+        if st:
+            self._handler._call(st)
+
+    def __del__(self):
+        try:
+            if self._id is not None and self._lib is not None:
+                self._lib.bship_rng_destroy(self._id)
+                self._id = None
+        except Exception:
+            pass
 
     def seed(self, seed=None):
         if seed is None:
@@ -48,6 +70,7 @@ class HipRandomState:
         seed = int(seed)
         if not 0 <= seed < 2 ** 32:
             raise ValueError("seed must be between 0 and 2**32 - 1")
+        self.select()
         self._handler._call(self._handler._lib.bship_rng_seed(seed))
         if self._handler.fast_masks:               # the optional mask stream restarts with it
             self._handler._call(self._handler._lib.bship_fast_rng_seed(seed))
@@ -67,6 +90,7 @@ class HipRandomState:
         key = (ctypes.c_uint32 * 624)()
         pos, has_gauss, gauss = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
         h = self._handler
+        self.select()
         h._call(h._lib.bship_rng_get_state(key, ctypes.byref(pos), ctypes.byref(has_gauss),
                                            ctypes.byref(gauss)))
         return ('MT19937', np.frombuffer(key, dtype=np.uint32).copy(), pos.value,
@@ -174,10 +198,15 @@ class HipHandler(Handler):
         self.rnd = HipRandomState(self, seed)
 
     def __describe__(self):
-        return {'@type': self.__class__.__name__}
+        # the constructor's settings travel with a saved network description, as NumpyHandler's
+        # dtype does (numpy_handler.py:25-33); the seed does not (the reference's does not either)
+        return {'@type': self.__class__.__name__, 'device': self.device,
+                'pitched_views': self.pitched_views, 'fast_masks': self.fast_masks}
 
     def __init_from_description__(self, description):
-        self.__init__()
+        self.__init__(device=int(description.get('device', 0)),
+                      pitched_views=bool(description.get('pitched_views', False)),
+                      fast_masks=bool(description.get('fast_masks', False)))
 
     # ------------------------------------------------------------- plumbing
     # parameters an operation writes (everything else is only read); operations that are not
@@ -359,6 +388,7 @@ class HipHandler(Handler):
         those around the replay. Arrays that ``fn`` allocates keep their memory for as long
         as the recording exists. Shapes and addresses are fixed at recording time.
         """
+        self.rnd.select()        # the recording's masks come from this handler's generator, on every replay
         self._call(self._lib.bship_graph_begin())
         try:
             fn()
@@ -585,9 +615,11 @@ class HipHandler(Handler):
 
     # ------------------------------------------------------------------- RNG
     def fill_gaussian(self, mean, std, out):
+        self.rnd.select()
         self._call(self._lib.bship_fill_gaussian_f32(out.ptr, out.size, mean, std))
 
     def generate_probability_mask(self, mask, probability):
+        self.rnd.select()
         if self.fast_masks:
             self._call(self._lib.bship_prob_mask_fast_f32(mask.ptr, mask.size, probability))
         else:
@@ -596,6 +628,7 @@ class HipHandler(Handler):
     def fast_mask_state(self):
         """(seed, next block) of the fast mask generator (fast_masks=True)."""
         seed, block = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        self.rnd.select()
         self._call(self._lib.bship_fast_rng_get_state(ctypes.byref(seed), ctypes.byref(block)))
         return seed.value, block.value
 
@@ -850,5 +883,6 @@ class HipHandler(Handler):
         out = scale * out (dropout_layer.py:41-45) with one pass behind the mask."""
         if not (inputs.shape == mask.shape == out.shape):
             raise ValueError("dropout_forward: inconsistent shapes")
+        self.rnd.select()
         fn = self._lib.bship_dropout_fwd_fast_f32 if self.fast_masks else self._lib.bship_dropout_fwd_f32
         self._call(fn(inputs.ptr, mask.ptr, out.ptr, out.size, float(keep_probability), float(scale)))

@@ -288,7 +288,20 @@ int bship_index_m_by_v_pitched_f32(const float* m, int64_t ld_m, const float* v,
 
 /* --------------------------------- RNG ----------------------------------- */
 
-/* Seeds the device-resident MT19937 state the way
+/* Generators: every handler object owns a random stream (`self.rnd`, numpy 21;
+ * randomness.py 10-80). bship_rng_create makes a new, unseeded generator;
+ * bship_rng_select makes it the one that bship_rng_seed, bship_rng_get_state, the
+ * mask draws, bship_fill_gaussian_f32 and the fast stream's calls use from then on
+ * (nothing happens if it is selected already; otherwise masks drawn ahead for the
+ * generator selected so far are given up, so every generator's stream stays the
+ * sequential one). A recorded step draws from the generator that was selected
+ * while it was recorded and selects it on every replay. Generator 0 exists from
+ * the start and is selected until another one is. bship_rng_destroy frees a
+ * generator's device state (generator 0 cannot be destroyed). */
+int bship_rng_create(int* generator_id);
+int bship_rng_select(int generator_id);
+int bship_rng_destroy(int generator_id);
+/* Seeds the selected generator's device-resident MT19937 state the way
  * numpy.random.RandomState(seed) does (randomness.py 66-80, numpy 21). Blocks. */
 int bship_rng_seed(uint32_t seed);
 /* generate_probability_mask (numpy 199-200): mask = (uniform[0,1) < p), drawing

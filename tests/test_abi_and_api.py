@@ -104,3 +104,25 @@ def test_interface_matches_the_reference_sources():
     assert list(inspect.signature(HipHandler.mult_add_mv).parameters)[1:] == numpy_methods["mult_add_mv"]
     for name in numpy_methods:
         assert hasattr(HipHandler, name), name
+
+
+def test_description_round_trips_the_constructor_settings():
+    # the reference handler describes its constructor argument and is rebuilt from it
+    # (numpy_handler.py:25-33, describable.py); ours does the same for its settings. No GPU needed:
+    # the constructor is replaced by a recorder.
+    from brainstorm_amd.hip_handler import HipHandler
+    h = object.__new__(HipHandler)
+    h.device, h.pitched_views, h.fast_masks = 2, True, True
+    desc = h.__describe__()
+    assert desc == {"@type": "HipHandler", "device": 2, "pitched_views": True, "fast_masks": True}
+    seen = {}
+
+    class Recorder(HipHandler):
+        def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False):
+            seen.update(seed=seed, device=device, pitched_views=pitched_views, fast_masks=fast_masks)
+
+    r = object.__new__(Recorder)
+    r.__init_from_description__(desc)
+    assert seen == {"seed": None, "device": 2, "pitched_views": True, "fast_masks": True}
+    r.__init_from_description__({"@type": "HipHandler"})                  # descriptions written before
+    assert seen == {"seed": None, "device": 0, "pitched_views": False, "fast_masks": False}
