@@ -104,9 +104,14 @@ def _matmul_shapes(op, a):
         _fail(op, "out has shape %r, expected %r" % (tuple(a["out"].shape), (a1, b2)))
 
 
+def _label_count(a):
+    """Number of classes the labels of binarize_v / index_m_by_v select from."""
+    return a["m"].shape[1] if "m" in a else a["out"].shape[1]
+
+
 def _labels_in_range(handler, a):
     labels = handler.get_numpy_copy(a["v"])
-    return labels.size == 0 or (labels.min() >= 0 and int(labels.max()) < a["out"].shape[1])
+    return labels.size == 0 or (labels.min() >= 0 and int(labels.max()) < _label_count(a))
 
 
 _POOL = [shape_tuple("window", 2), shape_tuple("stride", 2), padding_ok]
@@ -157,7 +162,8 @@ CONTRACTS = {
                    where(lambda a: tuple(a["v"].shape) == (a["out"].shape[0], 1), "v must be (rows of out, 1)"),
                    "labels"],
     "index_m_by_v": [same_shape("v", "out"), ndim("m", 2), ndim("v", 2),
-                     where(lambda a: tuple(a["v"].shape) == (a["m"].shape[0], 1), "v must be (rows of m, 1)")],
+                     where(lambda a: tuple(a["v"].shape) == (a["m"].shape[0], 1), "v must be (rows of m, 1)"),
+                     "labels"],
     "fill_gaussian": [where(lambda a: a["std"] >= 0.0, "std must not be negative")],
     "generate_probability_mask": [scalar("probability"),
                                   where(lambda a: 0.0 <= a["probability"] <= 1.0, "probability outside [0, 1]")],
@@ -206,7 +212,7 @@ def _make_method(name):
         for check in checks:
             if check == "labels":
                 if not _labels_in_range(self.handler, a):
-                    _fail(name, "labels outside [0, %d)" % a["out"].shape[1])
+                    _fail(name, "labels outside [0, %d)" % _label_count(a))
             else:
                 check(name, a)
         result = inner(*a.values())           # positionally: handlers differ in some parameter names

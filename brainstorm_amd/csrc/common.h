@@ -175,6 +175,18 @@ void rng_graph_destroyed(int id);
 // Enqueues mem[0:n] = val.
 int launch_fill(float* mem, float val, size_t n);
 
+// ---- integer labels stored as float32 (device) ----
+// Column selected by label v in a row of K columns: truncated toward zero like astype(int32);
+// labels in [-K, -1] count from the end, as NumPy's indexing does (numpy_handler.py:101, 203).
+// Anything else (beyond [-K, K), NaN, infinities) selects no column: -1. NumPy raises IndexError
+// there; a kernel cannot, so such a row gets no one-hot entry and gathers 0.
+__device__ __forceinline__ int64_t label_column(float v, int64_t K) {
+    if (!(v > -2147483648.0f && v < 2147483648.0f)) return -1;
+    int64_t j = static_cast<int64_t>(static_cast<int>(v));
+    if (j < 0) j += K;
+    return (j >= 0 && j < K) ? j : -1;
+}
+
 // ---- wavefront reductions (device) ----
 // All 64 lanes must be active. Four DPP steps (lane^1, lane^2, mirror inside 8 lanes, mirror inside
 // a row of 16) leave every lane of a row with the row's result without touching LDS (a shuffle is a

@@ -336,8 +336,8 @@ __global__ __launch_bounds__(kBlock) void softmax_ce_loss_kernel(const float* __
                                                                  float* __restrict__ loss, int64_t M, int64_t K) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (row >= M) return;
-    const int64_t j = static_cast<int64_t>(static_cast<int>(targets[row]));
-    float p = (j >= 0 && j < K) ? probs[row * K + j] : 0.0f;
+    const int64_t j = label_column(targets[row], K);
+    float p = j >= 0 ? probs[row * K + j] : 0.0f;
     p = ClipOp{1e-6f, 1.0f}.apply(p, 0.0f, 0.0f);
     p = LogOp{}.apply(p, 0.0f, 0.0f);
     loss[row] = MultStOp{-1.0f}.apply(p, 0.0f, 0.0f);
@@ -353,7 +353,7 @@ __global__ __launch_bounds__(kBlock) void softmax_ce_bwd_kernel(const float* __r
     if (i >= total) return;
     const int64_t row = i / K;
     const int64_t j = i - row * K;
-    float t = (j == static_cast<int64_t>(static_cast<int>(targets[row]))) ? 1.0f : 0.0f;
+    float t = (j == label_column(targets[row], K)) ? 1.0f : 0.0f;
     t = MultStOp{-1.0f}.apply(t, 0.0f, 0.0f);
     t = AddOp{}.apply(t, probs[i], 0.0f);
     t = MulOp{}.apply(t, dloss[row], 0.0f);

@@ -2,7 +2,9 @@
 // hipBLASLt is column-major, so C = op(A) op(B) is issued as
 // C^T = op(B)^T op(A)^T by swapping the operands. Descriptors and the algorithm
 // chosen by the heuristic are cached per problem shape, because recurrent
-// networks issue the same small product thousands of times per step.
+// networks issue the same small product thousands of times per step. The cache
+// holds the kMaxPlans most recently used shapes (workloads with varying batch or
+// sequence lengths would otherwise grow it without limit).
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
@@ -20,6 +22,7 @@ struct GemmPlan {
     hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
+    uint64_t last_use = 0;
 };
 
 typedef std::tuple<int, int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int> GemmKey;   // ..., with bias
@@ -27,6 +30,10 @@ typedef std::tuple<int, int, int64_t, int64_t, int64_t, int64_t, int64_t, int64_
 std::mutex g_gemm_mutex;
 hipblasLtHandle_t g_handle = nullptr;
 std::map<GemmKey, GemmPlan> g_plans;
+constexpr size_t kMaxPlans = 512;
+uint64_t g_use_counter = 0;
+// The products' workspace is not a pool block: the first product may arrive while a step is being
+// recorded, and blocks handed out then belong to that recording.
 void* g_workspace = nullptr;
 constexpr size_t kWorkspaceBytes = 64u << 20;
 
@@ -92,7 +99,7 @@ void gemm_release() {
     std::lock_guard<std::mutex> lock(g_gemm_mutex);
     for (auto& kv : g_plans) destroy_plan(kv.second);
     g_plans.clear();
-    if (g_workspace) { pool_free_raw(g_workspace); g_workspace = nullptr; }
+    if (g_workspace) { (void)hipFree(g_workspace); g_workspace = nullptr; }
     if (g_handle) { hipblasLtDestroy(g_handle); g_handle = nullptr; }
 }
 
@@ -106,8 +113,13 @@ static int gemm_impl(int transa, int transb, int64_t M, int64_t N, int64_t K, fl
     std::lock_guard<std::mutex> lock(g_gemm_mutex);
     if (!g_handle) BSHIP_BLAS(hipblasLtCreate(&g_handle));
     if (!g_workspace) {
-        int st = pool_alloc_raw(kWorkspaceBytes, &g_workspace);
-        if (st != 0) return st;
+        hipError_t e = hipMalloc(&g_workspace, kWorkspaceBytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            g_workspace = nullptr;
+            return set_error(BSHIP_ERR_OUT_OF_MEMORY, "hipMalloc of the %zu-byte product workspace failed: %s",
+                             kWorkspaceBytes, hipGetErrorString(e));
+        }
     }
     // Row-major C(MxN) = op(A) op(B)  <=>  column-major C^T(NxM) = op(B)^T op(A)^T.
     // A row-major matrix read as column-major is its transpose, so the first
@@ -120,8 +132,18 @@ static int gemm_impl(int transa, int transb, int64_t M, int64_t N, int64_t K, fl
         int st = make_plan(plan, transb ? HIPBLAS_OP_T : HIPBLAS_OP_N, transa ? HIPBLAS_OP_T : HIPBLAS_OP_N,
                            N, M, K, ldb, lda, ldc, bias != nullptr);
         if (st != 0) { destroy_plan(plan); return st; }
+        if (g_plans.size() >= kMaxPlans) {
+            // drop the shape that has not been used for the longest time (launches already
+            // enqueued keep no reference to a plan)
+            auto oldest = g_plans.begin();
+            for (auto jt = g_plans.begin(); jt != g_plans.end(); ++jt)
+                if (jt->second.last_use < oldest->second.last_use) oldest = jt;
+            destroy_plan(oldest->second);
+            g_plans.erase(oldest);
+        }
         it = g_plans.emplace(key, plan).first;
     }
+    it->second.last_use = ++g_use_counter;
     const GemmPlan& p = it->second;
     if (bias)
         BSHIP_BLAS(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));

@@ -1,21 +1,22 @@
 // Integer-label operations: one-hot rows (binarize_v) and the per-row gather
 // (index_m_by_v). Labels are float32-valued integers, truncated toward zero
-// like NumPy's astype(int32).
+// like NumPy's astype(int32); negative labels count from the last column, as
+// NumPy's indexing does (label_column in common.h).
 #include "common.h"
 
 namespace bship {
 
-// out[i, j] = (j == (int)v[i]). Write-only: one workgroup per tile of kBlock*W
+// out[i, j] = (j == label_column(v[i])). Write-only: one workgroup per tile of kBlock*W
 // columns of one row, one store per lane (the shape of the fill kernel).
 // WT selects write-through stores (large outputs). KW = K / W.
 template <int W, bool AL, bool WT>
 __global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restrict__ v, int64_t ldv,
                                                           float* __restrict__ out, int64_t ldo, int64_t KW,
-                                                          unsigned tiles_per_row) {
+                                                          int64_t K, unsigned tiles_per_row) {
     const int64_t row = blockIdx.x / tiles_per_row;
     const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
     if (c >= KW) return;
-    const int64_t hot = static_cast<int64_t>(static_cast<int>(v[row * ldv]));
+    const int64_t hot = label_column(v[row * ldv], K);
     float* q = out + row * ldo + c * W;         // ldv, ldo: elements from one row to the next
     typename VecT<W>::type r;
     if constexpr (W == 4) {
@@ -29,15 +30,15 @@ __global__ __launch_bounds__(kBlock) void binarize_kernel(const float* __restric
     else vstore<W, AL>(q, r);
 }
 
-// out[i] = m[i, (int)v[i]]; labels outside [0,K) read as 0.
+// out[i] = m[i, label_column(v[i])]; labels outside [-K,K) read as 0.
 __global__ __launch_bounds__(kBlock) void index_m_by_v_kernel(const float* __restrict__ m, int64_t ldm,
                                                               const float* __restrict__ v, int64_t ldv,
                                                               float* __restrict__ out, int64_t ldo, int64_t M,
                                                               int64_t K) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (row >= M) return;
-    const int64_t j = static_cast<int64_t>(static_cast<int>(v[row * ldv]));
-    out[row * ldo] = (j >= 0 && j < K) ? m[row * ldm + j] : 0.0f;
+    const int64_t j = label_column(v[row * ldv], K);
+    out[row * ldo] = j >= 0 ? m[row * ldm + j] : 0.0f;
 }
 
 }  // namespace bship
@@ -68,11 +69,11 @@ int bship_binarize_pitched_f32(const float* v, int64_t ld_v, float* out, int64_t
     const unsigned tpr = static_cast<unsigned>(tiles_per_row);
     const bool wt = static_cast<size_t>(M) * static_cast<size_t>(K) >= ctx().write_through_min;
     hipStream_t s = ctx().stream;
-    if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
-    else if (vec && al)              hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
-    else if (vec)                    hipLaunchKernelGGL((binarize_kernel<4, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
-    else if (wt)                     hipLaunchKernelGGL((binarize_kernel<1, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
-    else                             hipLaunchKernelGGL((binarize_kernel<1, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, tpr);
+    if (vec && wt)                   hipLaunchKernelGGL((binarize_kernel<4, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, K, tpr);
+    else if (vec && al)              hipLaunchKernelGGL((binarize_kernel<4, true, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, K, tpr);
+    else if (vec)                    hipLaunchKernelGGL((binarize_kernel<4, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, K, tpr);
+    else if (wt)                     hipLaunchKernelGGL((binarize_kernel<1, false, true>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, K, tpr);
+    else                             hipLaunchKernelGGL((binarize_kernel<1, false, false>), grid, blk, 0, s, v, ld_v, out, ld_out, KW, K, tpr);
     return check_launch("binarize_v");
 }
 

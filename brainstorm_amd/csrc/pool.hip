@@ -50,6 +50,7 @@ static void* g_bounce = nullptr;
 static void* g_bounce_dev = nullptr;
 static std::mutex g_bounce_mutex;
 static unsigned g_bounce_seq = 0;              // number of the last polled read-back (behind the buffer)
+static bool g_bounce_failed = false;           // coherent pinned memory could not be had: ordinary copies
 
 int pool_alloc_raw(size_t nbytes, void** out) {
     *out = nullptr;
@@ -154,6 +155,7 @@ void pool_release_all() {
         std::lock_guard<std::mutex> block(g_bounce_mutex);
         if (g_bounce) (void)hipHostFree(g_bounce);
         g_bounce = g_bounce_dev = nullptr;
+        g_bounce_failed = false;
     }
     std::lock_guard<std::mutex> lock(g_pool_mutex);
     trim_locked();
@@ -345,13 +347,19 @@ int bship_pool_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_
 }
 
 // Pinned host memory for small transfers, allocated on first use (the caller holds g_bounce_mutex).
+// Coherent (fine-grained) memory, asked for explicitly: the host polls a sequence number that a
+// running kernel writes behind its data, which needs the kernel's system-scope release to be visible
+// to the host while the kernel runs; with the default flag that depends on the environment. If such
+// memory cannot be had, small transfers take the runtime's ordinary copies.
 static bool bounce_ready() {
     if (g_bounce) return true;
-    if (hipHostMalloc(&g_bounce, kBounceBytes + 64, hipHostMallocDefault) != hipSuccess ||
+    if (g_bounce_failed) return false;
+    if (hipHostMalloc(&g_bounce, kBounceBytes + 64, hipHostMallocCoherent | hipHostMallocMapped) != hipSuccess ||
         hipHostGetDevicePointer(&g_bounce_dev, g_bounce, 0) != hipSuccess) {
         (void)hipGetLastError();
         if (g_bounce) (void)hipHostFree(g_bounce);
         g_bounce = g_bounce_dev = nullptr;
+        g_bounce_failed = true;
         return false;
     }
     memset(static_cast<char*>(g_bounce) + kBounceBytes, 0, 64);

@@ -108,3 +108,27 @@ def test_pool_limit_raises_memory_error(hip):
     big = hip.allocate((4 << 20,))                       # fine again without the cap
     hip.fill(big, 1.0)
     assert float(big[-1:].get()[0]) == 1.0
+
+
+def test_small_transfers_behind_a_long_queue(hip):
+    # Read-backs and uploads of a few bytes poll pinned memory for at most 1 ms and then wait for the
+    # stream the ordinary way. Several milliseconds of queued work in front of them take that second
+    # path; the values must be the same. Every kernel here runs to its normal end.
+    n = 1 << 28
+    a = hip.allocate((n,))
+    hip.fill(a, 1.0)
+    hip.synchronize()
+    for _ in range(12):                               # about 12 x 0.33 ms
+        hip.mult_st(1.0001, a, a)
+    one = hip.get_numpy_copy(a[12345:12346])          # read-back of one float behind the queue
+    want = np.float32(1.0)
+    for _ in range(12):
+        want = np.float32(want * np.float32(1.0001))
+    assert one[0] == want
+    for _ in range(12):
+        hip.mult_st(1.0001, a, a)
+    small = hip.allocate((3,))
+    hip.set_from_numpy(small, np.array([1.5, -2.5, 3.5], np.float32))       # upload behind the queue
+    assert small.get().tolist() == [1.5, -2.5, 3.5]
+    assert hip.is_fully_finite(a)
+    del a
