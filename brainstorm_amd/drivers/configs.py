@@ -28,16 +28,37 @@ from .net import Net
 F32 = np.float32
 
 
-def _init_parameters(net, rng, std, special=None):
-    """Gaussian weights, zero biases; `special` maps a parameter-name suffix to a constant."""
+def _init_parameters(net, rng, std, special=None, quick=None):
+    """Gaussian weights, zero biases; `special` maps a parameter-name suffix to a constant.
+
+    `quick(layer_name)` -> None or an int: weights of layers for which it returns an int are drawn
+    from a float32 PCG64 stream seeded with that int instead of `rng`, several layers at a time on
+    host threads (what makes a 1.7 G-parameter network quick to set up; RandomState's float64
+    polar method is sequential and takes minutes for it).
+    """
     flat = np.zeros(net.parameter_count(), dtype=F32)
+    jobs = []
     for name, (a, b, shape) in net.parameter_slices().items():
-        leaf = name.split(".")[-1]
+        layer, leaf = name.split(".")
         if special and leaf in special:
             flat[a:b] = special[leaf]
         elif len(shape) >= 2:
-            flat[a:b] = (rng.standard_normal(b - a) * std).astype(F32)
+            stream = quick(layer) if quick else None
+            if stream is None:
+                flat[a:b] = (rng.standard_normal(b - a) * std).astype(F32)
+            else:
+                jobs.append((stream, a, b))
         # 1-D parameters (biases) stay zero
+
+    def draw(job):
+        stream, a, b = job
+        np.random.Generator(np.random.PCG64(stream)).standard_normal(out=flat[a:b], dtype=F32)
+        flat[a:b] *= F32(std)
+
+    if jobs:
+        import concurrent.futures
+        with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
+            list(pool.map(draw, jobs))
     return flat
 
 
@@ -82,7 +103,12 @@ def build_lstm(handler, seed=2, time_steps=100, batch=100, symbols=205, hidden=1
     return _finish(net, data, _init_parameters(net, rng, 0.05))
 
 
-def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10, fused=False):
+def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10, fused=False,
+                  quick_init_from_block=None, parameters=None):
+    """quick_init_from_block: blocks from this index on (and the output layer) take their weights
+    from per-layer PCG64 streams (see _init_parameters), so the first blocks of a deep network have
+    the weights of the shallow network with the same seed. parameters: a flat float32 vector to
+    use instead of drawing one."""
     rng = np.random.RandomState(seed)
     data = {"default": rng.standard_normal((1, batch, width)).astype(F32),
             "targets": rng.randint(0, classes, (1, batch, 1)).astype(F32)}
@@ -103,7 +129,18 @@ def build_highway(handler, seed=3, blocks=50, batch=2048, width=4096, classes=10
         ("loss", Loss(), {"default": "ce.loss"}),
     ]
     net = Net(handler, layers)
-    flat = _init_parameters(net, rng, 1.0 / np.sqrt(width), special={"gamma": 1.0, "sigma": 1.0})
+    if parameters is not None:
+        return _finish(net, data, parameters)
+
+    def quick(layer):
+        if quick_init_from_block is None:
+            return None
+        if layer == "out":
+            return 1000 * seed + 999
+        block = int(layer[1:])                       # "H12", "T12"
+        return None if block < quick_init_from_block else 1000 * seed + 2 * block + (layer[0] == "T")
+
+    flat = _init_parameters(net, rng, 1.0 / np.sqrt(width), special={"gamma": 1.0, "sigma": 1.0}, quick=quick)
     return _finish(net, data, flat)
 
 

@@ -64,8 +64,25 @@ def compare_all(net_h, net_r, tol, exact=()):
     return max(worst.values())
 
 
-def test_mlp_training_steps(hip):
-    net_h, net_r = both(configs.build_mlp, hip, 21)
+def device_equal(hip, a, b):
+    """True if the device arrays a and b hold the same finite values everywhere (sum |a - b| == 0,
+    computed on the device: the deep network's buffers are too large to compare on the host)."""
+    n = a.size
+    if n == 0:
+        return True
+    diff = hip._scratch((n,))
+    hip.subtract_tt(a.reshape((n,)), b.reshape((n,)), diff)
+    hip.abs_t(diff, diff)
+    total = hip.allocate(())
+    hip.sum_t(diff, None, total)
+    return float(total.get()) == 0.0
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
+def test_mlp_training_steps(hip, fused):
+    # fused=True: dropout, bias + activation, softmax cross entropy and the momentum update through
+    # the fused entry points, held to the oracle's primitive sequence at the same bars
+    net_h, net_r = both(lambda h, **kw: configs.build_mlp(h, fused=fused and h is hip, **kw), hip, 21)
     net_h.forward_pass(training_pass=True)
     net_r.forward_pass(training_pass=True)
     net_h.backward_pass()
@@ -77,7 +94,7 @@ def test_mlp_training_steps(hip):
     g_err = scaled_err(net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients)
     assert g_err <= 1e-5, g_err
     # 20 momentum steps (lr 0.1, momentum 0.9 as in examples/mnist_pi.py:46) with fresh masks
-    st_h, st_r = MomentumStepper(0.1, 0.9), MomentumStepper(0.1, 0.9)
+    st_h, st_r = MomentumStepper(0.1, 0.9, fused=fused), MomentumStepper(0.1, 0.9)
     st_h.start(net_h)
     st_r.start(net_r)
     for _ in range(20):
@@ -89,7 +106,37 @@ def test_mlp_training_steps(hip):
     assert p_err <= 1e-4, p_err
     loss_h, loss_r = net_h.get("loss", "outputs", "loss")[0], net_r.get("loss", "outputs", "loss")[0]
     assert abs(loss_h - loss_r) <= 1e-4 * abs(loss_r)
-    print("mlp: worst buffer %.2e, gradient %.2e, parameters after 20 steps %.2e" % (worst, g_err, p_err))
+    print("mlp (fused=%s): worst buffer %.2e, gradient %.2e, parameters after 20 steps %.2e"
+          % (fused, worst, g_err, p_err))
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
+def test_mlp_recorded_training_steps(hip, fused):
+    # the step recorded into a HIP graph and replayed (masks drawn next to the replay, in parallel
+    # segments of the same MT19937 stream), against the oracle's eager steps: same masks, same bars
+    net_h, net_r = both(lambda h, **kw: configs.build_mlp(h, fused=fused and h is hip, **kw), hip, 27)
+    st_h, st_r = MomentumStepper(0.1, 0.9, fused=fused), MomentumStepper(0.1, 0.9)
+    st_h.start(net_h)
+    st_r.start(net_r)
+    st_h.run()                     # one ordinary step first: nothing is set up inside the recording
+    st_r.run()
+    try:
+        for step in range(12):
+            st_h.run_recorded()
+            st_r.run()
+            if step in (0, 5, 11):
+                for k in ("drop1", "drop2", "drop3"):
+                    assert_bit_equal(net_h.get(k, "internals", "mask"), net_r.get(k, "internals", "mask"),
+                                     "%s after replay %d" % (k, step))
+                loss_h = net_h.get("loss", "outputs", "loss")[0]
+                loss_r = net_r.get("loss", "outputs", "loss")[0]
+                assert abs(loss_h - loss_r) <= 1e-4 * abs(loss_r), (step, loss_h, loss_r)
+        worst = compare_all(net_h, net_r, 1e-4, {("drop1", "mask"), ("drop2", "mask"), ("drop3", "mask")})
+        p_err = scaled_err(hip.get_numpy_copy(net_h.parameters), net_r.parameters)
+        assert p_err <= 1e-4, p_err
+    finally:
+        st_h.release_recorded()
+    print("mlp recorded (fused=%s): worst buffer %.2e, parameters after 13 steps %.2e" % (fused, worst, p_err))
 
 
 def test_lstm_full_size_forward_backward(hip):
@@ -138,9 +185,13 @@ def test_lstm_full_size_forward_backward(hip):
           % (worst_p, d_err))
 
 
-def test_highway_batchnorm_blocks(hip):
-    # two blocks at the configuration's width and batch (the oracle's matrix products bound the size)
-    net_h, net_r = both(configs.build_highway, hip, 23, blocks=2)
+@pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
+def test_highway_batchnorm_blocks(hip, fused):
+    # two blocks at the configuration's width and batch (the oracle's matrix products bound the size);
+    # fused=True: BatchNorm, Highway, bias + activation and softmax cross entropy through the fused
+    # entry points, against the oracle's primitive sequence
+    net_h, net_r = both(lambda h, **kw: configs.build_highway(h, fused=fused and h is hip, **kw), hip, 23,
+                        blocks=2)
     net_h.forward_pass(training_pass=True)
     net_r.forward_pass(training_pass=True)
     worst_fwd = 0.0
@@ -168,11 +219,103 @@ def test_highway_batchnorm_blocks(hip):
     g_h, g_r = net_h.handler.get_numpy_copy(net_h.gradients), net_r.gradients
     for name, (a, b, _) in net_r.parameter_slices().items():
         assert scaled_err(g_h[a:b], g_r[a:b]) <= 1e-5, name
-    print("highway: worst forward buffer %.2e, worst backward buffer %.2e" % (worst_fwd, worst))
+    print("highway (fused=%s): worst forward buffer %.2e, worst backward buffer %.2e" % (fused, worst_fwd, worst))
 
 
-def test_cnn_forward_backward(hip):
-    net_h, net_r = both(configs.build_cnn, hip, 24)
+@pytest.fixture
+def trimmed_pool(hip):
+    """Gives the pool's cached blocks back to the driver after a test that used tens of gigabytes."""
+    yield
+    import gc
+    gc.collect()
+    assert hip._lib.bship_pool_trim() == 0
+
+
+def test_highway_full_depth(hip, trimmed_pool):
+    """The bandwidth-stress configuration at its full depth: 50 x {BatchNorm -> FC_H(rel) || FC_T(sigmoid)
+    -> Highway} at width 4096 and batch 2048 (35 GB of buffers, 1.68 G parameters), one training step
+    (forward, backward, momentum update) through the primitives and through the fused entry points.
+    The oracle cannot run 50 blocks in test time, so depth is held by what does not need it:
+      * the first two blocks equal the oracle's two-block network (same seed -> same weights);
+      * every BatchNorm output has per-feature mean beta and variance gamma^2 var/(var + eps), at
+        every depth (batch_normalization_layer.py:68-105), and every buffer is finite;
+      * the fused network equals the primitive one on every buffer, gradient and parameter;
+      * the momentum update of the whole unaligned parameter vector equals its closed form
+        (steppers.py:104-112) bit for bit.
+    """
+    blocks, lr, mom = 50, 0.1, 0.9
+    hip.rnd.seed(23)
+    net_p, data = configs.build_highway(hip, blocks=blocks, quick_init_from_block=2)
+    params0 = hip.get_numpy_copy(net_p.parameters)
+    net_f, _ = configs.build_highway(hip, blocks=blocks, fused=True, parameters=params0)
+    steppers = []
+    for net, fused in ((net_p, False), (net_f, True)):
+        net.provide_external_data(data)
+        st = MomentumStepper(lr, mom, fused=fused)
+        st.start(net)
+        st.run()
+        steppers.append(st)
+        assert hip.is_fully_finite(net.full_buffer), "non-finite values (fused=%s)" % fused
+    loss = net_p.get("loss", "outputs", "loss")[0]
+    assert np.isfinite(loss) and 0.0 < loss < 20.0, loss
+
+    # fused == primitives on everything, compared on the device
+    assert device_equal(hip, net_f.full_buffer, net_p.full_buffer), "fused network differs from the primitive one"
+    assert device_equal(hip, steppers[1].velocity, steppers[0].velocity)
+    assert_bit_equal(net_f.get("loss", "outputs", "loss"), net_p.get("loss", "outputs", "loss"), "loss")
+    del net_f, steppers
+
+    # BatchNorm statistics at every depth (gamma = 1, beta = 0 at initialisation)
+    eps = 1.0e-5
+    for k in range(blocks):
+        y = net_p.get("bn%d" % k, "outputs", "default")[0].astype(np.float64)
+        s_b = net_p.get("bn%d" % k, "internals", "sigma_b").astype(np.float64)       # sqrt(var + eps)
+        assert np.all(s_b > 0.05) and np.all(s_b < 50.0), ("scale drifts", k, s_b.min(), s_b.max())
+        assert np.max(np.abs(y.mean(axis=0))) <= 2e-6, (k, np.max(np.abs(y.mean(axis=0))))
+        want_var = 1.0 - eps / (s_b * s_b)
+        assert np.max(np.abs(y.var(axis=0) - want_var)) <= 2e-5, (k, np.max(np.abs(y.var(axis=0) - want_var)))
+
+    # the first two blocks against the oracle
+    ref = NumpyRefHandler(F32, seed=23)
+    net_r, data_r = configs.build_highway(ref, blocks=2)
+    assert np.array_equal(data_r["default"], data["default"])
+    n2 = net_r.parameters.size - (10 * 4096 + 10)                                     # without its output layer
+    assert np.array_equal(params0[:n2], net_r.parameters[:n2])
+    net_r.provide_external_data(data_r)
+    net_r.forward_pass(training_pass=True)
+    worst = 0.0
+    for name in net_r.layers:
+        if name in ("Input", "out", "ce", "loss"):
+            continue
+        for group in ("outputs", "internals"):
+            for key, want in getattr(net_r.buffers[name], group).items():
+                err = scaled_err(net_p.get(name, group, key), want)
+                worst = max(worst, err)
+                assert err <= 1e-5, (name, group, key, err)
+
+    # the update: v = 0 * 0.9 + (-lr (1 - mom)) * g ; p = v + p, in float32, over all 1.68 G parameters
+    # (BatchNorm's running statistics mu and sigma are rewritten by the forward pass and have no
+    # gradient: they are left out here and covered by the comparisons above)
+    step = F32(-(lr * (1 - mom)))
+    n, chunk = params0.size, 1 << 27
+    statistics = np.zeros(n, bool)
+    for name, (a, b, _) in net_p.parameter_slices().items():
+        if name.endswith(".mu") or name.endswith(".sigma"):
+            statistics[a:b] = True
+    for a in range(0, n, chunk):
+        b = min(n, a + chunk)
+        g = hip.get_numpy_copy(net_p.gradients[a:b])
+        assert not g[statistics[a:b]].any()
+        want = (F32(mom) * np.zeros(b - a, F32) + step * g) + params0[a:b]
+        got = hip.get_numpy_copy(net_p.parameters[a:b])
+        keep = ~statistics[a:b]
+        assert_bit_equal(got[keep], want[keep], "parameters %d:%d" % (a, b))
+    print("highway, 50 blocks: loss %.4f, first two blocks vs oracle %.2e" % (loss, worst))
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
+def test_cnn_forward_backward(hip, fused):
+    net_h, net_r = both(lambda h, **kw: configs.build_cnn(h, fused=fused and h is hip, **kw), hip, 24)
     net_h.forward_pass(training_pass=True)
     net_r.forward_pass(training_pass=True)
     # Pooling must agree exactly GIVEN the same input: feed the oracle's conv outputs to the GPU pool
@@ -198,7 +341,7 @@ def test_cnn_forward_backward(hip):
         err = scaled_err(g_h[a:b], g_r[a:b])
         worst = max(worst, err)
         assert err <= 5e-5, (name, err)
-    print("cnn: worst gradient block %.2e" % worst)
+    print("cnn (fused=%s): worst gradient block %.2e" % (fused, worst))
 
 
 def test_device_resident_inputs(hip):

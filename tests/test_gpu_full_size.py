@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import bench
-from util import assert_bit_equal, assert_max_ulp
+from util import assert_bit_equal, assert_max_ulp, ulp_distance
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -31,7 +31,7 @@ def chunks(hip, arr):
     return hip.get_numpy_copy(arr).reshape(REPS, BASE * BASE)
 
 
-def check_repeats(hip, out, want_base, what, max_ulp=0):
+def check_repeats(hip, out, want_base, what, max_ulp=0, min_within_2=None):
     got = chunks(hip, out)
     for k in range(1, REPS):
         assert np.array_equal(got[k].view(np.uint32), got[0].view(np.uint32)), "%s: copy %d differs from copy 0" % (what, k)
@@ -39,6 +39,9 @@ def check_repeats(hip, out, want_base, what, max_ulp=0):
         assert_bit_equal(got[0], want_base.ravel(), what)
     else:
         assert_max_ulp(got[0], want_base.ravel(), max_ulp, what)
+    if min_within_2 is not None:
+        within2 = float(np.mean(ulp_distance(got[0], want_base.ravel()) <= 2))
+        assert within2 >= min_within_2, "%s: only %.6f of the elements within 2 ulp of the oracle" % (what, within2)
 
 
 def test_elementwise_ops_at_2p28(hip, ref, sweep):
@@ -69,15 +72,18 @@ def test_elementwise_ops_at_2p28(hip, ref, sweep):
     ref.mult_add_st(0.5, a, want)
     ref.mult_add_st(0.5, a, want)
     check_repeats(hip, t["acc"], want, "mult_add_st")
-    # transcendentals: position independent, and as close to the oracle as the small-size tests require
+    # transcendentals: position independent, and at the bars of the small-size tests (test_gpu_parity.py):
+    # tanh within 2 ulp of the float32 oracle everywhere; sigmoid and log_t within 4 ulp everywhere and
+    # 99.9 % of the elements within 2 (NumPy's float32 exp/log are up to 3 ulp from the correctly rounded
+    # value themselves; the device result is within 1 ulp of it)
     for name, run, oracle, bound in [
             ("tanh", lambda: hip.tanh(t["a"], out), lambda w: ref.tanh(a, w), 2),
             ("sigmoid", lambda: hip.sigmoid(t["a"], out), lambda w: ref.sigmoid(a, w), 4),
-            ("log_t", lambda: hip.log_t(t["u"], out), lambda w: ref.log_t(u, w), 5)]:
+            ("log_t", lambda: hip.log_t(t["u"], out), lambda w: ref.log_t(u, w), 4)]:
         want = np.zeros((BASE, BASE), F32)
         oracle(want)
         run()
-        check_repeats(hip, out, want, name, max_ulp=bound)
+        check_repeats(hip, out, want, name, max_ulp=bound, min_within_2=0.999)
     # copy and fill
     hip.copy_to(t["a"], out)
     check_repeats(hip, out, a, "copy_to")

@@ -214,16 +214,19 @@ def test_set_from_numpy_casts_and_broadcasts(hip, ref):
 
 
 # -------------------------------------------------------------- transcendentals
-def _check_transcendental(hip, ref, op, x, exact_f64, label):
-    """Stated bound for float32 transcendentals.
+# The bars for float32 transcendentals against the float32 oracle (NumpyHandler's results):
+#   tanh:            every element within 2 ulp;
+#   sigmoid, log_t:  every element within 4 ulp, and at least 99.9 % of the elements of an array of
+#                    10^4 or more within 2 ulp.
+# and against the float64 evaluation of the reference formula rounded to float32: within 1 ulp, always.
+# A flat "2 ulp to NumpyHandler" cannot be met by any implementation for sigmoid and log_t: NumPy's
+# float32 SIMD exp/log are themselves up to 3 ulp from the correctly rounded value (which host CPU
+# decides where), and the result here is within 1 ulp of it.
+ORACLE_MAX_ULP = {"tanh": 2, "sigmoid": 4, "log_t": 4}
+ORACLE_MIN_FRACTION_WITHIN_2 = 0.999
 
-    HIP evaluates in float64 and rounds once, so it must be within 1 ulp of the float64
-    evaluation of the reference formula rounded to float32 (`truth`). NumPy's own float32
-    SIMD routines are measurably 1-4 ulp away from that truth (depending on the host CPU),
-    so the distance to the float32 oracle is bounded elementwise by 2 ulp + the oracle's own
-    distance from the truth; wherever the oracle is within 2 ulp of the truth this is the
-    plain "<= 2 ulp to NumpyHandler" bar... and the distance to the oracle is reported.
-    """
+
+def _check_transcendental(hip, ref, op, x, exact_f64, label):
     want32 = np.zeros_like(x)
     getattr(ref, op)(x.copy(), want32)
     xd = hip.create_from_numpy(x)
@@ -235,11 +238,13 @@ def _check_transcendental(hip, ref, op, x, exact_f64, label):
     d_truth = ulp_distance(got, truth)
     d_oracle = ulp_distance(got, want32)
     oracle_err = ulp_distance(want32, truth)
-    assert d_truth.max() <= 1, "%s %s: %d ulp from the float64 evaluation" % (op, label, d_truth.max())
-    assert np.all(d_oracle <= 2 + oracle_err), "%s %s: too far from the float32 oracle" % (op, label)
+    within2 = float(np.mean(d_oracle <= 2))
     print("%s %s: max ulp to float32 oracle %d (oracle itself %d from float64 truth), "
-          "fraction within 2 ulp %.6f" % (op, label, d_oracle.max(), oracle_err.max(),
-                                           np.mean(d_oracle <= 2)))
+          "fraction within 2 ulp %.6f" % (op, label, d_oracle.max(), oracle_err.max(), within2))
+    assert d_truth.max() <= 1, "%s %s: %d ulp from the float64 evaluation" % (op, label, d_truth.max())
+    assert d_oracle.max() <= ORACLE_MAX_ULP[op], "%s %s: %d ulp from the float32 oracle" % (op, label, d_oracle.max())
+    if x.size >= 10000:
+        assert within2 >= ORACLE_MIN_FRACTION_WITHIN_2, "%s %s: only %.6f within 2 ulp" % (op, label, within2)
     # in place must give the same bits
     getattr(hip, op)(xd, xd)
     assert_bit_equal(xd.get(), got, op + " in place")
@@ -483,7 +488,100 @@ def test_index_m_by_v_exact(hip, ref):
         operation_check(hip, ref, "index_m_by_v", (m, v, np.zeros((rows, 1), F32)))
 
 
+def test_negative_labels_count_from_the_last_column(hip, ref):
+    # NumPy's indexing wraps labels in [-K, -1] (numpy_handler.py:101, 203: eye[v], m[arange, v]);
+    # the kernels do the same, also the fused softmax cross entropy
+    rng = np.random.RandomState(23)
+    rows, k = 37, 11
+    v = rng.randint(-k, k, (rows, 1)).astype(F32)
+    v[:4, 0] = [-1, -k, k - 1, 0]
+    operation_check(hip, ref, "binarize_v", (v, np.full((rows, k), 7.0, F32)))
+    operation_check(hip, ref, "index_m_by_v", (rand(rng, (rows, k)), v, np.zeros((rows, 1), F32)))
+    x = rand(rng, (rows, k))
+    vd, xd = hip.create_from_numpy(v), hip.create_from_numpy(x)
+    probs, loss = hip.allocate((rows, k)), hip.allocate((rows, 1))
+    hip.softmax_ce_forward(xd, vd, probs, loss)
+    picked = hip.allocate((rows, 1))
+    hip.index_m_by_v(probs, vd, picked)
+    want = -np.log(np.clip(picked.get(), F32(1e-6), F32(1.0)).astype(np.float64))
+    np.testing.assert_allclose(loss.get(), want, rtol=1e-6)
+    t_bin, din = hip.allocate((rows, k)), hip.allocate((rows, k))
+    hip.softmax_ce_backward(probs, vd, hip.create_from_numpy(np.ones((rows, 1), F32)), t_bin, din)
+    onehot = np.zeros((rows, k), F32)
+    ref.binarize_v(v, onehot)
+    assert_bit_equal(din.get(), (-onehot + probs.get()) * F32(1.0), "softmax - onehot with wrapped labels")
+
+
+def test_documented_deviations_from_numpy(hip, ref):
+    """Two places where the device does something NumpyHandler cannot or does not:
+    labels beyond [-K, K) (NumPy raises IndexError; a kernel cannot raise, the row selects no column:
+    an all-zero one-hot row, a gathered 0) and sigmoid of NaN (NumPy's two masked assignments skip the
+    element and leave y's old value, numpy_handler.py:283-287; the device writes NaN)."""
+    k = 5
+    v = np.array([[5.0], [-6.0], [1e10], [np.nan], [np.inf], [2.0]], F32)
+    vd = hip.create_from_numpy(v)
+    out = hip.create_from_numpy(np.full((6, k), 7.0, F32))
+    hip.binarize_v(vd, out)
+    want = np.zeros((6, k), F32)
+    want[5, 2] = 1.0
+    assert_bit_equal(out.get(), want, "one-hot rows of labels out of range")
+    m = np.arange(30, dtype=F32).reshape(6, k) + 1
+    got = hip.allocate((6, 1))
+    hip.index_m_by_v(hip.create_from_numpy(m), vd, got)
+    assert_bit_equal(got.get(), np.array([[0], [0], [0], [0], [0], [m[5, 2]]], F32), "gather with labels out of range")
+    with pytest.raises(IndexError):
+        ref.index_m_by_v(m, v[:1], np.zeros((1, 1), F32))
+    # sigmoid(NaN)
+    x = np.array([0.5, np.nan, -0.5], F32)
+    y_ref = np.full(3, 9.0, F32)
+    with np.errstate(invalid="ignore"):
+        ref.sigmoid(x, y_ref)
+    assert y_ref[1] == 9.0                       # the oracle (like NumpyHandler) leaves the old value
+    y = hip.create_from_numpy(np.full(3, 9.0, F32))
+    hip.sigmoid(hip.create_from_numpy(x), y)
+    got = y.get()
+    assert np.isnan(got[1]) and got[0] == y_ref[0] and got[2] == y_ref[2]
+
+
 # ------------------------------------------------------------------------- RNG
+def test_handlers_alive_together_keep_their_own_streams(hip):
+    # every reference handler owns its random state (numpy_handler.py:21): two handlers with different
+    # seeds, their calls interleaved (masks, a repeating pattern that starts the look-ahead, gaussians,
+    # a reseed), each reproduce their own RandomState stream; the session's handler is not disturbed
+    from brainstorm_amd import HipHandler
+    hip.rnd.seed(99)
+    rs0 = np.random.RandomState(99)
+    m0 = hip.allocate((1000,))
+    hip.generate_probability_mask(m0, 0.5)
+    assert_bit_equal(m0.get(), (rs0.uniform(size=1000) < 0.5).astype(F32))
+    a, b = HipHandler(seed=7), HipHandler(seed=8)            # constructing them reseeds nobody else
+    ra, rb = np.random.RandomState(7), np.random.RandomState(8)
+    assert a.rnd.get_seed() == 7 and b.rnd.get_seed() == 8
+    ma, mb = a.allocate((3, 1200)), b.allocate((777,))
+    for step in range(8):
+        for _ in range(2):                                   # a: the same two requests every step (look-ahead)
+            a.generate_probability_mask(ma, 0.8)
+            assert_bit_equal(ma.get(), (ra.uniform(size=(3, 1200)) < 0.8).astype(F32), "handler a, step %d" % step)
+        b.generate_probability_mask(mb, 0.3)
+        assert_bit_equal(mb.get(), (rb.uniform(size=777) < 0.3).astype(F32), "handler b, step %d" % step)
+        if step == 3:
+            g = b.allocate((5,))
+            b.fill_gaussian(1.0, 2.0, g)
+            np.testing.assert_allclose(g.get(), 2.0 * rb.standard_normal(5) + 1.0, rtol=1e-6)
+        if step == 5:
+            a.rnd.seed(70)
+            ra = np.random.RandomState(70)
+        hip.generate_probability_mask(m0, 0.5)
+        assert_bit_equal(m0.get(), (rs0.uniform(size=1000) < 0.5).astype(F32), "session handler, step %d" % step)
+    for h, r in ((a, ra), (b, rb), (hip, rs0)):
+        _, key, pos, has_gauss, _ = h.rnd.get_state()
+        st = r.get_state()
+        assert pos == st[2] and np.array_equal(key, st[1]) and has_gauss == st[3]
+    del a, b                                                  # their generators are destroyed with them
+    hip.generate_probability_mask(m0, 0.5)
+    assert_bit_equal(m0.get(), (rs0.uniform(size=1000) < 0.5).astype(F32), "after the others are gone")
+
+
 def test_generate_probability_mask_matches_randomstate(hip):
     # Sizes chosen so that consecutive calls start at even and odd positions of the 624-word
     # MT19937 block and cross block boundaries (a 53-bit double takes two words).
@@ -614,6 +712,32 @@ def test_dot_mm_and_dot_add_mm(hip, ref):
             # 1e-5 relative to the magnitude of a length-k inner product
             scale = np.sqrt(k) + np.abs(want)
             assert np.max(np.abs(od.get() - want) / scale) <= 1e-5, (op, m, k, n, ta, tb)
+
+
+def test_dot_mm_with_operands_at_odd_elements(hip, ref):
+    # time-step slices and hub slices start at any element of a flat buffer: A, B and C 4-byte but not
+    # 16-byte aligned, each shape twice so that the second call runs the cached plan
+    rng = np.random.RandomState(29)
+    for (m, k, n), ta, tb in itertools.product([(100, 1000, 1000), (37, 129, 65), (5, 3, 2)], (False, True),
+                                               (False, True)):
+        a = rand(rng, (k, m) if ta else (m, k))
+        b = rand(rng, (n, k) if tb else (k, n))
+        out = rand(rng, (m, n))
+        for offs in ((1, 2, 3), (3, 1, 1)):
+            views = []
+            for arr, off in zip((a, b, out), offs):
+                flat = hip.allocate((arr.size + 4,))
+                assert flat.ptr % 16 == 0
+                v = flat[off:off + arr.size].reshape(arr.shape)
+                hip.set_from_numpy(v, arr)
+                views.append(v)
+            for op in ("dot_mm", "dot_add_mm"):
+                hip.set_from_numpy(views[2], out)
+                want = out.copy()
+                getattr(ref, op)(a, b, want, ta, tb)
+                getattr(hip, op)(views[0], views[1], views[2], ta, tb)
+                scale = np.sqrt(k) + np.abs(want)
+                assert np.max(np.abs(views[2].get() - want) / scale) <= 1e-5, (op, m, k, n, ta, tb, offs)
 
 
 # -------------------------------------------------------------- conv / pooling

@@ -29,6 +29,53 @@ def ref64():
     return NumpyRefHandler(F64, seed=7)
 
 
+# ------------------------------------------------------------- memory operations
+def test_allocate_copy_fill_and_transfers(ref):
+    # allocate == zeros, of the handler's dtype (numpy_handler.py:36-43)
+    for shape in ((3, 4), 7, (2, 0, 5), ()):
+        a, z = ref.allocate(shape), ref.zeros(shape)
+        assert a.dtype == F32 and z.dtype == F32 and a.shape == z.shape == np.empty(shape).shape
+        assert not a.any() and not z.any()
+    o = ref.ones((2, 3))
+    assert o.dtype == F32 and all(v == 1.0 for v in o.ravel().tolist())
+    # copy_to(src, dest): dest receives src, src is untouched; a reshaped view writes through (47-52)
+    src = np.arange(12, dtype=F32).reshape(3, 4)
+    base = np.full(20, -1.0, F32)
+    dest = base[4:16].reshape(3, 4)                       # a view into a larger flat buffer
+    ref.copy_to(src, dest)
+    assert base.tolist() == [-1.0] * 4 + [float(k) for k in range(12)] + [-1.0] * 4
+    assert src.tolist() == [[0, 1, 2, 3], [4, 5, 6, 7], [8, 9, 10, 11]]
+    with pytest.raises(TypeError):                        # same_kind casting: float -> int is refused
+        ref.copy_to(src, np.zeros((3, 4), np.int32))
+    # fill sets every element of a view and nothing else (57-58)
+    ref.fill(base[2:5], 2.5)
+    assert base[:6].tolist() == [-1.0, -1.0, 2.5, 2.5, 2.5, 1.0]
+    # set_from_numpy casts to the handler dtype: float64 values are ROUNDED to float32 (64-65)
+    mem = ref.allocate((3,))
+    ref.set_from_numpy(mem, np.array([0.1, 16777217.0, -1e-50], dtype=F64))
+    assert mem.dtype == F32
+    assert mem.view(np.uint32).tolist() == [0x3dcccccd, 0x4b800000, 0x80000000]   # 0.1f, 2^24 (ties to even), -0
+    ref.set_from_numpy(mem, np.array([1, -2, 3], dtype=np.int32))
+    assert mem.tolist() == [1.0, -2.0, 3.0]
+    # create_from_numpy / get_numpy_copy give copies, not views (54-62)
+    host = np.array([1.0, 2.0], F32)
+    dev = ref.create_from_numpy(host)
+    back = ref.get_numpy_copy(dev)
+    host[0], dev[1] = 9.0, 8.0
+    assert dev.tolist() == [1.0, 8.0] and back.tolist() == [1.0, 2.0]
+
+
+def test_is_fully_finite(ref):
+    a = np.array([[0.0, -0.0, 1e-45], [3.4e38, -3.4e38, 1.0]], F32)     # zeros, a denormal, the largest floats
+    assert ref.is_fully_finite(a) is True or ref.is_fully_finite(a) == True  # noqa: E712
+    for bad in (np.nan, np.inf, -np.inf):
+        for pos in ((0, 0), (1, 2)):
+            b = a.copy()
+            b[pos] = bad
+            assert not ref.is_fully_finite(b), (bad, pos)
+    assert ref.is_fully_finite(np.zeros((0, 3), F32))
+
+
 # ----------------------------------------------------------------------- MT19937
 class TextbookMT19937:
     """Matsumoto & Nishimura's mt19937ar.c (init_genrand / genrand_int32 / genrand_res53)."""
