@@ -96,7 +96,27 @@ struct ImgPlan {
     ImgGeom g;
     uint32_t lanes_per_image;
     FastDiv d_cv, d_w, d_ow, d_kcv, d_kwcv, d_sh, d_sw;
+    FastDiv d_pw;         // stride-aligned patches per image row (pooling backward)
+    // launch shape: `tiles` workgroups cover one image, `groups` sets of images; see img_block
+    uint32_t tiles, groups, per_xcd;
+    FastDiv d_tiles;
 };
+
+// Which (tile of an image, group of images) a workgroup of the 1-D grid works on. The hardware
+// hands workgroups to the 8 XCDs round-robin by their number, and each XCD has an L2 of its own:
+// with tile = blockIdx.x the neighbouring tiles of one image, whose windows overlap (a pooling
+// output row is needed by the workgroups of three input rows), ran on different XCDs and each
+// fetched the shared rows from HBM again (max-pool backward 32x32x32: 1.55x its algorithmic
+// traffic). Here XCD x works through the x-th contiguous eighth of the (group, tile) sequence, so
+// all tiles of an image group meet in one L2. The grid is 8 * per_xcd workgroups; numbers beyond
+// the sequence's end have nothing to do.
+constexpr uint32_t kXcdCount = 8;
+__device__ __forceinline__ bool img_block(const ImgPlan& pl, uint32_t& tile, uint32_t& group) {
+    const uint32_t v = (blockIdx.x % kXcdCount) * pl.per_xcd + blockIdx.x / kXcdCount;
+    if (v >= pl.tiles * pl.groups) return false;
+    pl.d_tiles.divmod(v, group, tile);
+    return true;
+}
 
 // col[(img, oy, ox), (ky, kx, ch)] = in[img, oy*sh-pad+ky, ox*sw-pad+kx, ch] or 0   (_cpuop 264-277)
 // One lane per W channels of one (oy, ox, ky, kx); lanes_per_image = oh*ow*kh*kw*cv.
@@ -105,7 +125,9 @@ template <int W, bool AL, bool WT>
 __device__ __forceinline__ void im2col_body(const float* __restrict__ in, float* __restrict__ col,
                                             int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t opix, r, oy, ox, ky, kxc, kx, chv;
     pl.d_kcv.divmod(p, opix, r);
@@ -119,8 +141,8 @@ __device__ __forceinline__ void im2col_body(const float* __restrict__ in, float*
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * W;
     // kImagesPerWorkgroup images at a time: all loads first, then all stores
-    for (int64_t img0 = static_cast<int64_t>(blockIdx.y) * kImagesPerWorkgroup; img0 < n;
-         img0 += static_cast<int64_t>(gridDim.y) * kImagesPerWorkgroup) {
+    for (int64_t img0 = static_cast<int64_t>(group) * kImagesPerWorkgroup; img0 < n;
+         img0 += static_cast<int64_t>(pl.groups) * kImagesPerWorkgroup) {
         typename VecT<W>::type v[kImagesPerWorkgroup];
 #pragma unroll
         for (int k = 0; k < kImagesPerWorkgroup; ++k) {
@@ -147,7 +169,9 @@ template <bool WT>
 __global__ __launch_bounds__(kBlock) void im2col_gather4(const float* __restrict__ in,
                                                          float* __restrict__ col, int64_t n, ImgPlan pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     int in_off[4];
 #pragma unroll
@@ -164,8 +188,8 @@ __global__ __launch_bounds__(kBlock) void im2col_gather4(const float* __restrict
     }
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * 4;
-    for (int64_t img0 = static_cast<int64_t>(blockIdx.y) * kImagesPerWorkgroup; img0 < n;
-         img0 += static_cast<int64_t>(gridDim.y) * kImagesPerWorkgroup) {
+    for (int64_t img0 = static_cast<int64_t>(group) * kImagesPerWorkgroup; img0 < n;
+         img0 += static_cast<int64_t>(pl.groups) * kImagesPerWorkgroup) {
         f4 v[kImagesPerWorkgroup];
 #pragma unroll
         for (int k = 0; k < kImagesPerWorkgroup; ++k) {
@@ -284,7 +308,9 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
                                                         float* __restrict__ in_deltas, int64_t n,
                                                         ImgPlan pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t pix, chv, yy, xx;
     pl.d_cv.divmod(p, pix, chv);
@@ -296,7 +322,7 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
     const int64_t kc = static_cast<int64_t>(g.kh) * g.kw * g.c;
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t col_img = static_cast<int64_t>(g.oh) * g.ow * kc;
-    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+    for (int64_t img = group; img < n; img += pl.groups) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
         typename VecT<W>::type acc = img_load<W, AL>(q);
         const float* cimg = col + img * col_img + chv * W;
@@ -519,7 +545,9 @@ template <int W, bool AL, int K>
 __device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, float* __restrict__ out,
                                                  float* __restrict__ argmax, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t opix, chv, oy, ox;
     pl.d_cv.divmod(p, opix, chv);
@@ -531,7 +559,7 @@ __device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, f
     const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
     const int ch0 = static_cast<int>(chv) * W;
     typedef typename VecT<W>::type R;
-    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+    for (int64_t img = group; img < n; img += pl.groups) {
         const float* base = in + img * in_img + ch0;
         R best = vsplat<W>(-FLT_MAX), where = vsplat<W>(-1.0f);
         auto take = [&](R v, int k) {
@@ -589,7 +617,9 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
                                                  const float* __restrict__ out_deltas,
                                                  float* __restrict__ in_deltas, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t pix, chv, yy, xx;
     pl.d_cv.divmod(p, pix, chv);
@@ -603,7 +633,7 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
     typedef typename VecT<W>::type R;
-    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+    for (int64_t img = group; img < n; img += pl.groups) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
         R acc = vload<W, AL>(q);
         auto take = [&](R am, R d) {
@@ -653,7 +683,9 @@ template <int W, bool AL, int K>
 __device__ __forceinline__ void avgpool_fwd_body(const float* __restrict__ in, float* __restrict__ out,
                                                  int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t opix, chv, oy, ox;
     pl.d_cv.divmod(p, opix, chv);
@@ -665,7 +697,7 @@ __device__ __forceinline__ void avgpool_fwd_body(const float* __restrict__ in, f
     const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
     const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
     typedef typename VecT<W>::type R;
-    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+    for (int64_t img = group; img < n; img += pl.groups) {
         const float* base = in + img * in_img + chv * W;
         R sum = vsplat<W>(0.0f);
         if constexpr (K > 0) {
@@ -706,7 +738,9 @@ template <int W, bool AL, int C>
 __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_deltas,
                                                  float* __restrict__ in_deltas, int64_t n, const ImgPlan& pl) {
     const ImgGeom& g = pl.g;
-    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
     if (p >= pl.lanes_per_image) return;
     uint32_t pix, chv, yy, xx;
     pl.d_cv.divmod(p, pix, chv);
@@ -725,7 +759,7 @@ __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_d
         const int nx = imin(wx + g.kw, g.w) - imax(wx, 0);
         return static_cast<float>(ny * nx);
     };
-    for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
+    for (int64_t img = group; img < n; img += pl.groups) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
         R acc = vload<W, AL>(q);
         const float* dimg = out_deltas + img * out_img + chv * W;
@@ -768,6 +802,120 @@ __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_d
 BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel, 0)
 BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel_c1, 1)
 BSHIP_AVG_BWD_KERNEL(avgpool_bwd_kernel_c2, 2)
+
+// Pooling backward for strides above 1 (_cpuop 103-115 and 187-202, gather form): one lane owns W
+// channels of a stride-aligned S x S patch of input pixels, (y + pad) / S = pi and (x + pad) / S = pj.
+// The windows that cover any pixel of the patch are the C x C output positions
+// (pi - C + 1 .. pi) x (pj - C + 1 .. pj) with C = (k - 1) / S + 1, so a lane reads C*C window
+// entries for S*S pixels (3x3 windows, stride 2: 2 per pixel) where a lane per pixel reads up to
+// C*C for each (8 of its 10 accesses, which kept the vector memory path busier than HBM). Every
+// pixel still adds its terms in (oy, ox) scan order. lanes_per_image = patch rows x patch columns x cv.
+// MAX: max pooling (argmax holds the winner's index), otherwise average pooling.
+template <int W, bool AL, int S, int C, bool MAX>
+__device__ __forceinline__ void pool_bwd_patch_body(const float* __restrict__ argmax,
+                                                    const float* __restrict__ out_deltas,
+                                                    float* __restrict__ in_deltas, int64_t n, const ImgPlan& pl) {
+    const ImgGeom& g = pl.g;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t patch, chv, pi, pj;
+    pl.d_cv.divmod(p, patch, chv);
+    pl.d_pw.divmod(patch, pi, pj);
+    const int ch0 = static_cast<int>(chv) * W;
+    const int y0 = static_cast<int>(pi) * S - g.pad, x0 = static_cast<int>(pj) * S - g.pad;
+    const int oyb = static_cast<int>(pi) - (C - 1), oxb = static_cast<int>(pj) - (C - 1);
+    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    typedef typename VecT<W>::type R;
+    bool valid[S * S];
+    int pix_off[S * S];
+#pragma unroll
+    for (int r = 0; r < S; ++r)
+#pragma unroll
+        for (int t = 0; t < S; ++t) {
+            const int y = y0 + r, x = x0 + t;
+            valid[r * S + t] = y >= 0 && y < g.h && x >= 0 && x < g.w;
+            pix_off[r * S + t] = (imin(imax(y, 0), g.h - 1) * g.w + imin(imax(x, 0), g.w - 1)) * g.c + ch0;
+        }
+    // window (a, b) of the cover: whether it exists, and for average pooling its pixel count
+    bool exists[C * C];
+    int win_off[C * C];
+    float win_size[C * C];
+#pragma unroll
+    for (int a = 0; a < C; ++a)
+#pragma unroll
+        for (int b = 0; b < C; ++b) {
+            const int oy = oyb + a, ox = oxb + b;
+            exists[a * C + b] = oy >= 0 && oy < g.oh && ox >= 0 && ox < g.ow;
+            win_off[a * C + b] = (imin(imax(oy, 0), g.oh - 1) * g.ow + imin(imax(ox, 0), g.ow - 1)) * g.c + ch0;
+            const int wy = oy * S - g.pad, wx = ox * S - g.pad;
+            win_size[a * C + b] = static_cast<float>((imin(wy + g.kh, g.h) - imax(wy, 0)) *
+                                                     (imin(wx + g.kw, g.w) - imax(wx, 0)));
+        }
+    for (int64_t img = group; img < n; img += pl.groups) {
+        float* q = in_deltas + img * in_img;
+        R acc[S * S], am[C * C], d[C * C];
+#pragma unroll
+        for (int k = 0; k < S * S; ++k)
+            if (valid[k]) acc[k] = vload<W, AL>(q + pix_off[k]);
+#pragma unroll
+        for (int k = 0; k < C * C; ++k) {
+            if constexpr (MAX) am[k] = img_load<W, AL>(argmax + img * out_img + win_off[k]);
+            d[k] = img_load<W, AL>(out_deltas + img * out_img + win_off[k]);
+        }
+        if constexpr (!MAX) {
+            // a window's share delta / size is the same quotient for every pixel under it
+#pragma unroll
+            for (int k = 0; k < C * C; ++k)
+#pragma unroll
+                for (int j = 0; j < W; ++j) comp<W>(d[k], j) = comp<W>(d[k], j) / win_size[k];
+        }
+#pragma unroll
+        for (int r = 0; r < S; ++r)
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                if (!valid[r * S + t]) continue;
+#pragma unroll
+                for (int a = 0; a < C; ++a)
+#pragma unroll
+                    for (int b = 0; b < C; ++b) {
+                        // the pixel's offset inside window (a, b): S * (C - 1 - a) + r rows down
+                        const bool covers = exists[a * C + b] && S * (C - 1 - a) + r < g.kh &&
+                                            S * (C - 1 - b) + t < g.kw;
+                        if (!covers) continue;
+#pragma unroll
+                        for (int j = 0; j < W; ++j) {
+                            if constexpr (MAX) {
+                                if (static_cast<int>(comp<W>(am[a * C + b], j)) == pix_off[r * S + t] + j)
+                                    comp<W>(acc[r * S + t], j) += comp<W>(d[a * C + b], j);
+                            } else {
+                                comp<W>(acc[r * S + t], j) += comp<W>(d[a * C + b], j);
+                            }
+                        }
+                    }
+            }
+#pragma unroll
+        for (int k = 0; k < S * S; ++k)
+            if (valid[k]) vstore<W, AL>(q + pix_off[k], acc[k]);
+    }
+}
+#define BSHIP_POOL_BWD_PATCH_KERNELS(suffix, S, C)                                                       \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void maxpool_bwd_patch_##suffix(                                \
+        const float* __restrict__ argmax, const float* __restrict__ out_deltas,                          \
+        float* __restrict__ in_deltas, int64_t n, ImgPlan pl) {                                          \
+        pool_bwd_patch_body<W, AL, S, C, true>(argmax, out_deltas, in_deltas, n, pl);                    \
+    }                                                                                                    \
+    template <int W, bool AL>                                                                            \
+    __global__ __launch_bounds__(kBlock) void avgpool_bwd_patch_##suffix(                                \
+        const float* __restrict__ out_deltas, float* __restrict__ in_deltas, int64_t n, ImgPlan pl) {    \
+        pool_bwd_patch_body<W, AL, S, C, false>(nullptr, out_deltas, in_deltas, n, pl);                  \
+    }
+BSHIP_POOL_BWD_PATCH_KERNELS(s2c1, 2, 1)
+BSHIP_POOL_BWD_PATCH_KERNELS(s2c2, 2, 2)
+BSHIP_POOL_BWD_PATCH_KERNELS(s3c1, 3, 1)
 
 static int check_geom(const char* fn, int64_t n, const ImgGeom& g) {
     if (n < 0 || g.h < 0 || g.w < 0 || g.c < 0 || g.oh < 0 || g.ow < 0 || g.kh < 1 || g.kw < 1 ||
@@ -920,6 +1068,12 @@ using namespace bship;
 // Launches kernel<W, AL> over lanes_per_image x n: W = 4 when the channels come in fours,
 // AL when additionally every pointer is 16-byte aligned.
 #define BSHIP_LAUNCH_IMG(kernel, name, positions, aligned, ...)                                         \
+    BSHIP_LAUNCH_IMG_N(kernel, name, positions, aligned, kImagesPerWorkgroup, __VA_ARGS__)
+// images_per_wg: how many images a workgroup walks through, one after the other (kernels whose image
+// loop is `img = group; img += groups`; im2col_body needs kImagesPerWorkgroup). Measured at batch 2048:
+// the pooling backward kernels (read-modify-write of in_deltas) want 1 (max 32x32x32: 0.75 -> 0.89 of
+// peak, avg 0.71 -> 0.80), max pooling forward 4 (0.90 against 0.82 with 1).
+#define BSHIP_LAUNCH_IMG_N(kernel, name, positions, aligned, images_per_wg, ...)                        \
     do {                                                                                                \
         const bool vec4_ = (g.c % 4 == 0);                                                              \
         const int cv_ = vec4_ ? g.c / 4 : g.c;                                                          \
@@ -936,9 +1090,15 @@ using namespace bship;
         pl_.d_kwcv = FastDiv(static_cast<uint32_t>(imax(g.kw * cv_, 1)));                               \
         pl_.d_sh = FastDiv(static_cast<uint32_t>(g.sh));                                                \
         pl_.d_sw = FastDiv(static_cast<uint32_t>(g.sw));                                                \
-        const int64_t gy_ = ceil_div(n, kImagesPerWorkgroup);                                           \
-        const dim3 grid_(static_cast<unsigned>(ceil_div(lanes_, kBlock)),                               \
-                         static_cast<unsigned>(gy_ < 65535 ? gy_ : 65535));                             \
+        pl_.d_pw = FastDiv(static_cast<uint32_t>(imax((g.w - 1 + g.pad) / g.sw + 1, 1)));               \
+        const int64_t gy_ = ceil_div(n, images_per_wg);                                                 \
+        pl_.tiles = static_cast<uint32_t>(ceil_div(lanes_, kBlock));                                    \
+        pl_.groups = static_cast<uint32_t>(gy_ < 65535 ? gy_ : 65535);                                  \
+        if (static_cast<int64_t>(pl_.tiles) * pl_.groups > 0x7ffffff0)                                  \
+            pl_.groups = static_cast<uint32_t>(imax(1, static_cast<int>(0x7ffffff0 / pl_.tiles)));      \
+        pl_.d_tiles = FastDiv(pl_.tiles);                                                               \
+        pl_.per_xcd = static_cast<uint32_t>(ceil_div(static_cast<int64_t>(pl_.tiles) * pl_.groups, kXcdCount)); \
+        const dim3 grid_(pl_.per_xcd * kXcdCount);                                                      \
         if (vec4_ && (aligned))                                                                         \
             hipLaunchKernelGGL((kernel<4, true>), grid_, dim3(kBlock), 0, ctx().stream, __VA_ARGS__, n, pl_); \
         else if (vec4_)                                                                                 \
@@ -988,7 +1148,13 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
         pl.d_kcv = FastDiv(static_cast<uint32_t>(kh * kw * c));
         pl.d_kwcv = FastDiv(static_cast<uint32_t>(kw * c));
         const int64_t gy = ceil_div(n, kImagesPerWorkgroup);
-        const dim3 grid(static_cast<unsigned>(ceil_div(per_image / 4, kBlock)), static_cast<unsigned>(gy < 65535 ? gy : 65535));
+        pl.tiles = static_cast<uint32_t>(ceil_div(per_image / 4, kBlock));
+        pl.groups = static_cast<uint32_t>(gy < 65535 ? gy : 65535);
+        if (static_cast<int64_t>(pl.tiles) * pl.groups > 0x7ffffff0)
+            pl.groups = static_cast<uint32_t>(imax(1, static_cast<int>(0x7ffffff0 / pl.tiles)));
+        pl.d_tiles = FastDiv(pl.tiles);
+        pl.per_xcd = static_cast<uint32_t>(ceil_div(static_cast<int64_t>(pl.tiles) * pl.groups, kXcdCount));
+        const dim3 grid(pl.per_xcd * kXcdCount);
         if (write_through) hipLaunchKernelGGL(im2col_gather4<true>, grid, dim3(kBlock), 0, ctx().stream, in, col, n, pl);
         else               hipLaunchKernelGGL(im2col_gather4<false>, grid, dim3(kBlock), 0, ctx().stream, in, col, n, pl);
         return check_launch("im2col");
@@ -1077,6 +1243,17 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
     BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     const bool al = aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas);
+    // square windows and strides above 1: a lane per stride-aligned patch of pixels
+    if (pool_h == pool_w && stride_h == stride_w && (stride_h == 2 || stride_h == 3)) {
+        const int64_t patches = static_cast<int64_t>((h - 1 + pad) / stride_h + 1) * ((w - 1 + pad) / stride_w + 1);
+        const int cover_patch = (pool_h - 1) / stride_h + 1;
+        if (stride_h == 2 && cover_patch == 1)
+            BSHIP_LAUNCH_IMG_N(maxpool_bwd_patch_s2c1, "maxpool2d_backward_batch", patches, al, 1, argmax, out_deltas, in_deltas);
+        if (stride_h == 2 && cover_patch == 2)
+            BSHIP_LAUNCH_IMG_N(maxpool_bwd_patch_s2c2, "maxpool2d_backward_batch", patches, al, 1, argmax, out_deltas, in_deltas);
+        if (stride_h == 3 && cover_patch == 1)
+            BSHIP_LAUNCH_IMG_N(maxpool_bwd_patch_s3c1, "maxpool2d_backward_batch", patches, al, 1, argmax, out_deltas, in_deltas);
+    }
     // how many output positions can cover one pixel along each axis
     const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
     if (cover == 1)
@@ -1101,9 +1278,9 @@ int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, in
     BSHIP_REQUIRE_F32_ALIGNED(out);
     const bool al = aligned16(in) && aligned16(out);
     if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
-        BSHIP_LAUNCH_IMG(avgpool_fwd_kernel_3x3, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
+        BSHIP_LAUNCH_IMG_N(avgpool_fwd_kernel_3x3, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, 1, in, out);
     if (pool_h == 2 && pool_w == 2 && h >= 1 && w >= 1)
-        BSHIP_LAUNCH_IMG(avgpool_fwd_kernel_2x2, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
+        BSHIP_LAUNCH_IMG_N(avgpool_fwd_kernel_2x2, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, 1, in, out);
     BSHIP_LAUNCH_IMG(avgpool_fwd_kernel, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out);
 }
 
@@ -1121,6 +1298,16 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_
     BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     const bool al = aligned16(out_deltas) && aligned16(in_deltas);
+    if (pool_h == pool_w && stride_h == stride_w && (stride_h == 2 || stride_h == 3)) {
+        const int64_t patches = static_cast<int64_t>((h - 1 + pad) / stride_h + 1) * ((w - 1 + pad) / stride_w + 1);
+        const int cover_patch = (pool_h - 1) / stride_h + 1;
+        if (stride_h == 2 && cover_patch == 1)
+            BSHIP_LAUNCH_IMG_N(avgpool_bwd_patch_s2c1, "avgpool2d_backward_batch", patches, al, 1, out_deltas, in_deltas);
+        if (stride_h == 2 && cover_patch == 2)
+            BSHIP_LAUNCH_IMG_N(avgpool_bwd_patch_s2c2, "avgpool2d_backward_batch", patches, al, 1, out_deltas, in_deltas);
+        if (stride_h == 3 && cover_patch == 1)
+            BSHIP_LAUNCH_IMG_N(avgpool_bwd_patch_s3c1, "avgpool2d_backward_batch", patches, al, 1, out_deltas, in_deltas);
+    }
     const int cover = imax((pool_h + stride_h - 1) / stride_h, (pool_w + stride_w - 1) / stride_w);
     if (cover == 1)
         BSHIP_LAUNCH_IMG(avgpool_bwd_kernel_c1, "avgpool2d_backward_batch", static_cast<int64_t>(h) * w, al, out_deltas, in_deltas);

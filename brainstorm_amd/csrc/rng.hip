@@ -360,13 +360,18 @@ static int rng_ensure_state() {
 // A mask costs a fixed sequential time on ONE compute unit and depends on
 // nothing but the stream position, while a training loop asks for the same
 // masks, in the same order, every step. Once the recent requests (n, p) repeat
-// with some period P, the next P masks are drawn ahead of time on a second
-// stream into staging buffers, overlapping the step's other kernels; a matching
-// request then is a wait on an event plus a device copy, and the entry is drawn
-// again for the step after. Each entry keeps the stream position from before
-// its draw, so any request that does not match the prediction (or any other use
-// of the generator) rewinds to exactly the position a purely sequential
-// generator would have, and results never depend on whether a prefetch hit.
+// with some period P, the next P masks (a "round") are drawn ahead of time on a
+// second stream into staging buffers, overlapping the step's other kernels: one
+// draw of the round's words (the masks are consecutive in the stream; long
+// enough, the draw is cut into parallel segments) and one kernel that turns them
+// into the P masks. A matching request then is a wait on an event plus a device
+// copy. Two rounds alternate: when the first mask of a round is asked for, the
+// draw of the following round is enqueued, so it has the whole step to finish.
+// A round keeps the stream position from before its draw, so any request that
+// does not match the prediction (or any other use of the generator) rewinds to
+// that position and re-draws the words of the masks already handed out: the
+// generator is exactly where a purely sequential one would be, and results never
+// depend on whether a request was served from a round.
 struct MaskPrefetch {
     size_t n;
     double p;
@@ -377,7 +382,6 @@ struct MaskPrefetch {
     hipEvent_t ready;      // second stream: the mask is in staging
     hipEvent_t consumed;   // main stream: staging has been copied out
 };
-static std::deque<MaskPrefetch> g_fifo;
 static std::vector<std::pair<size_t, double>> g_history;
 static hipStream_t g_side = nullptr;
 static hipEvent_t g_join = nullptr;          // orders one stream behind the other
@@ -526,82 +530,10 @@ static int order_streams(hipStream_t earlier, hipStream_t later) {
     return 0;
 }
 
-// Drops every prefetched mask and puts the generator back to the position before
-// the oldest of them. Afterwards the main stream owns the generator again.
-static int prefetch_flush(bool restore_position, bool wrong_guess = false) {
-    g_history.clear();
-    if (g_fifo.empty()) return 0;
-    // "A B B" looks like period 1 after its second B: when a guess turns out wrong, only
-    // longer periods are tried next (any multiple of the true period serves as well)
-    if (wrong_guess) g_min_period = g_fifo.size() + 1 > kMaxPeriod ? 1 : g_fifo.size() + 1;
-    int st = order_streams(g_side, ctx().stream);
-    if (st == 0 && restore_position) {
-        hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, ctx().stream,
-                           g_fifo.front().before, g_state);
-        st = check_launch("random stream rewind");
-    }
-    // the blocks go back to the pool; their next owners run on the main stream, which is
-    // ordered behind the second stream now
-    for (MaskPrefetch& e : g_fifo) free_entry(e);
-    g_fifo.clear();
-    return st;
-}
-
-// Enqueues the draw of one mask on the second stream and appends it to the queue. Once the
-// draw is enqueued the entry is queued in every case: it records how far the generator has run.
-static int prefetch_schedule(MaskPrefetch e, bool wait_consumed) {
-    if (wait_consumed && hipStreamWaitEvent(g_side, e.consumed, 0) != hipSuccess) {
-        // cannot order behind the reader of the staging buffer: wait for it on the host instead
-        int st = check_hip(hipStreamSynchronize(ctx().stream), "hipStreamSynchronize");
-        if (st != 0) { free_entry(e); return st; }
-    }
-    launch_mask(g_side, e.staging, e.n, e.p, e.before, e.raw);
-    int st = check_launch("mask prefetch");
-    if (st != 0) { free_entry(e); return st; }
-    if (hipEventRecord(e.ready, g_side) != hipSuccess)
-        (void)hipStreamSynchronize(g_side);      // no event to wait for later: finish the draw now
-    g_fifo.push_back(e);
-    return 0;
-}
-
-// After a mask was drawn directly: if the recent requests repeat with period P,
-// draw the next P masks ahead. Failures here only mean "no prefetch".
-static void prefetch_maybe_start() {
-    const size_t h = g_history.size();
-    size_t period = 0;
-    for (size_t P = g_min_period; P <= kMaxPeriod && 2 * P <= h; ++P) {
-        bool same = true;
-        for (size_t k = 0; k < P && same; ++k) same = g_history[h - 1 - k] == g_history[h - 1 - k - P];
-        if (same) { period = P; break; }
-    }
-    if (h > 4 * kMaxPeriod) g_history.erase(g_history.begin(), g_history.begin() + (h - 2 * kMaxPeriod));
-    if (period == 0) return;
-    size_t total = 0;
-    for (size_t k = 0; k < period; ++k) total += g_history[g_history.size() - period + k].first;
-    if (total > kMaxPrefetchFloats) return;
-    if (!g_side && hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking) != hipSuccess) { g_side = nullptr; return; }
-    if (order_streams(ctx().stream, g_side) != 0) return;
-    const std::vector<std::pair<size_t, double>> next(g_history.end() - period, g_history.end());
-    for (const auto& req : next) {
-        MaskPrefetch e = MaskPrefetch();
-        e.n = req.first;
-        e.p = req.second;
-        void* a = nullptr;
-        void* b = nullptr;
-        void* r = nullptr;
-        bool ok = pool_alloc_raw(e.n * sizeof(float), &a) == 0;
-        e.staging = static_cast<float*>(a);
-        ok = ok && pool_alloc_raw(2 * e.n * sizeof(uint32_t), &r) == 0;
-        e.raw = static_cast<uint32_t*>(r);
-        ok = ok && pool_alloc_raw(sizeof(RngState), &b) == 0;
-        e.before = static_cast<RngState*>(b);
-        ok = ok && hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) == hipSuccess;
-        ok = ok && hipEventCreateWithFlags(&e.consumed, hipEventDisableTiming) == hipSuccess;
-        if (!ok) { free_entry(e); break; }
-        // fresh pool blocks may still be in use by earlier main-stream work: already ordered above
-        if (prefetch_schedule(e, false) != 0) break;
-    }
-}
+// Gives up everything drawn ahead and puts the generator back to its sequential position (defined
+// behind the masks of recorded steps, whose helpers the look-ahead shares).
+static int prefetch_flush(bool restore_position, bool wrong_guess = false);
+static void prefetch_maybe_start();
 
 // --------------------------- masks of recorded steps ---------------------------
 // A recorded step (bship_graph_begin ... bship_graph_end) replays the same kernels with the same
@@ -729,6 +661,126 @@ __global__ __launch_bounds__(kBlock) void slot_copy_kernel(SlotCopies c) {
     }
 }
 
+
+// ------------------------------ look-ahead rounds ------------------------------
+struct Round {
+    GraphMasks gm;                    // the round's masks: slots (n, p, staging), raw words, snapshot in slots.front().before
+    hipEvent_t ready = nullptr;       // second stream: the masks are in the slots' staging buffers
+    hipEvent_t consumed = nullptr;    // main stream: the round's last mask has been read
+    bool drawn = false;               // the draw is enqueued and not yet used up
+    bool read = false;                // `consumed` has been recorded
+};
+static Round g_round[2];
+static int g_round_cur = 0;           // the round being handed out
+static size_t g_round_cursor = 0;     // its next slot
+static bool g_lookahead = false;
+
+static void free_round(Round& r) {
+    for (MaskPrefetch& e : r.gm.slots) free_entry(e);
+    if (r.gm.raw) pool_free_raw(r.gm.raw);
+    if (r.ready) (void)hipEventDestroy(r.ready);
+    if (r.consumed) (void)hipEventDestroy(r.consumed);
+    r = Round();
+}
+
+// Enqueues the draw of round r on the second stream, which owns the generator while rounds are in use.
+static int draw_round(Round& r) {
+    if (r.read) BSHIP_HIP(hipStreamWaitEvent(g_side, r.consumed, 0));    // its buffers were read on the main stream
+    int st = launch_graph_masks(g_side, r.gm, false);
+    if (st != 0) return st;
+    BSHIP_HIP(hipEventRecord(r.ready, g_side));
+    r.drawn = true;
+    return 0;
+}
+
+static int prefetch_flush(bool restore_position, bool wrong_guess) {
+    g_history.clear();
+    if (!g_lookahead) return 0;
+    Round& cur = g_round[g_round_cur];
+    // "A B B" looks like period 1 after its second B: when a guess turns out wrong, only
+    // longer periods are tried next (any multiple of the true period serves as well)
+    const size_t period = cur.gm.slots.size();
+    if (wrong_guess) g_min_period = period + 1 > kMaxPeriod ? 1 : period + 1;
+    int st = order_streams(g_side, ctx().stream);
+    if (st == 0 && restore_position && cur.drawn) {
+        hipLaunchKernelGGL(rng_copy_state_kernel, dim3(1), dim3(kBlock), 0, ctx().stream,
+                           cur.gm.slots.front().before, g_state);
+        st = check_launch("random stream rewind");
+        size_t used = 0;
+        for (size_t k = 0; k < g_round_cursor; ++k) used += 2 * cur.gm.slots[k].n;
+        if (st == 0 && used > 0) {
+            // the masks already handed out: their words again (into the round's own buffer, which
+            // nobody reads any more), so that the generator stands right behind them
+            hipLaunchKernelGGL(mt_raw_kernel, dim3(1), dim3(kRawThreads), 0, ctx().stream, g_state, cur.gm.raw,
+                               used, static_cast<RngState*>(nullptr));
+            st = check_launch("random stream rewind");
+        }
+    }
+    // the blocks go back to the pool; their next owners run on the main stream, which is
+    // ordered behind the second stream now
+    free_round(g_round[0]);
+    free_round(g_round[1]);
+    g_lookahead = false;
+    g_round_cur = 0;
+    g_round_cursor = 0;
+    return st;
+}
+
+// After a mask was drawn directly: if the recent requests repeat with period P, set up two
+// rounds of P masks and draw the first. Failures here only mean "no look-ahead".
+static void prefetch_maybe_start() {
+    const size_t h = g_history.size();
+    size_t period = 0;
+    for (size_t P = g_min_period; P <= kMaxPeriod && 2 * P <= h; ++P) {
+        bool same = true;
+        for (size_t k = 0; k < P && same; ++k) same = g_history[h - 1 - k] == g_history[h - 1 - k - P];
+        if (same) { period = P; break; }
+    }
+    if (h > 4 * kMaxPeriod) g_history.erase(g_history.begin(), g_history.begin() + (h - 2 * kMaxPeriod));
+    if (period == 0) return;
+    size_t total = 0;
+    for (size_t k = 0; k < period; ++k) total += g_history[g_history.size() - period + k].first;
+    if (2 * total > kMaxPrefetchFloats) return;
+    if (ensure_side_stream() != 0) { (void)hipGetLastError(); return; }
+    const std::vector<std::pair<size_t, double>> next(g_history.end() - period, g_history.end());
+    bool ok = true;
+    for (Round& r : g_round) {
+        r = Round();
+        for (const auto& req : next) {
+            MaskPrefetch e = MaskPrefetch();
+            e.n = req.first;
+            e.p = req.second;
+            void* a = nullptr;
+            ok = ok && pool_alloc_raw(e.n * sizeof(float), &a) == 0;
+            e.staging = static_cast<float*>(a);
+            r.gm.slots.push_back(e);
+            r.gm.words += 2 * e.n;
+        }
+        void* b = nullptr;
+        void* w = nullptr;
+        ok = ok && pool_alloc_raw(sizeof(RngState), &b) == 0;
+        r.gm.slots.front().before = static_cast<RngState*>(b);
+        ok = ok && pool_alloc_raw(r.gm.words * sizeof(uint32_t), &w) == 0;
+        r.gm.raw = static_cast<uint32_t*>(w);
+        ok = ok && hipEventCreateWithFlags(&r.ready, hipEventDisableTiming) == hipSuccess;
+        ok = ok && hipEventCreateWithFlags(&r.consumed, hipEventDisableTiming) == hipSuccess;
+    }
+    // fresh pool blocks may still be in use by earlier main-stream work, and the generator passes
+    // to the second stream: both are ordered here
+    ok = ok && order_streams(ctx().stream, g_side) == 0;
+    if (ok) {
+        g_lookahead = true;          // from here on the second stream has run the generator ahead
+        g_round_cur = 0;
+        g_round_cursor = 0;
+        ok = draw_round(g_round[0]) == 0;
+        if (!ok) (void)prefetch_flush(g_round[0].drawn);
+        return;
+    }
+    (void)hipGetLastError();
+    free_round(g_round[0]);
+    free_round(g_round[1]);
+}
+
 int rng_graph_begin(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     int st = ensure_side_stream();
@@ -827,8 +879,9 @@ void rng_graph_destroyed(int id) {
     g_graph_masks.erase(it);
 }
 
-// Serves a mask request: either hands back the queue's front entry (*is_hit; the caller reads
-// hit->staging on the main stream and then calls mask_end), or draws the mask into `mask` directly.
+// Serves a mask request: either hands back a drawn mask (*is_hit; the caller reads hit->staging on
+// the main stream and then calls mask_end, or mask_abort if it could not), or draws the mask into
+// `mask` directly.
 static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* is_hit) {
     *is_hit = false;
     if (g_recording_masks) {
@@ -837,13 +890,18 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
     }
     int ust = graph_masks_unprime();
     if (ust != 0) return ust;
-    if (!g_fifo.empty()) {
-        const MaskPrefetch& e = g_fifo.front();
+    if (g_lookahead) {
+        Round& cur = g_round[g_round_cur];
+        const MaskPrefetch& e = cur.gm.slots[g_round_cursor];
         if (e.n == n && e.p == p) {
-            BSHIP_HIP(hipStreamWaitEvent(ctx().stream, e.ready, 0));
+            if (g_round_cursor == 0) {
+                BSHIP_HIP(hipStreamWaitEvent(ctx().stream, cur.ready, 0));
+                // the round after this one: drawn while this one is handed out
+                int st = draw_round(g_round[g_round_cur ^ 1]);
+                if (st != 0) { (void)prefetch_flush(true); return st; }
+            }
             *hit = e;
             *is_hit = true;
-            g_fifo.pop_front();
             return 0;
         }
         int st = prefetch_flush(true, true);
@@ -862,13 +920,28 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
     return st;
 }
 
-// The main stream has enqueued its read of the entry's staging buffer: draw the entry again
-// for the step after.
+// The main stream has enqueued its read of the mask handed out by mask_begin.
 static int mask_end(MaskPrefetch& e) {
     if (g_recording_masks) return graph_mask_redraw(e);
-    hipError_t err = hipEventRecord(e.consumed, ctx().stream);
-    if (err != hipSuccess) { free_entry(e); return check_hip(err, "hipEventRecord"); }
-    return prefetch_schedule(e, true);
+    Round& cur = g_round[g_round_cur];
+    if (++g_round_cursor < cur.gm.slots.size()) return 0;
+    // the round is used up: its buffers may be drawn into again once this read has run
+    g_round_cursor = 0;
+    cur.drawn = false;
+    hipError_t err = hipEventRecord(cur.consumed, ctx().stream);
+    cur.read = true;
+    g_round_cur ^= 1;
+    if (err != hipSuccess) {
+        (void)prefetch_flush(true);
+        return check_hip(err, "hipEventRecord");
+    }
+    return 0;
+}
+
+// The read of the mask handed out by mask_begin could not be enqueued.
+static void mask_abort(MaskPrefetch& e) {
+    if (g_recording_masks) free_entry(e);      // a slot of its own, not yet part of the recording
+    // a round's slot stays where it is: the next request is served from it again
 }
 
 // Dropout forward (dropout_layer.py:41-45) behind the mask: mask = src (the mask as drawn),
@@ -1008,8 +1081,11 @@ static int launch_fast_mask(const float* in, float* mask, float* out, size_t n, 
 void rng_release() {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
     if (g_side) (void)hipStreamSynchronize(g_side);
-    for (MaskPrefetch& e : g_fifo) free_entry(e);
-    g_fifo.clear();
+    free_round(g_round[0]);
+    free_round(g_round[1]);
+    g_lookahead = false;
+    g_round_cur = 0;
+    g_round_cursor = 0;
     for (auto& kv : g_graph_masks) {
         for (MaskPrefetch& e : kv.second.slots) free_entry(e);
         if (kv.second.raw) pool_free_raw(kv.second.raw);
@@ -1129,7 +1205,7 @@ int bship_prob_mask_f32(float* mask, size_t n, double p) {
     int st = mask_begin(mask, n, p, &hit, &is_hit);
     if (st != 0 || !is_hit) return st;
     st = bship_d2d(mask, hit.staging, n * sizeof(float));
-    if (st != 0) { free_entry(hit); return st; }
+    if (st != 0) { mask_abort(hit); return st; }
     return mask_end(hit);
 }
 
@@ -1159,7 +1235,7 @@ int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, do
         hipLaunchKernelGGL(dropout_apply_kernel<false>, grid, blk, 0, ctx().stream, src, mask, in, out, scale, n);
     st = check_launch("dropout_forward");
     if (is_hit) {
-        if (st != 0) { free_entry(hit); return st; }
+        if (st != 0) { mask_abort(hit); return st; }
         st = mask_end(hit);
     }
     return st;

@@ -747,7 +747,7 @@ def _out_size(n, k, pad, stride):
 
 POOL_CASES = [(n, h, w, c, win, pad, stride)
               for (n, h, w, c) in [(1, 4, 4, 1), (2, 5, 7, 3), (3, 32, 32, 32), (2, 15, 15, 64)]
-              for win in [(1, 1), (2, 2), (3, 3), (2, 3), (3, 2)]
+              for win in [(1, 1), (2, 2), (3, 3), (2, 3), (3, 2), (4, 4)]
               for pad in (0, 1, 2)
               for stride in [(1, 1), (2, 2), (1, 2), (3, 3)]
               if win[0] <= h + 2 * pad and win[1] <= w + 2 * pad]
