@@ -260,7 +260,31 @@ def run_pitched_ops(rows=8192, cols=8192, reps=10):
              ("mult_mv_col", 8 * n, lambda: hip.mult_mv(a, col, o)),
              ("sum_t_axis0", 4 * n, lambda: hip.sum_t(a, 0, row)),
              ("sum_t_axis1", 4 * n, lambda: hip.sum_t(a, 1, col)),
-             ("copy_to", 8 * n, lambda: hip.copy_to(a, o))]
+             ("copy_to", 8 * n, lambda: hip.copy_to(a, o)),
+             ("generate_probability_mask", 4 * n, lambda: hip.generate_probability_mask(o, 0.5)),
+             ("broadcast_t_rows", 4 * n, lambda: hip.broadcast_t(row, 0, o)),
+             ("merge_tt", 8 * n, lambda: hip.merge_tt(a[:, :cols // 2], b[:, :cols // 2], o)),
+             ("split_add_tt", 12 * n, lambda: hip.split_add_tt(o, a[:, :cols // 2], b[:, :cols // 2]))]
+    # pooling on image slices: batch 2048 of 32x32x32 images and their 15x15x32 pooled outputs, each a
+    # feature slice of a hub that is half as wide again (the image operations' own benchmark shapes)
+    n_img, h, w, c, k, s = 2048, 32, 32, 32, 3, 2
+    oh = (h - k) // s + 1
+    fi, fo = h * w * c, oh * oh * c
+    hub_in, hub_din = hip.allocate((n_img, fi + fi // 2)), hip.allocate((n_img, fi + fi // 2))
+    hub_out, hub_arg, hub_dout = (hip.allocate((n_img, fo + fo // 2)) for _ in range(3))
+    noise = hip.allocate((1, 1 << 22))            # N(0,1) values: which pixel wins decides what max pooling touches
+    hip.fill_gaussian(0.0, 1.0, noise)
+    hip.broadcast_t(noise, 0, hub_in.reshape((hub_in.size // (1 << 22), 1 << 22)))
+    hip.copy_to(hub_in.reshape((hub_in.size,))[:hub_dout.size].reshape(hub_dout.shape), hub_dout)
+    x, dx = (t[:, :fi].reshape((n_img, h, w, c)) for t in (hub_in, hub_din))
+    y, am, dy = (t[:, :fo].reshape((n_img, oh, oh, c)) for t in (hub_out, hub_arg, hub_dout))
+    ni, no = n_img * fi, n_img * fo
+    cases += [("maxpool_fwd_32x32x32_k3s2", 4 * (ni + 2 * no), lambda: hip.maxpool2d_forward_batch(x, (k, k), y, 0, (s, s), am)),
+              ("maxpool_bwd_32x32x32_k3s2", 4 * (2 * ni + 2 * no),
+               lambda: hip.maxpool2d_backward_batch(x, (k, k), y, 0, (s, s), am, dx, dy)),
+              ("avgpool_fwd_32x32x32_k3s2", 4 * (ni + no), lambda: hip.avgpool2d_forward_batch(x, (k, k), y, 0, (s, s))),
+              ("avgpool_bwd_32x32x32_k3s2", 4 * (2 * ni + no),
+               lambda: hip.avgpool2d_backward_batch(x, (k, k), y, 0, (s, s), dx, dy))]
     out = {}
     for native in (True, False):
         hip.native_pitched = native

@@ -60,6 +60,7 @@ SIGNATURES = {
     "bship_elementwise_pitched_f32": [c_int, c_int, c_float, c_float, _P, _I64, c_int, _P, _I64, c_int,
                                       _P, _I64, _I64, _I64],
     "bship_broadcast_f32": [_P, _P, _I64, _I64, _I64],
+    "bship_broadcast_pitched_f32": [_P, _I64, _I64, _P, _I64, _I64, _I64, _I64, _I64],
     "bship_merge_f32": [_P, _P, _P, _I64, _I64, _I64],
     "bship_split_add_f32": [_P, _P, _P, _I64, _I64, _I64],
     "bship_sum_f32": [_P, _P, _I64, _I64, c_int],
@@ -77,6 +78,7 @@ SIGNATURES = {
     "bship_rng_destroy": [c_int],
     "bship_rng_seed": [c_uint32],
     "bship_prob_mask_f32": [_P, c_size_t, c_double],
+    "bship_prob_mask_pitched_f32": [_P, _I64, _I64, _I64, c_double],
     "bship_fill_gaussian_f32": [_P, c_size_t, c_double, c_double],
     "bship_fast_rng_seed": [ctypes.c_ulonglong],
     "bship_fast_rng_get_state": [POINTER(ctypes.c_ulonglong), POINTER(ctypes.c_ulonglong)],
@@ -91,6 +93,12 @@ SIGNATURES = {
     "bship_maxpool_bwd_nhwc_f32": [_P, _P, _P, _I64] + [c_int] * 10,
     "bship_avgpool_fwd_nhwc_f32": [_P, _P, _I64] + [c_int] * 10,
     "bship_avgpool_bwd_nhwc_f32": [_P, _P, _I64] + [c_int] * 10,
+    "bship_im2col_nhwc_pitched_f32": [_P, _I64, _P, _I64] + [c_int] * 8,
+    "bship_col2im_nhwc_pitched_f32": [_P, _P, _I64, _I64] + [c_int] * 8,
+    "bship_maxpool_fwd_nhwc_pitched_f32": [_P, _I64, _P, _I64, _P, _I64, _I64] + [c_int] * 10,
+    "bship_maxpool_bwd_nhwc_pitched_f32": [_P, _I64, _P, _I64, _P, _I64, _I64] + [c_int] * 10,
+    "bship_avgpool_fwd_nhwc_pitched_f32": [_P, _I64, _P, _I64, _I64] + [c_int] * 10,
+    "bship_avgpool_bwd_nhwc_pitched_f32": [_P, _I64, _P, _I64, _I64] + [c_int] * 10,
     "bship_lstm_fwd_step_f32": [c_int, _I64, _I64] + [_P] * 19,
     "bship_lstm_bwd_step_f32": [c_int, _I64, _I64] + [_P] * 24,
     "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,

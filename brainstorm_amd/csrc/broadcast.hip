@@ -205,6 +205,9 @@ int bship_broadcast_f32(const float* a, float* out, int64_t outer, int64_t bdim,
     BSHIP_REQUIRE_PTR(a);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_DIM(a != out);
+    // up to 2^32 - 1 elements: the vectorised kernel of the run-pitched form, with one run each
+    if (n <= 0xffffffffll)
+        return bship_broadcast_pitched_f32(a, outer * inner, outer * inner, out, n, n, outer, bdim, inner);
     hipLaunchKernelGGL(broadcast_kernel, dim3(stream_grid(ceil_div(n, kBlock))), dim3(kBlock), 0,
                        ctx().stream, a, out, outer, bdim, inner);
     return check_launch("broadcast_t");

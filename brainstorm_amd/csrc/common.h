@@ -175,6 +175,26 @@ void rng_graph_destroyed(int id);
 // Enqueues mem[0:n] = val.
 int launch_fill(float* mem, float val, size_t n);
 
+// n / d for 32-bit unsigned n by multiply and shift (Granlund-Montgomery, rounded-up
+// multiplier): with l = ceil(log2 d) and m = floor(2^32 (2^l - d) / d) + 1,
+// n / d = (mulhi(m, n) + n) >> l for every 32-bit n.
+struct FastDiv {
+    uint32_t d, magic, shift;
+    FastDiv() : d(1), magic(1), shift(0) {}
+    explicit FastDiv(uint32_t dd) : d(dd) {
+        shift = 0;
+        while ((uint64_t(1) << shift) < dd) ++shift;
+        magic = static_cast<uint32_t>(((uint64_t(1) << 32) * ((uint64_t(1) << shift) - dd)) / dd + 1);
+    }
+    __device__ __forceinline__ uint32_t div(uint32_t n) const {
+        return static_cast<uint32_t>((static_cast<uint64_t>(__umulhi(n, magic)) + n) >> shift);
+    }
+    __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
 // ---- integer labels stored as float32 (device) ----
 // Column selected by label v in a row of K columns: truncated toward zero like astype(int32);
 // labels in [-K, -1] count from the end, as NumPy's indexing does (numpy_handler.py:101, 203).

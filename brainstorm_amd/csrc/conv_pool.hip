@@ -37,26 +37,6 @@ struct ImgGeom {
 __host__ __device__ inline int imax(int a, int b) { return a > b ? a : b; }
 __host__ __device__ inline int imin(int a, int b) { return a < b ? a : b; }
 
-// n / d for 32-bit unsigned n by multiply and shift (Granlund-Montgomery, rounded-up
-// multiplier): with l = ceil(log2 d) and m = floor(2^32 (2^l - d) / d) + 1,
-// n / d = (mulhi(m, n) + n) >> l for every 32-bit n.
-struct FastDiv {
-    uint32_t d, magic, shift;
-    FastDiv() : d(1), magic(1), shift(0) {}
-    explicit FastDiv(uint32_t dd) : d(dd) {
-        shift = 0;
-        while ((uint64_t(1) << shift) < dd) ++shift;
-        magic = static_cast<uint32_t>(((uint64_t(1) << 32) * ((uint64_t(1) << shift) - dd)) / dd + 1);
-    }
-    __device__ __forceinline__ uint32_t div(uint32_t n) const {
-        return static_cast<uint32_t>((static_cast<uint64_t>(__umulhi(n, magic)) + n) >> shift);
-    }
-    __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
-        q = div(n);
-        r = n - q * d;
-    }
-};
-
 // Range [lo, hi) of output positions o with  o*stride - pad <= p < o*stride - pad + k.
 __device__ __forceinline__ void cover_range(int p, int pad, const FastDiv& stride, int k, int n_out,
                                             int& lo, int& hi) {
@@ -97,6 +77,10 @@ struct ImgPlan {
     uint32_t lanes_per_image;
     FastDiv d_cv, d_w, d_ow, d_kcv, d_kwcv, d_sh, d_sw;
     FastDiv d_pw;         // stride-aligned patches per image row (pooling backward)
+    // elements from one image to the next: arrays shaped like the input (in, in_deltas), like the
+    // output (out, out_deltas) and the argmax array. h*w*c / oh*ow*c for dense arrays; larger when
+    // the array is a feature slice of a wider hub (each image is contiguous, images lie a pitch apart)
+    int64_t in_pitch, out_pitch, aux_pitch;
     // launch shape: `tiles` workgroups cover one image, `groups` sets of images; see img_block
     uint32_t tiles, groups, per_xcd;
     FastDiv d_tiles;
@@ -138,7 +122,7 @@ __device__ __forceinline__ void im2col_body(const float* __restrict__ in, float*
     const int ix = static_cast<int>(ox) * g.sw - g.pad + static_cast<int>(kx);
     const bool inside = iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
     const int64_t in_off = (static_cast<int64_t>(iy) * g.w + ix) * g.c + chv * W;
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t in_img = pl.in_pitch;
     const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * W;
     // kImagesPerWorkgroup images at a time: all loads first, then all stores
     for (int64_t img0 = static_cast<int64_t>(group) * kImagesPerWorkgroup; img0 < n;
@@ -186,7 +170,7 @@ __global__ __launch_bounds__(kBlock) void im2col_gather4(const float* __restrict
         const bool inside = iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
         in_off[j] = inside ? (iy * g.w + ix) * g.c + static_cast<int>(ch) : -1;
     }
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t in_img = pl.in_pitch;
     const int64_t col_img = static_cast<int64_t>(pl.lanes_per_image) * 4;
     for (int64_t img0 = static_cast<int64_t>(group) * kImagesPerWorkgroup; img0 < n;
          img0 += static_cast<int64_t>(pl.groups) * kImagesPerWorkgroup) {
@@ -232,6 +216,7 @@ struct BandPlan {
     uint32_t per_image;    // oh*ow*kh*kw*c
     int tile_rows;         // most image rows a band looks at
     int wpc;               // (w + 2*pad) * c : LDS row pitch
+    int64_t in_pitch;      // elements from one input image to the next (h*w*c when dense)
     FastDiv d_k, d_ow, d_kwc, d_wpc, d_owk;
 };
 
@@ -250,7 +235,7 @@ __global__ __launch_bounds__(kBlock) void im2col_band(const float* __restrict__ 
     const int tile_cap = pl.tile_rows * pl.wpc;
     const int wc = g.w * g.c, padc = g.pad * g.c, swc = g.sw * g.c;
     const uint32_t kwc = static_cast<uint32_t>(g.kw * g.c);
-    const int64_t in_img = static_cast<int64_t>(g.h) * wc;
+    const int64_t in_img = pl.in_pitch;
     int buf = 0;
     for (int64_t img = blockIdx.y; img < n; img += gridDim.y) {
         float* t = band_tile + buf * tile_cap;
@@ -320,7 +305,7 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
     cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
     cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
     const int64_t kc = static_cast<int64_t>(g.kh) * g.kw * g.c;
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
+    const int64_t in_img = pl.in_pitch;
     const int64_t col_img = static_cast<int64_t>(g.oh) * g.ow * kc;
     for (int64_t img = group; img < n; img += pl.groups) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
@@ -362,6 +347,7 @@ struct Col2imBandPlan {
     int bands;             // workgroups per image
     int ring;              // col rows held in LDS
     uint32_t owk;          // ow*kh*kw*c : floats per col row
+    int64_t in_pitch;      // elements from one image of in_deltas to the next (h*w*c when dense)
     FastDiv d_bands, d_wc, d_w, d_sh, d_sw, d_ring, d_owk4;
 };
 
@@ -410,7 +396,7 @@ __global__ __launch_bounds__(kCol2imThreads) void col2im_band(const float* __res
     const int kc = g.kh * g.kw * g.c, wc = g.w * g.c;
     const int pitch = static_cast<int>(pl.owk);
     const float* cimg = col + img * (static_cast<int64_t>(g.oh) * pl.owk);
-    float* dimg = in_deltas + img * (static_cast<int64_t>(g.h) * wc);
+    float* dimg = in_deltas + img * pl.in_pitch;
     // Lane index o of a phase -> image element: within an image row the lanes are ordered channel
     // first, then x, so that neighbouring lanes read LDS words kh*kw*c apart (an odd stride for
     // RGB images: no bank conflicts) rather than runs of c words with gaps.
@@ -555,8 +541,8 @@ __device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, f
     const int y = static_cast<int>(oy) * g.sh - g.pad, x = static_cast<int>(ox) * g.sw - g.pad;
     const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
     const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
-    const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    const int64_t in_img = pl.in_pitch;
+    const int64_t out_img = pl.out_pitch;
     const int ch0 = static_cast<int>(chv) * W;
     typedef typename VecT<W>::type R;
     for (int64_t img = group; img < n; img += pl.groups) {
@@ -596,7 +582,7 @@ __device__ __forceinline__ void maxpool_fwd_body(const float* __restrict__ in, f
         for (int j = 0; j < W; ++j)
             if (comp<W>(where, j) < 0.0f) comp<W>(best, j) = 0.0f;
         vstore<W, AL>(out + img * out_img + static_cast<int64_t>(p) * W, best);
-        vstore<W, AL>(argmax + img * out_img + static_cast<int64_t>(p) * W, where);
+        vstore<W, AL>(argmax + img * pl.aux_pitch + static_cast<int64_t>(p) * W, where);
     }
 }
 #define BSHIP_POOL_FWD_KERNEL(name, K)                                                                   \
@@ -630,8 +616,8 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
     int oy0, oy1, ox0, ox1;
     cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
     cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
-    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    const int64_t in_img = pl.in_pitch;
+    const int64_t out_img = pl.out_pitch;
     typedef typename VecT<W>::type R;
     for (int64_t img = group; img < n; img += pl.groups) {
         float* q = in_deltas + img * in_img + static_cast<int64_t>(p) * W;
@@ -648,9 +634,9 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
 #pragma unroll
                 for (int b = 0; b < C; ++b) {
                     const int oy = imin(oy0 + a, g.oh - 1), ox = imin(ox0 + b, g.ow - 1);
-                    const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
-                    am[a * C + b] = img_load<W, AL>(argmax + o);
-                    d[a * C + b] = img_load<W, AL>(out_deltas + o);
+                    const int64_t o = (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
+                    am[a * C + b] = img_load<W, AL>(argmax + img * pl.aux_pitch + o);
+                    d[a * C + b] = img_load<W, AL>(out_deltas + img * out_img + o);
                 }
 #pragma unroll
             for (int a = 0; a < C; ++a)
@@ -660,8 +646,8 @@ __device__ __forceinline__ void maxpool_bwd_body(const float* __restrict__ argma
         } else {
             for (int oy = oy0; oy < oy1; ++oy)
                 for (int ox = ox0; ox < ox1; ++ox) {
-                    const int64_t o = img * out_img + (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
-                    take(img_load<W, AL>(argmax + o), img_load<W, AL>(out_deltas + o));
+                    const int64_t o = (static_cast<int64_t>(oy) * g.ow + ox) * g.c + ch0;
+                    take(img_load<W, AL>(argmax + img * pl.aux_pitch + o), img_load<W, AL>(out_deltas + img * out_img + o));
                 }
         }
         vstore<W, AL>(q, acc);
@@ -694,8 +680,8 @@ __device__ __forceinline__ void avgpool_fwd_body(const float* __restrict__ in, f
     const int y0 = imax(y, 0), y1 = imin(y + g.kh, g.h);
     const int x0 = imax(x, 0), x1 = imin(x + g.kw, g.w);
     const float size = static_cast<float>(imax((y1 - y0) * (x1 - x0), 1));
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
-    const int64_t out_img = static_cast<int64_t>(pl.lanes_per_image) * W;
+    const int64_t in_img = pl.in_pitch;
+    const int64_t out_img = pl.out_pitch;
     typedef typename VecT<W>::type R;
     for (int64_t img = group; img < n; img += pl.groups) {
         const float* base = in + img * in_img + chv * W;
@@ -749,8 +735,8 @@ __device__ __forceinline__ void avgpool_bwd_body(const float* __restrict__ out_d
     int oy0, oy1, ox0, ox1;
     cover_range(y, g.pad, pl.d_sh, g.kh, g.oh, oy0, oy1);
     cover_range(x, g.pad, pl.d_sw, g.kw, g.ow, ox0, ox1);
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
-    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    const int64_t in_img = pl.in_pitch;
+    const int64_t out_img = pl.out_pitch;
     typedef typename VecT<W>::type R;
     // number of image pixels under the window at output position (oy, ox)
     auto window_size = [&](int oy, int ox) {
@@ -826,8 +812,8 @@ __device__ __forceinline__ void pool_bwd_patch_body(const float* __restrict__ ar
     const int ch0 = static_cast<int>(chv) * W;
     const int y0 = static_cast<int>(pi) * S - g.pad, x0 = static_cast<int>(pj) * S - g.pad;
     const int oyb = static_cast<int>(pi) - (C - 1), oxb = static_cast<int>(pj) - (C - 1);
-    const int64_t in_img = static_cast<int64_t>(g.h) * g.w * g.c;
-    const int64_t out_img = static_cast<int64_t>(g.oh) * g.ow * g.c;
+    const int64_t in_img = pl.in_pitch;
+    const int64_t out_img = pl.out_pitch;
     typedef typename VecT<W>::type R;
     bool valid[S * S];
     int pix_off[S * S];
@@ -862,7 +848,7 @@ __device__ __forceinline__ void pool_bwd_patch_body(const float* __restrict__ ar
             if (valid[k]) acc[k] = vload<W, AL>(q + pix_off[k]);
 #pragma unroll
         for (int k = 0; k < C * C; ++k) {
-            if constexpr (MAX) am[k] = img_load<W, AL>(argmax + img * out_img + win_off[k]);
+            if constexpr (MAX) am[k] = img_load<W, AL>(argmax + img * pl.aux_pitch + win_off[k]);
             d[k] = img_load<W, AL>(out_deltas + img * out_img + win_off[k]);
         }
         if constexpr (!MAX) {
@@ -1066,7 +1052,8 @@ static bool allow_dynamic_lds(K kernel, size_t bytes) {
 using namespace bship;
 
 // Launches kernel<W, AL> over lanes_per_image x n: W = 4 when the channels come in fours,
-// AL when additionally every pointer is 16-byte aligned.
+// AL when additionally every pointer is 16-byte aligned. The image pitches of the plan are the
+// caller's local variables in_pitch, out_pitch and aux_pitch.
 #define BSHIP_LAUNCH_IMG(kernel, name, positions, aligned, ...)                                         \
     BSHIP_LAUNCH_IMG_N(kernel, name, positions, aligned, kImagesPerWorkgroup, __VA_ARGS__)
 // images_per_wg: how many images a workgroup walks through, one after the other (kernels whose image
@@ -1091,6 +1078,9 @@ using namespace bship;
         pl_.d_sh = FastDiv(static_cast<uint32_t>(g.sh));                                                \
         pl_.d_sw = FastDiv(static_cast<uint32_t>(g.sw));                                                \
         pl_.d_pw = FastDiv(static_cast<uint32_t>(imax((g.w - 1 + g.pad) / g.sw + 1, 1)));               \
+        pl_.in_pitch = in_pitch;                                                                        \
+        pl_.out_pitch = out_pitch;                                                                      \
+        pl_.aux_pitch = aux_pitch;                                                                      \
         const int64_t gy_ = ceil_div(n, images_per_wg);                                                 \
         pl_.tiles = static_cast<uint32_t>(ceil_div(lanes_, kBlock));                                    \
         pl_.groups = static_cast<uint32_t>(gy_ < 65535 ? gy_ : 65535);                                  \
@@ -1112,12 +1102,19 @@ extern "C" {
 
 int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, int c, int kh,
                           int kw, int pad, int stride_h, int stride_w) {
+    return bship_im2col_nhwc_pitched_f32(in, static_cast<int64_t>(h) * w * c, col, n, h, w, c, kh, kw, pad,
+                                         stride_h, stride_w);
+}
+
+int bship_im2col_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* col, int64_t n, int h, int w,
+                                  int c, int kh, int kw, int pad, int stride_h, int stride_w) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(kh >= 1 && kw >= 1 && stride_h >= 1 && stride_w >= 1 && pad >= 0);
     BSHIP_REQUIRE_DIM(h + 2 * pad >= kh && w + 2 * pad >= kw);
     ImgGeom g{h, w, c, conv_out(h, kh, pad, stride_h), conv_out(w, kw, pad, stride_w), kh, kw, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c);
     const int64_t total = n * g.oh * g.ow * kh * kw * c;
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
@@ -1126,8 +1123,10 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
     BSHIP_REQUIRE_F32_ALIGNED(col);
     const bool write_through = static_cast<size_t>(total) >= (size_t(1) << 26);   // 256 MiB: beyond the last-level cache
     const int64_t per_image = static_cast<int64_t>(g.oh) * g.ow * kh * kw * c;
+    const int64_t out_pitch = per_image, aux_pitch = 0;
     BandPlan bp;
     if (plan_im2col_band(g, n, per_image, &bp)) {
+        bp.in_pitch = in_pitch;
         const size_t lds = 2 * static_cast<size_t>(bp.tile_rows) * bp.wpc * sizeof(float);
         const dim3 grid(static_cast<unsigned>(ceil_div(per_image, bp.band)), static_cast<unsigned>(n < 65535 ? n : 65535));
         if (c % 4 == 0) {
@@ -1147,6 +1146,9 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
         pl.d_ow = FastDiv(static_cast<uint32_t>(g.ow));
         pl.d_kcv = FastDiv(static_cast<uint32_t>(kh * kw * c));
         pl.d_kwcv = FastDiv(static_cast<uint32_t>(kw * c));
+        pl.in_pitch = in_pitch;
+        pl.out_pitch = out_pitch;
+        pl.aux_pitch = 0;
         const int64_t gy = ceil_div(n, kImagesPerWorkgroup);
         pl.tiles = static_cast<uint32_t>(ceil_div(per_image / 4, kBlock));
         pl.groups = static_cast<uint32_t>(gy < 65535 ? gy : 65535);
@@ -1159,30 +1161,38 @@ int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w, 
         else               hipLaunchKernelGGL(im2col_gather4<false>, grid, dim3(kBlock), 0, ctx().stream, in, col, n, pl);
         return check_launch("im2col");
     }
+    const bool al = aligned16(in) && aligned16(col) && in_pitch % 4 == 0;
     if (write_through)
-        BSHIP_LAUNCH_IMG(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,
-                         aligned16(in) && aligned16(col), in, col);
-    BSHIP_LAUNCH_IMG(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw,
-                     aligned16(in) && aligned16(col), in, col);
+        BSHIP_LAUNCH_IMG(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
+    BSHIP_LAUNCH_IMG(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
 }
 
 int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, int w, int c,
                           int kh, int kw, int pad, int stride_h, int stride_w) {
+    return bship_col2im_nhwc_pitched_f32(col, in_deltas, static_cast<int64_t>(h) * w * c, n, h, w, c, kh, kw,
+                                         pad, stride_h, stride_w);
+}
+
+int bship_col2im_nhwc_pitched_f32(const float* col, float* in_deltas, int64_t in_pitch, int64_t n, int h,
+                                  int w, int c, int kh, int kw, int pad, int stride_h, int stride_w) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(kh >= 1 && kw >= 1 && stride_h >= 1 && stride_w >= 1 && pad >= 0);
     BSHIP_REQUIRE_DIM(h + 2 * pad >= kh && w + 2 * pad >= kw);
     ImgGeom g{h, w, c, conv_out(h, kh, pad, stride_h), conv_out(w, kw, pad, stride_w), kh, kw, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c);
     const int64_t total = n * h * w * c;
     if (total == 0) return 0;
     BSHIP_REQUIRE_PTR(col);
     BSHIP_REQUIRE_PTR(in_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(col);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
+    const int64_t out_pitch = 0, aux_pitch = 0;
     Col2imBandPlan bp;
     size_t lds = 0;
     if (plan_col2im_band(g, n, &bp, &lds)) {
+        bp.in_pitch = in_pitch;
         const int ks = (kh == kw && stride_h == 1 && stride_w == 1 && (kh == 3 || kh == 5)) ? kh : 0;
         const int64_t groups = ceil_div(n, kXcds) * bp.bands;
         if (groups * kXcds <= 0x7fffffff) {
@@ -1201,25 +1211,35 @@ int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, 
         (void)hipGetLastError();   // the attribute was refused: use the kernel without LDS
     }
     BSHIP_LAUNCH_IMG(col2im_kernel, "col2im", static_cast<int64_t>(h) * w,
-                     aligned16(col) && aligned16(in_deltas), col, in_deltas);
+                     aligned16(col) && aligned16(in_deltas) && in_pitch % 4 == 0, col, in_deltas);
 }
 
 int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64_t n, int h, int w,
                                int c, int out_h, int out_w, int pool_h, int pool_w, int pad,
                                int stride_h, int stride_w) {
+    const int64_t o = static_cast<int64_t>(out_h) * out_w * c;
+    return bship_maxpool_fwd_nhwc_pitched_f32(in, static_cast<int64_t>(h) * w * c, out, o, argmax, o, n, h, w, c,
+                                              out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w);
+}
+
+int bship_maxpool_fwd_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* out, int64_t out_pitch,
+                                       float* argmax, int64_t aux_pitch, int64_t n, int h, int w, int c,
+                                       int out_h, int out_w, int pool_h, int pool_w, int pad, int stride_h,
+                                       int stride_w) {
     BSHIP_REQUIRE_INIT();
     ImgGeom g{h, w, c, out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
-    const int64_t total = n * out_h * out_w * c;
-    if (total == 0) return 0;
+    const int64_t out_image = static_cast<int64_t>(out_h) * out_w * c;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c && out_pitch >= out_image && aux_pitch >= out_image);
+    if (n * out_image == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_PTR(argmax);
     BSHIP_REQUIRE_F32_ALIGNED(in);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     BSHIP_REQUIRE_F32_ALIGNED(argmax);
-    const bool al = aligned16(in) && aligned16(out) && aligned16(argmax);
+    const bool al = aligned16(in) && aligned16(out) && aligned16(argmax) && (in_pitch | out_pitch | aux_pitch) % 4 == 0;
     if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
         BSHIP_LAUNCH_IMG(maxpool_fwd_kernel_3x3, "maxpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, in, out, argmax);
     if (pool_h == 2 && pool_w == 2 && h >= 1 && w >= 1)
@@ -1230,10 +1250,21 @@ int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64
 int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, float* in_deltas,
                                int64_t n, int h, int w, int c, int out_h, int out_w, int pool_h,
                                int pool_w, int pad, int stride_h, int stride_w) {
+    const int64_t o = static_cast<int64_t>(out_h) * out_w * c;
+    return bship_maxpool_bwd_nhwc_pitched_f32(argmax, o, out_deltas, o, in_deltas, static_cast<int64_t>(h) * w * c, n,
+                                              h, w, c, out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w);
+}
+
+int bship_maxpool_bwd_nhwc_pitched_f32(const float* argmax, int64_t aux_pitch, const float* out_deltas,
+                                       int64_t out_pitch, float* in_deltas, int64_t in_pitch, int64_t n, int h,
+                                       int w, int c, int out_h, int out_w, int pool_h, int pool_w, int pad,
+                                       int stride_h, int stride_w) {
     BSHIP_REQUIRE_INIT();
     ImgGeom g{h, w, c, out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
+    const int64_t out_image = static_cast<int64_t>(out_h) * out_w * c;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c && out_pitch >= out_image && aux_pitch >= out_image);
     const int64_t total = n * h * w * c;
     if (total == 0 || out_h == 0 || out_w == 0) return 0;
     BSHIP_REQUIRE_PTR(argmax);
@@ -1242,7 +1273,8 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
     BSHIP_REQUIRE_F32_ALIGNED(argmax);
     BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
-    const bool al = aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas);
+    const bool al = aligned16(argmax) && aligned16(out_deltas) && aligned16(in_deltas) &&
+                    (in_pitch | out_pitch | aux_pitch) % 4 == 0;
     // square windows and strides above 1: a lane per stride-aligned patch of pixels
     if (pool_h == pool_w && stride_h == stride_w && (stride_h == 2 || stride_h == 3)) {
         const int64_t patches = static_cast<int64_t>((h - 1 + pad) / stride_h + 1) * ((w - 1 + pad) / stride_w + 1);
@@ -1266,17 +1298,27 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* out_deltas, flo
 int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, int w, int c,
                                int out_h, int out_w, int pool_h, int pool_w, int pad, int stride_h,
                                int stride_w) {
+    return bship_avgpool_fwd_nhwc_pitched_f32(in, static_cast<int64_t>(h) * w * c, out,
+                                              static_cast<int64_t>(out_h) * out_w * c, n, h, w, c, out_h, out_w,
+                                              pool_h, pool_w, pad, stride_h, stride_w);
+}
+
+int bship_avgpool_fwd_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* out, int64_t out_pitch, int64_t n,
+                                       int h, int w, int c, int out_h, int out_w, int pool_h, int pool_w, int pad,
+                                       int stride_h, int stride_w) {
     BSHIP_REQUIRE_INIT();
     ImgGeom g{h, w, c, out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
-    const int64_t total = n * out_h * out_w * c;
-    if (total == 0) return 0;
+    const int64_t out_image = static_cast<int64_t>(out_h) * out_w * c;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c && out_pitch >= out_image);
+    if (n * out_image == 0) return 0;
     BSHIP_REQUIRE_PTR(in);
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(in);
     BSHIP_REQUIRE_F32_ALIGNED(out);
-    const bool al = aligned16(in) && aligned16(out);
+    const int64_t aux_pitch = 0;
+    const bool al = aligned16(in) && aligned16(out) && (in_pitch | out_pitch) % 4 == 0;
     if (pool_h == 3 && pool_w == 3 && h >= 1 && w >= 1)
         BSHIP_LAUNCH_IMG_N(avgpool_fwd_kernel_3x3, "avgpool2d_forward_batch", static_cast<int64_t>(out_h) * out_w, al, 1, in, out);
     if (pool_h == 2 && pool_w == 2 && h >= 1 && w >= 1)
@@ -1287,17 +1329,28 @@ int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int h, in
 int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas, int64_t n, int h, int w,
                                int c, int out_h, int out_w, int pool_h, int pool_w, int pad,
                                int stride_h, int stride_w) {
+    return bship_avgpool_bwd_nhwc_pitched_f32(out_deltas, static_cast<int64_t>(out_h) * out_w * c, in_deltas,
+                                              static_cast<int64_t>(h) * w * c, n, h, w, c, out_h, out_w, pool_h,
+                                              pool_w, pad, stride_h, stride_w);
+}
+
+int bship_avgpool_bwd_nhwc_pitched_f32(const float* out_deltas, int64_t out_pitch, float* in_deltas, int64_t in_pitch,
+                                       int64_t n, int h, int w, int c, int out_h, int out_w, int pool_h, int pool_w,
+                                       int pad, int stride_h, int stride_w) {
     BSHIP_REQUIRE_INIT();
     ImgGeom g{h, w, c, out_h, out_w, pool_h, pool_w, pad, stride_h, stride_w};
     int st = check_geom(__func__, n, g);
     if (st != 0) return st;
+    BSHIP_REQUIRE_DIM(in_pitch >= static_cast<int64_t>(h) * w * c &&
+                      out_pitch >= static_cast<int64_t>(out_h) * out_w * c);
     const int64_t total = n * h * w * c;
     if (total == 0 || out_h == 0 || out_w == 0) return 0;
     BSHIP_REQUIRE_PTR(out_deltas);
     BSHIP_REQUIRE_PTR(in_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(out_deltas);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
-    const bool al = aligned16(out_deltas) && aligned16(in_deltas);
+    const int64_t aux_pitch = 0;
+    const bool al = aligned16(out_deltas) && aligned16(in_deltas) && (in_pitch | out_pitch) % 4 == 0;
     if (pool_h == pool_w && stride_h == stride_w && (stride_h == 2 || stride_h == 3)) {
         const int64_t patches = static_cast<int64_t>((h - 1 + pad) / stride_h + 1) * ((w - 1 + pad) / stride_w + 1);
         const int cover_patch = (pool_h - 1) / stride_h + 1;

@@ -117,11 +117,76 @@ static int launch_map2d(const char* name, F f, Operand2d in0, Operand2d in1, Ope
     return check_launch(name);
 }
 
+// broadcast_t (numpy 103-105) between arrays made of contiguous runs: element e of the dense
+// order of `out`, e = (o * bdim + b) * inner + i, is element o * inner + i of the dense order of
+// `a`; dense element k of an array lies at (k / run) * pitch + k % run. W = 4 when inner and both
+// runs are multiples of 4: four consecutive elements then share their rows on both sides.
+struct BroadcastPlan {
+    uint32_t groups;             // lanes: n / W
+    uint32_t inner;
+    int64_t ld_a, ld_out;
+    FastDiv d_inner, d_bdim, d_arun, d_orun;
+};
+// WT: write-through stores (outputs too large to be read again from the caches soon).
+template <int W, bool WT>
+__global__ __launch_bounds__(kBlock) void broadcast_pitched_kernel(const float* __restrict__ a,
+                                                                   float* __restrict__ out, BroadcastPlan pl) {
+    const uint32_t g = blockIdx.x * kBlock + threadIdx.x;
+    if (g >= pl.groups) return;
+    const uint32_t e = g * W;
+    uint32_t ob, i, o, b, ar, ac, orow, oc;
+    pl.d_inner.divmod(e, ob, i);
+    pl.d_bdim.divmod(ob, o, b);
+    pl.d_arun.divmod(o * pl.inner + i, ar, ac);
+    pl.d_orun.divmod(e, orow, oc);
+    const float* src = a + static_cast<int64_t>(ar) * pl.ld_a + ac;
+    float* dst = out + static_cast<int64_t>(orow) * pl.ld_out + oc;
+    if constexpr (W == 4) {
+        const f4 v = *reinterpret_cast<const f4u*>(src);        // the source is read bdim times: cached
+        if constexpr (WT) vstore_writeonly<4>(dst, v);
+        else vstore<4, false>(dst, v);
+    } else {
+        *dst = *src;
+    }
+}
+
 }  // namespace bship
 
 using namespace bship;
 
 extern "C" {
+
+int bship_broadcast_pitched_f32(const float* a, int64_t a_run, int64_t ld_a, float* out, int64_t out_run,
+                                int64_t ld_out, int64_t outer, int64_t bdim, int64_t inner) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(outer >= 0 && bdim >= 0 && inner >= 0);
+    const int64_t n = outer * bdim * inner;
+    if (n == 0) return 0;
+    BSHIP_REQUIRE_DIM(a_run >= 1 && out_run >= 1 && ld_a >= a_run && ld_out >= out_run);
+    BSHIP_REQUIRE_DIM((outer * inner) % a_run == 0 && n % out_run == 0);
+    BSHIP_REQUIRE_DIM(n <= 0xffffffffll);
+    BSHIP_REQUIRE_PTR(a);
+    BSHIP_REQUIRE_PTR(out);
+    BSHIP_REQUIRE_F32_ALIGNED(a);
+    BSHIP_REQUIRE_F32_ALIGNED(out);
+    BSHIP_REQUIRE_DIM(a != out);
+    const bool vec = inner % 4 == 0 && a_run % 4 == 0 && out_run % 4 == 0;
+    BroadcastPlan pl;
+    pl.groups = static_cast<uint32_t>(vec ? n / 4 : n);
+    pl.inner = static_cast<uint32_t>(inner);
+    pl.ld_a = ld_a;
+    pl.ld_out = ld_out;
+    pl.d_inner = FastDiv(static_cast<uint32_t>(inner));
+    pl.d_bdim = FastDiv(static_cast<uint32_t>(bdim));
+    pl.d_arun = FastDiv(static_cast<uint32_t>(a_run));
+    pl.d_orun = FastDiv(static_cast<uint32_t>(out_run));
+    const dim3 grid(static_cast<unsigned>(ceil_div(pl.groups, kBlock)));
+    const bool wt = static_cast<size_t>(n) >= ctx().write_through_min;
+    if (vec && wt) hipLaunchKernelGGL((broadcast_pitched_kernel<4, true>), grid, dim3(kBlock), 0, ctx().stream, a, out, pl);
+    else if (vec)  hipLaunchKernelGGL((broadcast_pitched_kernel<4, false>), grid, dim3(kBlock), 0, ctx().stream, a, out, pl);
+    else           hipLaunchKernelGGL((broadcast_pitched_kernel<1, false>), grid, dim3(kBlock), 0, ctx().stream, a, out, pl);
+    return check_launch("broadcast_t");
+}
 
 int bship_elementwise_pitched_f32(int family, int op, float s0, float s1,
                                   const float* a, int64_t a_row_stride, int a_col_stride,

@@ -246,14 +246,23 @@ __device__ __forceinline__ uint64_t raw_to_k53(const uint32_t* __restrict__ raw,
     const uint32_t w0 = mt_temper(raw[2 * i]), w1 = mt_temper(raw[2 * i + 1]);
     return (static_cast<uint64_t>(w0 >> 5) << 26) | static_cast<uint64_t>(w1 >> 6);
 }
+// Element i of the mask goes to row i / cols, column i % cols of a matrix whose rows lie ld elements
+// apart (ld == cols: the dense mask).
 __global__ __launch_bounds__(kBlock) void raw_to_mask_kernel(const uint32_t* __restrict__ raw,
-                                                             float* __restrict__ mask, size_t n, double p) {
+                                                             float* __restrict__ mask, size_t n, double p,
+                                                             size_t cols, size_t ld) {
     uint64_t threshold;
     if (!(p > 0.0)) threshold = 0;
     else if (p >= 1.0) threshold = ~static_cast<uint64_t>(0);
     else threshold = static_cast<uint64_t>(ceil(p * 9007199254740992.0));
     const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (i < n) mask[i] = raw_to_k53(raw, i) < threshold ? 1.0f : 0.0f;
+    if (i >= n) return;
+    size_t at = i;
+    if (ld != cols) {
+        const size_t row = i / cols;
+        at = row * ld + (i - row * cols);
+    }
+    mask[at] = raw_to_k53(raw, i) < threshold ? 1.0f : 0.0f;
 }
 __global__ __launch_bounds__(kBlock) void raw_to_doubles_kernel(const uint32_t* __restrict__ raw,
                                                                 double* __restrict__ u, size_t n) {
@@ -491,10 +500,13 @@ static void launch_raw_words(hipStream_t stream, uint32_t* raw, size_t nw, RngSt
 }
 
 // Enqueues mask[0..n) = (next n doubles of the stream < p) on `stream`; raw is scratch for 2n words.
-static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw) {
+// The mask is a matrix of `cols` columns whose rows lie `ld` elements apart (0: dense).
+static void launch_mask(hipStream_t stream, float* mask, size_t n, double p, RngState* before, uint32_t* raw,
+                        size_t cols = 0, size_t ld = 0) {
     launch_raw_words(stream, raw, 2 * n, before);
+    if (cols == 0) cols = ld = n;
     hipLaunchKernelGGL(raw_to_mask_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(n), kBlock))),
-                       dim3(kBlock), 0, stream, raw, mask, n, p);
+                       dim3(kBlock), 0, stream, raw, mask, n, p, cols, ld);
 }
 
 // Enqueues u[0..n) = the next n doubles of the stream on the main stream (raw: scratch for 2n words).
@@ -882,7 +894,8 @@ void rng_graph_destroyed(int id) {
 // Serves a mask request: either hands back a drawn mask (*is_hit; the caller reads hit->staging on
 // the main stream and then calls mask_end, or mask_abort if it could not), or draws the mask into
 // `mask` directly.
-static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* is_hit) {
+static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* is_hit, size_t cols = 0,
+                      size_t ld = 0) {
     *is_hit = false;
     if (g_recording_masks) {
         *is_hit = true;
@@ -910,7 +923,7 @@ static int mask_begin(float* mask, size_t n, double p, MaskPrefetch* hit, bool* 
     void* raw = nullptr;
     int st = pool_alloc_raw(2 * n * sizeof(uint32_t), &raw);
     if (st != 0) return st;
-    launch_mask(ctx().stream, mask, n, p, nullptr, static_cast<uint32_t*>(raw));
+    launch_mask(ctx().stream, mask, n, p, nullptr, static_cast<uint32_t*>(raw), cols, ld);
     st = check_launch("generate_probability_mask");
     pool_free_raw(raw);               // its next owner runs on this stream, after the two kernels
     if (st == 0 && prefetch_enabled()) {
@@ -1194,17 +1207,23 @@ int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, 
 }
 
 int bship_prob_mask_f32(float* mask, size_t n, double p) {
+    return bship_prob_mask_pitched_f32(mask, static_cast<int64_t>(n), 1, static_cast<int64_t>(n), p);
+}
+
+int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p) {
     BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_DIM(rows >= 0 && cols >= 0 && ld_mask >= cols);
+    const size_t n = static_cast<size_t>(rows) * static_cast<size_t>(cols);
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(mask);
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
-    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_prob_mask_f32: bship_rng_seed() has not been called");
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "%s: bship_rng_seed() has not been called", __func__);
     MaskPrefetch hit;
     bool is_hit = false;
-    int st = mask_begin(mask, n, p, &hit, &is_hit);
+    int st = mask_begin(mask, n, p, &hit, &is_hit, static_cast<size_t>(cols), static_cast<size_t>(ld_mask));
     if (st != 0 || !is_hit) return st;
-    st = bship_d2d(mask, hit.staging, n * sizeof(float));
+    st = bship_copy2d_f32(mask, ld_mask, hit.staging, cols, rows, cols);
     if (st != 0) { mask_abort(hit); return st; }
     return mask_end(hit);
 }

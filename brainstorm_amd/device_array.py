@@ -250,51 +250,64 @@ class PitchedViewError(TypeError):
 
 
 class PitchedDeviceArray(DeviceArray):
-    """A view whose rows (the last axis) are contiguous but lie ``pitch`` elements apart.
+    """A view made of contiguous runs of ``run`` elements that lie ``pitch`` elements apart.
 
     brainstorm lets several layers write side by side into one hub and hands each of
-    them the feature slice ``hub[:, :, a:b]`` (buffer_structure.py:232-245); NumPy
-    addresses such a slice with strides. The kernels of this library work on dense
-    arrays, so a handler created with ``pitched_views=True`` moves a pitched operand
-    into a dense temporary before an operation and moves written operands back
-    (``bship_copy2d_f32``): correct everywhere, two extra passes over the operand.
+    them the feature slice ``hub[:, :, a:b]`` (buffer_structure.py:232-245), reshaped
+    to the layer's own feature shape (an image layer gets ``(T, B, H, W, C)`` whose
+    H*W*C elements are one run); NumPy addresses such a slice with strides. Here the
+    trailing axes whose sizes multiply to ``run`` are dense, and the axes in front of
+    them count the runs ("rows") in C order. A handler created with
+    ``pitched_views=True`` passes such views to kernels that take the pitch, or moves
+    them through a dense temporary where no such kernel exists.
     Reading ``ptr`` raises, so that no code path can mistake the view for a dense array.
     """
 
-    __slots__ = ("_base", "pitch")
+    __slots__ = ("_base", "pitch", "run")
 
-    def __init__(self, base, shape, pitch, owner, handler):
+    def __init__(self, base, shape, pitch, owner, handler, run=None):
         # DeviceArray.__init__ would assign self.ptr, which is read-only here
         self._base = base
         self.shape = shape
         self.size = _prod(shape)
         self.pitch = pitch
+        self.run = shape[-1] if run is None else run
         self._owner = owner
         self._handler = handler
 
     @property
     def ptr(self):
         raise PitchedViewError(
-            "row-pitched view of shape %r (pitch %d) used where a dense array is needed"
-            % (self.shape, self.pitch))
+            "row-pitched view of shape %r (runs of %d, pitch %d) used where a dense array is needed"
+            % (self.shape, self.run, self.pitch))
 
     @property
     def rows(self):
-        return self.size // self.shape[-1] if self.shape[-1] else 0
+        return self.size // self.run if self.run else 0
 
     def _address(self):
         return self._base
 
     def _strides(self):
         strides = [1] * len(self.shape)
-        acc = self.pitch
-        for ax in range(len(self.shape) - 2, -1, -1):
+        acc = 1
+        ax = len(self.shape) - 1
+        while ax >= 0 and acc < self.run:          # the axes of one run: dense
             strides[ax] = acc
             acc *= self.shape[ax]
+            ax -= 1
+        while ax >= 0 and self.shape[ax] == 1 and acc == self.run:
+            strides[ax] = acc                      # size-1 axes next to the run: any stride serves
+            ax -= 1
+        acc = self.pitch
+        for k in range(ax, -1, -1):
+            strides[k] = acc
+            acc *= self.shape[k]
         return strides
 
     def __repr__(self):
-        return "PitchedDeviceArray(shape=%r, pitch=%d, ptr=0x%x)" % (self.shape, self.pitch, self._base)
+        return "PitchedDeviceArray(shape=%r, run=%d, pitch=%d, ptr=0x%x)" % (self.shape, self.run, self.pitch,
+                                                                            self._base)
 
     def __getitem__(self, key):
         return self._getitem_general(key)
@@ -310,10 +323,16 @@ class PitchedDeviceArray(DeviceArray):
             new_shape = tuple(self.size // known if s == -1 else s for s in new_shape)
         if any(s < 0 for s in new_shape) or _prod(new_shape) != self.size:
             raise ValueError("cannot reshape array of size %d into shape %r" % (self.size, new_shape))
-        if not new_shape or new_shape[-1] != self.shape[-1]:
-            raise NotImplementedError("a row-pitched view can only be reshaped over its leading axes "
-                                      "(%r -> %r)" % (self.shape, new_shape))
-        return PitchedDeviceArray(self._base, new_shape, self.pitch, self._owner, self._handler)
+        # some trailing axes of the new shape must make up exactly one run
+        acc = 1
+        for s in reversed(new_shape):
+            if acc >= self.run:
+                break
+            acc *= s
+        if acc != self.run:
+            raise NotImplementedError("a row-pitched view can only be reshaped within its runs of %d elements and "
+                                      "over the axes that count them (%r -> %r)" % (self.run, self.shape, new_shape))
+        return PitchedDeviceArray(self._base, new_shape, self.pitch, self._owner, self._handler, self.run)
 
 
 def _view(parent, offset, shape, strides, key):
@@ -324,12 +343,16 @@ def _view(parent, offset, shape, strides, key):
     owner, handler = parent._owner, parent._handler
     if _prod(shape) == 0 or not shape:
         return DeviceArray(ptr if _prod(shape) else 0, shape, owner, handler)
-    cols = shape[-1]
-    # the leading axes must advance like the rows of one matrix: stride = pitch * rows below
+    # the longest dense suffix of axes is the contiguous run
+    run, k = 1, len(shape)
+    while k > 0 and (shape[k - 1] == 1 or strides[k - 1] == run):
+        run *= shape[k - 1]
+        k -= 1
+    # the axes in front of it must advance like the rows of one matrix: stride = pitch * rows below
     pitch = None
     below = 1
-    ok = cols == 1 or strides[-1] == 1
-    for n, st in zip(reversed(shape[:-1]), reversed(strides[:-1])):
+    ok = True
+    for n, st in zip(reversed(shape[:k]), reversed(strides[:k])):
         if n != 1:
             if pitch is None:
                 if st % below:
@@ -341,10 +364,10 @@ def _view(parent, offset, shape, strides, key):
     if not ok:
         raise NotImplementedError("slicing %r out of shape %r leaves more than a row pitch; "
                                   "such views are not supported" % (key, parent.shape))
-    if pitch is None or pitch == cols:
+    if pitch is None or pitch == run:
         return DeviceArray(ptr, shape, owner, handler)
     if not getattr(handler, "pitched_views", False):
         raise NotImplementedError(
             "slicing %r out of shape %r needs a row pitch; create the handler with "
-            "pitched_views=True to work on such views through dense temporaries" % (key, parent.shape))
-    return PitchedDeviceArray(ptr, shape, pitch, owner, handler)
+            "pitched_views=True to work on such views" % (key, parent.shape))
+    return PitchedDeviceArray(ptr, shape, pitch, owner, handler, run)

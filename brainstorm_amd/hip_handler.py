@@ -127,6 +127,10 @@ class _NoNativePath(Exception):
     """The operands of a call on row-pitched views do not fit the row-pitched kernels."""
 
 
+def _without_self(arguments):
+    return {k: v for k, v in arguments.items() if k != "self"}
+
+
 def _native_pitched_table():
     """Handler operation -> function(handler, arguments) that runs it on row-pitched operands as they
     are (bship_elementwise_pitched_f32, bship_sum_pitched_f32, bship_copy2d_f32)."""
@@ -152,7 +156,17 @@ def _native_pitched_table():
              "softmax_m": lambda h, A: h._pitched_softmax(A["m"], A["out"]),
              "binarize_v": lambda h, A: h._pitched_binarize(A["v"], A["out"]),
              "index_m_by_v": lambda h, A: h._pitched_index(A["m"], A["v"], A["out"]),
-             "sum_t": lambda h, A: h._pitched_sum(A["a"], A["axis"], A["out"])}
+             "sum_t": lambda h, A: h._pitched_sum(A["a"], A["axis"], A["out"]),
+             "generate_probability_mask": lambda h, A: h._pitched_mask(A["mask"], A["probability"]),
+             "broadcast_t": lambda h, A: h._pitched_broadcast(A["a"], A["axis"], A["out"]),
+             "merge_tt": lambda h, A: h._pitched_merge(A["a"], A["b"], A["out"]),
+             "split_add_tt": lambda h, A: h._pitched_split_add(A["x"], A["out_a"], A["out_b"]),
+             "maxpool2d_forward_batch": lambda h, A: h._pitched_maxpool_fwd(**_without_self(A)),
+             "maxpool2d_backward_batch": lambda h, A: h._pitched_maxpool_bwd(**_without_self(A)),
+             "avgpool2d_forward_batch": lambda h, A: h._pitched_avgpool_fwd(**_without_self(A)),
+             "avgpool2d_backward_batch": lambda h, A: h._pitched_avgpool_bwd(**_without_self(A)),
+             "conv2d_forward_batch": lambda h, A: h._pitched_conv_fwd(**_without_self(A)),
+             "conv2d_backward_batch": lambda h, A: h._pitched_conv_bwd(**_without_self(A))}
     for name, op in (("add", ADD), ("subtract", SUB), ("mult", MUL), ("divide", DIV)):
         table[name + "_tt"] = ew(PITCHED_BINARY, op, "out", "a", "b")
         table[name + "_mv"] = mv(PITCHED_BINARY, op)
@@ -245,7 +259,7 @@ class HipHandler(Handler):
             setattr(self, name, functools.partial(self._dense_call, fn, sig, written))
 
     def _copy2d(self, pitched, dense, to_dense):
-        cols = pitched.shape[-1]
+        cols = pitched.run
         args = ((dense.ptr, cols, pitched._base, pitched.pitch) if to_dense
                 else (pitched._base, pitched.pitch, dense.ptr, cols))
         self._call(self._lib.bship_copy2d_f32(*args, pitched.rows, cols))
@@ -255,15 +269,30 @@ class HipHandler(Handler):
     def _as_matrix(self, a, rows, cols):
         """(address, elements from row to row) of `a` read as a (rows, cols) matrix."""
         if type(a) is PitchedDeviceArray:
-            if a.shape[-1] != cols or a.rows != rows:
+            if a.run != cols or a.rows != rows:
                 raise _NoNativePath()
             return a._base, a.pitch
         if a.size != rows * cols:
             raise _NoNativePath()
         return a.ptr, cols
 
+    @staticmethod
+    def _common_run(*arrays):
+        """The row length operands are read with: the run of the pitched ones (the same for all
+        of them), else the last axis of the first."""
+        runs = {x.run for x in arrays if type(x) is PitchedDeviceArray}
+        if len(runs) > 1:
+            raise _NoNativePath()
+        if runs:
+            return runs.pop()
+        first = arrays[0]
+        return first.shape[-1] if first.shape else 1
+
     def _pitched_elementwise(self, family, op, out, a, b, s0, s1, b_is_vector=False):
-        cols = out.shape[-1] if out.shape else 1
+        if b_is_vector:
+            cols = out.shape[-1] if out.shape else 1        # the matrix of a matrix-vector operation
+        else:
+            cols = self._common_run(*[x for x in (out, a, b) if x is not None])
         rows = out.size // cols if cols else 0
         po, ldo = self._as_matrix(out, rows, cols)
         pa, lda = self._as_matrix(a, rows, cols) if a is not None else (None, 0)
@@ -283,7 +312,7 @@ class HipHandler(Handler):
                                                            po, ldo, rows, cols))
 
     def _pitched_copy(self, src, dest):
-        cols = dest.shape[-1] if dest.shape else 1
+        cols = self._common_run(dest, src)
         rows = dest.size // cols if cols else 0
         pd, ldd = self._as_matrix(dest, rows, cols)
         ps, lds = self._as_matrix(src, rows, cols)
@@ -294,7 +323,7 @@ class HipHandler(Handler):
         if v.size != rows:
             raise _NoNativePath()
         if type(v) is PitchedDeviceArray:
-            if v.shape[-1] != 1:
+            if v.run != 1:
                 raise _NoNativePath()
             return v._base, v.pitch
         return v.ptr, 1
@@ -328,9 +357,124 @@ class HipHandler(Handler):
         if (type(a) is not PitchedDeviceArray or type(out) is PitchedDeviceArray
                 or (axis is not None and (a.ndim != 2 or axis not in (0, 1)))):
             raise _NoNativePath()
-        cols = a.shape[-1]
+        cols = a.run
+        if axis is not None and cols != a.shape[-1]:
+            raise _NoNativePath()
         self._call(self._lib.bship_sum_pitched_f32(a._base, a.pitch, out.ptr, a.rows, cols,
                                                    -1 if axis is None else axis))
+
+    # ---- operations on image-pitched and run-pitched views, no dense temporaries ----
+    def _pitched_mask(self, mask, probability):
+        if self.fast_masks or type(mask) is not PitchedDeviceArray:
+            raise _NoNativePath()
+        self.rnd.select()
+        self._call(self._lib.bship_prob_mask_pitched_f32(mask._base, mask.pitch, mask.rows, mask.run, probability))
+
+    @staticmethod
+    def _runs(a):
+        """(address, run, elements from run to run) of any array."""
+        if type(a) is PitchedDeviceArray:
+            return a._base, a.run, a.pitch
+        return a.ptr, max(a.size, 1), max(a.size, 1)
+
+    def _pitched_broadcast(self, a, axis, out):
+        assert (out.shape[:axis] + (1,) + out.shape[axis + 1:]) == a.shape
+        if out.size >= 2 ** 32:
+            raise _NoNativePath()
+        outer = _prod(out.shape[:axis])
+        inner = _prod(out.shape[axis + 1:])
+        pa, ra, lda = self._runs(a)
+        po, ro, ldo = self._runs(out)
+        self._call(self._lib.bship_broadcast_pitched_f32(pa, ra, lda, po, ro, ldo, outer, out.shape[axis], inner))
+
+    def _as_rows(self, a, cols):
+        """`a` as a (rows, cols) matrix view that can be sliced by columns."""
+        if type(a) is PitchedDeviceArray and a.run != cols:
+            raise _NoNativePath()
+        return a.reshape((a.size // cols, cols))
+
+    def _pitched_merge(self, a, b, out):
+        # out[..., :na] = a; out[..., na:] = b   (numpy 221-225): two strided copies
+        na, nb = a.shape[-1], b.shape[-1]
+        assert na + nb == out.shape[-1]
+        if 0 in (na, nb, out.size):
+            raise _NoNativePath()
+        o2 = self._as_rows(out, na + nb)
+        self._pitched_copy(self._as_rows(a, na), o2[:, :na])
+        self._pitched_copy(self._as_rows(b, nb), o2[:, na:])
+
+    def _pitched_split_add(self, x, out_a, out_b):
+        # out_a += x[..., :na]; out_b += x[..., na:]   (numpy 251-256): two strided additions
+        na, nb = out_a.shape[-1], out_b.shape[-1]
+        assert na + nb == x.shape[-1]
+        if 0 in (na, nb, x.size):
+            raise _NoNativePath()
+        x2 = self._as_rows(x, na + nb)
+        oa, ob = self._as_rows(out_a, na), self._as_rows(out_b, nb)
+        self._pitched_elementwise(PITCHED_BINARY, ADD, oa, x2[:, :na], oa, 0.0, 0.0)
+        self._pitched_elementwise(PITCHED_BINARY, ADD, ob, x2[:, na:], ob, 0.0, 0.0)
+
+    @staticmethod
+    def _images(a):
+        """(address, elements from image to image) of an (n, h, w, c) array."""
+        image = _prod(a.shape[1:])
+        if type(a) is PitchedDeviceArray:
+            if a.run != image:
+                raise _NoNativePath()
+            return a._base, a.pitch
+        return a.ptr, image
+
+    def _pitched_maxpool_fwd(self, inputs, window, outputs, padding, stride, argmax, **_):
+        n, h, w, c = inputs.shape
+        (pi, li), (po, lo), (pa, la) = self._images(inputs), self._images(outputs), self._images(argmax)
+        self._call(self._lib.bship_maxpool_fwd_nhwc_pitched_f32(
+            pi, li, po, lo, pa, la, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
+            padding, stride[0], stride[1]))
+
+    def _pitched_maxpool_bwd(self, inputs, window, outputs, padding, stride, argmax, in_deltas, out_deltas, **_):
+        n, h, w, c = inputs.shape
+        (pa, la), (pd, ld), (pi, li) = self._images(argmax), self._images(out_deltas), self._images(in_deltas)
+        self._call(self._lib.bship_maxpool_bwd_nhwc_pitched_f32(
+            pa, la, pd, ld, pi, li, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
+            padding, stride[0], stride[1]))
+
+    def _pitched_avgpool_fwd(self, inputs, window, outputs, padding, stride, **_):
+        n, h, w, c = inputs.shape
+        (pi, li), (po, lo) = self._images(inputs), self._images(outputs)
+        self._call(self._lib.bship_avgpool_fwd_nhwc_pitched_f32(
+            pi, li, po, lo, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
+            padding, stride[0], stride[1]))
+
+    def _pitched_avgpool_bwd(self, inputs, window, outputs, padding, stride, in_deltas, out_deltas, **_):
+        n, h, w, c = inputs.shape
+        (pd, ld), (pi, li) = self._images(out_deltas), self._images(in_deltas)
+        self._call(self._lib.bship_avgpool_bwd_nhwc_pitched_f32(
+            pd, ld, pi, li, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
+            padding, stride[0], stride[1]))
+
+    def _densified(self, a):
+        """A dense copy of a pitched array (for operands of the convolutions' matrix products)."""
+        if type(a) is not PitchedDeviceArray:
+            return a
+        t = self._scratch(a.shape)
+        self._copy2d(a, t, True)
+        return t
+
+    def _pitched_conv_fwd(self, inputs, weights, bias, outputs, padding, stride, **_):
+        # im2col reads the image-pitched inputs as they are; the product's result is a matrix over
+        # all images, so pitched outputs receive it through one dense block and one strided copy
+        weights, bias = self._densified(weights), self._densified(bias)
+        out = self._scratch(outputs.shape) if type(outputs) is PitchedDeviceArray else outputs
+        self._conv_forward(inputs, weights, bias, out, padding, stride)
+        if out is not outputs:
+            self._copy2d(outputs, out, False)
+
+    def _pitched_conv_bwd(self, inputs, weights, padding, stride, in_deltas, out_deltas, weight_deltas,
+                          bias_deltas, **_):
+        if type(weight_deltas) is PitchedDeviceArray or type(bias_deltas) is PitchedDeviceArray:
+            raise _NoNativePath()
+        self._conv_backward(inputs, self._densified(weights), padding, stride, in_deltas,
+                            self._densified(out_deltas), weight_deltas, bias_deltas)
 
     def _dense_call(self, fn, sig, written, *args, **kwargs):
         """Runs fn on row-pitched operands: with the row-pitched kernels where they cover the call,
@@ -655,37 +799,48 @@ class HipHandler(Handler):
         self._gemm(a, b, out, transa, transb, 1.0)
 
     def conv2d_forward_batch(self, inputs, weights, bias, outputs, padding, stride):
+        self._conv_forward(inputs, weights, bias, outputs, padding, stride)
+
+    def _conv_forward(self, inputs, weights, bias, outputs, padding, stride):
         # numpy 149-171, with the per-image loop folded into one im2col and one product:
-        # col (N*oh*ow, kh*kw*C) . W(F, kh*kw*C)^T -> outputs (N*oh*ow, F), then + bias
+        # col (N*oh*ow, kh*kw*C) . W(F, kh*kw*C)^T -> outputs (N*oh*ow, F), then + bias.
+        # inputs may be image-pitched (images a hub's full feature count apart); outputs is dense.
         n, h, w, c = inputs.shape
         f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
         oh, ow = outputs.shape[1], outputs.shape[2]
         kc = kh * kw * c
         rows = n * oh * ow
         col = self._scratch((rows, kc))       # im2col writes every element
-        self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
-                                                   padding, stride[0], stride[1]))
+        p_in, ld_in = self._images(inputs)
+        self._call(self._lib.bship_im2col_nhwc_pitched_f32(p_in, ld_in, col.ptr, n, h, w, c, kh, kw,
+                                                           padding, stride[0], stride[1]))
         # product and bias in one call (the bias goes into the product's epilogue)
         self._call(self._lib.bship_gemm_bias_f32(0, 1, rows, f, kc, col.ptr, kc, weights.ptr, kc,
                                                  bias.ptr, outputs.ptr, f))
 
     def conv2d_backward_batch(self, inputs, weights, padding, stride, in_deltas, out_deltas,
                               weight_deltas, bias_deltas):
-        # numpy 110-147: weight_deltas and bias_deltas are overwritten, in_deltas accumulated
+        self._conv_backward(inputs, weights, padding, stride, in_deltas, out_deltas, weight_deltas, bias_deltas)
+
+    def _conv_backward(self, inputs, weights, padding, stride, in_deltas, out_deltas, weight_deltas, bias_deltas):
+        # numpy 110-147: weight_deltas and bias_deltas are overwritten, in_deltas accumulated.
+        # inputs and in_deltas may be image-pitched; everything else is dense.
         n, h, w, c = inputs.shape
         f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
         oh, ow = out_deltas.shape[1], out_deltas.shape[2]
         kc = kh * kw * c
         rows = n * oh * ow
         col = self._scratch((rows, kc))       # im2col writes every element
-        self._call(self._lib.bship_im2col_nhwc_f32(inputs.ptr, col.ptr, n, h, w, c, kh, kw,
-                                                   padding, stride[0], stride[1]))
+        p_in, ld_in = self._images(inputs)
+        self._call(self._lib.bship_im2col_nhwc_pitched_f32(p_in, ld_in, col.ptr, n, h, w, c, kh, kw,
+                                                           padding, stride[0], stride[1]))
         dy = out_deltas.reshape((rows, f))
         self._gemm(dy, col, weight_deltas.reshape((f, kc)), True, False, 0.0)
         self._call(self._lib.bship_sum_f32(dy.ptr, bias_deltas.ptr, rows, f, 0))
         self._gemm(dy, weights.reshape((f, kc)), col, False, False, 0.0)
-        self._call(self._lib.bship_col2im_nhwc_f32(col.ptr, in_deltas.ptr, n, h, w, c, kh, kw,
-                                                   padding, stride[0], stride[1]))
+        p_din, ld_din = self._images(in_deltas)
+        self._call(self._lib.bship_col2im_nhwc_pitched_f32(col.ptr, p_din, ld_din, n, h, w, c, kh, kw,
+                                                           padding, stride[0], stride[1]))
 
     # --------------------------------------------------------------- pooling
     def maxpool2d_forward_batch(self, inputs, window, outputs, padding, stride, argmax):

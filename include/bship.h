@@ -197,6 +197,13 @@ int bship_mv_f32(int op, const float* m, const float* v, float* out,
 int bship_broadcast_f32(const float* a, float* out, int64_t outer,
                         int64_t bdim, int64_t inner);
 
+/* broadcast_t between arrays made of contiguous runs (feature slices of wider hubs):
+ * dense element k of an array lies at (k / run) * ld + k % run. outer * inner must be a
+ * whole number of runs of a, the whole output a whole number of runs of out. At most
+ * 2^32 - 1 output elements. */
+int bship_broadcast_pitched_f32(const float* a, int64_t a_run, int64_t ld_a, float* out,
+                                int64_t out_run, int64_t ld_out, int64_t outer, int64_t bdim,
+                                int64_t inner);
 /* merge_tt (numpy 221-225, pycuda 317-323): out[:, :na] = a, out[:, na:] = b */
 int bship_merge_f32(const float* a, const float* b, float* out, int64_t rows,
                     int64_t na, int64_t nb);
@@ -307,6 +314,10 @@ int bship_rng_seed(uint32_t seed);
 /* generate_probability_mask (numpy 199-200): mask = (uniform[0,1) < p), drawing
  * the same 53-bit doubles, in the same order, as RandomState.uniform. */
 int bship_prob_mask_f32(float* mask, size_t n, double p);
+/* The same mask, written to a (rows, cols) matrix whose rows lie ld_mask elements apart
+ * (a feature slice of a wider hub): element i of the draw goes to row i / cols, column
+ * i % cols, exactly what `mask[:] = (uniform(size=shape) < p)` does on a strided view. */
+int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p);
 /* fill_gaussian (numpy 193-194): out = std*standard_normal + mean with the
  * legacy polar method of RandomState.standard_normal. Blocks. */
 int bship_fill_gaussian_f32(float* out, size_t n, double mean, double std);
@@ -364,6 +375,38 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
                                int64_t n, int h, int w, int c, int out_h,
                                int out_w, int pool_h, int pool_w, int pad,
                                int stride_h, int stride_w);
+
+/* The image operations on image-pitched arrays. A layer whose input or output is
+ * a feature slice of a hub that several layers share (buffer_structure.py
+ * 232-245) sees images that are contiguous (h*w*c elements) but lie a pitch of
+ * the hub's full feature count apart; NumpyHandler's _cpuop routines take such
+ * strided views as they are. Every *_pitch is the number of elements from one
+ * image to the next in that array (at least the image size; the image size
+ * itself gives the dense functions above). col stays dense. */
+int bship_im2col_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* col, int64_t n,
+                                  int h, int w, int c, int kh, int kw, int pad,
+                                  int stride_h, int stride_w);
+int bship_col2im_nhwc_pitched_f32(const float* col, float* in_deltas, int64_t in_deltas_pitch,
+                                  int64_t n, int h, int w, int c, int kh, int kw, int pad,
+                                  int stride_h, int stride_w);
+int bship_maxpool_fwd_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* out,
+                                       int64_t out_pitch, float* argmax, int64_t argmax_pitch,
+                                       int64_t n, int h, int w, int c, int out_h, int out_w,
+                                       int pool_h, int pool_w, int pad, int stride_h,
+                                       int stride_w);
+int bship_maxpool_bwd_nhwc_pitched_f32(const float* argmax, int64_t argmax_pitch,
+                                       const float* out_deltas, int64_t out_deltas_pitch,
+                                       float* in_deltas, int64_t in_deltas_pitch, int64_t n,
+                                       int h, int w, int c, int out_h, int out_w, int pool_h,
+                                       int pool_w, int pad, int stride_h, int stride_w);
+int bship_avgpool_fwd_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* out,
+                                       int64_t out_pitch, int64_t n, int h, int w, int c,
+                                       int out_h, int out_w, int pool_h, int pool_w, int pad,
+                                       int stride_h, int stride_w);
+int bship_avgpool_bwd_nhwc_pitched_f32(const float* out_deltas, int64_t out_deltas_pitch,
+                                       float* in_deltas, int64_t in_deltas_pitch, int64_t n,
+                                       int h, int w, int c, int out_h, int out_w, int pool_h,
+                                       int pool_w, int pad, int stride_h, int stride_w);
 
 /* --------------------------- fused layer steps --------------------------- */
 

@@ -152,17 +152,23 @@ def test_random_index_chains_match_numpy(data):
                 dev[key]
             return
         dense = want.size == 0 or want.ndim == 0 or want.flags["C_CONTIGUOUS"]
-        # a row-pitched view: last axis contiguous (or of length 1), leading axes like the rows of one matrix
+        # a row-pitched view: the longest dense suffix of axes is one run, the axes in front of it
+        # advance like the rows of one matrix
         representable = dense
-        if not dense and pitched and (want.shape[-1] == 1 or want.strides[-1] == 4):
+        if not dense and pitched:
+            strides = [s // 4 for s in want.strides]
+            run, k = 1, want.ndim
+            while k > 0 and (want.shape[k - 1] == 1 or strides[k - 1] == run):
+                run *= want.shape[k - 1]
+                k -= 1
             pitch, below, ok = None, 1, True
-            for n, s in zip(reversed(want.shape[:-1]), reversed(want.strides[:-1])):
+            for n, s in zip(reversed(want.shape[:k]), reversed(strides[:k])):
                 if n != 1:
                     if pitch is None:
-                        ok = ok and (s // 4) % below == 0
-                        pitch = (s // 4) // below
+                        ok = ok and s % below == 0
+                        pitch = s // below
                     else:
-                        ok = ok and s // 4 == pitch * below
+                        ok = ok and s == pitch * below
                 below *= n
             representable = ok
         if not representable:
@@ -177,7 +183,40 @@ def test_random_index_chains_match_numpy(data):
             if dense:
                 assert type(got) is DeviceArray
             else:
-                assert got.pitch == [s // 4 for n, s in zip(want.shape[:-1], want.strides[:-1]) if n != 1][-1]
+                assert got.pitch == pitch and got.run == run and got.rows * got.run == got.size
+                # element strides agree with NumPy's wherever an axis has more than one entry
+                for n, mine, theirs in zip(want.shape, got._strides(), want.strides):
+                    assert n == 1 or mine == theirs // 4
         dev, host = got, want
         if type(dev) is not DeviceArray:
             return                                   # chains continue on dense views only here
+
+
+def test_feature_slice_of_a_hub_reshaped_to_images():
+    # buffer_structure.py:232-245: hub[:, :, a:b] of a (T, B, F) hub, reshaped to the layer's own
+    # feature shape; the H*W*C elements of one image are one contiguous run
+    T, B, F = 3, 4, 50
+    host = np.arange(T * B * F, dtype=np.float32).reshape(T, B, F)
+    dev = DeviceArray(BASE_PTR, (T, B, F), None, _PitchedHandler())
+    sl = dev[:, :, 6:30]
+    assert (sl.shape, sl.run, sl.pitch, sl.rows) == ((T, B, 24), 24, F, T * B)
+    img = sl.reshape((T, B, 2, 3, 4))
+    want = host[:, :, 6:30].reshape(T, B, 2, 3, 4)
+    assert (img.shape, img.run, img.pitch, img.rows) == ((T, B, 2, 3, 4), 24, F, T * B)
+    assert img._strides() == [s // 4 for s in want.strides]
+    flat = img.reshape((T * B, 2, 3, 4))                       # flatten_time
+    assert flat.shape == (T * B, 2, 3, 4) and flat.run == 24 and flat.rows == T * B
+    assert img.reshape((T * B, 24)).shape == (T * B, 24)
+    one = img[1]                                                # a time step: still pitched
+    assert one.shape == (B, 2, 3, 4) and one.run == 24 and one.pitch == F
+    assert (one._address() - BASE_PTR) // 4 == int(want[1, 0, 0, 0, 0])
+    row = img[1, 2]                                             # one image: dense
+    assert type(row) is DeviceArray and row.shape == (2, 3, 4)
+    assert (row.ptr - BASE_PTR) // 4 == int(want[1, 2, 0, 0, 0])
+    with pytest.raises(NotImplementedError):
+        img[:, :, :, :, 1:3]                                    # a channel slice of the images: no single pitch
+    with pytest.raises(NotImplementedError):
+        sl.reshape((T, B, 4, 6))[:, :, 1:3, 1:3]
+    for bad in ((T * B * 2, 12), (T, B * 24), (24, T * B)):    # would split or merge runs across the pitch
+        with pytest.raises(NotImplementedError):
+            sl.reshape(bad)

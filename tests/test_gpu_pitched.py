@@ -253,3 +253,160 @@ def test_two_layers_writing_one_hub(php):
     got, want = run(php), run(NumpyRefHandler(F32, seed=0))
     for g, w in zip(got, want):
         np.testing.assert_allclose(g, w, rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------------ images, masks, broadcast, merge / split
+class _NoTemporaries:
+    """Fails the test if the handler makes a dense temporary (allocate or _scratch) inside the block."""
+
+    def __init__(self, handler, allowed=0):
+        self.h, self.allowed, self.made = handler, allowed, []
+
+    def __enter__(self):
+        self.real = (self.h.allocate, self.h._scratch)
+        self.h.allocate = lambda shape: self.made.append(shape) or self.real[0](shape)
+        self.h._scratch = lambda shape: self.made.append(shape) or self.real[1](shape)
+        return self
+
+    def __exit__(self, *exc):
+        self.h.allocate, self.h._scratch = self.real
+        if exc[0] is None:
+            assert len(self.made) <= self.allowed, self.made
+
+
+def _hub_pair(php, rng, n, width):
+    host = rng.standard_normal((n, width)).astype(F32)
+    return host, php.create_from_numpy(host)
+
+
+@pytest.mark.parametrize("n,h,w,c,win,pad,stride", [(5, 9, 9, 4, 3, 0, 2), (3, 8, 8, 3, 2, 1, 2), (4, 7, 6, 8, 3, 1, 1),
+                                                    (2, 32, 32, 32, 3, 0, 2)])
+def test_pooling_on_image_slices_of_hubs(php, n, h, w, c, win, pad, stride):
+    # inputs, outputs, argmax and both delta arrays are feature slices of wider hubs, reshaped to
+    # images (buffer_structure.py:232-245): same bits as the oracle, nothing else in the hubs changes
+    rng = np.random.RandomState(31)
+    ref = NumpyRefHandler(F32, seed=0)
+    oh, ow = (h + 2 * pad - win) // stride + 1, (w + 2 * pad - win) // stride + 1
+    fi, fo = h * w * c, oh * ow * c
+    off_i, off_o = 5, 3
+    hubs = {k: _hub_pair(php, rng, n, width) for k, width in
+            (("in", fi + 11), ("out", fo + 7), ("arg", fo + 9), ("din", fi + 11), ("dout", fo + 7))}
+
+    def views(which):
+        sl = {"in": (off_i, fi, (n, h, w, c)), "din": (off_i, fi, (n, h, w, c)), "out": (off_o, fo, (n, oh, ow, c)),
+              "arg": (off_o, fo, (n, oh, ow, c)), "dout": (off_o, fo, (n, oh, ow, c))}
+        return {k: hubs[k][which][:, a:a + f].reshape(shape) for k, (a, f, shape) in sl.items()}
+
+    dev, host = views(1), views(0)
+    assert all(type(v) is PitchedDeviceArray for v in dev.values())
+    # the oracle's C routines take contiguous arrays: run them on copies and put the results back
+    x, out, arg = (np.ascontiguousarray(host[k]) for k in ("in", "out", "arg"))
+    din, dout = np.ascontiguousarray(host["din"]), np.ascontiguousarray(host["dout"])
+    ref.maxpool2d_forward_batch(x, (win, win), out, pad, (stride, stride), arg)
+    ref.maxpool2d_backward_batch(x, (win, win), out, pad, (stride, stride), arg, din, dout)
+    out_avg = out.copy()
+    ref.avgpool2d_forward_batch(x, (win, win), out_avg, pad, (stride, stride))
+    din_avg = din.copy()
+    ref.avgpool2d_backward_batch(x, (win, win), out_avg, pad, (stride, stride), din_avg, dout)
+    with _NoTemporaries(php):
+        php.maxpool2d_forward_batch(dev["in"], (win, win), dev["out"], pad, (stride, stride), dev["arg"])
+        php.maxpool2d_backward_batch(dev["in"], (win, win), dev["out"], pad, (stride, stride), dev["arg"],
+                                     dev["din"], dev["dout"])
+    want = {k: hubs[k][0].copy() for k in hubs}
+    want["out"][:, off_o:off_o + fo] = out.reshape(n, fo)
+    want["arg"][:, off_o:off_o + fo] = arg.reshape(n, fo)
+    want["din"][:, off_i:off_i + fi] = din.reshape(n, fi)
+    for k in hubs:
+        assert_bit_equal(hubs[k][1].get(), want[k], "max pooling, hub %s" % k)
+    with _NoTemporaries(php):
+        php.avgpool2d_forward_batch(dev["in"], (win, win), dev["out"], pad, (stride, stride))
+        php.avgpool2d_backward_batch(dev["in"], (win, win), dev["out"], pad, (stride, stride), dev["din"], dev["dout"])
+    want["out"][:, off_o:off_o + fo] = out_avg.reshape(n, fo)
+    want["din"][:, off_i:off_i + fi] = din_avg.reshape(n, fi)
+    for k in hubs:
+        assert_bit_equal(hubs[k][1].get(), want[k], "average pooling, hub %s" % k)
+
+
+@pytest.mark.parametrize("n,h,w,c,f,k,pad", [(4, 8, 8, 3, 5, 3, 1), (3, 6, 7, 8, 4, 5, 2), (2, 32, 32, 3, 8, 5, 2)])
+def test_convolution_on_image_slices_of_hubs(php, n, h, w, c, f, k, pad):
+    rng = np.random.RandomState(32)
+    ref = NumpyRefHandler(F32, seed=0)
+    oh, ow = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    fi, fo = h * w * c, oh * ow * f
+    hubs = {key: _hub_pair(php, rng, n, width) for key, width in
+            (("in", fi + 6), ("out", fo + 10), ("din", fi + 6), ("dout", fo + 10))}
+    wts, bias = rng.standard_normal((f, k, k, c)).astype(F32), rng.standard_normal((f,)).astype(F32)
+    dev = {"in": hubs["in"][1][:, 2:2 + fi].reshape((n, h, w, c)), "din": hubs["din"][1][:, 2:2 + fi].reshape((n, h, w, c)),
+           "out": hubs["out"][1][:, 7:7 + fo].reshape((n, oh, ow, f)), "dout": hubs["dout"][1][:, 7:7 + fo].reshape((n, oh, ow, f))}
+    x = np.ascontiguousarray(hubs["in"][0][:, 2:2 + fi].reshape(n, h, w, c))
+    din = np.ascontiguousarray(hubs["din"][0][:, 2:2 + fi].reshape(n, h, w, c))
+    dout = np.ascontiguousarray(hubs["dout"][0][:, 7:7 + fo].reshape(n, oh, ow, f))
+    out = np.zeros((n, oh, ow, f), F32)
+    dw, db = np.zeros_like(wts), np.zeros_like(bias)
+    ref.conv2d_forward_batch(x, wts, bias, out, pad, (1, 1))
+    ref.conv2d_backward_batch(x, wts, pad, (1, 1), din, dout, dw, db)
+    wd, bd = php.create_from_numpy(wts), php.create_from_numpy(bias)
+    dwd, dbd = php.allocate(wts.shape), php.allocate(bias.shape)
+    php.conv2d_forward_batch(dev["in"], wd, bd, dev["out"], pad, (1, 1))
+    php.conv2d_backward_batch(dev["in"], wd, pad, (1, 1), dev["din"], dev["dout"], dwd, dbd)
+    want = {key: hubs[key][0].copy() for key in hubs}
+    want["out"][:, 7:7 + fo] = out.reshape(n, fo)
+    want["din"][:, 2:2 + fi] = din.reshape(n, fi)
+    scale = np.sqrt(k * k * c)
+    for key in hubs:
+        got = hubs[key][1].get()
+        assert np.max(np.abs(got - want[key])) <= 1e-5 * scale * max(1.0, np.max(np.abs(want[key]))), key
+    untouched = np.ones(fo + 10, bool)
+    untouched[7:7 + fo] = False
+    assert_bit_equal(hubs["out"][1].get()[:, untouched], hubs["out"][0][:, untouched], "outside the output slice")
+    assert_bit_equal(hubs["in"][1].get(), hubs["in"][0], "inputs")
+    np.testing.assert_allclose(dwd.get(), dw, rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(dbd.get(), db, rtol=1e-4, atol=1e-4)
+
+
+def test_masks_broadcast_merge_split_on_slices(php):
+    rng = np.random.RandomState(33)
+    ref = NumpyRefHandler(F32, seed=9)
+    php.rnd.seed(9)
+    t, b, width = 3, 7, 61
+    hub, dhub = rng.standard_normal((t, b, width)).astype(F32), None
+    dhub = php.create_from_numpy(hub)
+    want = hub.copy()
+    # masks: a 3-d feature slice, the same slice seen as images, and again (the look-ahead sees a pattern)
+    for _ in range(4):
+        with _NoTemporaries(php):
+            php.generate_probability_mask(dhub[:, :, 4:28], 0.7)
+            php.generate_probability_mask(dhub[:, :, 30:54].reshape((t, b, 2, 3, 4)), 0.4)
+        ref.generate_probability_mask(want[:, :, 4:28], 0.7)
+        ref.generate_probability_mask(want[:, :, 30:54].reshape(t, b, 2, 3, 4), 0.4)
+        assert_bit_equal(dhub.get(), want, "masks in slices")
+    # broadcast_t: over the batch axis into a slice, over the last axis, and from a pitched source
+    src = rng.standard_normal((t, 1, 24)).astype(F32)
+    col = rng.standard_normal((t, b, 1)).astype(F32)
+    dsrc, dcol = php.create_from_numpy(src), php.create_from_numpy(col)
+    with _NoTemporaries(php):
+        php.broadcast_t(dsrc, 1, dhub[:, :, 4:28])
+        php.broadcast_t(dcol, 2, dhub[:, :, 30:54])
+        php.broadcast_t(dhub[:, :, 57:58], 2, dhub[:, :, 0:3])
+    ref.broadcast_t(src, 1, want[:, :, 4:28])
+    ref.broadcast_t(col, 2, want[:, :, 30:54])
+    ref.broadcast_t(want[:, :, 57:58].copy(), 2, want[:, :, 0:3])
+    assert_bit_equal(dhub.get(), want, "broadcast_t into slices")
+    # merge_tt and split_add_tt with every operand a slice
+    with _NoTemporaries(php):
+        php.merge_tt(dhub[:, :, 4:14], dhub[:, :, 30:37], dhub[:, :, 40:57])
+        php.split_add_tt(dhub[:, :, 40:57], dhub[:, :, 4:14], dhub[:, :, 20:27])
+    ref.merge_tt(want[:, :, 4:14], want[:, :, 30:37], want[:, :, 40:57])
+    ref.split_add_tt(want[:, :, 40:57], want[:, :, 4:14], want[:, :, 20:27])
+    assert_bit_equal(dhub.get(), want, "merge_tt / split_add_tt on slices")
+    # dense operands mixed with slices
+    a, bb = rng.standard_normal((t, b, 10)).astype(F32), rng.standard_normal((t, b, 7)).astype(F32)
+    da, db = php.create_from_numpy(a), php.create_from_numpy(bb)
+    with _NoTemporaries(php):
+        php.merge_tt(da, db, dhub[:, :, 40:57])
+        php.split_add_tt(dhub[:, :, 40:57], da, db)
+    ref.merge_tt(a, bb, want[:, :, 40:57])
+    ref.split_add_tt(want[:, :, 40:57], a, bb)
+    assert_bit_equal(dhub.get(), want, "merge_tt with dense sources")
+    assert_bit_equal(da.get(), a, "split_add_tt into a dense array")
+    assert_bit_equal(db.get(), bb, "split_add_tt into a dense array")
