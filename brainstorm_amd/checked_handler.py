@@ -104,6 +104,11 @@ def _matmul_shapes(op, a):
         _fail(op, "out has shape %r, expected %r" % (tuple(a["out"].shape), (a1, b2)))
 
 
+def _broadcastable(src, dest):
+    """NumPy's rule for np.copyto(dest, src): trailing axes agree or are 1 in src."""
+    return len(src) <= len(dest) and all(s in (1, d) for s, d in zip(reversed(src), reversed(dest)))
+
+
 def _label_count(a):
     """Number of classes the labels of binarize_v / index_m_by_v select from."""
     return a["m"].shape[1] if "m" in a else a["out"].shape[1]
@@ -122,7 +127,7 @@ _DERIV = [same_shape("x", "y", "dy", "dx")]          # x may be None (the handle
 # every parameter that is not named in NON_ARRAY must be an array of the handler's array type.
 CONTRACTS = {
     "allocate": [shape_tuple("shape")], "ones": [shape_tuple("shape")], "zeros": [shape_tuple("shape")],
-    "copy_to": [same_shape("src", "dest")],
+    "copy_to": [where(lambda a: _broadcastable(a["src"].shape, a["dest"].shape), "src does not broadcast into dest")],
     "copy_to_if": [same_shape("src", "dest", "cond")],
     "create_from_numpy": [where(lambda a: isinstance(a["arr"], np.ndarray), "arr must be a numpy array")],
     "fill": [scalar("val")],

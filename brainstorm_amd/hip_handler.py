@@ -586,9 +586,26 @@ class HipHandler(Handler):
     # --------------------------------------------------------- copy and fill
     def copy_to(self, src, dest):
         # numpy 47-52 / pycuda 83-85
-        if src.size != dest.size:
-            raise ValueError("copy_to: size mismatch %r -> %r" % (src.shape, dest.shape))
-        self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
+        # np.copyto broadcasts src to dest's shape: a scalar, a row for every row, a column for every
+        # column ... Served when the axes that repeat are neighbours (one broadcast_t), which covers those.
+        if src.shape == dest.shape or (src.size == dest.size and src.ndim <= 1):
+            self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
+            return
+        if src.ndim > dest.ndim:
+            raise ValueError("copy_to: could not broadcast %r into %r" % (src.shape, dest.shape))
+        padded = (1,) * (dest.ndim - src.ndim) + tuple(src.shape)
+        repeat = [k for k, (s, d) in enumerate(zip(padded, dest.shape)) if s != d]
+        if any(padded[k] != 1 for k in repeat):
+            raise ValueError("copy_to: could not broadcast %r into %r" % (src.shape, dest.shape))
+        if dest.size == 0:
+            return
+        if repeat[-1] - repeat[0] + 1 != len(repeat):
+            raise NotImplementedError("copy_to: broadcasting %r into %r repeats axes that are not neighbours"
+                                      % (src.shape, dest.shape))
+        outer = _prod(dest.shape[:repeat[0]])
+        inner = _prod(dest.shape[repeat[-1] + 1:])
+        times = _prod(dest.shape[repeat[0]:repeat[-1] + 1])
+        self._call(self._lib.bship_broadcast_f32(src.ptr, dest.ptr, outer, times, inner))
 
     def copy_to_if(self, src, dest, cond):
         self._call(self._lib.bship_cond_f32(COPY_IF, src.ptr, 0.0, dest.ptr, cond.ptr, dest.size))
@@ -737,13 +754,33 @@ class HipHandler(Handler):
     def sum_t(self, a, axis, out):
         # numpy 268-273; the shape of `out` decides keepdims, which does not change the layout
         if axis is None or a.ndim <= 1:
-            rows, cols, ax = 1, a.size, -1
-        elif a.ndim == 2 and axis in (0, 1):
-            rows, cols = a.shape
-            ax = axis
+            self._call(self._lib.bship_sum_f32(a.ptr, out.ptr, 1, a.size, -1))
+            return
+        if not isinstance(axis, (int, np.integer)):
+            raise NotImplementedError("sum_t over axes %r" % (axis,))
+        axis = int(axis) + (a.ndim if axis < 0 else 0)
+        if not 0 <= axis < a.ndim:
+            raise ValueError("sum_t: axis %d out of range for a %d-d array" % (axis, a.ndim))
+        # any array is (outer, length of the axis, inner)
+        outer, length, inner = _prod(a.shape[:axis]), a.shape[axis], _prod(a.shape[axis + 1:])
+        lib = self._lib
+        if outer * inner == 0:
+            return
+        if inner == 1:
+            self._call(lib.bship_sum_f32(a.ptr, out.ptr, outer, length, 1))
+        elif outer == 1:
+            self._call(lib.bship_sum_f32(a.ptr, out.ptr, length, inner, 0))
+        elif outer <= length:
+            # a column sum per outer index: slab o is a contiguous (length, inner) matrix
+            for o in range(outer):
+                self._call(lib.bship_sum_f32(a.ptr + o * length * inner * 4, out.ptr + o * inner * 4, length, inner, 0))
         else:
-            raise NotImplementedError("sum_t over axis %r of a %d-d array" % (axis, a.ndim))
-        self._call(self._lib.bship_sum_f32(a.ptr, out.ptr, rows, cols, ax))
+            # entry k of the axis is an (outer, inner) matrix with row pitch length * inner: add them up in order
+            pitch = length * inner
+            self._call(lib.bship_copy2d_f32(out.ptr, inner, a.ptr, pitch, outer, inner))
+            for k in range(1, length):
+                self._call(lib.bship_elementwise_pitched_f32(PITCHED_BINARY, ADD, 0.0, 0.0, out.ptr, inner, 1,
+                                                             a.ptr + k * inner * 4, pitch, 1, out.ptr, inner, outer, inner))
 
     def softmax_m(self, m, out):
         n_cols = m.shape[-1]

@@ -49,7 +49,7 @@ def test_bad_arguments_return_errors_not_crashes(hip):
     with pytest.raises(ValueError):
         hip.add_mv(hip.allocate((2, 3)), hip.allocate((1, 4)), hip.allocate((2, 3)))
     with pytest.raises(NotImplementedError):
-        hip.sum_t(hip.allocate((2, 3, 4)), 1, hip.allocate((2, 4)))
+        hip.sum_t(hip.allocate((2, 3, 4)), (0, 1), hip.allocate((4,)))
     # the handler is still usable afterwards
     hip.fill(x, 3.0)
     assert np.array_equal(x.get(), np.full(8, 3.0, np.float32))

@@ -401,6 +401,37 @@ def test_sum_t(hip, ref):
     _check_sum(hip, ref, rand(rng, ((1 << 22) + 13,)), None, ())
 
 
+def test_sum_t_over_an_axis_of_arrays_with_more_axes(hip, ref):
+    # NumpyHandler takes whatever np.sum takes (numpy_handler.py:268-273): any axis of any array,
+    # negative axes, out with or without the summed axis kept
+    rng = np.random.RandomState(18)
+    for shape in ((2, 3, 4), (5, 300, 7), (300, 5, 260), (3, 4, 5, 6), (1, 2049, 3), (4, 1, 9), (40, 3, 1)):
+        a = rand(rng, shape)
+        for axis in list(range(len(shape))) + [-1, -2]:
+            want = np.sum(a.astype(np.float64), axis=axis)
+            for out_shape in (want.shape, np.sum(a, axis=axis, keepdims=True).shape):
+                _check_sum(hip, ref, a, axis, out_shape)
+    with pytest.raises(ValueError):
+        hip.sum_t(hip.allocate((2, 3, 4)), 3, hip.allocate((2, 3)))
+
+
+def test_copy_to_broadcasts_like_numpy(hip, ref):
+    # np.copyto(dest, src) broadcasts src (numpy_handler.py:47-52)
+    rng = np.random.RandomState(19)
+    cases = [((1, 7), (5, 7)), ((7,), (5, 7)), ((5, 1), (5, 7)), ((1,), (5, 7)), ((), (3, 4, 5)), ((1, 1), (3, 4)),
+             ((3, 1, 1, 6), (3, 4, 5, 6)), ((4, 260), (3, 4, 260)), ((2, 1, 1028), (2, 300, 1028)), ((5, 7), (5, 7)),
+             ((35,), (35,))]
+    for src_shape, dest_shape in cases:
+        operation_check(hip, ref, "copy_to", (rand(rng, src_shape), rand(rng, dest_shape)))
+    for src_shape, dest_shape in [((3,), (5, 7)), ((2, 7), (5, 7)), ((5, 7, 1), (5, 7))]:
+        with pytest.raises(ValueError):
+            hip.copy_to(hip.allocate(src_shape), hip.allocate(dest_shape))
+        with pytest.raises(ValueError):
+            ref.copy_to(np.zeros(src_shape, F32), np.zeros(dest_shape, F32))
+    with pytest.raises(NotImplementedError):
+        hip.copy_to(hip.allocate((1, 4, 1)), hip.allocate((3, 4, 5)))      # repeats two axes that are not neighbours
+
+
 def test_sum_t_is_deterministic(hip):
     rng = np.random.RandomState(18)
     a = hip.create_from_numpy(rand(rng, (2048, 4096)))
