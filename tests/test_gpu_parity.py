@@ -895,7 +895,9 @@ def test_im2col_col2im_exact(hip, ref):
 BAND_CASES = [(260, 40, 32, 3, 5, 5, 2, (1, 1)), (210, 40, 256, 3, 3, 3, 1, (2, 2)), (1030, 28, 28, 1, 5, 5, 2, (1, 1)),
               (9, 40, 32, 3, 5, 5, 2, (1, 1)), (130, 17, 12, 8, 3, 3, 0, (1, 1)), (70, 30, 30, 6, 3, 3, 1, (3, 1)),
               (300, 19, 16, 12, 2, 2, 0, (2, 2)), (33, 15, 15, 32, 5, 5, 2, (1, 1)), (40, 11, 9, 5, 3, 3, 1, (1, 1)),
-              (20, 10, 10, 3, 3, 3, 1, (1, 1)), (20, 12, 10, 3, 3, 3, 1, (2, 1))]
+              (20, 10, 10, 3, 3, 3, 1, (1, 1)), (20, 12, 10, 3, 3, 3, 1, (2, 1)),
+              # 4 output pixels = kh*kw*c stores: 245 of them (one lane each), 294 (too many: general kernel), 2 groups a row
+              (12, 20, 16, 5, 7, 7, 3, (1, 1)), (12, 20, 16, 6, 7, 7, 3, (1, 1)), (50, 9, 8, 3, 2, 3, 1, (1, 2))]
 
 
 def test_im2col_col2im_banded_exact(hip, ref):
