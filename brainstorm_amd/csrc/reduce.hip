@@ -307,6 +307,13 @@ static void launch_softmax_threads(bool vec, bool al, int per, dim3 grid, const 
 }
 
 constexpr int kWideBlock = 1024;
+// Rows of up to this many accesses per lane are held by 256 lanes (8 workgroups fit a compute unit and
+// overlap each other's load, arithmetic and store phases); measured at 8192 columns: 8 accesses x 256
+// lanes reach 0.78 of peak, 2 x 1024 lanes 0.76. At 16384 columns 16 x 256 lanes fall to 0.67 against
+// 0.70-0.72 for 4 x 1024, so longer rows take the wide workgroups.
+#ifndef BSHIP_SM_NARROW_MAX
+#define BSHIP_SM_NARROW_MAX 8
+#endif
 
 static int launch_softmax(const float* m, float* out, int64_t M, int64_t N, int64_t ldm, int64_t ldo) {
     const bool vec = (N % 4 == 0);
@@ -322,7 +329,7 @@ static int launch_softmax(const float* m, float* out, int64_t M, int64_t N, int6
         // a wavefront per row, 4 rows per workgroup
         launch_softmax_threads<kBlock, kWave>(vec, al, per_for(kWave),
                                               dim3(static_cast<unsigned>(ceil_div(M, kBlock / kWave))), m, out, M, N, ldm, ldo);
-    } else if (NW <= static_cast<int64_t>(kBlock) * 4) {
+    } else if (NW <= static_cast<int64_t>(kBlock) * BSHIP_SM_NARROW_MAX) {
         launch_softmax_threads<kBlock, kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo);
     } else if (NW <= static_cast<int64_t>(kWideBlock) * 16) {
         launch_softmax_threads<kWideBlock, kWideBlock>(vec, al, per_for(kWideBlock),
