@@ -23,6 +23,8 @@ COPY_IF, FILL_IF, ADD_IF = 0, 1, 2
  PITCHED_FILL) = range(8)
 
 ERR_OUT_OF_MEMORY = -5
+ERR_UNSUPPORTED = -6
+ERR_TIMEOUT = -9
 
 _P = c_void_p          # device pointers travel as plain integers
 _I64 = c_int64
@@ -103,6 +105,7 @@ SIGNATURES = {
     "bship_lstm_bwd_step_f32": [c_int, _I64, _I64] + [_P] * 24,
     "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,
     "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
+    "bship_lstm_fwd_sequence_f32": [c_int, _I64, _I64, _I64] + [_P] * 19,
     "bship_softmax_ce_fwd_f32": [_P, _P, _P, _P, _I64, _I64],
     "bship_softmax_ce_bwd_f32": [_P, _P, _P, _P, _P, _I64, _I64],
     "bship_momentum_update_f32": [c_float, c_float, _P, _P, _P, c_size_t],

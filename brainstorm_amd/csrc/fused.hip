@@ -9,21 +9,9 @@
 #include "colsum.h"
 #include "common.h"
 #include "functors.h"
+#include "lstm_cell.h"
 
 namespace bship {
-
-enum { kActSigmoid = 0, kActTanh = 1, kActRel = 2, kActLinear = 3, kActEl = 4 };
-
-// act_func[...] (base_handler.py:57-63); 'linear' is copy_to
-__device__ __forceinline__ float act_forward(int act, float x) {
-    switch (act) {
-        case kActSigmoid: return SigmoidOp{}.apply(x, 0.0f, 0.0f);
-        case kActTanh:    return TanhOp{}.apply(x, 0.0f, 0.0f);
-        case kActRel:     return RelOp{}.apply(x, 0.0f, 0.0f);
-        case kActEl:      return ElOp{}.apply(x, 0.0f, 0.0f);
-        default:          return x;
-    }
-}
 
 // act_func_deriv[...](x, y, dy, dx) (base_handler.py:65-71); 'linear' copies dy
 __device__ __forceinline__ float act_backward(int act, float y, float dy) {
@@ -74,23 +62,14 @@ __global__ __launch_bounds__(kBlock) void lstm_fwd_step_kernel(LstmFwdArgs a, in
         fa = fa + ldg(r + 2 * static_cast<int64_t>(n));
         oa = oa + ldg(r + 3 * static_cast<int64_t>(n));
     }
-    za = za + a.bz[j];
-    const float zb = act_forward(act, za);
-    { const float p = c_prev * a.pi[j]; ia = ia + p; }
-    ia = ia + a.bi[j];
-    const float ib = SigmoidOp{}.apply(ia, 0.0f, 0.0f);
-    { const float p = c_prev * a.pf[j]; fa = fa + p; }
-    fa = fa + a.bf[j];
-    const float fb = SigmoidOp{}.apply(fa, 0.0f, 0.0f);
-    float ca = ib * zb;
-    { const float p = fb * c_prev; ca = ca + p; }
-    { const float p = ca * a.po[j]; oa = oa + p; }
-    oa = oa + a.bo[j];
-    const float ob = SigmoidOp{}.apply(oa, 0.0f, 0.0f);
-    const float cb = act_forward(act, ca);
+    LstmCell c;
+    c.za = za; c.ia = ia; c.fa = fa; c.oa = oa;
+    lstm_cell_forward(c, act, c_prev, a.pi[j], a.pf[j], a.po[j], a.bz[j], a.bi[j], a.bf[j], a.bo[j]);
+    za = c.za; ia = c.ia; fa = c.fa; oa = c.oa;
+    const float zb = c.zb, ib = c.ib, fb = c.fb, ca = c.ca, ob = c.ob, cb = c.cb;
     stg(a.Za + e, za); stg(a.Zb + e, zb); stg(a.Ia + e, ia); stg(a.Ib + e, ib); stg(a.Fa + e, fa); stg(a.Fb + e, fb);
     stg(a.Ca + e, ca); stg(a.Oa + e, oa); stg(a.Ob + e, ob); stg(a.Cb + e, cb);
-    a.y[e] = ob * cb;
+    a.y[e] = c.y;
 }
 
 struct LstmBwdArgs {

@@ -1,0 +1,345 @@
+// The forward recurrence of a peephole LSTM layer (lstm_layer.py:115-145) for ALL time steps in one
+// persistent launch.
+//
+// Step by step through the library, a time step is one float32 product y[t-1] (B,H) x [Rz;Ri;Rf;Ro]^T
+// (4H,H) and one elementwise kernel: for B = 100, H = 1000 the product alone takes 13.7 us, re-reads the
+// 16 MB of recurrent weights from the L2s every step and is followed by a launch gap. Here the weights
+// stay on chip for the whole sequence: a workgroup owns 4 hidden units, i.e. the 16 rows
+// {z,i,f,o} x {4 units} of the stacked matrix (64 KB in LDS), and up to 64 rows of the batch. It computes
+// the (rows,16) slab of pre-activations of its units with float32 matrix-core instructions
+// (v_mfma_f32_16x16x4f32), applies the cell update to its (rows,4) elements, writes y[t] and the ten
+// internals, and meets the other workgroups of its batch group at one grid barrier per time step.
+//
+// Batch groups: the rows of a batch are independent sequences, so a batch of more than 64 rows is split
+// into two groups that run as two independent recurrences with a barrier each. A compute unit holds one
+// workgroup of either group (the LDS they ask for fits twice, not three times), and while one of them
+// waits at its barrier or evaluates activations, the other one keeps the matrix cores and the L2 busy.
+//
+// The operand y[t-1] is kept TRANSPOSED (k-major, 128 columns of batch) in a small double buffer beside
+// the layer's own y, because the matrix-core operand layout gives neighbouring lanes neighbouring batch
+// rows: v_mfma_f32_16x16x4f32 (A 16x4, B 4x16, D 16x16, one float of A and B and four of D per lane)
+// takes A[l % 16][l / 16] and B[l / 16][l % 16] from lane l and returns D[4 * (l / 16) + r][l % 16], r = 0..3.
+// Read from the (B,H) array, the 16 lanes of a group would touch 16 different rows with one load; read
+// from the transposed copy, lane (m = l % 16, g = l / 16) loads the NT consecutive batch rows
+// base + NT*m .. + NT-1 of row k of the copy, and component r of that load is its operand for row tile r,
+// whose 16 rows are the batch rows base + NT*m' + r (a tile need not be contiguous). NT = 1..4 is the number
+// of 16-row tiles the group's rows need.
+//
+// Work split inside a workgroup (256 lanes = 4 wavefronts): wavefront w takes the K-quarter w of the inner
+// dimension for all tiles; the four K-partial sums of an element meet in LDS and are added in a fixed
+// order.
+//
+// The grid barrier: y[t] goes to the transposed buffer with write-through stores; every wavefront waits
+// for its stores, the workgroup's first wavefront raises the workgroup's flag in device memory to the step
+// number and polls the flags of its group (64 per load), then invalidates the compute unit's and the L2's
+// stale lines. The wait is bounded: after `spin_limit` polls a workgroup sets *failed and every workgroup
+// exits at its next poll, so the kernel ends in any case; the host then reports the failure. All
+// workgroups must be resident together: the host checks the occupancy the runtime reports against the
+// grid before it launches.
+#pragma clang fp contract(off)
+
+#include <cstdlib>
+
+#include "common.h"
+#include "functors.h"
+#include "lstm_cell.h"
+
+namespace bship {
+
+constexpr int kSeqThreads = 256;
+constexpr int kSeqUnits = 4;                      // hidden units per workgroup
+constexpr int kSeqCols = 4 * kSeqUnits;           // one 16-column tile: gates z, i, f, o of the units
+constexpr int kSeqGroupRows = 64;                 // batch rows per group: up to 4 row tiles of 16
+constexpr int kSeqMaxBatch = 2 * kSeqGroupRows;   // columns of the transposed operand
+constexpr int kSeqFlagStride = 256;               // flags per batch group
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct LstmSeqArgs {
+    float *Za, *Zb, *Ia, *Ib, *Fa, *Fb, *Oa, *Ob, *Ca, *Cb, *y;   // (T + 1, B, H) each; slab T is the context slot
+    const float *R;                                               // (4H, H): [Rz; Ri; Rf; Ro]
+    const float *pi, *pf, *po, *bz, *bi, *bf, *bo;                // (H,) each
+    float* yT;             // two (krows, 128) buffers, zero on entry: y[t-1] transposed, by step parity
+    unsigned* flags;       // kSeqFlagStride per batch group, zero on entry
+    int* failed;           // zero on entry; 1 if a wait ran out
+    int T, B, H, act;
+    int ugroups;           // workgroups per batch group: ceil(H / 4)
+    int base1;             // first batch row of group 1 (group 0 starts at row 0)
+    int nt0, nt1;          // row tiles of group 0 and group 1
+    int kpitch;            // floats from one weight row to the next in LDS
+    int kquarter;          // k values per wavefront (a multiple of 16)
+    int krows;             // 4 * kquarter: rows of a transposed-operand buffer
+    unsigned spin_limit;
+};
+
+// NT consecutive floats, aligned to 4 bytes only
+template <int NT> struct RowPiece { float v[NT]; };
+
+template <int NT>
+__device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* Rs, float* P, int* s_go, int group,
+                                                   int ug, int base, int rows) {
+    const int tid = static_cast<int>(threadIdx.x);
+    const int lane = tid & 63, kq = tid >> 6;
+    const int m = lane & 15, g = lane >> 4;
+    const int H = a.H;
+    const int u0 = ug * kSeqUnits;
+    const int64_t slab = static_cast<int64_t>(a.B) * H;
+    const unsigned members = static_cast<unsigned>(a.ugroups);
+    unsigned* flags = a.flags + group * kSeqFlagStride;
+
+    // `between` runs after the workgroup has announced its arrival and before it looks for the others:
+    // the place for stores nobody waits for.
+    auto grid_barrier = [&](unsigned target, auto between) -> bool {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // this wavefront's write-through stores have reached memory
+        __syncthreads();
+        if (tid == 0) __hip_atomic_store(flags + ug, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        between();
+        if (kq == 0) {
+            int go = 1;
+            unsigned spins = 0;
+            for (;;) {
+                // a limit of 0 polls gives up at once: the way to exercise this path from the host
+                if (spins++ >= a.spin_limit || __hip_atomic_load(a.failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+                    if (lane == 0) __hip_atomic_store(a.failed, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    go = 0;
+                    break;
+                }
+                bool here = true;
+                for (unsigned w = lane; w < members; w += 64)
+                    here = here && __hip_atomic_load(flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target;
+                if (__all(here)) break;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");    // drops this compute unit's and this L2's stale lines
+            if (lane == 0) *s_go = go;
+        }
+        __syncthreads();
+        return *s_go != 0;                                        // the same for every lane of the workgroup
+    };
+
+    // this workgroup's 16 weight rows -> LDS (row c = gate * 4 + unit), zero beyond H and for missing units
+    for (int c = 0; c < kSeqCols; ++c) {
+        const int unit = u0 + (c & 3), gate = c >> 2;
+        const float* src = a.R + (static_cast<int64_t>(gate) * H + unit) * H;
+        for (int k = tid; k < a.kpitch; k += kSeqThreads)
+            Rs[c * a.kpitch + k] = (unit < H && k < H) ? src[k] : 0.0f;
+    }
+    // the element of the (rows, 4) slab this lane updates, its previous cell state and its input products
+    // (fetched a step ahead: they do not depend on other workgroups)
+    const int el = tid >> 2, eu = tid & 3;          // row inside the group, unit inside the workgroup
+    const int eb = base + el, ej = u0 + eu;
+    const bool owns = el < rows && ej < H;
+    float c_prev = 0.0f, p_i = 0.0f, p_f = 0.0f, p_o = 0.0f, b_z = 0.0f, b_i = 0.0f, b_f = 0.0f, b_o = 0.0f;
+    float in_z = 0.0f, in_i = 0.0f, in_f = 0.0f, in_o = 0.0f;
+    float* const yT0 = a.yT;                                     // the buffer of even steps; the odd one follows it
+    const int yT_step = a.krows * kSeqMaxBatch;
+    if (owns) {
+        const int64_t e0 = static_cast<int64_t>(eb) * H + ej;
+        c_prev = a.Ca[static_cast<int64_t>(a.T) * slab + e0];                                   // Ca[-1]
+        p_i = a.pi[ej]; p_f = a.pf[ej]; p_o = a.po[ej];
+        b_z = a.bz[ej]; b_i = a.bi[ej]; b_f = a.bf[ej]; b_o = a.bo[ej];
+        in_z = a.Za[e0]; in_i = a.Ia[e0]; in_f = a.Fa[e0]; in_o = a.Oa[e0];
+        // y[-1], transposed, is what step 0 multiplies
+        __hip_atomic_store(yT0 + ej * kSeqMaxBatch + eb, a.y[static_cast<int64_t>(a.T) * slab + e0], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!grid_barrier(1u, [] {})) return;
+
+    const int k_begin = kq * a.kquarter;
+    const int k_limit = (H + 15) & ~15;
+    const int k_end = k_begin + a.kquarter < k_limit ? k_begin + a.kquarter : k_limit;
+    const int nblocks = k_end > k_begin ? (k_end - k_begin) / 16 : 0;
+    // All workgroups of an XCD read the same y[t-1] out of the same L2 at the same time; if they also walked
+    // it in the same order, every request of a moment would go to the same L2 channel. Each workgroup
+    // therefore starts its k blocks at a different one (and wraps around).
+    const int rot = nblocks > 0 ? static_cast<int>((blockIdx.x / 8u) % static_cast<unsigned>(nblocks)) : 0;
+    for (int t = 0; t < a.T; ++t) {
+        const float* yprev = yT0 + (t & 1) * yT_step + base + NT * m;
+        v4f acc[NT];
+#pragma unroll
+        for (int r = 0; r < NT; ++r) acc[r] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        // A k block is 16 wide. Lane (m, g) takes k = kb + 4g + j, j = 0..3: four weights with one LDS read,
+        // and for each j its NT batch rows of row k of the transposed operand with one load (16 neighbouring
+        // lanes read 64 * NT contiguous bytes).
+        struct Block { RowPiece<NT> ya[4]; v4f rb; };
+        auto load_block = [&](int ib, Block& blk) {
+            int b = (ib < nblocks ? ib : nblocks - 1) + rot;       // past the end: the last block again (not used)
+            if (b >= nblocks) b -= nblocks;
+            const int k = k_begin + 16 * b + 4 * g;
+            blk.rb = *reinterpret_cast<const v4f*>(Rs + m * a.kpitch + k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) blk.ya[j] = *reinterpret_cast<const RowPiece<NT>*>(yprev + (k + j) * kSeqMaxBatch);
+        };
+        auto multiply = [&](const Block& blk) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int r = 0; r < NT; ++r)
+                    acc[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(blk.ya[j].v[r], blk.rb[j], acc[r], 0, 0, 0);
+            }
+        };
+        // The L2 answers in about a microsecond and a block is multiplied in a fifth of that, so loads run
+        // THREE blocks ahead (four register sets in turn). Every load is issued unconditionally, which lets
+        // the compiler wait for exactly the set it needs and leave the younger ones in flight.
+        if (nblocks > 0) {
+            Block b0, b1, b2, b3;
+            load_block(0, b0);
+            load_block(1, b1);
+            load_block(2, b2);
+            for (int ib = 0;; ib += 4) {
+                load_block(ib + 3, b3);
+                multiply(b0);
+                if (ib + 1 >= nblocks) break;
+                load_block(ib + 4, b0);
+                multiply(b1);
+                if (ib + 2 >= nblocks) break;
+                load_block(ib + 5, b1);
+                multiply(b2);
+                if (ib + 3 >= nblocks) break;
+                load_block(ib + 6, b2);
+                multiply(b3);
+                if (ib + 4 >= nblocks) break;
+            }
+        }
+        // lane (m, g) holds, of tile r, the rows m' = 4g + q (q = 0..3) of column m: group row NT * m' + r
+#pragma unroll
+        for (int r = 0; r < NT; ++r) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) P[(kq * kSeqGroupRows + NT * (4 * g + q) + r) * kSeqCols + m] = acc[r][q];
+        }
+        __syncthreads();
+        const int64_t e = static_cast<int64_t>(t) * slab + static_cast<int64_t>(eb) * H + ej;
+        LstmCell cell;
+        if (owns) {
+            float rec[4];
+#pragma unroll
+            for (int gate = 0; gate < 4; ++gate) {
+                const int col = gate * 4 + eu;
+                const float p0 = P[(0 * kSeqGroupRows + el) * kSeqCols + col], p1 = P[(1 * kSeqGroupRows + el) * kSeqCols + col];
+                const float p2 = P[(2 * kSeqGroupRows + el) * kSeqCols + col], p3 = P[(3 * kSeqGroupRows + el) * kSeqCols + col];
+                rec[gate] = (p0 + p1) + (p2 + p3);
+            }
+            cell.za = in_z + rec[0];
+            cell.ia = in_i + rec[1];
+            cell.fa = in_f + rec[2];
+            cell.oa = in_o + rec[3];
+            if (t + 1 < a.T) { in_z = a.Za[e + slab]; in_i = a.Ia[e + slab]; in_f = a.Fa[e + slab]; in_o = a.Oa[e + slab]; }
+            lstm_cell_forward(cell, a.act, c_prev, p_i, p_f, p_o, b_z, b_i, b_f, b_o);
+            // the next step's operand first, written through to memory
+            if (t + 1 < a.T)
+                __hip_atomic_store(yT0 + ((t + 1) & 1) * yT_step + ej * kSeqMaxBatch + eb, cell.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            c_prev = cell.ca;
+        }
+        // y[t] and the internals are nobody's operand: they are stored while the barrier waits
+        auto store_results = [&] {
+            if (owns) {
+                a.y[e] = cell.y;
+                a.Za[e] = cell.za; a.Zb[e] = cell.zb; a.Ia[e] = cell.ia; a.Ib[e] = cell.ib; a.Fa[e] = cell.fa; a.Fb[e] = cell.fb;
+                a.Ca[e] = cell.ca; a.Oa[e] = cell.oa; a.Ob[e] = cell.ob; a.Cb[e] = cell.cb;
+            }
+        };
+        if (t + 1 == a.T) { store_results(); break; }              // nothing follows the last step
+        if (!grid_barrier(static_cast<unsigned>(t) + 2u, store_results)) return;
+    }
+}
+
+__global__ __launch_bounds__(kSeqThreads) void lstm_fwd_sequence_kernel(LstmSeqArgs a) {
+    extern __shared__ float seq_lds[];
+    float* Rs = seq_lds;                                                     // [16][kpitch]
+    float* P = seq_lds + kSeqCols * a.kpitch;                                // [4][kSeqGroupRows][16]
+    __shared__ int s_go;
+    const int group = static_cast<int>(blockIdx.x) / a.ugroups;
+    const int ug = static_cast<int>(blockIdx.x) - group * a.ugroups;
+    const int base = group == 0 ? 0 : a.base1;
+    const int nt = group == 0 ? a.nt0 : a.nt1;
+    const int rows = (group == 0 && a.nt1 > 0 ? a.base1 : a.B) - base;
+    switch (nt) {
+        case 1: lstm_sequence_body<1>(a, Rs, P, &s_go, group, ug, base, rows); break;
+        case 2: lstm_sequence_body<2>(a, Rs, P, &s_go, group, ug, base, rows); break;
+        case 3: lstm_sequence_body<3>(a, Rs, P, &s_go, group, ug, base, rows); break;
+        default: lstm_sequence_body<4>(a, Rs, P, &s_go, group, ug, base, rows); break;
+    }
+}
+
+}  // namespace bship
+
+using namespace bship;
+
+extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t batch, int64_t n, const float* R_all,
+                                           float* Za, float* Zb, float* Ia, float* Ib, float* Fa, float* Fb,
+                                           float* Oa, float* Ob, float* Ca, float* Cb, float* y, const float* pi,
+                                           const float* pf, const float* po, const float* bz, const float* bi,
+                                           const float* bf, const float* bo) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_EAGER();
+    BSHIP_REQUIRE_DIM(time_steps >= 0 && batch >= 0 && n >= 0);
+    if (act < 0 || act > 4) return set_error(BSHIP_ERR_BAD_OP, "%s: unknown activation %d", __func__, act);
+    if (time_steps == 0 || batch == 0 || n == 0) return 0;
+    const float* ins[] = {R_all, pi, pf, po, bz, bi, bf, bo};
+    float* outs[] = {Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y};
+    for (const float* p : ins) { BSHIP_REQUIRE_PTR(p); BSHIP_REQUIRE_F32_ALIGNED(p); }
+    for (float* p : outs) { BSHIP_REQUIRE_PTR(p); BSHIP_REQUIRE_F32_ALIGNED(p); }
+    const Context& c = ctx();
+    const int64_t ugroups = ceil_div(n, kSeqUnits);
+    if (n % 4 != 0 || batch > kSeqMaxBatch || ugroups > kSeqFlagStride || time_steps > 0x3fffff)
+        return set_error(BSHIP_ERR_UNSUPPORTED, "%s: needs n %% 4 == 0, batch <= %d and n <= %d; got batch %lld, n %lld",
+                         __func__, kSeqMaxBatch, kSeqUnits * kSeqFlagStride, static_cast<long long>(batch),
+                         static_cast<long long>(n));
+    LstmSeqArgs a;
+    a.Za = Za; a.Zb = Zb; a.Ia = Ia; a.Ib = Ib; a.Fa = Fa; a.Fb = Fb; a.Oa = Oa; a.Ob = Ob; a.Ca = Ca; a.Cb = Cb; a.y = y;
+    a.R = R_all; a.pi = pi; a.pf = pf; a.po = po; a.bz = bz; a.bi = bi; a.bf = bf; a.bo = bo;
+    a.T = static_cast<int>(time_steps); a.B = static_cast<int>(batch); a.H = static_cast<int>(n); a.act = act;
+    a.ugroups = static_cast<int>(ugroups);
+    // row tiles: one group of up to 4, or two groups that share them as evenly as they divide
+    const int tiles = static_cast<int>(ceil_div(batch, 16));
+    a.nt0 = tiles <= 4 ? tiles : (tiles + 1) / 2;
+    a.nt1 = tiles - a.nt0;
+    a.base1 = 16 * a.nt0;
+    const int ngroups = a.nt1 > 0 ? 2 : 1;
+    const int k16 = (a.H + 15) & ~15;
+    a.kquarter = ((k16 / 16 + 3) / 4) * 16;
+    a.krows = 4 * a.kquarter;
+    int kpitch = k16;                                  // covers every k a wavefront reads
+    if ((kpitch / 4) % 2 == 0) kpitch += 4;            // an odd number of 16-byte units per row spreads the rows over the banks
+    a.kpitch = kpitch;
+    const char* spins = getenv("BSHIP_GRID_BARRIER_SPINS");
+    a.spin_limit = spins && spins[0] ? static_cast<unsigned>(strtoul(spins, nullptr, 10)) : (1u << 21);
+    const size_t lds = (static_cast<size_t>(kSeqCols) * kpitch + 4 * kSeqGroupRows * kSeqCols) * sizeof(float);
+    static bool lds_granted = false;
+    if (!lds_granted) {
+        BSHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(lstm_fwd_sequence_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024));
+        lds_granted = true;
+    }
+    // Never three workgroups on a compute unit (160 KB of LDS): a third one would take matrix-core time
+    // from the two groups' pair without shortening anybody's step.
+    const size_t lds_ask = lds < 56 * 1024 ? 56 * 1024 : lds;
+    const int64_t grid = ugroups * ngroups;
+    int per_cu = 0;
+    if (lds_ask <= 159 * 1024)
+        BSHIP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(lstm_fwd_sequence_kernel),
+                                                               kSeqThreads, lds_ask));
+    if (static_cast<int64_t>(per_cu) * c.num_cus < grid)
+        return set_error(BSHIP_ERR_UNSUPPORTED, "%s: batch %d, n %d needs %lld workgroups with %zu bytes of LDS resident "
+                         "together; the device holds %d per compute unit", __func__, a.B, a.H,
+                         static_cast<long long>(grid), lds_ask, per_cu);
+    // zero-filled: the failure flag, 256 bytes on the flags of both groups, 4 KB on the two transposed buffers
+    const size_t yt_bytes = 2 * static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
+    void* sync = nullptr;
+    int st = bship_malloc(4096 + yt_bytes, &sync);
+    if (st != 0) return st;
+    a.failed = static_cast<int*>(sync);
+    a.flags = reinterpret_cast<unsigned*>(static_cast<char*>(sync) + 256);
+    a.yT = reinterpret_cast<float*>(static_cast<char*>(sync) + 4096);
+    hipLaunchKernelGGL(lstm_fwd_sequence_kernel, dim3(static_cast<unsigned>(grid)), dim3(kSeqThreads), lds_ask,
+                       c.stream, a);
+    st = check_launch("lstm_forward_sequence");
+    int failed = 0;
+    if (st == 0) st = bship_d2h(&failed, a.failed, sizeof(int));     // waits for the kernel
+    bship_free(sync);
+    if (st != 0) return st;
+    if (failed)
+        return set_error(BSHIP_ERR_TIMEOUT, "%s: the workgroups did not all meet at a time step's barrier within %u "
+                         "polls (the device was shared with other work?); the layer's buffers hold an unfinished pass",
+                         __func__, a.spin_limit);
+    return 0;
+}

@@ -247,15 +247,17 @@ class Lstm(Layer):
         # handler's lstm_forward_step / lstm_backward_step (one launch each, same bits) when it
         # has them. fused="packed": additionally the four recurrent products of a step become
         # one product over the stacked matrices [Rz;Ri;Rf;Ro] (same values up to the summation
-        # order inside the matrix product).
+        # order inside the matrix product). fused="sequence": as "packed", and the whole forward
+        # recurrence is one launch of the handler's lstm_forward_sequence when it has one and the
+        # shape fits it.
         self.fused = "steps" if fused is True else (fused or False)
-        assert self.fused in (False, "steps", "packed")
+        assert self.fused in (False, "steps", "packed", "sequence")
 
     def _use_fused(self):
         return bool(self.fused) and hasattr(self.handler, "lstm_forward_step")
 
     def _stacked_recurrent(self, Rz, Ri, Rf, Ro):
-        if self.fused != "packed" or not hasattr(self.handler, "stack_adjacent"):
+        if self.fused not in ("packed", "sequence") or not hasattr(self.handler, "stack_adjacent"):
             return None
         return self.handler.stack_adjacent([Rz, Ri, Rf, Ro])
 
@@ -288,6 +290,11 @@ class Lstm(Layer):
         _h.dot_mm(flat_x, Wo, flatten_time(Oa[:-1]), transb=True)
 
         R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
+        if (R_all is not None and self.fused == "sequence" and hasattr(_h, "lstm_forward_sequence")
+                and Za.shape[0] == time_size + 1
+                and _h.lstm_forward_sequence(self.activation, R_all, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y,
+                                             pi, pf, po, bz, bi, bf, bo)):
+            return
         if R_all is not None:
             rec = _h.allocate((x.shape[1], 4 * n))
             for t in range(time_size):

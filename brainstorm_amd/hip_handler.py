@@ -986,6 +986,31 @@ class HipHandler(Handler):
         self._call(self._lib.bship_lstm_fwd_step_packed_f32(
             self._ACT_CODES[activation], batch, n, rec.ptr, *[a.ptr for a in mats + vecs]))
 
+    def lstm_forward_sequence(self, activation, R_all, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y,
+                              pi, pf, po, bz, bi, bf, bo):
+        """The whole forward recurrence of lstm_layer.py:115-145 in one launch: Za, Ia, Fa, Oa hold the
+        input products on entry; every array is (time + 1, batch, n) with its context slot last; R_all is
+        the stacked (4n, n) recurrent matrix (stack_adjacent). Returns False, with nothing done, when the
+        shape does not fit the kernel (n % 4, batch > 128, n > 1024, or more workgroups than the device
+        holds at once): the caller then takes the step-by-step path. Raises BshipError (status
+        BSHIP_ERR_TIMEOUT) if the workgroups did not meet at a time step's barrier. Waits for the
+        device."""
+        steps = Za.shape[0] - 1
+        batch, n = Za.shape[1], Za.shape[2]
+        mats = (Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y)
+        vecs = (pi, pf, po, bz, bi, bf, bo)
+        if (R_all.shape != (4 * n, n) or any(m.shape != (steps + 1, batch, n) for m in mats)
+                or any(v.size != n for v in vecs)):
+            raise ValueError("lstm_forward_sequence: inconsistent shapes")
+        if n % 4 or batch > 128 or n > 1024:
+            return False
+        status = self._lib.bship_lstm_fwd_sequence_f32(
+            self._ACT_CODES[activation], steps, batch, n, R_all.ptr, *[a.ptr for a in mats + vecs])
+        if status == _lib.ERR_UNSUPPORTED:
+            return False
+        self._call(status)
+        return True
+
     def lstm_backward_step_packed(self, activation, deltas, dy, packed_out, Zb, Ib, Fb, Ob, Cb,
                                   Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next, dZa, dZb, dIa,
                                   dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po):

@@ -44,6 +44,7 @@ extern "C" {
 #define BSHIP_ERR_UNSUPPORTED     (-6)
 #define BSHIP_ERR_BAD_POINTER     (-7)
 #define BSHIP_ERR_BLAS            (-8)
+#define BSHIP_ERR_TIMEOUT         (-9)   /* a bounded wait inside a kernel ran out; every kernel has exited */
 
 /* ------------------------------ lifecycle -------------------------------- */
 
@@ -375,6 +376,29 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
                                int64_t n, int h, int w, int c, int out_h,
                                int out_w, int pool_h, int pool_w, int pad,
                                int stride_h, int stride_w);
+
+/* The forward recurrence of a peephole LSTM layer for all time steps in one launch
+ * (lstm_layer.py 115-145: per time step the four recurrent products y[t-1] R^T accumulated into
+ * Za, Ia, Fa, Oa, then the elementwise part that bship_lstm_fwd_step_f32 does). On entry Za, Ia,
+ * Fa, Oa hold the input products x W^T (lstm_layer.py 110-113). Every array of the first group is
+ * (time_steps + 1, batch, n), dense; slab `time_steps` is the context slot that y[t-1] and
+ * Ca[t-1] mean at t = 0. R_all is the stacked (4n, n) matrix [Rz; Ri; Rf; Ro] (the four matrices
+ * are adjacent in the layer's parameter vector). The recurrent weights stay in LDS for the whole
+ * sequence, one workgroup per 4 hidden units and per group of up to 64 batch rows (a larger batch
+ * runs as two independent groups), and the workgroups of a group meet at one grid barrier per
+ * time step whose wait is bounded (BSHIP_GRID_BARRIER_SPINS polls, default 2^21): if it runs out,
+ * e.g. because other work kept some workgroups off the device, every workgroup exits, the call
+ * returns BSHIP_ERR_TIMEOUT and the buffers hold an unfinished pass. Needs n % 4 == 0,
+ * batch <= 128, n <= 1024 and all workgroups resident together (two per compute unit need
+ * n <= 1008 for a batch above 64); otherwise BSHIP_ERR_UNSUPPORTED before anything is launched.
+ * Takes 4 KB + 1 KB per hidden unit from the pool for the flags and the transposed operand.
+ * Results equal the step-by-step path up to the summation order of the products. Blocks; not
+ * recordable. */
+int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t batch, int64_t n,
+                                const float* R_all, float* Za, float* Zb, float* Ia, float* Ib,
+                                float* Fa, float* Fb, float* Oa, float* Ob, float* Ca, float* Cb,
+                                float* y, const float* pi, const float* pf, const float* po,
+                                const float* bz, const float* bi, const float* bf, const float* bo);
 
 /* The image operations on image-pitched arrays. A layer whose input or output is
  * a feature slice of a hub that several layers share (buffer_structure.py

@@ -183,6 +183,21 @@ def test_lstm_full_size_forward_backward(hip):
     assert d_err <= 1e-4, d_err
     print("lstm, fused steps + stacked recurrent product: worst gradient block %.2e, input deltas %.2e"
           % (worst_p, d_err))
+    # and with the whole forward recurrence in one launch (weights resident in LDS, one grid barrier
+    # per time step): every internal and the outputs at the oracle's bar
+    hip.rnd.seed(22)
+    net_s, data = configs.build_lstm(hip, fused="sequence")
+    net_s.provide_external_data(data)
+    net_s.forward_pass(training_pass=True)
+    loss_s = net_s.get("loss", "outputs", "loss")[0]
+    assert abs(loss_s - loss_r) <= 1e-5 * abs(loss_r), (loss_s, loss_r)
+    worst_s = 0.0
+    for key in ("Za", "Zb", "Ia", "Ib", "Fa", "Fb", "Oa", "Ob", "Ca", "Cb"):
+        err = scaled_err(net_s.get("lstm", "internals", key), net_r.get("lstm", "internals", key))
+        worst_s = max(worst_s, err)
+        assert err <= 1e-5, (key, err)
+    assert scaled_err(net_s.get("lstm", "outputs", "default"), net_r.get("lstm", "outputs", "default")) <= 1e-5
+    print("lstm, whole-sequence forward kernel: worst internal %.2e" % worst_s)
 
 
 @pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
