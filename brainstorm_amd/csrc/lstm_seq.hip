@@ -75,6 +75,22 @@ struct LstmSeqArgs {
 // NT consecutive floats, aligned to 4 bytes only
 template <int NT> struct RowPiece { float v[NT]; };
 
+// One load of NT floats at byte offset `voff` of the buffer (zeros, and no memory access, beyond its end)
+template <int NT>
+__device__ __forceinline__ RowPiece<NT> load_row_piece(__amdgpu_buffer_rsrc_t rsrc, int voff) {
+    if constexpr (NT == 1) return __builtin_bit_cast(RowPiece<1>, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, 0, 0));
+    else if constexpr (NT == 2) return __builtin_bit_cast(RowPiece<2>, __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, 0, 0));
+    else if constexpr (NT == 3) {
+        // four floats loaded, three kept (the 96-bit builtin does not load all three with this compiler);
+        // the fourth is the next lane's first or, for the last lane, a column inside the same row
+        const RowPiece<4> q = __builtin_bit_cast(RowPiece<4>, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0));
+        RowPiece<3> p;
+        p.v[0] = q.v[0]; p.v[1] = q.v[1]; p.v[2] = q.v[2];
+        return p;
+    }
+    else return __builtin_bit_cast(RowPiece<4>, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0));
+}
+
 template <int NT>
 __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* Rs, float* P, int* s_go, int group,
                                                    int ug, int base, int rows) {
@@ -104,9 +120,17 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
                     go = 0;
                     break;
                 }
+                // the group's flags, four per lane, all four loads in flight together (a lane beyond the last
+                // workgroup reads the last one's flag again)
+                unsigned seen[kSeqFlagStride / 64];
+#pragma unroll
+                for (int i = 0; i < kSeqFlagStride / 64; ++i) {
+                    const unsigned w = static_cast<unsigned>(lane) + 64u * i;
+                    seen[i] = __hip_atomic_load(flags + (w < members ? w : members - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
                 bool here = true;
-                for (unsigned w = lane; w < members; w += 64)
-                    here = here && __hip_atomic_load(flags + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target;
+#pragma unroll
+                for (int i = 0; i < kSeqFlagStride / 64; ++i) here = here && seen[i] >= target;
                 if (__all(here)) break;
             }
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");    // drops this compute unit's and this L2's stale lines
@@ -132,6 +156,7 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
     float in_z = 0.0f, in_i = 0.0f, in_f = 0.0f, in_o = 0.0f;
     float* const yT0 = a.yT;                                     // the buffer of even steps; the odd one follows it
     const int yT_step = a.krows * kSeqMaxBatch;
+    const int yT_bytes = yT_step * static_cast<int>(sizeof(float));
     if (owns) {
         const int64_t e0 = static_cast<int64_t>(eb) * H + ej;
         c_prev = a.Ca[static_cast<int64_t>(a.T) * slab + e0];                                   // Ca[-1]
@@ -152,8 +177,28 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
     // it in the same order, every request of a moment would go to the same L2 channel. Each workgroup
     // therefore starts its k blocks at a different one (and wraps around).
     const int rot = nblocks > 0 ? static_cast<int>((blockIdx.x / 8u) % static_cast<unsigned>(nblocks)) : 0;
+    // What a step leaves besides its operand for the next one (y[t] and the ten internals) is stored while
+    // the workgroup waits at the barrier.
+    LstmCell cell = {};
+    int64_t e = 0;
+    auto store_results = [&] {
+        if (owns) {
+            a.y[e] = cell.y;
+            a.Za[e] = cell.za; a.Zb[e] = cell.zb; a.Ia[e] = cell.ia; a.Ib[e] = cell.ib; a.Fa[e] = cell.fa; a.Fb[e] = cell.fb;
+            a.Ca[e] = cell.ca; a.Oa[e] = cell.oa; a.Ob[e] = cell.ob; a.Cb[e] = cell.cb;
+        }
+    };
     for (int t = 0; t < a.T; ++t) {
-        const float* yprev = yT0 + (t & 1) * yT_step + base + NT * m;
+        e = static_cast<int64_t>(t) * slab + static_cast<int64_t>(eb) * H + ej;
+        // The step's operand as a buffer resource: a load whose offset lies beyond the buffer returns zeros
+        // without touching memory, which is how the loads past the last k block are switched off without a
+        // branch around them.
+        // (the address is the same in every lane; saying so keeps the descriptor in scalar registers)
+        const uint64_t yaddr = reinterpret_cast<uint64_t>(yT0 + (t & 1) * yT_step);
+        float* const ybase = reinterpret_cast<float*>(
+            (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(yaddr >> 32))) << 32) |
+            static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(yaddr))));
+        const __amdgpu_buffer_rsrc_t yprev = __builtin_amdgcn_make_buffer_rsrc(ybase, 0, __builtin_amdgcn_readfirstlane(yT_bytes), 0x00020000);
         v4f acc[NT];
 #pragma unroll
         for (int r = 0; r < NT; ++r) acc[r] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
@@ -162,12 +207,13 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
         // lanes read 64 * NT contiguous bytes).
         struct Block { RowPiece<NT> ya[4]; v4f rb; };
         auto load_block = [&](int ib, Block& blk) {
-            int b = (ib < nblocks ? ib : nblocks - 1) + rot;       // past the end: the last block again (not used)
+            int b = (ib < nblocks ? ib : nblocks - 1) + rot;       // past the end: the last block's weights (not used)
             if (b >= nblocks) b -= nblocks;
             const int k = k_begin + 16 * b + 4 * g;
             blk.rb = *reinterpret_cast<const v4f*>(Rs + m * a.kpitch + k);
+            const int voff = ib < nblocks ? (k * kSeqMaxBatch + base + NT * m) * 4 : 0x40000000;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) blk.ya[j] = *reinterpret_cast<const RowPiece<NT>*>(yprev + (k + j) * kSeqMaxBatch);
+            for (int j = 0; j < 4; ++j) blk.ya[j] = load_row_piece<NT>(yprev, voff + j * kSeqMaxBatch * 4);
         };
         auto multiply = [&](const Block& blk) {
 #pragma unroll
@@ -177,27 +223,21 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
                     acc[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(blk.ya[j].v[r], blk.rb[j], acc[r], 0, 0, 0);
             }
         };
-        // The L2 answers in about a microsecond and a block is multiplied in a fifth of that, so loads run
-        // THREE blocks ahead (four register sets in turn). Every load is issued unconditionally, which lets
-        // the compiler wait for exactly the set it needs and leave the younger ones in flight.
-        if (nblocks > 0) {
-            Block b0, b1, b2, b3;
-            load_block(0, b0);
-            load_block(1, b1);
-            load_block(2, b2);
-            for (int ib = 0;; ib += 4) {
-                load_block(ib + 3, b3);
-                multiply(b0);
-                if (ib + 1 >= nblocks) break;
-                load_block(ib + 4, b0);
-                multiply(b1);
-                if (ib + 2 >= nblocks) break;
-                load_block(ib + 5, b1);
-                multiply(b2);
-                if (ib + 3 >= nblocks) break;
-                load_block(ib + 6, b2);
-                multiply(b3);
-                if (ib + 4 >= nblocks) break;
+        // With every compute unit of an XCD pulling the same operand out of one L2, a load takes about two
+        // microseconds to come back and a block is multiplied in a seventh of that: loads run kSeqSets - 1
+        // blocks ahead, in kSeqSets register sets used in turn. Every load is issued unconditionally, which
+        // lets the compiler wait for exactly the set it needs and leave the younger ones in flight.
+        {
+            constexpr int kSeqSets = NT == 4 ? 6 : 8;              // what 256 registers per lane hold
+            Block blk[kSeqSets];
+#pragma unroll
+            for (int s = 0; s < kSeqSets - 1; ++s) load_block(s, blk[s]);
+            for (int ib = 0; ib < nblocks; ib += kSeqSets) {
+#pragma unroll
+                for (int s = 0; s < kSeqSets; ++s) {
+                    load_block(ib + s + kSeqSets - 1, blk[(s + kSeqSets - 1) % kSeqSets]);
+                    if (ib + s < nblocks) multiply(blk[s]);
+                }
             }
         }
         // lane (m, g) holds, of tile r, the rows m' = 4g + q (q = 0..3) of column m: group row NT * m' + r
@@ -207,8 +247,6 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
             for (int q = 0; q < 4; ++q) P[(kq * kSeqGroupRows + NT * (4 * g + q) + r) * kSeqCols + m] = acc[r][q];
         }
         __syncthreads();
-        const int64_t e = static_cast<int64_t>(t) * slab + static_cast<int64_t>(eb) * H + ej;
-        LstmCell cell;
         if (owns) {
             float rec[4];
 #pragma unroll
@@ -229,20 +267,13 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
                 __hip_atomic_store(yT0 + ((t + 1) & 1) * yT_step + ej * kSeqMaxBatch + eb, cell.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             c_prev = cell.ca;
         }
-        // y[t] and the internals are nobody's operand: they are stored while the barrier waits
-        auto store_results = [&] {
-            if (owns) {
-                a.y[e] = cell.y;
-                a.Za[e] = cell.za; a.Zb[e] = cell.zb; a.Ia[e] = cell.ia; a.Ib[e] = cell.ib; a.Fa[e] = cell.fa; a.Fb[e] = cell.fb;
-                a.Ca[e] = cell.ca; a.Oa[e] = cell.oa; a.Ob[e] = cell.ob; a.Cb[e] = cell.cb;
-            }
-        };
         if (t + 1 == a.T) { store_results(); break; }              // nothing follows the last step
         if (!grid_barrier(static_cast<unsigned>(t) + 2u, store_results)) return;
     }
 }
 
-__global__ __launch_bounds__(kSeqThreads) void lstm_fwd_sequence_kernel(LstmSeqArgs a) {
+// two wavefronts per SIMD: a compute unit holds one workgroup of each batch group
+__global__ __launch_bounds__(kSeqThreads, 2) void lstm_fwd_sequence_kernel(LstmSeqArgs a) {
     extern __shared__ float seq_lds[];
     float* Rs = seq_lds;                                                     // [16][kpitch]
     float* P = seq_lds + kSeqCols * a.kpitch;                                // [4][kSeqGroupRows][16]
