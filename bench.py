@@ -362,6 +362,9 @@ def run_nets_gpu(hip):
         # ... and the four recurrent matrix products of a step as one over the stacked matrices
         "lstm_205-1000-205_T100_batch100_fused_packed": time_net(hip, configs.build_lstm, 5, 1,
                                                                 hip.synchronize, fused="packed"),
+        # ... with the backward recurrent product through the thin-operand kernel (dot_small_tn)
+        "lstm_205-1000-205_T100_batch100_fused_thin": time_net(hip, configs.build_lstm, 5, 1,
+                                                              hip.synchronize, fused="thin"),
         # ... and the whole forward recurrence as one persistent launch (weights resident in LDS, one grid
         # barrier per time step); the backward pass is the packed one
         "lstm_205-1000-205_T100_batch100_fused_sequence": time_net(hip, configs.build_lstm, 5, 1,

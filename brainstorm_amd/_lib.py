@@ -106,6 +106,9 @@ SIGNATURES = {
     "bship_lstm_fwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 20,
     "bship_lstm_bwd_step_packed_f32": [c_int, _I64, _I64] + [_P] * 26,
     "bship_lstm_fwd_sequence_f32": [c_int, _I64, _I64, _I64] + [_P] * 19,
+    "bship_dot_small_tn_f32": [_P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int, _I64],
+    "bship_transpose_f32": [_P, _I64, _I64, _I64, _P, _I64],
+    "bship_lstm_bwd_step_thin_f32": [c_int, _I64, _I64, _P, _P, c_int, _I64] + [_P] * 25,
     "bship_softmax_ce_fwd_f32": [_P, _P, _P, _P, _I64, _I64],
     "bship_softmax_ce_bwd_f32": [_P, _P, _P, _P, _P, _I64, _I64],
     "bship_momentum_update_f32": [c_float, c_float, _P, _P, _P, c_size_t],

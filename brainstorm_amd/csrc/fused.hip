@@ -83,6 +83,35 @@ struct LstmBwdArgs {
     float* packed_out;
 };
 
+struct LstmBwdCell { float dob, doa, dcb, dca, dfb, dfa, dib, dia, dzb, dza; };
+
+// The backward step's arithmetic for element e (column j), given dy = deltas + recurrent deltas; shared by
+// the step kernels so that all of them apply the same float32 operations in the same order.
+__device__ __forceinline__ LstmBwdCell lstm_cell_backward(const LstmBwdArgs& a, int act, int64_t e, unsigned j, float dy) {
+    LstmBwdCell c;
+    float dca = ldg(a.dCa + e);
+    { const float p = ldg(a.dIa_next + e) * a.pi[j]; dca = dca + p; }
+    { const float p = ldg(a.dFa_next + e) * a.pf[j]; dca = dca + p; }
+    const float ob = ldg(a.Ob + e), cb = ldg(a.Cb + e);
+    c.dob = dy * cb;
+    c.doa = SigmoidDerivOp{}.apply(ob, c.dob, 0.0f);
+    { const float p = c.doa * a.po[j]; dca = dca + p; }
+    float dcb = dy * ob;
+    dcb = act_backward(act, cb, dcb);
+    c.dcb = dcb;
+    dca = dca + dcb;
+    { const float p = ldg(a.dCa_next + e) * ldg(a.Fb_next + e); dca = dca + p; }
+    c.dca = dca;
+    c.dfb = dca * ldg(a.Ca_prev + e);
+    c.dfa = SigmoidDerivOp{}.apply(ldg(a.Fb + e), c.dfb, 0.0f);
+    const float zb = ldg(a.Zb + e), ib = ldg(a.Ib + e);
+    c.dib = dca * zb;
+    c.dia = SigmoidDerivOp{}.apply(ib, c.dib, 0.0f);
+    c.dzb = dca * ib;
+    c.dza = act_backward(act, zb, c.dzb);
+    return c;
+}
+
 // The elementwise part of one LSTM backward time step (lstm_layer.py:180-205),
 // after the recurrent deltas have been accumulated into dy:
 //   mult_add_mv(dIa_next, pi, dCa); mult_add_mv(dFa_next, pf, dCa)
@@ -102,24 +131,9 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
         dy = ldg(a.deltas + e) + dy;
         a.dy_out[e] = dy;
     }
-    float dca = ldg(a.dCa + e);
-    { const float p = ldg(a.dIa_next + e) * a.pi[j]; dca = dca + p; }
-    { const float p = ldg(a.dFa_next + e) * a.pf[j]; dca = dca + p; }
-    const float ob = ldg(a.Ob + e), cb = ldg(a.Cb + e);
-    const float dob = dy * cb;
-    const float doa = SigmoidDerivOp{}.apply(ob, dob, 0.0f);
-    { const float p = doa * a.po[j]; dca = dca + p; }
-    float dcb = dy * ob;
-    dcb = act_backward(act, cb, dcb);
-    dca = dca + dcb;
-    { const float p = ldg(a.dCa_next + e) * ldg(a.Fb_next + e); dca = dca + p; }
-    const float dfb = dca * ldg(a.Ca_prev + e);
-    const float dfa = SigmoidDerivOp{}.apply(ldg(a.Fb + e), dfb, 0.0f);
-    const float zb = ldg(a.Zb + e), ib = ldg(a.Ib + e);
-    const float dib = dca * zb;
-    const float dia = SigmoidDerivOp{}.apply(ib, dib, 0.0f);
-    const float dzb = dca * ib;
-    const float dza = act_backward(act, zb, dzb);
+    const LstmBwdCell c = lstm_cell_backward(a, act, e, j, dy);
+    const float dob = c.dob, doa = c.doa, dcb = c.dcb, dca = c.dca, dfb = c.dfb, dfa = c.dfa, dib = c.dib, dia = c.dia,
+                dzb = c.dzb, dza = c.dza;
     // the gate deltas feed the matrix products that follow and dCa the next step: those stay cached
     stg(a.dOb + e, dob); a.dOa[e] = doa; stg(a.dCb + e, dcb); a.dCa[e] = dca; stg(a.dFb + e, dfb); a.dFa[e] = dfa;
     stg(a.dIb + e, dib); a.dIa[e] = dia; stg(a.dZb + e, dzb); a.dZa[e] = dza;
@@ -132,6 +146,58 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
     }
 }
 
+
+// The backward step behind bship_dot_small_tn_f32: the recurrent deltas arrive as `parts` partial
+// products (slabs of (batch, n), `part_stride` floats apart) that are added here in ascending order, and
+// [dZa|dIa|dFa|dOa] leaves TRANSPOSED, as the (4n, 128) left operand of the next step's product
+// (row g*n + j, column b; columns >= batch are never written). A workgroup owns an 8 x 32 tile of (batch, n),
+// one element per lane; the four gate deltas turn through LDS and leave as 32-byte pieces of the operand's rows.
+constexpr int kThinMaxParts = 8;
+
+struct LstmBwdThinArgs {
+    LstmBwdArgs s;               // s.dy = the partial products, s.packed_out = the transposed operand
+    int parts;
+    int64_t part_stride;
+};
+
+__global__ __launch_bounds__(256) void lstm_bwd_step_thin_kernel(LstmBwdThinArgs t, int act, int batch, unsigned n,
+                                                                 unsigned col_tiles) {
+    __shared__ float turn[4][8][33];
+    const LstmBwdArgs& a = t.s;
+    const int tid = static_cast<int>(threadIdx.x);
+    const int b0 = static_cast<int>(blockIdx.x / col_tiles) * 8;
+    const unsigned j0 = (blockIdx.x % col_tiles) * 32u;
+    {
+        const int tx = tid & 31, ty = tid >> 5;
+        const int b = b0 + ty;
+        const unsigned j = j0 + tx;
+        if (b < batch && j < n) {
+            const int64_t e = static_cast<int64_t>(b) * n + j;
+            // all partial products are requested before the first is used (a slab beyond the last one
+            // reads the last one again and is not added)
+            float part[kThinMaxParts];
+#pragma unroll
+            for (int p = 0; p < kThinMaxParts; ++p) part[p] = ldg(a.dy + (p < t.parts ? p : t.parts - 1) * t.part_stride + e);
+            float rec = part[0];
+#pragma unroll
+            for (int p = 1; p < kThinMaxParts; ++p) rec = p < t.parts ? rec + part[p] : rec;
+            const float dy = ldg(a.deltas + e) + rec;
+            a.dy_out[e] = dy;
+            const LstmBwdCell c = lstm_cell_backward(a, act, e, j, dy);
+            stg(a.dOb + e, c.dob); a.dOa[e] = c.doa; stg(a.dCb + e, c.dcb); a.dCa[e] = c.dca; stg(a.dFb + e, c.dfb);
+            a.dFa[e] = c.dfa; stg(a.dIb + e, c.dib); a.dIa[e] = c.dia; stg(a.dZb + e, c.dzb); a.dZa[e] = c.dza;
+            turn[0][ty][tx] = c.dza; turn[1][ty][tx] = c.dia; turn[2][ty][tx] = c.dfa; turn[3][ty][tx] = c.doa;
+        }
+    }
+    __syncthreads();
+    const int bb = tid & 7;
+    const unsigned jj = static_cast<unsigned>(tid >> 3);
+    if (b0 + bb < batch && j0 + jj < n) {
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate)
+            a.packed_out[(static_cast<int64_t>(gate) * n + j0 + jj) * 128 + b0 + bb] = turn[gate][bb][jj];
+    }
+}
 
 // =================== generic multi-operand streaming kernels ===================
 // Bodies describe one element: apply(v, in, out) with v = the row-vector operands
@@ -588,6 +654,30 @@ int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n, const floa
                   dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po,
                   deltas, dy, packed_out};
     return lstm_bwd_launch(__func__, true, act, batch, n, a);
+}
+
+int bship_lstm_bwd_step_thin_f32(int act, int64_t batch, int64_t n, const float* deltas, const float* dy_parts,
+                                 int parts, int64_t part_stride, float* dy, float* packed_t_out, const float* Zb,
+                                 const float* Ib, const float* Fb, const float* Ob, const float* Cb,
+                                 const float* Ca_prev, const float* Fb_next, const float* dIa_next,
+                                 const float* dFa_next, const float* dCa_next, float* dZa, float* dZb, float* dIa,
+                                 float* dIb, float* dFa, float* dFb, float* dOa, float* dOb, float* dCa, float* dCb,
+                                 const float* pi, const float* pf, const float* po) {
+    LstmBwdThinArgs t{{dy_parts, Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next,
+                       dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po, deltas, dy, packed_t_out},
+                      parts, part_stride};
+    const void* ptrs[] = {dy_parts, Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next, dZa, dZb, dIa,
+                          dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po, deltas, dy, packed_t_out};
+    int st = check_step_args(__func__, act, batch, n, ptrs, 27);
+    if (st != 0 || batch * n == 0) return st;
+    if (batch > 128 || parts < 1 || parts > kThinMaxParts || (parts > 1 && part_stride < batch * n))
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: batch %lld (at most 128), parts %d (1..8), part_stride %lld",
+                         __func__, (long long)batch, parts, (long long)part_stride);
+    const int64_t row_tiles = ceil_div(batch, 8), col_tiles = ceil_div(n, 32);
+    hipLaunchKernelGGL(lstm_bwd_step_thin_kernel, dim3(static_cast<unsigned>(row_tiles * col_tiles)), dim3(256), 0,
+                       ctx().stream, t, act, static_cast<int>(batch), static_cast<unsigned>(n),
+                       static_cast<unsigned>(col_tiles));
+    return check_launch("lstm_backward_step_thin");
 }
 
 int bship_highway_fwd_f32(const float* H, const float* T, const float* x, float* y, size_t n) {

@@ -40,6 +40,7 @@
 
 #include <cstdlib>
 
+#include "buffer_loads.h"
 #include "common.h"
 #include "functors.h"
 #include "lstm_cell.h"
@@ -71,25 +72,6 @@ struct LstmSeqArgs {
     int krows;             // 4 * kquarter: rows of a transposed-operand buffer
     unsigned spin_limit;
 };
-
-// NT consecutive floats, aligned to 4 bytes only
-template <int NT> struct RowPiece { float v[NT]; };
-
-// One load of NT floats at byte offset `voff` of the buffer (zeros, and no memory access, beyond its end)
-template <int NT>
-__device__ __forceinline__ RowPiece<NT> load_row_piece(__amdgpu_buffer_rsrc_t rsrc, int voff) {
-    if constexpr (NT == 1) return __builtin_bit_cast(RowPiece<1>, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, 0, 0));
-    else if constexpr (NT == 2) return __builtin_bit_cast(RowPiece<2>, __builtin_amdgcn_raw_buffer_load_b64(rsrc, voff, 0, 0));
-    else if constexpr (NT == 3) {
-        // four floats loaded, three kept (the 96-bit builtin does not load all three with this compiler);
-        // the fourth is the next lane's first or, for the last lane, a column inside the same row
-        const RowPiece<4> q = __builtin_bit_cast(RowPiece<4>, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0));
-        RowPiece<3> p;
-        p.v[0] = q.v[0]; p.v[1] = q.v[1]; p.v[2] = q.v[2];
-        return p;
-    }
-    else return __builtin_bit_cast(RowPiece<4>, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, 0, 0));
-}
 
 template <int NT>
 __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* Rs, float* P, int* s_go, int group,
@@ -193,27 +175,22 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
         // The step's operand as a buffer resource: a load whose offset lies beyond the buffer returns zeros
         // without touching memory, which is how the loads past the last k block are switched off without a
         // branch around them.
-        // (the address is the same in every lane; saying so keeps the descriptor in scalar registers)
-        const uint64_t yaddr = reinterpret_cast<uint64_t>(yT0 + (t & 1) * yT_step);
-        float* const ybase = reinterpret_cast<float*>(
-            (static_cast<uint64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(yaddr >> 32))) << 32) |
-            static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(yaddr))));
-        const __amdgpu_buffer_rsrc_t yprev = __builtin_amdgcn_make_buffer_rsrc(ybase, 0, __builtin_amdgcn_readfirstlane(yT_bytes), 0x00020000);
+        const __amdgpu_buffer_rsrc_t yprev = uniform_rsrc(yT0 + (t & 1) * yT_step, yT_bytes);
         v4f acc[NT];
 #pragma unroll
         for (int r = 0; r < NT; ++r) acc[r] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         // A k block is 16 wide. Lane (m, g) takes k = kb + 4g + j, j = 0..3: four weights with one LDS read,
         // and for each j its NT batch rows of row k of the transposed operand with one load (16 neighbouring
         // lanes read 64 * NT contiguous bytes).
-        struct Block { RowPiece<NT> ya[4]; v4f rb; };
+        struct Block { Piece<NT> ya[4]; v4f rb; };
         auto load_block = [&](int ib, Block& blk) {
             int b = (ib < nblocks ? ib : nblocks - 1) + rot;       // past the end: the last block's weights (not used)
             if (b >= nblocks) b -= nblocks;
             const int k = k_begin + 16 * b + 4 * g;
             blk.rb = *reinterpret_cast<const v4f*>(Rs + m * a.kpitch + k);
-            const int voff = ib < nblocks ? (k * kSeqMaxBatch + base + NT * m) * 4 : 0x40000000;
+            const int voff = ib < nblocks ? (k * kSeqMaxBatch + base + NT * m) * 4 : kBufferOob;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) blk.ya[j] = load_row_piece<NT>(yprev, voff + j * kSeqMaxBatch * 4);
+            for (int j = 0; j < 4; ++j) blk.ya[j] = load_piece<NT>(yprev, voff + j * kSeqMaxBatch * 4);
         };
         auto multiply = [&](const Block& blk) {
 #pragma unroll

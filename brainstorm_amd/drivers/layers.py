@@ -249,15 +249,17 @@ class Lstm(Layer):
         # one product over the stacked matrices [Rz;Ri;Rf;Ro] (same values up to the summation
         # order inside the matrix product). fused="sequence": as "packed", and the whole forward
         # recurrence is one launch of the handler's lstm_forward_sequence when it has one and the
-        # shape fits it.
+        # shape fits it. fused="thin": as "packed", and for batches of at most 128 rows the backward
+        # recurrent product goes through the handler's dot_small_tn (a product kernel for a thin left
+        # operand kept transposed, its K range cut into partial products that the step kernel adds).
         self.fused = "steps" if fused is True else (fused or False)
-        assert self.fused in (False, "steps", "packed", "sequence")
+        assert self.fused in (False, "steps", "packed", "sequence", "thin")
 
     def _use_fused(self):
         return bool(self.fused) and hasattr(self.handler, "lstm_forward_step")
 
     def _stacked_recurrent(self, Rz, Ri, Rf, Ro):
-        if self.fused not in ("packed", "sequence") or not hasattr(self.handler, "stack_adjacent"):
+        if self.fused not in ("packed", "sequence", "thin") or not hasattr(self.handler, "stack_adjacent"):
             return None
         return self.handler.stack_adjacent([Rz, Ri, Rf, Ro])
 
@@ -359,10 +361,28 @@ class Lstm(Layer):
         time_size = x.shape[0]
         fused = self._use_fused()
         R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
-        if R_all is not None:
+        batch = x.shape[1]
+        thin = R_all is not None and self.fused == "thin" and hasattr(_h, "dot_small_tn") and batch <= 128
+        if thin:
+            # the same, transposed ((4n, 128), columns beyond the batch stay zero), and the partial
+            # products of as many K ranges as fill the device with workgroups of 64 rows x 32 columns
+            n = self.size
+            packed_t = [_h.allocate((4 * n, 128)) for _ in range(2)]
+            groups = -(-n // 32) * (2 if batch > 64 else 1)
+            splits = max(1, min(8, _h.device_info()[1] // groups))
+            parts = _h.allocate((splits, batch, n) if splits > 1 else (batch, n))
+        elif R_all is not None:
             # [dZa|dIa|dFa|dOa] of the step after the current one, double-buffered; zero beyond the end
             packed = [_h.allocate((x.shape[1], 4 * self.size)) for _ in range(2)]
         for t in range(time_size - 1, -1, -1):
+            if thin:
+                _h.dot_small_tn(packed_t[(t + 1) % 2], batch, R_all, parts, splits)
+                _h.lstm_backward_step_thin(self.activation, deltas[t], parts, dy[t], packed_t[t % 2],
+                                           Zb[t], Ib[t], Fb[t], Ob[t], Cb[t], Ca[t - 1],
+                                           Fb[t + 1], dIa[t + 1], dFa[t + 1], dCa[t + 1],
+                                           dZa[t], dZb[t], dIa[t], dIb[t], dFa[t], dFb[t],
+                                           dOa[t], dOb[t], dCa[t], dCb[t], pi, pf, po)
+                continue
             if R_all is not None:
                 dy_t = dy[t]
                 _h.dot_mm(packed[(t + 1) % 2], R_all, dy_t)

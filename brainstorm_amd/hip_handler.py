@@ -835,6 +835,26 @@ class HipHandler(Handler):
     def dot_add_mm(self, a, b, out, transa=False, transb=False):
         self._gemm(a, b, out, transa, transb, 1.0)
 
+    def transpose(self, a, out):
+        """out[:a.shape[1], :a.shape[0]] = a.T for 2-D dense arrays; out may have more columns than a
+        has rows (they are left alone): the layout dot_small_tn wants is out of shape (k, 128)."""
+        rows, cols = a.shape
+        if len(out.shape) != 2 or out.shape[0] < cols or out.shape[1] < rows:
+            raise ValueError("transpose: %r does not hold the transpose of %r" % (out.shape, a.shape))
+        self._call(self._lib.bship_transpose_f32(a.ptr, rows, cols, cols, out.ptr, out.shape[1]))
+
+    def dot_small_tn(self, a_t, rows, b, out, splits=1):
+        """out = A . b for a thin A (rows <= 128) given transposed: a_t is (k, 128) with A[i][kk] at
+        [kk, i] and zero columns from `rows` on. splits > 1: out is (splits, rows, n) and receives the
+        partial products of `splits` ranges of k, to be added by the consumer in a fixed order."""
+        k, n = b.shape
+        if a_t.shape != (k, 128) or rows > 128:
+            raise ValueError("dot_small_tn: the transposed operand must be (%d, 128), rows <= 128" % k)
+        want = (rows, n) if splits == 1 else (splits, rows, n)
+        if out.shape != want:
+            raise ValueError("dot_small_tn: out must be %r, got %r" % (want, out.shape))
+        self._call(self._lib.bship_dot_small_tn_f32(a_t.ptr, b.ptr, out.ptr, rows, n, k, n, n, splits, rows * n))
+
     def conv2d_forward_batch(self, inputs, weights, bias, outputs, padding, stride):
         self._conv_forward(inputs, weights, bias, outputs, padding, stride)
 
@@ -1027,6 +1047,26 @@ class HipHandler(Handler):
         self._call(self._lib.bship_lstm_bwd_step_packed_f32(
             self._ACT_CODES[activation], batch, n, deltas.ptr, dy.ptr, packed_out.ptr,
             *[a.ptr for a in mats[2:] + vecs]))
+
+    def lstm_backward_step_thin(self, activation, deltas, dy_parts, dy, packed_t_out, Zb, Ib, Fb, Ob, Cb,
+                                Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next, dZa, dZb, dIa,
+                                dIb, dFa, dFb, dOa, dOb, dCa, dCb, pi, pf, po):
+        """lstm_backward_step_packed behind dot_small_tn: dy_parts holds the partial products of
+        packed[t+1] . [Rz;Ri;Rf;Ro], shape (batch, n) or (parts, batch, n); dy receives deltas + their
+        sum; packed_t_out (4n, 128) receives [dZa|dIa|dFa|dOa] of this step transposed (the left
+        operand of the next product)."""
+        batch, n = dy.shape
+        mats = (Zb, Ib, Fb, Ob, Cb, Ca_prev, Fb_next, dIa_next, dFa_next, dCa_next,
+                dZa, dZb, dIa, dIb, dFa, dFb, dOa, dOb, dCa, dCb)
+        vecs = (pi, pf, po)
+        parts = 1 if len(dy_parts.shape) == 2 else dy_parts.shape[0]
+        if (packed_t_out.shape != (4 * n, 128) or tuple(dy_parts.shape[-2:]) != (batch, n) or batch > 128
+                or deltas.shape != (batch, n) or any(m.shape != (batch, n) for m in mats)
+                or any(v.size != n for v in vecs)):
+            raise ValueError("lstm_backward_step_thin: inconsistent shapes")
+        self._call(self._lib.bship_lstm_bwd_step_thin_f32(
+            self._ACT_CODES[activation], batch, n, deltas.ptr, dy_parts.ptr, parts, batch * n, dy.ptr,
+            packed_t_out.ptr, *[a.ptr for a in mats + vecs]))
 
     def softmax_ce_forward(self, inputs, targets, probs, loss):
         """softmax_m(inputs, probs) and loss = -log(clip(probs[i, targets[i]], 1e-6, 1)) with the roundings of

@@ -400,6 +400,40 @@ int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t batch, int6
                                 float* y, const float* pi, const float* pf, const float* po,
                                 const float* bz, const float* bi, const float* bf, const float* bo);
 
+/* bship_lstm_bwd_step_packed_f32 behind bship_dot_small_tn_f32 (batch <= 128): the recurrent deltas
+ * packed[t+1] . [Rz;Ri;Rf;Ro] arrive as `parts` partial products (slabs of (batch, n), part_stride
+ * floats apart, added in ascending order), dy receives deltas + their sum, and [dZa|dIa|dFa|dOa]
+ * of this step leaves transposed: packed_t_out is (4n, 128), row g*n + j, column b; columns >= batch
+ * are not written (allocate it zeroed). The arithmetic is lstm_layer.py 186-214, as in
+ * bship_lstm_bwd_step_f32. */
+int bship_lstm_bwd_step_thin_f32(int act, int64_t batch, int64_t n, const float* deltas, const float* dy_parts,
+                                 int parts, int64_t part_stride, float* dy, float* packed_t_out, const float* Zb,
+                                 const float* Ib, const float* Fb, const float* Ob, const float* Cb,
+                                 const float* Ca_prev, const float* Fb_next, const float* dIa_next,
+                                 const float* dFa_next, const float* dCa_next, float* dZa, float* dZb, float* dIa,
+                                 float* dIb, float* dFa, float* dFb, float* dOa, float* dOb, float* dCa, float* dCb,
+                                 const float* pi, const float* pf, const float* po);
+
+/* Matrix product with a thin left operand that is stored transposed, for the per-time-step
+ * recurrent products of lstm_layer.py 115-145 and 180-205 (dot_mm / dot_add_mm of a (batch, n)
+ * slab, numpy_handler.py 211-229, with batch <= 128):
+ *     c[s] (M x N, row pitch ldc) = A[:, K-range s] . b[K-range s, :]     for s = 0 .. splits-1
+ * where aT holds A transposed: K rows of 128 floats, element (k, i) = A[i][k], columns >= M zero,
+ * 16-byte aligned; b is (K, N) with row pitch ldb. splits > 1 cuts K into that many ranges of whole
+ * 16-blocks whose results go to the slabs c + s * c_split_stride (floats), for the caller to add in
+ * a fixed order; splits == 1 writes the whole product to c. Sums run over k in ascending blocks per
+ * wavefront quarter, ((q0 + q1) + (q2 + q3)): equal to a float32 BLAS product up to summation order.
+ * M > 128 or operands of 1 GiB and more: BSHIP_ERR_UNSUPPORTED. Recordable. */
+int bship_dot_small_tn_f32(const float* aT, const float* b, float* c, int64_t M, int64_t N, int64_t K,
+                           int64_t ldb, int64_t ldc, int splits, int64_t c_split_stride);
+
+/* dst[c][r] = src[r][c] for r < rows, c < cols (row pitches ld_src >= cols, ld_dst >= rows);
+ * columns >= rows of dst are left as they are. Produces the transposed operands of
+ * bship_dot_small_tn_f32 (ld_dst = 128) and transposed weight matrices. No counterpart in
+ * base_handler.py: NumPy callers write a.T. */
+int bship_transpose_f32(const float* src, int64_t rows, int64_t cols, int64_t ld_src, float* dst,
+                        int64_t ld_dst);
+
 /* The image operations on image-pitched arrays. A layer whose input or output is
  * a feature slice of a hub that several layers share (buffer_structure.py
  * 232-245) sees images that are contiguous (h*w*c elements) but lie a pitch of

@@ -183,6 +183,21 @@ def test_lstm_full_size_forward_backward(hip):
     assert d_err <= 1e-4, d_err
     print("lstm, fused steps + stacked recurrent product: worst gradient block %.2e, input deltas %.2e"
           % (worst_p, d_err))
+    # the backward recurrent product through the thin-operand kernel and its step kernel
+    hip.rnd.seed(22)
+    net_t, data = configs.build_lstm(hip, fused="thin")
+    net_t.provide_external_data(data)
+    net_t.forward_pass(training_pass=True)
+    net_t.backward_pass()
+    g_t = hip.get_numpy_copy(net_t.gradients)
+    worst_t = 0.0
+    for name, (a, b, _) in net_r.parameter_slices().items():
+        err = scaled_err(g_t[a:b], g_r[a:b])
+        worst_t = max(worst_t, err)
+        assert err <= 1e-4, (name, err)
+    d_err = scaled_err(net_t.get("Input", "output_deltas", "default"), net_r.get("Input", "output_deltas", "default"))
+    assert d_err <= 1e-4, d_err
+    print("lstm, thin backward product: worst gradient block %.2e, input deltas %.2e" % (worst_t, d_err))
     # and with the whole forward recurrence in one launch (weights resident in LDS, one grid barrier
     # per time step): every internal and the outputs at the oracle's bar
     hip.rnd.seed(22)
