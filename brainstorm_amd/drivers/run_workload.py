@@ -3,7 +3,8 @@
     python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded]
 
 ``fused`` is passed to the workload's builder ("0" for single handler operations, "1" for the fused
-entry points, "packed" for the LSTM's stacked recurrent product). With a fourth argument "recorded"
+entry points; for the LSTM "packed" (stacked recurrent product), "thin" (packed, backward product
+through the thin-operand kernel) or "sequence" (packed, forward recurrence in one launch)). With a fourth argument "recorded"
 the step is recorded after one ordinary step and replayed. One step = forward + backward + momentum
 update.
 """
@@ -21,7 +22,7 @@ def main(argv):
     kw = {}
     recorded = len(argv) > 4 and argv[4] == "recorded"
     if fused and fused != "0":
-        kw["fused"] = "packed" if fused == "packed" else True
+        kw["fused"] = fused if fused in ("packed", "thin", "sequence") else True
     handler = HipHandler(seed=0)
     net, data = getattr(configs, "build_" + name)(handler, **kw)
     net.provide_external_data(data)
