@@ -60,7 +60,9 @@ struct LstmSeqArgs {
     float *Za, *Zb, *Ia, *Ib, *Fa, *Fb, *Oa, *Ob, *Ca, *Cb, *y;   // (T + 1, B, H) each; slab T is the context slot
     const float *R;                                               // (4H, H): [Rz; Ri; Rf; Ro]
     const float *pi, *pf, *po, *bz, *bi, *bf, *bo;                // (H,) each
-    float* yT;             // two (krows, 128) buffers, zero on entry: y[t-1] transposed, by step parity
+    float* yT;             // nbuf (krows, 128) buffers, zero on entry: step t reads y[t-1] transposed from buffer t % nbuf
+    int nbuf;              // T + 1 when that fits the scratch limit (no buffer is ever rewritten), else at least 2
+    int reuse;             // nbuf < T + 1: buffers are rewritten, caches must drop their old lines at every barrier
     unsigned* flags;       // kSeqFlagStride per batch group, zero on entry
     int* failed;           // zero on entry; 1 if a wait ran out
     int T, B, H, act;
@@ -115,7 +117,10 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
                 for (int i = 0; i < kSeqFlagStride / 64; ++i) here = here && seen[i] >= target;
                 if (__all(here)) break;
             }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");    // drops this compute unit's and this L2's stale lines
+            // With a buffer per time step nobody has read the operand's lines before they were written, so no
+            // cache holds a stale copy; with fewer buffers than steps this compute unit's and this L2's stale
+            // lines are dropped here (which also costs the other batch group its cached lines).
+            if (a.reuse) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             if (lane == 0) *s_go = go;
         }
         __syncthreads();
@@ -136,9 +141,9 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
     const bool owns = el < rows && ej < H;
     float c_prev = 0.0f, p_i = 0.0f, p_f = 0.0f, p_o = 0.0f, b_z = 0.0f, b_i = 0.0f, b_f = 0.0f, b_o = 0.0f;
     float in_z = 0.0f, in_i = 0.0f, in_f = 0.0f, in_o = 0.0f;
-    float* const yT0 = a.yT;                                     // the buffer of even steps; the odd one follows it
-    const int yT_step = a.krows * kSeqMaxBatch;
-    const int yT_bytes = yT_step * static_cast<int>(sizeof(float));
+    float* const yT0 = a.yT;                                     // buffer 0; the others follow it
+    const int64_t yT_step = static_cast<int64_t>(a.krows) * kSeqMaxBatch;
+    const int yT_bytes = static_cast<int>(yT_step) * static_cast<int>(sizeof(float));
     if (owns) {
         const int64_t e0 = static_cast<int64_t>(eb) * H + ej;
         c_prev = a.Ca[static_cast<int64_t>(a.T) * slab + e0];                                   // Ca[-1]
@@ -175,7 +180,7 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
         // The step's operand as a buffer resource: a load whose offset lies beyond the buffer returns zeros
         // without touching memory, which is how the loads past the last k block are switched off without a
         // branch around them.
-        const __amdgpu_buffer_rsrc_t yprev = uniform_rsrc(yT0 + (t & 1) * yT_step, yT_bytes);
+        const __amdgpu_buffer_rsrc_t yprev = uniform_rsrc(yT0 + (t % a.nbuf) * yT_step, yT_bytes);
         v4f acc[NT];
 #pragma unroll
         for (int r = 0; r < NT; ++r) acc[r] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
@@ -241,7 +246,7 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
             lstm_cell_forward(cell, a.act, c_prev, p_i, p_f, p_o, b_z, b_i, b_f, b_o);
             // the next step's operand first, written through to memory
             if (t + 1 < a.T)
-                __hip_atomic_store(yT0 + ((t + 1) & 1) * yT_step + ej * kSeqMaxBatch + eb, cell.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(yT0 + ((t + 1) % a.nbuf) * yT_step + ej * kSeqMaxBatch + eb, cell.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             c_prev = cell.ca;
         }
         if (t + 1 == a.T) { store_results(); break; }              // nothing follows the last step
@@ -255,6 +260,10 @@ __global__ __launch_bounds__(kSeqThreads, 2) void lstm_fwd_sequence_kernel(LstmS
     float* Rs = seq_lds;                                                     // [16][kpitch]
     float* P = seq_lds + kSeqCols * a.kpitch;                                // [4][kSeqGroupRows][16]
     __shared__ int s_go;
+    // Workgroups 0 .. ugroups-1 are batch group 0, the rest group 1: the dispatcher puts one workgroup on every
+    // compute unit before it gives any a second one, so a compute unit ends up with one workgroup of each
+    // group (other numberings that pair workgroups of the SAME group on a compute unit were measured 3 us per
+    // time step slower).
     const int group = static_cast<int>(blockIdx.x) / a.ugroups;
     const int ug = static_cast<int>(blockIdx.x) - group * a.ugroups;
     const int base = group == 0 ? 0 : a.base1;
@@ -330,8 +339,15 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
         return set_error(BSHIP_ERR_UNSUPPORTED, "%s: batch %d, n %d needs %lld workgroups with %zu bytes of LDS resident "
                          "together; the device holds %d per compute unit", __func__, a.B, a.H,
                          static_cast<long long>(grid), lds_ask, per_cu);
-    // zero-filled: the failure flag, 256 bytes on the flags of both groups, 4 KB on the two transposed buffers
-    const size_t yt_bytes = 2 * static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
+    // zero-filled: the failure flag, 256 bytes on the flags of both groups, 4 KB on the transposed buffers:
+    // one per time step and one for y[-1] if that stays below 256 MB, else as many as do (at least two)
+    const size_t one = static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
+    const size_t cap = static_cast<size_t>(256) << 20;
+    int64_t nbuf = time_steps + 1;
+    if (static_cast<size_t>(nbuf) * one > cap) nbuf = static_cast<int64_t>(cap / one) < 2 ? 2 : static_cast<int64_t>(cap / one);
+    a.nbuf = static_cast<int>(nbuf);
+    a.reuse = nbuf < time_steps + 1 ? 1 : 0;
+    const size_t yt_bytes = static_cast<size_t>(nbuf) * one;
     void* sync = nullptr;
     int st = bship_malloc(4096 + yt_bytes, &sync);
     if (st != 0) return st;

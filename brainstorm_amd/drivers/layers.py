@@ -249,7 +249,7 @@ class Lstm(Layer):
         # one product over the stacked matrices [Rz;Ri;Rf;Ro] (same values up to the summation
         # order inside the matrix product). fused="sequence": as "packed", and the whole forward
         # recurrence is one launch of the handler's lstm_forward_sequence when it has one and the
-        # shape fits it. fused="thin": as "packed", and for batches of at most 128 rows the backward
+        # shape fits it. fused="thin": as "sequence", and for batches of at most 128 rows the backward
         # recurrent product goes through the handler's dot_small_tn (a product kernel for a thin left
         # operand kept transposed, its K range cut into partial products that the step kernel adds).
         self.fused = "steps" if fused is True else (fused or False)
@@ -292,7 +292,7 @@ class Lstm(Layer):
         _h.dot_mm(flat_x, Wo, flatten_time(Oa[:-1]), transb=True)
 
         R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
-        if (R_all is not None and self.fused == "sequence" and hasattr(_h, "lstm_forward_sequence")
+        if (R_all is not None and self.fused in ("sequence", "thin") and hasattr(_h, "lstm_forward_sequence")
                 and Za.shape[0] == time_size + 1
                 and _h.lstm_forward_sequence(self.activation, R_all, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y,
                                              pi, pf, po, bz, bi, bf, bo)):
