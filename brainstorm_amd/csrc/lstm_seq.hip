@@ -342,7 +342,8 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
     // zero-filled: the failure flag, 256 bytes on the flags of both groups, 4 KB on the transposed buffers:
     // one per time step and one for y[-1] if that stays below 256 MB, else as many as do (at least two)
     const size_t one = static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
-    const size_t cap = static_cast<size_t>(256) << 20;
+    const char* cap_mb = getenv("BSHIP_LSTM_SEQ_SCRATCH_MB");       // default 256; small values force buffers to be reused
+    const size_t cap = static_cast<size_t>(cap_mb && cap_mb[0] ? strtoul(cap_mb, nullptr, 10) : 256) << 20;
     int64_t nbuf = time_steps + 1;
     if (static_cast<size_t>(nbuf) * one > cap) nbuf = static_cast<int64_t>(cap / one) < 2 ? 2 : static_cast<int64_t>(cap / one);
     a.nbuf = static_cast<int>(nbuf);

@@ -391,8 +391,10 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
  * returns BSHIP_ERR_TIMEOUT and the buffers hold an unfinished pass. Needs n % 4 == 0,
  * batch <= 128, n <= 1024 and all workgroups resident together (two per compute unit need
  * n <= 1008 for a batch above 64); otherwise BSHIP_ERR_UNSUPPORTED before anything is launched.
- * Takes 4 KB + 512 bytes per hidden unit and time step (at most 256 MB) from the pool for the flags and
- * the transposed operand, one buffer per time step so that no cache ever holds a stale line of it.
+ * Takes 4 KB + 512 bytes per hidden unit and time step from the pool for the flags and the
+ * transposed operand, one buffer per time step so that no cache ever holds a stale line of it;
+ * beyond BSHIP_LSTM_SEQ_SCRATCH_MB (default 256) megabytes the buffers are reused in turn and
+ * the caches are invalidated at every barrier instead.
  * Results equal the step-by-step path up to the summation order of the products. Blocks; not
  * recordable. */
 int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t batch, int64_t n,

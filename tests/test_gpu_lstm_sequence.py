@@ -141,6 +141,29 @@ def test_sequence_kernel_declines_shapes_it_does_not_fit(hip, batch, n):
         assert scaled_err(net_h.get("lstm", "outputs", "default"), net_r.get("lstm", "outputs", "default")) <= 1e-5
 
 
+def test_sequence_kernel_with_reused_operand_buffers(hip, monkeypatch):
+    # a scratch limit of 1 MB leaves two operand buffers for 1000 units: they are rewritten every other step
+    # and the caches invalidated at every barrier; same results as with one buffer per step
+    steps, batch, n = 9, 100, 1000
+    rng = np.random.RandomState(4)
+    R = hip.create_from_numpy((rng.standard_normal((4 * n, n)) * 0.03).astype(F32))
+    host = {k: np.zeros((steps + 1, batch, n), F32) for k in INTERNALS + ("y",)}
+    for k in ("Za", "Ia", "Fa", "Oa"):
+        host[k][:steps] = (rng.standard_normal((steps, batch, n)) * 0.5).astype(F32)
+    vecs = [hip.create_from_numpy((rng.standard_normal(n) * 0.3).astype(F32)) for _ in range(7)]
+
+    def run():
+        dev = {k: hip.create_from_numpy(v) for k, v in host.items()}
+        assert hip.lstm_forward_sequence("tanh", R, *[dev[k] for k in INTERNALS], dev["y"], *vecs) is True
+        return {k: hip.get_numpy_copy(v) for k, v in dev.items()}
+
+    want = run()
+    monkeypatch.setenv("BSHIP_LSTM_SEQ_SCRATCH_MB", "1")
+    got = run()
+    for k in want:
+        assert np.array_equal(got[k], want[k]), k
+
+
 _TIMEOUT_SCRIPT = r"""
 import sys
 import numpy as np
