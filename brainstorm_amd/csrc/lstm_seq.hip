@@ -60,7 +60,7 @@ struct LstmSeqArgs {
     float *Za, *Zb, *Ia, *Ib, *Fa, *Fb, *Oa, *Ob, *Ca, *Cb, *y;   // (T + 1, B, H) each; slab T is the context slot
     const float *R;                                               // (4H, H): [Rz; Ri; Rf; Ro]
     const float *pi, *pf, *po, *bz, *bi, *bf, *bo;                // (H,) each
-    float* yT;             // nbuf (krows, 128) buffers, zero on entry: step t reads y[t-1] transposed from buffer t % nbuf
+    float* yT;             // nbuf (krows, 128) buffers: step t reads y[t-1] transposed from buffer t % nbuf
     int nbuf;              // T + 1 when that fits the scratch limit (no buffer is ever rewritten), else at least 2
     int reuse;             // nbuf < T + 1: buffers are rewritten, caches must drop their old lines at every barrier
     unsigned* flags;       // kSeqFlagStride per batch group, zero on entry
@@ -143,7 +143,10 @@ __device__ __forceinline__ void lstm_sequence_body(const LstmSeqArgs& a, float* 
     float in_z = 0.0f, in_i = 0.0f, in_f = 0.0f, in_o = 0.0f;
     float* const yT0 = a.yT;                                     // buffer 0; the others follow it
     const int64_t yT_step = static_cast<int64_t>(a.krows) * kSeqMaxBatch;
-    const int yT_bytes = static_cast<int>(yT_step) * static_cast<int>(sizeof(float));
+    // what a load may touch of a buffer: the rows of real hidden units. Rows beyond them read zeros (the k
+    // padding of the last block), so the buffers need no clearing: columns beyond the batch hold whatever the
+    // pool block held, and those only reach rows of the product that nobody reads.
+    const int yT_bytes = H * kSeqMaxBatch * static_cast<int>(sizeof(float));
     if (owns) {
         const int64_t e0 = static_cast<int64_t>(eb) * H + ej;
         c_prev = a.Ca[static_cast<int64_t>(a.T) * slab + e0];                                   // Ca[-1]
@@ -339,7 +342,7 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
         return set_error(BSHIP_ERR_UNSUPPORTED, "%s: batch %d, n %d needs %lld workgroups with %zu bytes of LDS resident "
                          "together; the device holds %d per compute unit", __func__, a.B, a.H,
                          static_cast<long long>(grid), lds_ask, per_cu);
-    // zero-filled: the failure flag, 256 bytes on the flags of both groups, 4 KB on the transposed buffers:
+    // the failure flag, 256 bytes on the flags of both groups (zero-filled), 4 KB on the transposed buffers:
     // one per time step and one for y[-1] if that stays below 256 MB, else as many as do (at least two)
     const size_t one = static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
     const char* cap_mb = getenv("BSHIP_LSTM_SEQ_SCRATCH_MB");       // default 256; small values force buffers to be reused
@@ -350,8 +353,10 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
     a.reuse = nbuf < time_steps + 1 ? 1 : 0;
     const size_t yt_bytes = static_cast<size_t>(nbuf) * one;
     void* sync = nullptr;
-    int st = bship_malloc(4096 + yt_bytes, &sync);
+    int st = pool_alloc_raw(4096 + yt_bytes, &sync);
     if (st != 0) return st;
+    st = launch_fill(static_cast<float*>(sync), 0.0f, 1024);       // the flags; the operand buffers need no clearing
+    if (st != 0) { pool_free_raw(sync); return st; }
     a.failed = static_cast<int*>(sync);
     a.flags = reinterpret_cast<unsigned*>(static_cast<char*>(sync) + 256);
     a.yT = reinterpret_cast<float*>(static_cast<char*>(sync) + 4096);
@@ -360,7 +365,7 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
     st = check_launch("lstm_forward_sequence");
     int failed = 0;
     if (st == 0) st = bship_d2h(&failed, a.failed, sizeof(int));     // waits for the kernel
-    bship_free(sync);
+    pool_free_raw(sync);
     if (st != 0) return st;
     if (failed)
         return set_error(BSHIP_ERR_TIMEOUT, "%s: the workgroups did not all meet at a time step's barrier within %u "
