@@ -64,6 +64,26 @@ def test_dot_small_tn_matches_float64(hip, m, k, n, splits):
     assert scaled_err(got, want) <= 1e-5
 
 
+def test_dot_small_tn_and_transpose_on_pitched_operands(hip):
+    # b, c and the transpose's source as column slices of wider matrices (row pitches above the widths),
+    # straight through the C ABI
+    rng = np.random.RandomState(9)
+    m, k, n, ldb, ldc, lda = 70, 203, 45, 61, 50, 230
+    a_wide = rng.standard_normal((m, lda)).astype(F32)
+    b_wide = rng.standard_normal((k, ldb)).astype(F32)
+    c_wide = np.full((2, m, ldc), -3.0, F32)
+    da, db, dc = hip.create_from_numpy(a_wide), hip.create_from_numpy(b_wide), hip.create_from_numpy(c_wide)
+    a_t = hip.zeros((k, 128))
+    lib = hip._lib
+    hip._call(lib.bship_transpose_f32(da.ptr + 4 * 11, m, k, lda, a_t.ptr, 128))            # a = a_wide[:, 11:11+k]
+    assert_bit_equal(hip.get_numpy_copy(a_t)[:, :m], a_wide[:, 11:11 + k].T, "pitched transpose")
+    hip._call(lib.bship_dot_small_tn_f32(a_t.ptr, db.ptr + 4 * 7, dc.ptr + 4 * 2, m, n, k, ldb, ldc, 2, m * ldc))
+    got = hip.get_numpy_copy(dc)
+    assert np.all(got[:, :, :2] == -3.0) and np.all(got[:, :, 2 + n:] == -3.0), "columns outside the slice were written"
+    want = a_wide[:, 11:11 + k].astype(np.float64) @ b_wide[:, 7:7 + n].astype(np.float64)
+    assert scaled_err(got[:, :, 2:2 + n].astype(np.float64).sum(axis=0), want) <= 1e-5
+
+
 def test_dot_small_tn_is_deterministic_and_rejects_what_it_does_not_take(hip):
     rng = np.random.RandomState(3)
     a = rng.standard_normal((100, 4000)).astype(F32)
