@@ -15,9 +15,9 @@
 // workgroup of either group (the LDS they ask for fits twice, not three times), and while one of them
 // waits at its barrier or evaluates activations, the other one keeps the matrix cores and the L2 busy.
 //
-// The operand y[t-1] is kept TRANSPOSED (k-major, 128 columns of batch) in a small double buffer beside
-// the layer's own y, because the matrix-core operand layout gives neighbouring lanes neighbouring batch
-// rows: v_mfma_f32_16x16x4f32 (A 16x4, B 4x16, D 16x16, one float of A and B and four of D per lane)
+// The operand y[t-1] is kept TRANSPOSED (k-major, 128 columns of batch) in scratch buffers beside the
+// layer's own y, one per time step, because the matrix-core operand layout gives neighbouring lanes
+// neighbouring batch rows: v_mfma_f32_16x16x4f32 (A 16x4, B 4x16, D 16x16, one float of A and B and four of D per lane)
 // takes A[l % 16][l / 16] and B[l / 16][l % 16] from lane l and returns D[4 * (l / 16) + r][l % 16], r = 0..3.
 // Read from the (B,H) array, the 16 lanes of a group would touch 16 different rows with one load; read
 // from the transposed copy, lane (m = l % 16, g = l / 16) loads the NT consecutive batch rows
@@ -29,10 +29,12 @@
 // dimension for all tiles; the four K-partial sums of an element meet in LDS and are added in a fixed
 // order.
 //
-// The grid barrier: y[t] goes to the transposed buffer with write-through stores; every wavefront waits
-// for its stores, the workgroup's first wavefront raises the workgroup's flag in device memory to the step
-// number and polls the flags of its group (64 per load), then invalidates the compute unit's and the L2's
-// stale lines. The wait is bounded: after `spin_limit` polls a workgroup sets *failed and every workgroup
+// The grid barrier: y[t] goes to the step's transposed buffer with write-through stores; every wavefront
+// waits for its stores, the workgroup's first wavefront raises the workgroup's flag in device memory to the
+// step number and polls the flags of its group (all of them with four loads in flight). No cache is
+// invalidated: a buffer is written once and read only afterwards, so no L1 or L2 can hold an older copy of
+// its lines (only when the sequence needs more scratch than the limit are buffers reused, and then the
+// compute unit's and the L2's lines are dropped at every barrier). The wait is bounded: after `spin_limit` polls a workgroup sets *failed and every workgroup
 // exits at its next poll, so the kernel ends in any case; the host then reports the failure. All
 // workgroups must be resident together: the host checks the occupancy the runtime reports against the
 // grid before it launches.
