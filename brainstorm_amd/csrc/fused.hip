@@ -160,6 +160,9 @@ struct LstmBwdThinArgs {
     int64_t part_stride;
 };
 
+// PARTS: the number of slabs when it is 1, 2 or 4; 8 stands for "up to 8" (a slab beyond the last one reads the
+// last one again and is not added).
+template <int PARTS>
 __global__ __launch_bounds__(256) void lstm_bwd_step_thin_kernel(LstmBwdThinArgs t, int act, int batch, unsigned n,
                                                                  unsigned col_tiles) {
     __shared__ float turn[4][8][33];
@@ -173,14 +176,14 @@ __global__ __launch_bounds__(256) void lstm_bwd_step_thin_kernel(LstmBwdThinArgs
         const unsigned j = j0 + tx;
         if (b < batch && j < n) {
             const int64_t e = static_cast<int64_t>(b) * n + j;
-            // all partial products are requested before the first is used (a slab beyond the last one
-            // reads the last one again and is not added)
-            float part[kThinMaxParts];
+            // all partial products are requested before the first is used
+            float part[PARTS];
 #pragma unroll
-            for (int p = 0; p < kThinMaxParts; ++p) part[p] = ldg(a.dy + (p < t.parts ? p : t.parts - 1) * t.part_stride + e);
+            for (int p = 0; p < PARTS; ++p)
+                part[p] = ldg(a.dy + (PARTS < kThinMaxParts || p < t.parts ? p : t.parts - 1) * t.part_stride + e);
             float rec = part[0];
 #pragma unroll
-            for (int p = 1; p < kThinMaxParts; ++p) rec = p < t.parts ? rec + part[p] : rec;
+            for (int p = 1; p < PARTS; ++p) rec = (PARTS < kThinMaxParts || p < t.parts) ? rec + part[p] : rec;
             const float dy = ldg(a.deltas + e) + rec;
             a.dy_out[e] = dy;
             const LstmBwdCell c = lstm_cell_backward(a, act, e, j, dy);
@@ -674,9 +677,17 @@ int bship_lstm_bwd_step_thin_f32(int act, int64_t batch, int64_t n, const float*
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: batch %lld (at most 128), parts %d (1..8), part_stride %lld",
                          __func__, (long long)batch, parts, (long long)part_stride);
     const int64_t row_tiles = ceil_div(batch, 8), col_tiles = ceil_div(n, 32);
-    hipLaunchKernelGGL(lstm_bwd_step_thin_kernel, dim3(static_cast<unsigned>(row_tiles * col_tiles)), dim3(256), 0,
-                       ctx().stream, t, act, static_cast<int>(batch), static_cast<unsigned>(n),
-                       static_cast<unsigned>(col_tiles));
+    const dim3 grid(static_cast<unsigned>(row_tiles * col_tiles));
+#define BSHIP_THIN_STEP(P_)                                                                                        \
+    hipLaunchKernelGGL(lstm_bwd_step_thin_kernel<P_>, grid, dim3(256), 0, ctx().stream, t, act, static_cast<int>(batch), \
+                       static_cast<unsigned>(n), static_cast<unsigned>(col_tiles))
+    switch (parts) {
+        case 1: BSHIP_THIN_STEP(1); break;
+        case 2: BSHIP_THIN_STEP(2); break;
+        case 4: BSHIP_THIN_STEP(4); break;
+        default: BSHIP_THIN_STEP(8); break;
+    }
+#undef BSHIP_THIN_STEP
     return check_launch("lstm_backward_step_thin");
 }
 
