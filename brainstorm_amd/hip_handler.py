@@ -1011,8 +1011,8 @@ class HipHandler(Handler):
         """The whole forward recurrence of lstm_layer.py:115-145 in one launch: Za, Ia, Fa, Oa hold the
         input products on entry; every array is (time + 1, batch, n) with its context slot last; R_all is
         the stacked (4n, n) recurrent matrix (stack_adjacent). Returns False, with nothing done, when the
-        shape does not fit the kernel (n % 4, batch > 128, n > 1024, or more workgroups than the device
-        holds at once): the caller then takes the step-by-step path. Raises BshipError (status
+        shape does not fit the kernel (n % 4, batch > 128, n > 1024, or fewer compute units than
+        n / 4): the caller then takes the step-by-step path. Raises BshipError (status
         BSHIP_ERR_TIMEOUT) if the workgroups did not meet at a time step's barrier. Waits for the
         device."""
         steps = Za.shape[0] - 1

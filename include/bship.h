@@ -384,13 +384,13 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
  * (time_steps + 1, batch, n), dense; slab `time_steps` is the context slot that y[t-1] and
  * Ca[t-1] mean at t = 0. R_all is the stacked (4n, n) matrix [Rz; Ri; Rf; Ro] (the four matrices
  * are adjacent in the layer's parameter vector). The recurrent weights stay in LDS for the whole
- * sequence, one workgroup per 4 hidden units and per group of up to 64 batch rows (a larger batch
- * runs as two independent groups), and the workgroups of a group meet at one grid barrier per
- * time step whose wait is bounded (BSHIP_GRID_BARRIER_SPINS polls, default 2^21): if it runs out,
- * e.g. because other work kept some workgroups off the device, every workgroup exits, the call
- * returns BSHIP_ERR_TIMEOUT and the buffers hold an unfinished pass. Needs n % 4 == 0,
- * batch <= 128, n <= 1024 and all workgroups resident together (two per compute unit need
- * n <= 1008 for a batch above 64); otherwise BSHIP_ERR_UNSUPPORTED before anything is launched.
+ * sequence, one workgroup per 4 hidden units on a compute unit of its own (a batch above 64 rows
+ * is two row sets of four wavefronts each in the same workgroup), and the workgroups meet at one
+ * grid barrier per time step whose wait is bounded (BSHIP_GRID_BARRIER_SPINS polls, default 2^21):
+ * if it runs out, e.g. because other work kept some workgroups off the device, every workgroup
+ * exits, the call returns BSHIP_ERR_TIMEOUT and the buffers hold an unfinished pass. Needs
+ * n % 4 == 0, batch <= 128, n <= 1024 and n / 4 workgroups resident together (one per compute
+ * unit); otherwise BSHIP_ERR_UNSUPPORTED before anything is launched.
  * Takes 4 KB + 512 bytes per hidden unit and time step from the pool for the flags and the
  * transposed operand, one buffer per time step so that no cache ever holds a stale line of it;
  * beyond BSHIP_LSTM_SEQ_SCRATCH_MB (default 256) megabytes the buffers are reused in turn and
