@@ -185,7 +185,16 @@ extern "C" int bship_dot_small_tn_f32(const float* aT, const float* b, float* c,
         return set_error(BSHIP_ERR_UNSUPPORTED, "%s: operands of 1 GiB and more are not addressed", __func__);
     if (M == 0 || N == 0) return 0;
     BSHIP_REQUIRE_PTR(c); BSHIP_REQUIRE_F32_ALIGNED(c);
-    if (K > 0) { BSHIP_REQUIRE_PTR(aT); BSHIP_REQUIRE_PTR(b); BSHIP_REQUIRE_F32_ALIGNED(aT); BSHIP_REQUIRE_F32_ALIGNED(b); }
+    if (K == 0) {
+        // an empty sum: zeros, without a launch that would build descriptors over nothing
+        for (int sp = 0; sp < splits; ++sp)
+            for (int64_t r = 0; r < M; ++r) {
+                const int st = launch_fill(c + sp * c_split_stride + r * ldc, 0.0f, static_cast<size_t>(N));
+                if (st != 0) return st;
+            }
+        return 0;
+    }
+    BSHIP_REQUIRE_PTR(aT); BSHIP_REQUIRE_PTR(b); BSHIP_REQUIRE_F32_ALIGNED(aT); BSHIP_REQUIRE_F32_ALIGNED(b);
     if ((reinterpret_cast<uintptr_t>(aT) & 15) != 0)
         return set_error(BSHIP_ERR_BAD_POINTER, "%s: the transposed operand must be aligned to 16 bytes", __func__);
     DotSmallArgs a;

@@ -84,6 +84,14 @@ def test_dot_small_tn_and_transpose_on_pitched_operands(hip):
     assert scaled_err(got[:, :, 2:2 + n].astype(np.float64).sum(axis=0), want) <= 1e-5
 
 
+def test_dot_small_tn_with_nothing_to_add_writes_zeros(hip):
+    out = hip.create_from_numpy(np.full((2, 5, 9), 3.0, F32))
+    lib = hip._lib
+    hip._call(lib.bship_dot_small_tn_f32(0, 0, out.ptr, 5, 7, 0, 7, 9, 2, 45))      # K = 0: no operands are read
+    got = hip.get_numpy_copy(out)
+    assert np.all(got[:, :, :7] == 0.0) and np.all(got[:, :, 7:] == 3.0)
+
+
 def test_dot_small_tn_is_deterministic_and_rejects_what_it_does_not_take(hip):
     rng = np.random.RandomState(3)
     a = rng.standard_normal((100, 4000)).astype(F32)
