@@ -1026,8 +1026,8 @@ class HipHandler(Handler):
             return False
         status = self._lib.bship_lstm_fwd_sequence_f32(
             self._ACT_CODES[activation], steps, batch, n, R_all.ptr, *[a.ptr for a in mats + vecs])
-        if status == _lib.ERR_UNSUPPORTED:
-            return False
+        if status in (_lib.ERR_UNSUPPORTED, _lib.ERR_OUT_OF_MEMORY):
+            return False            # nothing was launched (the scratch for the operand buffers did not fit the pool)
         self._call(status)
         return True
 
