@@ -5,8 +5,17 @@
 // networks issue the same small product thousands of times per step. The cache
 // holds the kMaxPlans most recently used shapes (workloads with varying batch or
 // sequence lengths would otherwise grow it without limit).
+//
+// Thin products (one side of the result at most 128 long: a batch of 100 rows against a weight
+// matrix) are where the library's heuristic is furthest from its own best kernel (measured on MI355X
+// for 100x4000 . 4000x1000: first choice 18.1 us, best of the offered 14.1 us), and they are issued
+// hundreds of times per step by recurrent layers. For those the candidates are timed once, on the
+// caller's operands and a scratch result, when the shape is first seen outside a recording
+// (BSHIP_GEMM_AUTOTUNE=0 keeps the heuristic's first choice).
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -55,10 +64,66 @@ void destroy_plan(GemmPlan& p) {
     p = GemmPlan();
 }
 
+// The operands of the call that creates a plan, for timing the candidates on them.
+struct TuneOperands { const float* a; const float* b; const float* bias; };
+
+// BSHIP_GEMM_AUTOTUNE: 0 = the heuristic's first choice, 2 = timed choice and a line on stderr per shape.
+int tune_mode() {
+    static const int mode = [] { const char* e = getenv("BSHIP_GEMM_AUTOTUNE"); return e && e[0] ? atoi(e) : 1; }();
+    return mode;
+}
+bool tune_verbose() { return tune_mode() >= 2; }
+
+// Index of the candidate that runs fastest: each is launched four times untimed and 32 times between two
+// events on the library's stream, into a scratch result (the caller's result may be an accumulator). The
+// heuristic's first choice is kept unless another candidate is more than 1 % faster.
+// Candidates that need more workspace than the library keeps are skipped; if the scratch block or an
+// event cannot be had, or a candidate fails, the heuristic's first choice stands.
+int fastest_candidate(const GemmPlan& p, const hipblasLtMatmulHeuristicResult_t* res, int found, const float* a,
+                      const float* b, const float* bias, int64_t c_elements) {
+    void* scratch = nullptr;
+    if (pool_alloc_raw(static_cast<size_t>(c_elements) * sizeof(float), &scratch) != 0 || scratch == nullptr) return 0;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int best = 0, fastest = 0;
+    if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+        if (bias) (void)hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+        const float alpha = 1.0f, beta = 0.0f;
+        float* c = static_cast<float*>(scratch);
+        float best_ms = 1e30f, first_ms = 1e30f;
+        hipStream_t stream = ctx().stream;
+        for (int i = 0; i < found; ++i) {
+            if (res[i].workspaceSize > kWorkspaceBytes) continue;
+            bool ok = true;
+            for (int r = 0; r < 36 && ok; ++r) {
+                if (r == 4) (void)hipEventRecord(e0, stream);
+                ok = hipblasLtMatmul(g_handle, p.desc, &alpha, a, p.la, b, p.lb, &beta, c, p.lc, c, p.lc, &res[i].algo,
+                                     g_workspace, kWorkspaceBytes, stream) == HIPBLAS_STATUS_SUCCESS;
+            }
+            float ms = 1e30f;
+            if (hipEventRecord(e1, stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+                ok = false;
+            if (i == 0 && ok) first_ms = ms;
+            if (ok && ms < best_ms) { best_ms = ms; best = i; fastest = i; }
+        }
+        // differences below one per cent are within the noise of 32 launches
+        if (best_ms > 0.99f * first_ms) best = 0;
+        if (tune_verbose())
+            fprintf(stderr, "bship product plan: %lld result elements, %d candidates, first choice %.2f us, fastest (no. %d) %.2f us -> no. %d\n",
+                    (long long)c_elements, found, first_ms * 1000.0f / 32.0f, fastest, best_ms * 1000.0f / 32.0f, best);
+        (void)hipGetLastError();
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    pool_free_raw(scratch);
+    return best;
+}
+
 // Column-major problem: D(m x n) = opA(A) opB(B), leading dimensions lda/ldb/ldc.
+// tune: time the candidates on these operands instead of taking the heuristic's first choice.
 // with_bias: the epilogue adds a vector of m elements to every column of D (the pointer is set per call).
 int make_plan(GemmPlan& p, hipblasOperation_t opa, hipblasOperation_t opb, int64_t m, int64_t n,
-              int64_t k, int64_t lda, int64_t ldb, int64_t ldc, bool with_bias) {
+              int64_t k, int64_t lda, int64_t ldb, int64_t ldc, bool with_bias, const TuneOperands* tune) {
     BSHIP_BLAS(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
     if (with_bias) {
         const uint32_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
@@ -78,18 +143,22 @@ int make_plan(GemmPlan& p, hipblasOperation_t opa, hipblasOperation_t opb, int64
     uint64_t ws = kWorkspaceBytes;
     hipblasStatus_t s = hipblasLtMatmulPreferenceSetAttribute(
         pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-    hipblasLtMatmulHeuristicResult_t res[1];
+    constexpr int kCandidates = 24;
+    hipblasLtMatmulHeuristicResult_t res[kCandidates];
     int found = 0;
+    const int want = tune ? kCandidates : 1;
     if (s == HIPBLAS_STATUS_SUCCESS)
-        s = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, res, &found);
+        s = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.la, p.lb, p.lc, p.lc, pref, want, res, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (s != HIPBLAS_STATUS_SUCCESS) return blas_error(s, "hipblasLtMatmulAlgoGetHeuristic");
     if (found < 1)
         return set_error(BSHIP_ERR_BLAS,
                          "hipBLASLt has no float32 algorithm for m=%lld n=%lld k=%lld opA=%d opB=%d",
                          (long long)m, (long long)n, (long long)k, (int)opa, (int)opb);
-    p.algo = res[0].algo;
-    p.workspace = res[0].workspaceSize;
+    int best = 0;
+    if (tune && found > 1) best = fastest_candidate(p, res, found, tune->a, tune->b, tune->bias, ldc * n);
+    p.algo = res[best].algo;
+    p.workspace = res[best].workspaceSize;
     return 0;
 }
 
@@ -129,8 +198,13 @@ static int gemm_impl(int transa, int transb, int64_t M, int64_t N, int64_t K, fl
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
         GemmPlan plan;
+        // thin and small enough that a few dozen trial runs cost milliseconds; not while a step is recorded
+        const bool autotune = tune_mode() >= 1;
+        const bool thin = (M <= 128 || N <= 128) && 2.0 * M * N * K <= 8e9 && M * N >= 1024;
+        const TuneOperands operands{B, A, bias};
         int st = make_plan(plan, transb ? HIPBLAS_OP_T : HIPBLAS_OP_N, transa ? HIPBLAS_OP_T : HIPBLAS_OP_N,
-                           N, M, K, ldb, lda, ldc, bias != nullptr);
+                           N, M, K, ldb, lda, ldc, bias != nullptr,
+                           autotune && thin && !graph_recording() ? &operands : nullptr);
         if (st != 0) { destroy_plan(plan); return st; }
         if (g_plans.size() >= kMaxPlans) {
             // drop the shape that has not been used for the longest time (launches already

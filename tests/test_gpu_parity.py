@@ -771,6 +771,30 @@ def test_dot_mm_with_operands_at_odd_elements(hip, ref):
                 assert np.max(np.abs(views[2].get() - want) / scale) <= 1e-5, (op, m, k, n, ta, tb, offs)
 
 
+def test_first_call_of_a_thin_product_touches_the_result_once(hip, ref):
+    # a thin shape is timed over several candidate kernels when it is first seen; those trial runs go to a
+    # scratch result, so an accumulating first call adds the product exactly once, and the later calls
+    # (cached choice) repeat the first bit for bit
+    rng = np.random.RandomState(31)
+    for (m, k, n), ta, tb in itertools.product([(100, 4003, 1001), (7, 333, 4001), (2003, 77, 96)], (False, True),
+                                               (False, True)):
+        a = rand(rng, (k, m) if ta else (m, k))
+        b = rand(rng, (n, k) if tb else (k, n))
+        out = rand(rng, (m, n)) * F32(100.0)
+        want = out.copy()
+        ref.dot_add_mm(a, b, want, ta, tb)
+        ad, bd = hip.create_from_numpy(a), hip.create_from_numpy(b)
+        results = []
+        for _ in range(3):
+            od = hip.create_from_numpy(out)
+            hip.dot_add_mm(ad, bd, od, ta, tb)
+            results.append(od.get())
+        scale = np.sqrt(k) + np.abs(want)
+        assert np.max(np.abs(results[0] - want) / scale) <= 1e-5, (m, k, n, ta, tb)
+        assert_bit_equal(results[1], results[0], "second call")
+        assert_bit_equal(results[2], results[0], "third call")
+
+
 # -------------------------------------------------------------- conv / pooling
 def _out_size(n, k, pad, stride):
     return (n + 2 * pad - k) // stride + 1
