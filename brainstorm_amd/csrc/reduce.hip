@@ -187,13 +187,20 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
 // The launcher guarantees N % W == 0 and N / W <= THREADS * PER.
 template <int W, bool AL, int BLOCK, int THREADS, int PER>
 __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, float* out, int64_t M,
-                                                            int64_t N, int64_t ldm, int64_t ldo) {
+                                                            int64_t N, int64_t ldm, int64_t ldo, unsigned chunk) {
     constexpr int ROWS = BLOCK / THREADS;
     constexpr int WAVES = BLOCK / kWave;
     typedef typename VecT<W>::type R;
     __shared__ float lds[2][WAVES];
     const int t = threadIdx.x % THREADS;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * ROWS + threadIdx.x / THREADS;
+    // chunk > 1: the eight workgroups that the dispatcher deals to the eight XCDs in turn take rows
+    // `chunk` apart, so that each XCD works on runs of `chunk` adjacent rows (see launch_softmax)
+    unsigned bid = blockIdx.x;
+    if (chunk > 1) {
+        const unsigned full = gridDim.x / (8 * chunk) * (8 * chunk);
+        if (bid < full) bid = (bid % 8) * chunk + (bid / 8) % chunk + (bid / (8 * chunk)) * (8 * chunk);
+    }
+    const int64_t row = static_cast<int64_t>(bid) * ROWS + threadIdx.x / THREADS;
     const bool live = row < M;
     const int64_t NW = N / W;
     const float* p = m + (live ? row : 0) * ldm;       // ldm, ldo: elements from one row to the next
@@ -286,24 +293,24 @@ __global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, fl
 
 template <int W, bool AL, int BLOCK, int THREADS>
 static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N, int64_t ldm,
-                               int64_t ldo) {
+                               int64_t ldo, unsigned chunk) {
     hipStream_t s = ctx().stream;
     const dim3 b(BLOCK);
     switch (per) {
-        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
-        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
-        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
-        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
-        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N, ldm, ldo); break;
+        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
+        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
+        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
+        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
+        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
     }
 }
 
 template <int BLOCK, int THREADS>
 static void launch_softmax_threads(bool vec, bool al, int per, dim3 grid, const float* m, float* out,
-                                   int64_t M, int64_t N, int64_t ldm, int64_t ldo) {
-    if (vec && al) launch_softmax_per<4, true, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
-    else if (vec)  launch_softmax_per<4, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
-    else           launch_softmax_per<1, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo);
+                                   int64_t M, int64_t N, int64_t ldm, int64_t ldo, unsigned chunk = 0) {
+    if (vec && al) launch_softmax_per<4, true, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo, chunk);
+    else if (vec)  launch_softmax_per<4, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo, chunk);
+    else           launch_softmax_per<1, false, BLOCK, THREADS>(per, grid, m, out, M, N, ldm, ldo, chunk);
 }
 
 constexpr int kWideBlock = 1024;
@@ -332,8 +339,17 @@ static int launch_softmax(const float* m, float* out, int64_t M, int64_t N, int6
     } else if (NW <= static_cast<int64_t>(kBlock) * BSHIP_SM_NARROW_MAX) {
         launch_softmax_threads<kBlock, kBlock>(vec, al, per_for(kBlock), dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo);
     } else if (NW <= static_cast<int64_t>(kWideBlock) * 16) {
+        // Rows a multiple of 64 KiB apart: with one row per workgroup in index order, an XCD (every
+        // eighth workgroup) would only ever see addresses that agree in bits 16-18, which costs 4-5 % at
+        // 16384 x 16384 (0.71 -> 0.74 of peak with runs of 512 KiB per XCD; other pitches lose with runs).
+        unsigned chunk = 0;
+        if ((ldm * 4) % 65536 == 0 && (ldo * 4) % 65536 == 0) {
+            const char* e = getenv("BSHIP_SM_CHUNK_KB");
+            const int64_t run = (e ? atoll(e) : 512) * 1024;
+            chunk = static_cast<unsigned>(std::max<int64_t>(1, run / (ldm * 4)));
+        }
         launch_softmax_threads<kWideBlock, kWideBlock>(vec, al, per_for(kWideBlock),
-                                                       dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo);
+                                                       dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo, chunk);
     } else {
         hipLaunchKernelGGL(softmax_long_kernel, dim3(static_cast<unsigned>(M)), dim3(kBlock), 0,
                            ctx().stream, m, out, M, N, ldm, ldo);

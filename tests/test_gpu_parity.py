@@ -447,7 +447,10 @@ def test_sum_t_is_deterministic(hip):
 def test_softmax_m(hip, ref):
     rng = np.random.RandomState(19)
     shapes = some_2d_shapes + ((100, 10), (10000, 205), (64, 64), (37, 1031), (16, 4096), (5, 5000),
-                               (3, 16384), (2, 70001), (2, 70000), (300, 256), (9, 1024), (9, 1025))
+                               (3, 16384), (2, 70001), (2, 70000), (300, 256), (9, 1024), (9, 1025),
+                               # rows 64 KiB or 128 KiB apart: workgroups take the rows in another order,
+                               # all of them, some of them and (3 rows) none
+                               (64, 16384), (100, 16384), (70, 32768))
     for shape in shapes:
         for scale in (1.0, 20.0):
             m = (rand(rng, shape) * scale).astype(F32)
