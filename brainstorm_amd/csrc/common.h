@@ -28,10 +28,23 @@ struct Context {
     int blocks_per_cu = 8;     // streaming kernels launch num_cus*blocks_per_cu blocks
     int colsum_blocks_per_cu = 3;   // column sums: row bands are chosen to reach this many workgroups per CU (measured optimum)
     size_t write_through_min = size_t(1) << 22;   // elements from which write-only kernels store write-through
+    size_t ew_run_bytes = size_t(512) << 10;      // elementwise kernels with two inputs: bytes per stream that an XCD takes in one run (BSHIP_EW_RUN_KB)
     char name[256] = {0};
 };
 
 Context& ctx();
+
+// The dispatcher deals consecutive workgroups of a 1-D grid to the 8 XCDs in turn. With run > 1
+// the tiles are renumbered so that each XCD takes runs of `run` adjacent tiles instead of every
+// eighth tile; the tiles beyond the last whole group of 8 runs keep their numbers.
+__device__ __forceinline__ unsigned xcd_run_tile(unsigned run) {
+    unsigned tile = blockIdx.x;
+    if (run > 1) {
+        const unsigned group = 8 * run;
+        if (tile < gridDim.x / group * group) tile = (tile % 8) * run + (tile / 8) % run + tile / group * group;
+    }
+    return tile;
+}
 
 // Records a formatted message for bship_last_error() and returns `code`.
 int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -22,10 +22,11 @@ constexpr size_t kTile = static_cast<size_t>(kBlock) * 4;   // floats per workgr
 // of its operands before it stores. VPL = 128-bit vectors per lane: 1 for the
 // cheap operations, more for the float64 transcendentals so that a wavefront
 // has enough loads in flight to hide its long arithmetic phase.
+// run: tiles that one XCD takes in a row (xcd_run_tile).
 template <int NIN, bool AL, int VPL, typename F>
 __global__ __launch_bounds__(kBlock) void ew_kernel(F f, const float* p0, const float* p1,
-                                                    const float* p2, float* out, size_t n) {
-    const size_t base = static_cast<size_t>(blockIdx.x) * (kTile * VPL) + threadIdx.x * 4;
+                                                    const float* p2, float* out, size_t n, unsigned run) {
+    const size_t base = static_cast<size_t>(xcd_run_tile(run)) * (kTile * VPL) + threadIdx.x * 4;
     f4 r0[VPL], r1[VPL], r2[VPL];
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
@@ -66,14 +67,19 @@ int launch_ew(const char* name, F f, const float* p0, const float* p1, const flo
     if (tiles > 0x7fffffffu)
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", name, n);
     const dim3 grid(static_cast<unsigned>(tiles));
+    // Measured on MI355X in the sweep, 2^28 and 2^26 elements: kernels with three or more streams (two
+    // inputs and the output) gain 2-2.5 % (sigmoid_deriv at 2^26: 7 %) when an XCD works on runs of
+    // 512 KiB-1 MiB per stream, kernels with one input lose 2-4 % with any run length, and runs of
+    // 256 KiB (which leave an XCD with addresses that agree in bits 18-20) cost every kernel 4-5 %.
+    const unsigned run = NIN >= 2 ? static_cast<unsigned>(ctx().ew_run_bytes / (kTile * VPL * sizeof(float))) : 0;
     bool al = aligned16(p0) && aligned16(out) && (NIN < 2 || aligned16(p1)) &&
               (NIN < 3 || aligned16(p2));
     if (al)
         hipLaunchKernelGGL((ew_kernel<NIN, true, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
-                           p0, p1, p2, out, n);
+                           p0, p1, p2, out, n, run);
     else
         hipLaunchKernelGGL((ew_kernel<NIN, false, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
-                           p0, p1, p2, out, n);
+                           p0, p1, p2, out, n, run);
     return check_launch(name);
 }
 

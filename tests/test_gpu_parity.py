@@ -25,7 +25,9 @@ F32 = np.float32
 some_2d_shapes = ((1, 1), (4, 1), (1, 4), (5, 5), (3, 4), (4, 3))
 some_nd_shapes = ((1, 1, 4), (1, 1, 3, 3), (3, 4, 2, 1))
 # ... plus shapes that exercise whole tiles, tile tails and odd row lengths
-big_shapes = ((64, 64), (37, 1031), (4096,), (3, 5000), (1000, 205), (100, 1200), (513, 2048))
+# ((1201, 2049): 2404 tiles of 1024 floats, i.e. two whole groups of tiles that the kernels with two
+# inputs deal to the XCDs in runs, and a rest that keeps its order)
+big_shapes = ((64, 64), (37, 1031), (4096,), (3, 5000), (1000, 205), (100, 1200), (513, 2048), (1201, 2049))
 
 
 def rand(rng, shape):
