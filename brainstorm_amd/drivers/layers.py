@@ -356,12 +356,17 @@ class Lstm(Layer):
         y = buffers.outputs["default"]
         deltas = buffers.output_deltas["default"]
 
-        dy = _h.allocate(y.shape)          # zeros: dy[-1] is read below without ever being written
+        # arbitrary content where the handler can allocate that: every time step of dy is written before
+        # it is read; dy[-1], the slot behind the last step, is read below without ever being written
+        empty = getattr(_h, "empty", _h.allocate)
+        dy = empty(y.shape)
+        _h.fill(dy[-1], 0.0)
         _h.fill(dCa, 0.0)
         time_size = x.shape[0]
         fused = self._use_fused()
         R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
         batch = x.shape[1]
+        packed_all = None
         thin = R_all is not None and self.fused == "thin" and hasattr(_h, "dot_small_tn") and batch <= 128
         if thin:
             # the same, transposed ((4n, 128), columns beyond the batch stay zero), and the partial
@@ -372,8 +377,20 @@ class Lstm(Layer):
             splits = max(1, min(8, _h.device_info()[1] // groups))
             parts = _h.allocate((splits, batch, n) if splits > 1 else (batch, n))
         elif R_all is not None:
-            # [dZa|dIa|dFa|dOa] of the step after the current one, double-buffered; zero beyond the end
-            packed = [_h.allocate((x.shape[1], 4 * self.size)) for _ in range(2)]
+            # [dZa|dIa|dFa|dOa] of the step after the current one; zero beyond the end. When the input
+            # weights, their gradients, the recurrent gradients and the bias gradients are stacked in
+            # memory like R_all, the packed deltas of all steps are kept and the products and sums over
+            # time below become one each instead of one per gate (same terms, summed in the order of
+            # one product instead of four); otherwise two buffers alternate.
+            stacks = [_h.stack_adjacent(list(group)) for group in
+                      ((Wz, Wi, Wf, Wo), (dWz, dWi, dWf, dWo), (dRz, dRi, dRf, dRo), (dbz, dbi, dbf, dbo))]
+            if all(a is not None for a in stacks):
+                W_all, dW_all, dR_all, db_all = stacks
+                packed_all = empty((time_size + 1, batch, 4 * self.size))
+                _h.fill(packed_all[time_size], 0.0)
+                packed = None
+            else:
+                packed = [_h.allocate((x.shape[1], 4 * self.size)) for _ in range(2)]
         # the backward product packed[t+1] . R_all reads the weights against their rows; with a handler
         # that can transpose, it is given R_all^T and transb instead (same product; on MI355X the
         # library's kernel for that layout takes 16 us per step instead of 20)
@@ -392,11 +409,13 @@ class Lstm(Layer):
                 continue
             if R_all is not None:
                 dy_t = dy[t]
+                packed_next = packed_all[t + 1] if packed_all is not None else packed[(t + 1) % 2]
+                packed_now = packed_all[t] if packed_all is not None else packed[t % 2]
                 if R_all_t is not None:
-                    _h.dot_mm(packed[(t + 1) % 2], R_all_t, dy_t, transb=True)
+                    _h.dot_mm(packed_next, R_all_t, dy_t, transb=True)
                 else:
-                    _h.dot_mm(packed[(t + 1) % 2], R_all, dy_t)
-                _h.lstm_backward_step_packed(self.activation, deltas[t], dy_t, packed[t % 2],
+                    _h.dot_mm(packed_next, R_all, dy_t)
+                _h.lstm_backward_step_packed(self.activation, deltas[t], dy_t, packed_now,
                                              Zb[t], Ib[t], Fb[t], Ob[t], Cb[t], Ca[t - 1],
                                              Fb[t + 1], dIa[t + 1], dFa[t + 1], dCa[t + 1],
                                              dZa[t], dZb[t], dIa[t], dIb[t], dFa[t], dFb[t],
@@ -450,29 +469,37 @@ class Lstm(Layer):
         flat_dZa = flatten_time(dZa[:-1])
 
         # input deltas and input-weight gradients
-        _h.dot_add_mm(flat_dIa, Wi, flat_dinputs)
-        _h.dot_add_mm(flat_dFa, Wf, flat_dinputs)
-        _h.dot_add_mm(flat_dOa, Wo, flat_dinputs)
-        _h.dot_add_mm(flat_dZa, Wz, flat_dinputs)
-        _h.dot_add_mm(flat_dIa, flat_inputs, dWi, transa=True)
-        _h.dot_add_mm(flat_dFa, flat_inputs, dWf, transa=True)
-        _h.dot_add_mm(flat_dOa, flat_inputs, dWo, transa=True)
-        _h.dot_add_mm(flat_dZa, flat_inputs, dWz, transa=True)
+        if packed_all is not None:
+            flat_packed = flatten_time(packed_all[:-1])
+            _h.dot_add_mm(flat_packed, W_all, flat_dinputs)
+            _h.dot_add_mm(flat_packed, flat_inputs, dW_all, transa=True)
+            dbias_tmp = _h.allocate(db_all.shape)
+            _h.sum_t(flat_packed, axis=0, out=dbias_tmp)
+            _h.add_tt(db_all, dbias_tmp, db_all)
+        else:
+            _h.dot_add_mm(flat_dIa, Wi, flat_dinputs)
+            _h.dot_add_mm(flat_dFa, Wf, flat_dinputs)
+            _h.dot_add_mm(flat_dOa, Wo, flat_dinputs)
+            _h.dot_add_mm(flat_dZa, Wz, flat_dinputs)
+            _h.dot_add_mm(flat_dIa, flat_inputs, dWi, transa=True)
+            _h.dot_add_mm(flat_dFa, flat_inputs, dWf, transa=True)
+            _h.dot_add_mm(flat_dOa, flat_inputs, dWo, transa=True)
+            _h.dot_add_mm(flat_dZa, flat_inputs, dWz, transa=True)
 
-        dbias_tmp = _h.allocate(dbz.shape)
-        _h.sum_t(flat_dIa, axis=0, out=dbias_tmp)
-        _h.add_tt(dbi, dbias_tmp, dbi)
-        _h.sum_t(flat_dFa, axis=0, out=dbias_tmp)
-        _h.add_tt(dbf, dbias_tmp, dbf)
-        _h.sum_t(flat_dOa, axis=0, out=dbias_tmp)
-        _h.add_tt(dbo, dbias_tmp, dbo)
-        _h.sum_t(flat_dZa, axis=0, out=dbias_tmp)
-        _h.add_tt(dbz, dbias_tmp, dbz)
+            dbias_tmp = _h.allocate(dbz.shape)
+            _h.sum_t(flat_dIa, axis=0, out=dbias_tmp)
+            _h.add_tt(dbi, dbias_tmp, dbi)
+            _h.sum_t(flat_dFa, axis=0, out=dbias_tmp)
+            _h.add_tt(dbf, dbias_tmp, dbf)
+            _h.sum_t(flat_dOa, axis=0, out=dbias_tmp)
+            _h.add_tt(dbo, dbias_tmp, dbo)
+            _h.sum_t(flat_dZa, axis=0, out=dbias_tmp)
+            _h.add_tt(dbz, dbias_tmp, dbz)
 
         flat_outputs = flatten_time(y[:-2])
         flat_cell = flatten_time(Ca[:-2])
         flat_cell2 = flatten_time(Ca[:-1])
-        dWco_tmp = _h.allocate(flat_cell2.shape)
+        dWco_tmp = empty(flat_cell2.shape)            # written by the products below before it is read
         dWc_tmp = _h.allocate(dpo.shape)
         # output-gate peephole
         _h.mult_tt(flat_cell2, flat_dOa, dWco_tmp)
@@ -484,17 +511,21 @@ class Lstm(Layer):
         flat_dOa = flatten_time(dOa[1:-1])
         flat_dZa = flatten_time(dZa[1:-1])
         # recurrent-weight gradients
-        _h.dot_add_mm(flat_dIa, flat_outputs, dRi, transa=True)
-        _h.dot_add_mm(flat_dFa, flat_outputs, dRf, transa=True)
-        _h.dot_add_mm(flat_dOa, flat_outputs, dRo, transa=True)
-        _h.dot_add_mm(flat_dZa, flat_outputs, dRz, transa=True)
-        _h.dot_add_mm(dIa[0], dy[-1], dRi, transa=True)
-        _h.dot_add_mm(dFa[0], dy[-1], dRf, transa=True)
-        _h.dot_add_mm(dOa[0], dy[-1], dRo, transa=True)
-        _h.dot_add_mm(dZa[0], dy[-1], dRz, transa=True)
+        if packed_all is not None:
+            _h.dot_add_mm(flatten_time(packed_all[1:-1]), flat_outputs, dR_all, transa=True)
+            _h.dot_add_mm(packed_all[0], dy[-1], dR_all, transa=True)
+        else:
+            _h.dot_add_mm(flat_dIa, flat_outputs, dRi, transa=True)
+            _h.dot_add_mm(flat_dFa, flat_outputs, dRf, transa=True)
+            _h.dot_add_mm(flat_dOa, flat_outputs, dRo, transa=True)
+            _h.dot_add_mm(flat_dZa, flat_outputs, dRz, transa=True)
+            _h.dot_add_mm(dIa[0], dy[-1], dRi, transa=True)
+            _h.dot_add_mm(dFa[0], dy[-1], dRf, transa=True)
+            _h.dot_add_mm(dOa[0], dy[-1], dRo, transa=True)
+            _h.dot_add_mm(dZa[0], dy[-1], dRz, transa=True)
 
         # input- and forget-gate peepholes
-        dWcif_tmp = _h.allocate(flat_cell.shape)
+        dWcif_tmp = empty(flat_cell.shape)
         _h.mult_tt(flat_cell, flat_dIa, dWcif_tmp)
         _h.sum_t(dWcif_tmp, axis=0, out=dWc_tmp)
         _h.add_tt(dpi, dWc_tmp, dpi)

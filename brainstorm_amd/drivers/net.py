@@ -74,13 +74,18 @@ class Net:
         n_params = len(items)
         for key, shape, _, _ in list(items[:n_params]):
             items.append((("grad",) + key[1:], shape, True, 0))
+        rest = []
         for name, (outputs, _, internals) in self.specs.items():
             for o, buf in outputs.items():
-                items.append((("out", name, o), buf.shape(time_size, batch_size), False, buf.context))
-                items.append((("delta", name, o), buf.shape(time_size, batch_size), True, buf.context))
+                rest.append((("out", name, o), buf.shape(time_size, batch_size), False, buf.context))
+                rest.append((("delta", name, o), buf.shape(time_size, batch_size), True, buf.context))
             for i, buf in internals.items():
-                items.append((("internal", name, i), buf.shape(time_size, batch_size), buf.backward_only,
-                              buf.context if buf.scales == "TB" else 0))
+                rest.append((("internal", name, i), buf.shape(time_size, batch_size), buf.backward_only,
+                             buf.context if buf.scales == "TB" else 0))
+        # the backward-only buffers lie together, behind the gradients, so that one fill clears them all
+        # (the reference sorts its buffers into hubs by kind as well, structure/layout.py, and clears
+        # each backward-only hub with one fill, structure/buffers.py:147-150)
+        items += [it for it in rest if it[2]] + [it for it in rest if not it[2]]
         return items
 
     def resize(self, time_size, batch_size):
@@ -94,20 +99,23 @@ class Net:
         self.full_buffer = self.handler.allocate((total,))
         views, offset = {}, 0
         self._backward_only, self._with_context = [], []
+        runs = []                                  # [first, end) of adjacent backward-only buffers
         for key, shape, backward_only, context in items:
             n = _prod(shape)
             view = self.full_buffer[offset:offset + n].reshape(shape)
             views[key] = view
-            if backward_only and key[0] != "grad":
-                self._backward_only.append(view)
+            if backward_only and n:
+                if runs and runs[-1][1] == offset:
+                    runs[-1][1] = offset + n
+                else:
+                    runs.append([offset, offset + n])
             if context:
                 self._with_context.append((view, context))
             offset += n
         n_param = sum(_prod(s) for k, s, _, _ in items if k[0] == "param")
         self.parameters = self.full_buffer[0:n_param]
         self.gradients = self.full_buffer[n_param:2 * n_param]
-        if n_param:
-            self._backward_only.insert(0, self.gradients)        # the gradients hub is one fill
+        self._backward_only = [self.full_buffer[first:end] for first, end in runs]
         self.time_size, self.batch_size = time_size, batch_size
         self.buffers = OrderedDict()
         for name, (outputs, params, internals) in self.specs.items():

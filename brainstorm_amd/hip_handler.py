@@ -573,6 +573,13 @@ class HipHandler(Handler):
         self._call(self._lib.bship_malloc_scratch(n * 4, ctypes.byref(p)))
         return DeviceArray(p.value, tuple(shape), _Block(p.value, self._free), self)
 
+    def empty(self, shape):
+        """Like :meth:`allocate`, but with arbitrary content: for buffers that are overwritten completely
+        before they are read (allocate's zero fill of a large buffer is a pass over memory)."""
+        if isinstance(shape, (int, np.integer)):
+            shape = (int(shape),)
+        return self._scratch(tuple(int(s) for s in shape))
+
     def zeros(self, shape):
         return self.allocate(shape)
 
