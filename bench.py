@@ -39,12 +39,12 @@ F32 = np.float32
 # the same counters read for the sweep's 1 GiB copy_to (factors 2.000 and 0.999); the table and
 # the commands are in profiles/op_sweep_2p28_hbm_traffic.md. MiB per launch.
 MEASURED_TRAFFIC_MIB_2P28 = {
-    "add_tt": 3071.1, "mult_tt": 3071.1, "divide_tt": 3071.1, "mult_add_st": 3071.1,
-    "sigmoid_deriv": 3071.1, "tanh_deriv": 3071.1, "rel_deriv": 3071.1,
-    "sigmoid": 2047.2, "tanh": 2047.2, "log_t": 2047.2, "rel": 2047.7, "clip_t": 2047.2,
-    "sqrt_t": 2047.2, "copy_to": 2048.0, "fill": 1023.2, "softmax_m": 2047.9,
-    "add_mv_row": 2047.2, "mult_mv_row": 2047.2, "add_mv_col": 2049.5, "mult_mv_col": 2049.3,
-    "sum_t_axis0": 1024.8, "sum_t_axis1": 1024.5, "sum_t_all": 1024.1, "binarize_v": 1024.2,
+    "add_tt": 3071.3, "mult_tt": 3071.3, "divide_tt": 3071.3, "mult_add_st": 3071.3,
+    "sigmoid_deriv": 3071.3, "tanh_deriv": 3071.3, "rel_deriv": 3071.3,
+    "sigmoid": 2047.4, "tanh": 2047.4, "log_t": 2047.4, "rel": 2048.0, "clip_t": 2047.4,
+    "sqrt_t": 2047.3, "copy_to": 2048.0, "fill": 1023.4, "softmax_m": 2050.4,
+    "add_mv_row": 2047.4, "mult_mv_row": 2047.4, "add_mv_col": 2049.4, "mult_mv_col": 2049.6,
+    "sum_t_axis0": 1024.8, "sum_t_axis1": 1024.5, "sum_t_all": 1024.1, "binarize_v": 1024.3,
 }
 
 
