@@ -1089,3 +1089,56 @@ def test_device_array_views_alias(hip):
     hip.fill(flat[3:5], 9.0)
     host.reshape(24)[3:5] = 9.0
     np.testing.assert_array_equal(base.get(), host)
+
+
+# ---------------------------------------------------------- environment switches
+_SWITCH_SCRIPT = r"""
+import hashlib, sys
+sys.path.insert(0, %r)
+import numpy as np
+from brainstorm_amd import HipHandler
+h = HipHandler(seed=0)
+rng = np.random.RandomState(5)
+a = rng.standard_normal((1201, 2049)).astype(np.float32)
+b = rng.standard_normal((1201, 2049)).astype(np.float32)
+ad, bd, od = h.create_from_numpy(a), h.create_from_numpy(b), h.allocate(a.shape)
+h.add_tt(ad, bd, od)
+print("ADD", hashlib.sha256(od.get().tobytes()).hexdigest())
+h.mult_add_tt(ad, bd, od)
+print("MULTADD", hashlib.sha256(od.get().tobytes()).hexdigest())
+m = rng.standard_normal((72, 16384)).astype(np.float32)
+md, sd = h.create_from_numpy(m), h.allocate(m.shape)
+h.softmax_m(md, sd)
+print("SOFTMAX", hashlib.sha256(sd.get().tobytes()).hexdigest())
+x = rng.standard_normal((100, 4003)).astype(np.float32)
+w = rng.standard_normal((4003, 1001)).astype(np.float32)
+out = h.allocate((100, 1001))
+h.dot_mm(h.create_from_numpy(x), h.create_from_numpy(w), out)
+err = np.abs(out.get() - x.astype(np.float64) @ w.astype(np.float64)).max()
+print("DOT_OK", bool(err <= 1e-5 * np.sqrt(4003) * 10))
+"""
+
+
+def _run_with(env_extra):
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", _SWITCH_SCRIPT % root], env=dict(os.environ, **env_extra),
+                         capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    return dict(line.split(" ", 1) for line in res.stdout.strip().splitlines()), res.stderr
+
+
+def test_launch_order_switches_leave_the_results_alone():
+    # the order in which tiles and rows are dealt to the XCDs is a matter of speed only: elementwise
+    # results and softmax rows are the same bits with and without it; the product's kernel choice may
+    # change the summation order, so products are held to the float64 value with either setting
+    default, _ = _run_with({})
+    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_GEMM_AUTOTUNE": "0"})
+    for key in ("ADD", "MULTADD", "SOFTMAX"):
+        assert default[key] == plain[key], key
+    assert default["DOT_OK"] == "True" and plain["DOT_OK"] == "True"
+    verbose, err = _run_with({"BSHIP_GEMM_AUTOTUNE": "2"})
+    assert verbose["DOT_OK"] == "True"
+    assert "bship product plan" in err
