@@ -33,7 +33,7 @@ template <bool ACC> struct MvDiv { __device__ float apply(float m, float v, floa
 template <int W, bool AL, bool ACC, int R, typename F>
 __global__ __launch_bounds__(kBlock) void mv_rowvec_kernel(F f, const float* m, const float* v,
                                                            float* out, int64_t M, int64_t NW,
-                                                           unsigned col_tiles) {
+                                                           unsigned col_tiles, bool through) {
     typedef typename VecT<W>::type T;
     const unsigned ct = blockIdx.x % col_tiles;
     const int64_t r0 = static_cast<int64_t>(blockIdx.x / col_tiles) * R;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kBlock) void mv_rowvec_kernel(F f, const float* m, 
     for (int u = 0; u < R; ++u) {
         if (r0 + u < M) {
             const int64_t e = ((r0 + u) * NW + c) * W;
-            vstore<W, AL>(out + e, vmap(f, a[u], vv, ACC ? o[u] : a[u]));
+            vstore<W, AL>(out + e, vmap(f, a[u], vv, ACC ? o[u] : a[u]), through);
         }
     }
 }
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void mv_rowvec_kernel(F f, const float* m, 
 template <int W, bool AL, bool ACC, typename F>
 __global__ __launch_bounds__(kBlock) void mv_colvec_kernel(F f, const float* m, const float* v,
                                                            float* out, int64_t M, int64_t NW,
-                                                           unsigned tiles_per_row) {
+                                                           unsigned tiles_per_row, bool through) {
     typedef typename VecT<W>::type T;
     const int64_t row = blockIdx.x / tiles_per_row;
     const int64_t c = static_cast<int64_t>(blockIdx.x % tiles_per_row) * kBlock + threadIdx.x;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kBlock) void mv_colvec_kernel(F f, const float* m, 
     const T a = vload<W, AL>(m + e);
     T o = a;
     if (ACC) o = vload<W, AL>(out + e);
-    vstore<W, AL>(out + e, vmap(f, a, splat(a, s), o));
+    vstore<W, AL>(out + e, vmap(f, a, splat(a, s), o), through);
 }
 
 // rows per workgroup; measured at 8192^2 / 16384^2: add_mv 0.79/0.76 of peak with 1 row,
@@ -88,6 +88,7 @@ int launch_mv(const char* name, F f, const float* m, const float* v, float* out,
     const int64_t NW = vec ? N / 4 : N;
     const dim3 blk(kBlock);
     const int64_t col_tiles = ceil_div(NW, kBlock);
+    const bool through = store_through(static_cast<size_t>(M) * static_cast<size_t>(N));
     if (!v_is_col) {
         const bool al = aligned16(m) && aligned16(out) && aligned16(v);
         const int64_t blocks = col_tiles * ceil_div(M, kMvRows);
@@ -96,11 +97,11 @@ int launch_mv(const char* name, F f, const float* m, const float* v, float* out,
         const dim3 grid(static_cast<unsigned>(blocks));
         const unsigned ctl = static_cast<unsigned>(col_tiles);
         if (vec && al)
-            hipLaunchKernelGGL((mv_rowvec_kernel<4, true, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, true, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl, through);
         else if (vec)
-            hipLaunchKernelGGL((mv_rowvec_kernel<4, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
+            hipLaunchKernelGGL((mv_rowvec_kernel<4, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl, through);
         else
-            hipLaunchKernelGGL((mv_rowvec_kernel<1, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl);
+            hipLaunchKernelGGL((mv_rowvec_kernel<1, false, ACC, kMvRows, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, ctl, through);
     } else {
         const bool al = aligned16(m) && aligned16(out);
         const int64_t blocks = col_tiles * M;
@@ -109,11 +110,11 @@ int launch_mv(const char* name, F f, const float* m, const float* v, float* out,
         const dim3 grid(static_cast<unsigned>(blocks));
         const unsigned tpr = static_cast<unsigned>(col_tiles);
         if (vec && al)
-            hipLaunchKernelGGL((mv_colvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+            hipLaunchKernelGGL((mv_colvec_kernel<4, true, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr, through);
         else if (vec)
-            hipLaunchKernelGGL((mv_colvec_kernel<4, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+            hipLaunchKernelGGL((mv_colvec_kernel<4, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr, through);
         else
-            hipLaunchKernelGGL((mv_colvec_kernel<1, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr);
+            hipLaunchKernelGGL((mv_colvec_kernel<1, false, ACC, F>), grid, blk, 0, c.stream, f, m, v, out, M, NW, tpr, through);
     }
     return check_launch(name);
 }

@@ -88,6 +88,10 @@ int bship_init(int device) {
     if (cpc && atoi(cpc) > 0 && atoi(cpc) <= 64) g_ctx.colsum_blocks_per_cu = atoi(cpc);
     const char* wtm = getenv("BSHIP_WRITE_THROUGH_MIN");
     if (wtm && wtm[0]) g_ctx.write_through_min = static_cast<size_t>(strtoull(wtm, nullptr, 10));
+    const char* stm = getenv("BSHIP_STORE_THROUGH_MIN");
+    if (stm && stm[0]) g_ctx.store_through_min = static_cast<size_t>(strtoull(stm, nullptr, 10));
+    const char* stx = getenv("BSHIP_STORE_THROUGH_MAX");
+    if (stx && stx[0]) g_ctx.store_through_max = static_cast<size_t>(strtoull(stx, nullptr, 10));
     const char* erk = getenv("BSHIP_EW_RUN_KB");
     if (erk && erk[0]) g_ctx.ew_run_bytes = static_cast<size_t>(strtoull(erk, nullptr, 10)) << 10;
     g_ctx.device = device;

@@ -25,7 +25,7 @@ constexpr size_t kTile = static_cast<size_t>(kBlock) * 4;   // floats per workgr
 // run: tiles that one XCD takes in a row (xcd_run_tile).
 template <int NIN, bool AL, int VPL, typename F>
 __global__ __launch_bounds__(kBlock) void ew_kernel(F f, const float* p0, const float* p1,
-                                                    const float* p2, float* out, size_t n, unsigned run) {
+                                                    const float* p2, float* out, size_t n, unsigned run, bool through) {
     const size_t base = static_cast<size_t>(xcd_run_tile(run)) * (kTile * VPL) + threadIdx.x * 4;
     f4 r0[VPL], r1[VPL], r2[VPL];
 #pragma unroll
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kBlock) void ew_kernel(F f, const float* p0, const 
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 o[k] = f.apply(r0[u][k], NIN > 1 ? r1[u][k] : 0.0f, NIN > 2 ? r2[u][k] : 0.0f);
-            vstore<4, AL>(out + i, o);
+            vstore<4, AL>(out + i, o, through);
         } else {
             for (size_t j = i; j < n; ++j)     // the last, partial vector of the array
                 out[j] = f.apply(p0[j], NIN > 1 ? p1[j] : 0.0f, NIN > 2 ? p2[j] : 0.0f);
@@ -67,6 +67,7 @@ int launch_ew(const char* name, F f, const float* p0, const float* p1, const flo
     if (tiles > 0x7fffffffu)
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", name, n);
     const dim3 grid(static_cast<unsigned>(tiles));
+    const bool through = store_through(n);
     // Measured on MI355X in the sweep, 2^28 and 2^26 elements: kernels with three or more streams (two
     // inputs and the output) gain 2-2.5 % (sigmoid_deriv at 2^26: 7 %) when an XCD works on runs of
     // 512 KiB-1 MiB per stream, kernels with one input lose 2-4 % with any run length, and runs of
@@ -76,10 +77,10 @@ int launch_ew(const char* name, F f, const float* p0, const float* p1, const flo
               (NIN < 3 || aligned16(p2));
     if (al)
         hipLaunchKernelGGL((ew_kernel<NIN, true, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
-                           p0, p1, p2, out, n, run);
+                           p0, p1, p2, out, n, run, through);
     else
         hipLaunchKernelGGL((ew_kernel<NIN, false, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f,
-                           p0, p1, p2, out, n, run);
+                           p0, p1, p2, out, n, run, through);
     return check_launch(name);
 }
 

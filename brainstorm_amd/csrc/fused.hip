@@ -211,7 +211,7 @@ constexpr int kFusedRows = 2;   // as kMvRows of the matrix-vector kernels
 
 template <int W, bool AL, typename Body>
 __global__ __launch_bounds__(kBlock) void rowvec_fused_kernel(Body b, int64_t M, int64_t NW,
-                                                              unsigned col_tiles) {
+                                                              unsigned col_tiles, bool through) {
     typedef typename VecT<W>::type T;
     constexpr int KV = Body::kVecs > 0 ? Body::kVecs : 1;
     constexpr int R = kFusedRows;
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(kBlock) void rowvec_fused_kernel(Body b, int64_t M,
                 }
             }
 #pragma unroll
-            for (int k = 0; k < Body::kOut; ++k) vstore<W, AL>(b.outs[k] + e, o[k]);
+            for (int k = 0; k < Body::kOut; ++k) vstore<W, AL>(b.outs[k] + e, o[k], through);
         }
     }
 }
@@ -280,18 +280,19 @@ int launch_rowvec_fused(const char* name, const Body& b, int64_t M, int64_t N) {
     const dim3 grid(static_cast<unsigned>(blocks)), blk(kBlock);
     const unsigned ctl = static_cast<unsigned>(col_tiles);
     hipStream_t s = ctx().stream;
+    const bool through = store_through(static_cast<size_t>(M) * static_cast<size_t>(N));
     // (runs of adjacent tiles per XCD, which help the flat kernels below, cost these 2-4 %: measured on
     // the batch normalisation passes at 2048 x 4096 and 8192 x 8192)
-    if (vec && al) hipLaunchKernelGGL((rowvec_fused_kernel<4, true, Body>), grid, blk, 0, s, b, M, NW, ctl);
-    else if (vec)  hipLaunchKernelGGL((rowvec_fused_kernel<4, false, Body>), grid, blk, 0, s, b, M, NW, ctl);
-    else           hipLaunchKernelGGL((rowvec_fused_kernel<1, false, Body>), grid, blk, 0, s, b, M, NW, ctl);
+    if (vec && al) hipLaunchKernelGGL((rowvec_fused_kernel<4, true, Body>), grid, blk, 0, s, b, M, NW, ctl, through);
+    else if (vec)  hipLaunchKernelGGL((rowvec_fused_kernel<4, false, Body>), grid, blk, 0, s, b, M, NW, ctl, through);
+    else           hipLaunchKernelGGL((rowvec_fused_kernel<1, false, Body>), grid, blk, 0, s, b, M, NW, ctl, through);
     return check_launch(name);
 }
 
 // Flat arrays: one workgroup per tile of 1024 floats, one 128-bit vector per lane
 // and operand; the array's last, partial vector is handled element by element.
 template <bool AL, typename Body>
-__global__ __launch_bounds__(kBlock) void flat_fused_kernel(Body b, size_t n, unsigned run) {
+__global__ __launch_bounds__(kBlock) void flat_fused_kernel(Body b, size_t n, unsigned run, bool through) {
     const size_t i = (static_cast<size_t>(xcd_run_tile(run)) * kBlock + threadIdx.x) * 4;
     if (i >= n) return;
     if (i + 4 <= n) {
@@ -308,7 +309,7 @@ __global__ __launch_bounds__(kBlock) void flat_fused_kernel(Body b, size_t n, un
             for (int k = 0; k < Body::kOut; ++k) o[k][q] = os[k];
         }
 #pragma unroll
-        for (int k = 0; k < Body::kOut; ++k) vstore<4, AL>(b.outs[k] + i, o[k]);
+        for (int k = 0; k < Body::kOut; ++k) vstore<4, AL>(b.outs[k] + i, o[k], through);
     } else {
         for (size_t j = i; j < n; ++j) {
             float is[Body::kIn], os[Body::kOut];
@@ -333,8 +334,8 @@ int launch_flat_fused(const char* name, const Body& b, size_t n) {
     const dim3 grid(static_cast<unsigned>(tiles)), blk(kBlock);
     // three or more streams: an XCD takes runs of adjacent tiles, as in the elementwise kernels
     const unsigned run = Body::kIn + Body::kOut >= 3 ? static_cast<unsigned>(ctx().ew_run_bytes / (kBlock * 4 * sizeof(float))) : 0;
-    if (al) hipLaunchKernelGGL((flat_fused_kernel<true, Body>), grid, blk, 0, ctx().stream, b, n, run);
-    else    hipLaunchKernelGGL((flat_fused_kernel<false, Body>), grid, blk, 0, ctx().stream, b, n, run);
+    if (al) hipLaunchKernelGGL((flat_fused_kernel<true, Body>), grid, blk, 0, ctx().stream, b, n, run, store_through(n));
+    else    hipLaunchKernelGGL((flat_fused_kernel<false, Body>), grid, blk, 0, ctx().stream, b, n, run, store_through(n));
     return check_launch(name);
 }
 

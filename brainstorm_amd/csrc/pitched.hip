@@ -55,7 +55,7 @@ static inline int row_lanes_log2(int64_t cols) {
 template <int NIN, int VPL, typename F>
 __global__ __launch_bounds__(kBlock) void map2d_kernel(F f, Operand2d in0, Operand2d in1, Operand2d in2,
                                                        float* out, int64_t ldo, int64_t rows, int64_t cols,
-                                                       unsigned tiles_per_row, int L) {
+                                                       unsigned tiles_per_row, int L, bool through) {
     const int64_t row = (static_cast<int64_t>(blockIdx.x / tiles_per_row) << (8 - L)) + (threadIdx.x >> L);
     const int64_t c0 = ((static_cast<int64_t>(blockIdx.x % tiles_per_row) * VPL << L) + (threadIdx.x & ((1u << L) - 1))) * 4;
     if (row >= rows) return;
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kBlock) void map2d_kernel(F f, Operand2d in0, Opera
             f4 o;
 #pragma unroll
             for (int k = 0; k < 4; ++k) o[k] = f.apply(v0[u][k], v1[u][k], v2[u][k]);
-            vstore<4, false>(q, o);
+            vstore<4, false>(q, o, through);
         } else {
             for (int64_t j = 0; c + j < cols; ++j)
                 q[j] = f.apply(NIN > 0 ? load1(in0, row, c + j) : 0.0f, NIN > 1 ? load1(in1, row, c + j) : 0.0f,
@@ -108,12 +108,13 @@ static int launch_map2d(const char* name, F f, Operand2d in0, Operand2d in1, Ope
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %lld x %lld elements exceed one launch", name,
                          static_cast<long long>(rows), static_cast<long long>(cols));
     const dim3 grid(static_cast<unsigned>(tiles_per_row * row_groups));
+    const bool through = store_through(static_cast<size_t>(rows) * static_cast<size_t>(cols));
     if (wide)
         hipLaunchKernelGGL((map2d_kernel<NIN, VPL, F>), grid, dim3(kBlock), 0, ctx().stream, f, in0, in1, in2, out, ldo,
-                           rows, cols, static_cast<unsigned>(tiles_per_row), L);
+                           rows, cols, static_cast<unsigned>(tiles_per_row), L, through);
     else
         hipLaunchKernelGGL((map2d_kernel<NIN, 1, F>), grid, dim3(kBlock), 0, ctx().stream, f, in0, in1, in2, out, ldo,
-                           rows, cols, static_cast<unsigned>(tiles_per_row), L);
+                           rows, cols, static_cast<unsigned>(tiles_per_row), L, through);
     return check_launch(name);
 }
 

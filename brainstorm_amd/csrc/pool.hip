@@ -189,10 +189,10 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(float* __restrict__ p, flo
 
 template <bool AL>
 __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ s,
-                                                      float* __restrict__ d, size_t n) {
+                                                      float* __restrict__ d, size_t n, bool through) {
     const size_t i = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) * 4;
     if (i + 4 <= n) {
-        vstore<4, AL>(d + i, vload<4, AL>(s + i));
+        vstore<4, AL>(d + i, vload<4, AL>(s + i), through);
     } else {
         for (size_t j = i; j < n; ++j) d[j] = s[j];
     }
@@ -204,14 +204,14 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const float* __restrict__ 
 // start anywhere: the accesses promise 4-byte alignment only.
 __global__ __launch_bounds__(kBlock) void copy2d_kernel(const float* __restrict__ src, int64_t ld_src,
                                                         float* __restrict__ dst, int64_t ld_dst, int64_t rows,
-                                                        int64_t cols, unsigned tiles_per_row, int L) {
+                                                        int64_t cols, unsigned tiles_per_row, int L, bool through) {
     const int64_t row = (static_cast<int64_t>(blockIdx.x / tiles_per_row) << (8 - L)) + (threadIdx.x >> L);
     const int64_t c = ((static_cast<int64_t>(blockIdx.x % tiles_per_row) << L) + (threadIdx.x & ((1u << L) - 1))) * 4;
     if (row >= rows || c >= cols) return;
     const float* s = src + row * ld_src + c;
     float* d = dst + row * ld_dst + c;
     if (c + 4 <= cols) {
-        vstore<4, false>(d, vload<4, false>(s));
+        vstore<4, false>(d, vload<4, false>(s), through);
     } else {
         for (int64_t j = 0; c + j < cols; ++j) d[j] = s[j];
     }
@@ -426,7 +426,7 @@ int bship_d2h(void* dst_host, const void* src, size_t nbytes) {
             } else {
                 hipLaunchKernelGGL(copy_kernel<false>, dim3(static_cast<unsigned>((n + kCopyTile - 1) / kCopyTile)),
                                    dim3(kBlock), 0, ctx().stream, static_cast<const float*>(src),
-                                   static_cast<float*>(g_bounce_dev), n);
+                                   static_cast<float*>(g_bounce_dev), n, false);
                 int st = check_launch("read-back");
                 if (st != 0) return st;
                 BSHIP_HIP(hipStreamSynchronize(ctx().stream));
@@ -457,9 +457,9 @@ int bship_d2d(void* dst, const void* src, size_t nbytes) {
     const float* s = static_cast<const float*>(src);
     float* d = static_cast<float*>(dst);
     if (aligned16(s) && aligned16(d))
-        hipLaunchKernelGGL(copy_kernel<true>, grid, dim3(kBlock), 0, ctx().stream, s, d, n);
+        hipLaunchKernelGGL(copy_kernel<true>, grid, dim3(kBlock), 0, ctx().stream, s, d, n, store_through(n));
     else
-        hipLaunchKernelGGL(copy_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, s, d, n);
+        hipLaunchKernelGGL(copy_kernel<false>, grid, dim3(kBlock), 0, ctx().stream, s, d, n, store_through(n));
     return check_launch("copy_kernel");
 }
 
@@ -480,7 +480,8 @@ int bship_copy2d_f32(float* dst, int64_t ld_dst, const float* src, int64_t ld_sr
     const int64_t row_groups = ceil_div(rows, int64_t(1) << (8 - L));
     BSHIP_REQUIRE_DIM(tiles_per_row * row_groups <= 0x7fffffff);
     hipLaunchKernelGGL(copy2d_kernel, dim3(static_cast<unsigned>(tiles_per_row * row_groups)), dim3(kBlock), 0,
-                       ctx().stream, src, ld_src, dst, ld_dst, rows, cols, static_cast<unsigned>(tiles_per_row), L);
+                       ctx().stream, src, ld_src, dst, ld_dst, rows, cols, static_cast<unsigned>(tiles_per_row), L,
+                       store_through(static_cast<size_t>(rows) * static_cast<size_t>(cols)));
     return check_launch("copy2d");
 }
 

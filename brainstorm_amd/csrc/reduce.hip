@@ -187,7 +187,7 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
 // The launcher guarantees N % W == 0 and N / W <= THREADS * PER.
 template <int W, bool AL, int BLOCK, int THREADS, int PER>
 __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, float* out, int64_t M,
-                                                            int64_t N, int64_t ldm, int64_t ldo, unsigned chunk) {
+                                                            int64_t N, int64_t ldm, int64_t ldo, unsigned chunk, bool through) {
     constexpr int ROWS = BLOCK / THREADS;
     constexpr int WAVES = BLOCK / kWave;
     typedef typename VecT<W>::type R;
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_reg_kernel(const float* m, floa
             } else {
                 r = x[k] * inv;
             }
-            vstore<W, AL>(q + i * W, r);
+            vstore<W, AL>(q + i * W, r, through);
         }
     }
 }
@@ -294,14 +294,15 @@ __global__ __launch_bounds__(kBlock) void softmax_long_kernel(const float* m, fl
 template <int W, bool AL, int BLOCK, int THREADS>
 static void launch_softmax_per(int per, dim3 grid, const float* m, float* out, int64_t M, int64_t N, int64_t ldm,
                                int64_t ldo, unsigned chunk) {
+    const bool through = store_through(static_cast<size_t>(M) * static_cast<size_t>(N));
     hipStream_t s = ctx().stream;
     const dim3 b(BLOCK);
     switch (per) {
-        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
-        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
-        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
-        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
-        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk); break;
+        case 1:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 1>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk, through); break;
+        case 2:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 2>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk, through); break;
+        case 4:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 4>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk, through); break;
+        case 8:  hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 8>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk, through); break;
+        default: hipLaunchKernelGGL((softmax_reg_kernel<W, AL, BLOCK, THREADS, 16>), grid, b, 0, s, m, out, M, N, ldm, ldo, chunk, through); break;
     }
 }
 

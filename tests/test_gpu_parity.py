@@ -1131,11 +1131,13 @@ def _run_with(env_extra):
 
 
 def test_launch_order_switches_leave_the_results_alone():
-    # the order in which tiles and rows are dealt to the XCDs is a matter of speed only: elementwise
-    # results and softmax rows are the same bits with and without it; the product's kernel choice may
+    # the order in which tiles and rows are dealt to the XCDs and the kind of store (write-through for
+    # outputs of 2^18 to 2^26 elements, as the three here) are a matter of speed only: elementwise results
+    # and softmax rows are the same bits with and without them; the product's kernel choice may
     # change the summation order, so products are held to the float64 value with either setting
     default, _ = _run_with({})
-    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_GEMM_AUTOTUNE": "0"})
+    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_GEMM_AUTOTUNE": "0",
+                          "BSHIP_STORE_THROUGH_MIN": str(2 ** 40)})
     for key in ("ADD", "MULTADD", "SOFTMAX"):
         assert default[key] == plain[key], key
     assert default["DOT_OK"] == "True" and plain["DOT_OK"] == "True"
