@@ -434,6 +434,7 @@ struct CenterSquareSrc {
     const float* x;
     const float* mu;
     float* centered;
+    bool through;           // store centered write-through (store_through of the matrix size)
     bool aligned() const { return aligned16(x) && aligned16(mu) && aligned16(centered); }
     template <int W, bool AL> __device__ typename VecT<W>::type prep(int64_t col) const {
         return vload<W, AL>(mu + col);
@@ -441,7 +442,7 @@ struct CenterSquareSrc {
     template <int W, bool AL>
     __device__ typename VecT<W>::type load(int64_t off, typename VecT<W>::type m) const {
         const typename VecT<W>::type c = vload<W, AL>(x + off) + m;
-        vstore<W, AL>(centered + off, c);
+        vstore<W, AL>(centered + off, c, through);
         return c * c;
     }
 };
@@ -806,7 +807,8 @@ int bship_batchnorm_fwd_f32(int training, const float* inputs, const float* gamm
     hipLaunchKernelGGL(bn_mean_update_kernel, vgrid, blk, 0, s, sigma_b, mu, neg_inv_m, dec, omd, N);
     if ((st = check_launch("batchnorm mean")) != 0) return st;
     // centered = inputs + mu_b while summing centered^2 down the columns
-    st = launch_colsum(CenterSquareSrc{inputs, sigma_b, centered}, sigma_b, M, N);
+    st = launch_colsum(CenterSquareSrc{inputs, sigma_b, centered,
+                                       store_through(static_cast<size_t>(M) * static_cast<size_t>(N))}, sigma_b, M, N);
     if (st != 0) return st;
     hipLaunchKernelGGL(bn_sigma_update_kernel, vgrid, blk, 0, s, sigma_b, sigma, inv_m, eps, dec, omd, N);
     if ((st = check_launch("batchnorm deviation")) != 0) return st;
