@@ -139,8 +139,12 @@ NATIVE_OPS = [
 
 
 @pytest.mark.parametrize("rows,width,cuts", [(37, 790, (3, 260, 517, 774)), (5, 40, (1, 8, 15, 22)),
-                                             (300, 4100, (4, 1028, 2052, 3076)), (9, 7600, (5, 2530, 5055, 7580))],
-                         ids=["257 columns at odd offsets", "7 columns", "1024 columns, aligned", "2525 columns"])
+                                             (300, 4100, (4, 1028, 2052, 3076)), (9, 7600, (5, 2530, 5055, 7580)),
+                                             # 260 x 1027 = 267 020 elements per slice: above the 2^18 from which
+                                             # the kernels store write-through, rows at odd offsets
+                                             (260, 4200, (3, 1030, 2057, 3084))],
+                         ids=["257 columns at odd offsets", "7 columns", "1024 columns, aligned", "2525 columns",
+                              "1027 columns at odd offsets, write-through size"])
 @pytest.mark.parametrize("name,call", NATIVE_OPS, ids=[n for n, _ in NATIVE_OPS])
 def test_row_pitched_kernels(php, name, call, rows, width, cuts):
     # the kernels that take row-pitched operands as they are: same bits as NumPy on strided views,
