@@ -777,9 +777,9 @@ def test_dot_mm_with_operands_at_odd_elements(hip, ref):
 
 
 def test_first_call_of_a_thin_product_touches_the_result_once(hip, ref):
-    # a thin shape is timed over several candidate kernels when it is first seen; those trial runs go to a
-    # scratch result, so an accumulating first call adds the product exactly once, and the later calls
-    # (cached choice) repeat the first bit for bit
+    # the first call of a shape makes its plan (with BSHIP_GEMM_AUTOTUNE set, after trial runs into a
+    # scratch result): an accumulating first call adds the product exactly once, and the later calls
+    # (cached plan) repeat the first bit for bit
     rng = np.random.RandomState(31)
     for (m, k, n), ta, tb in itertools.product([(100, 4003, 1001), (7, 333, 4001), (2003, 77, 96)], (False, True),
                                                (False, True)):
@@ -1113,9 +1113,19 @@ print("SOFTMAX", hashlib.sha256(sd.get().tobytes()).hexdigest())
 x = rng.standard_normal((100, 4003)).astype(np.float32)
 w = rng.standard_normal((4003, 1001)).astype(np.float32)
 out = h.allocate((100, 1001))
-h.dot_mm(h.create_from_numpy(x), h.create_from_numpy(w), out)
-err = np.abs(out.get() - x.astype(np.float64) @ w.astype(np.float64)).max()
+xd, wd = h.create_from_numpy(x), h.create_from_numpy(w)
+h.dot_mm(xd, wd, out)
+exact = x.astype(np.float64) @ w.astype(np.float64)
+err = np.abs(out.get() - exact).max()
 print("DOT_OK", bool(err <= 1e-5 * np.sqrt(4003) * 10))
+# the first call of another thin shape accumulates: with the timed choice of the product's kernel its
+# trial runs must not touch the result
+x2 = x[:, :3001].copy(); w2 = w[:3001, :997].copy()
+acc0 = rng.standard_normal((100, 997)).astype(np.float32) * np.float32(100)
+acc = h.create_from_numpy(acc0)
+h.dot_add_mm(h.create_from_numpy(x2), h.create_from_numpy(w2), acc)
+err = np.abs(acc.get() - (acc0 + x2.astype(np.float64) @ w2.astype(np.float64))).max()
+print("DOTADD_OK", bool(err <= 1e-5 * (np.sqrt(3001) * 10 + 400)))
 """
 
 
@@ -1136,11 +1146,12 @@ def test_launch_order_switches_leave_the_results_alone():
     # and softmax rows are the same bits with and without them; the product's kernel choice may
     # change the summation order, so products are held to the float64 value with either setting
     default, _ = _run_with({})
-    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_GEMM_AUTOTUNE": "0",
-                          "BSHIP_STORE_THROUGH_MIN": str(2 ** 40)})
+    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_STORE_THROUGH_MIN": str(2 ** 40)})
     for key in ("ADD", "MULTADD", "SOFTMAX"):
         assert default[key] == plain[key], key
-    assert default["DOT_OK"] == "True" and plain["DOT_OK"] == "True"
-    verbose, err = _run_with({"BSHIP_GEMM_AUTOTUNE": "2"})
-    assert verbose["DOT_OK"] == "True"
-    assert "bship product plan" in err
+    for res in (default, plain):
+        assert res["DOT_OK"] == "True" and res["DOTADD_OK"] == "True"
+    # the optional timed choice of a thin product's kernel: same bars, a line per shape on stderr
+    timed, err = _run_with({"BSHIP_GEMM_AUTOTUNE": "2"})
+    assert timed["DOT_OK"] == "True" and timed["DOTADD_OK"] == "True"
+    assert err.count("bship product plan") >= 2
