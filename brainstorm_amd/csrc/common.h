@@ -31,6 +31,7 @@ struct Context {
     // kernels that read and write store write-through when their output has between these many elements
     // (BSHIP_STORE_THROUGH_MIN, BSHIP_STORE_THROUGH_MAX): at least 1 MB, at most the 256 MB of the last-level cache
     size_t store_through_min = size_t(1) << 18, store_through_max = size_t(1) << 26;
+    size_t softmax_run_bytes = size_t(512) << 10;  // softmax rows a multiple of 64 KiB apart: bytes of adjacent rows that an XCD takes in one run (BSHIP_SM_CHUNK_KB)
     size_t ew_run_bytes = size_t(512) << 10;      // elementwise kernels with two inputs: bytes per stream that an XCD takes in one run (BSHIP_EW_RUN_KB)
     char name[256] = {0};
 };

@@ -92,6 +92,8 @@ int bship_init(int device) {
     if (stm && stm[0]) g_ctx.store_through_min = static_cast<size_t>(strtoull(stm, nullptr, 10));
     const char* stx = getenv("BSHIP_STORE_THROUGH_MAX");
     if (stx && stx[0]) g_ctx.store_through_max = static_cast<size_t>(strtoull(stx, nullptr, 10));
+    const char* smk = getenv("BSHIP_SM_CHUNK_KB");
+    if (smk && smk[0]) g_ctx.softmax_run_bytes = static_cast<size_t>(strtoull(smk, nullptr, 10)) << 10;
     const char* erk = getenv("BSHIP_EW_RUN_KB");
     if (erk && erk[0]) g_ctx.ew_run_bytes = static_cast<size_t>(strtoull(erk, nullptr, 10)) << 10;
     g_ctx.device = device;

@@ -345,9 +345,7 @@ static int launch_softmax(const float* m, float* out, int64_t M, int64_t N, int6
         // 16384 x 16384 (0.71 -> 0.74 of peak with runs of 512 KiB per XCD; other pitches lose with runs).
         unsigned chunk = 0;
         if ((ldm * 4) % 65536 == 0 && (ldo * 4) % 65536 == 0) {
-            const char* e = getenv("BSHIP_SM_CHUNK_KB");
-            const int64_t run = (e ? atoll(e) : 512) * 1024;
-            chunk = static_cast<unsigned>(std::max<int64_t>(1, run / (ldm * 4)));
+            chunk = static_cast<unsigned>(std::max<int64_t>(1, static_cast<int64_t>(ctx().softmax_run_bytes) / (ldm * 4)));
         }
         launch_softmax_threads<kWideBlock, kWideBlock>(vec, al, per_for(kWideBlock),
                                                        dim3(static_cast<unsigned>(M)), m, out, M, N, ldm, ldo, chunk);
