@@ -150,8 +150,8 @@ __device__ __forceinline__ void vstore_writeonly(float* p, typename VecT<W>::typ
     // stores, but does not know that this statement is one)
     else asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
-// Context::write_through_min is the element count from which write-only kernels use it: below,
-// the data is likely to be read again soon and is better left to the default cache policy.
+// Context::write_through_min is the element count from which write-only kernels use it (16 MB; lowering it
+// to 1 MB changed none of the network workloads' step times).
 
 // Store of a kernel that reads as well: write-through when `through`, non-temporal otherwise. Outputs of
 // Context::store_through_min to store_through_max elements go through (store_through above): the
