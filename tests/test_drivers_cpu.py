@@ -204,3 +204,31 @@ def test_backward_clears_then_adds():
     np.testing.assert_allclose(net.get("Input", "output_deltas", "default"), first, rtol=1e-12)
     net.layers["fc"].backward_pass(net.buffers["fc"])   # a second layer pass alone adds on top
     assert not np.allclose(net.get("Input", "output_deltas", "default"), first)
+
+
+def test_backward_only_buffers_lie_together_and_one_fill_clears_them():
+    # gradients, deltas and the backward-only internals of every layer form one contiguous region of the
+    # flat buffer (the reference sorts its buffers into hubs by kind and clears each backward-only hub with
+    # one fill, structure/buffers.py:147-150); forward buffers keep their values through a backward pass
+    net, data, params = make_net([("lstm", Lstm(4), {"default": "Input.default"})], (3,), 2, time_steps=3)
+    assert len(net._backward_only) == 1
+    region = net._backward_only[0]
+    backward = [net.gradients] + [v for b in net.buffers.values() for v in b.output_deltas.values()]
+    is_backward = lambda layer, k: net.specs[layer][2][k].backward_only
+    backward += [v for layer, b in net.buffers.items() for k, v in b.internals.items() if is_backward(layer, k)]
+    assert all(np.shares_memory(region, v) for v in backward)
+    forward = [v for b in net.buffers.values() for v in b.outputs.values()] + [net.parameters]
+    forward += [v for layer, b in net.buffers.items() for k, v in b.internals.items() if not is_backward(layer, k)]
+    assert not any(np.shares_memory(region, v) for v in forward)
+    net.forward_pass(training_pass=True)
+    before = {name: {k: np.array(v, copy=True) for k, v in b.outputs.items()} for name, b in net.buffers.items()}
+    net.backward_pass()
+    assert np.any(net.handler.get_numpy_copy(net.gradients) != 0.0)
+    for name, outs in before.items():
+        for k, v in outs.items():
+            np.testing.assert_array_equal(net.handler.get_numpy_copy(net.buffers[name].outputs[k]), v)
+    net.handler.fill(region, 0.0)
+    assert not np.any(net.handler.get_numpy_copy(net.gradients))
+    for name, outs in before.items():
+        for k, v in outs.items():
+            np.testing.assert_array_equal(net.handler.get_numpy_copy(net.buffers[name].outputs[k]), v)
