@@ -392,6 +392,61 @@ __global__ __launch_bounds__(kBlock) void col2im_kernel(const float* __restrict_
     }
 }
 
+// The same for kh = kw = KS with stride 1, KS known at compile time: the covering positions are oy = y + pad -
+// (KS-1) + a, ox = x + pad - (KS-1) + b for a, b in [0, KS), so the KS*KS terms of an element are loaded
+// together (a term outside the col matrix reads a clamped address and is not added) and added in the same
+// scan order. With the run-time loops above a lane waits for each of its up to 25 loads in turn, which at
+// batch 100 (too few wavefronts to hide it) made the kernel 2.0 TB/s slow.
+template <int W, bool AL, int KS>
+__device__ __forceinline__ void col2im_ks_body(const float* __restrict__ col, float* __restrict__ in_deltas,
+                                               int64_t n, const ImgPlan& pl) {
+    const ImgGeom& g = pl.g;
+    uint32_t tile, group;
+    if (!img_block(pl, tile, group)) return;
+    const uint32_t p = tile * kBlock + threadIdx.x;
+    if (p >= pl.lanes_per_image) return;
+    uint32_t pix, chv, yy, xx;
+    pl.d_cv.divmod(p, pix, chv);
+    pl.d_w.divmod(pix, yy, xx);
+    const int oy_first = static_cast<int>(yy) + g.pad - (KS - 1), ox_first = static_cast<int>(xx) + g.pad - (KS - 1);
+    const int64_t kc = static_cast<int64_t>(KS) * KS * g.c;
+    const int64_t col_img = static_cast<int64_t>(g.oh) * g.ow * kc;
+    int off[KS * KS];
+    bool ok[KS * KS];
+#pragma unroll
+    for (int a = 0; a < KS; ++a)
+#pragma unroll
+        for (int b = 0; b < KS; ++b) {
+            const int oy = oy_first + a, ox = ox_first + b;
+            const bool in = oy >= 0 && oy < g.oh && ox >= 0 && ox < g.ow;
+            ok[a * KS + b] = in;
+            // ky = KS-1-a, kx = KS-1-b
+            off[a * KS + b] = in ? static_cast<int>((static_cast<int64_t>(oy) * g.ow + ox) * kc) +
+                                       ((KS - 1 - a) * KS + (KS - 1 - b)) * g.c
+                                 : 0;
+        }
+    for (int64_t img = group; img < n; img += pl.groups) {
+        float* q = in_deltas + img * pl.in_pitch + static_cast<int64_t>(p) * W;
+        const float* cimg = col + img * col_img + chv * W;
+        typename VecT<W>::type v[KS * KS];
+#pragma unroll
+        for (int i = 0; i < KS * KS; ++i) v[i] = img_load<W, AL>(cimg + off[i]);
+        typename VecT<W>::type acc = img_load<W, AL>(q);
+#pragma unroll
+        for (int i = 0; i < KS * KS; ++i)
+            if (ok[i]) acc += v[i];
+        img_store<W, AL>(q, acc);
+    }
+}
+#define BSHIP_COL2IM_KS_KERNEL(name, KS)                                                                   \
+    template <int W, bool AL>                                                                              \
+    __global__ __launch_bounds__(kBlock) void name(const float* __restrict__ col,                          \
+                                                   float* __restrict__ in_deltas, int64_t n, ImgPlan pl) { \
+        col2im_ks_body<W, AL, KS>(col, in_deltas, n, pl);                                                  \
+    }
+BSHIP_COL2IM_KS_KERNEL(col2im_kernel_k3, 3)
+BSHIP_COL2IM_KS_KERNEL(col2im_kernel_k5, 5)
+
 // col2im through LDS, for narrow channel counts: there a lane's 4*c-byte pieces of the col
 // matrix lie kh*kw*c floats apart and every cache line would be fetched several times.
 // A workgroup walks down a band of image rows, `rows` of them per phase. The col rows (oy) that
@@ -1300,8 +1355,21 @@ int bship_col2im_nhwc_pitched_f32(const float* col, float* in_deltas, int64_t in
         }
         (void)hipGetLastError();   // the attribute was refused: use the kernel without LDS
     }
-    BSHIP_LAUNCH_IMG_ORDER(col2im_kernel, "col2im", static_cast<int64_t>(h) * w,
-                           aligned16(col) && aligned16(in_deltas) && in_pitch % 4 == 0, true, col, in_deltas);
+    const bool al = aligned16(col) && aligned16(in_deltas) && in_pitch % 4 == 0;
+    // one image's col matrix must be addressable with 32-bit offsets for the compile-time windows
+    const bool small_image = static_cast<int64_t>(g.oh) * g.ow * kh * kw * c <= 0x7fffffff;
+    // for launches of up to 8 workgroups per compute unit: with more, enough wavefronts wait side by side and the
+    // plain loops are as fast (15x15x32, 5x5: batch 100 35.7 -> 18 us, CNN step 0.457 -> 0.437 ms; batch 2048
+    // 0.756 against 0.751 of peak)
+    const int64_t workgroups = ceil_div(static_cast<int64_t>(h) * w * (c % 4 == 0 ? c / 4 : c), kBlock) *
+                               ceil_div(n, kImagesPerWorkgroup);
+    const int ks_gather = (kh == kw && stride_h == 1 && stride_w == 1 && small_image &&
+                           workgroups <= 8 * static_cast<int64_t>(ctx().num_cus)) ? kh : 0;
+    if (ks_gather == 5)
+        BSHIP_LAUNCH_IMG_ORDER(col2im_kernel_k5, "col2im", static_cast<int64_t>(h) * w, al, true, col, in_deltas);
+    if (ks_gather == 3)
+        BSHIP_LAUNCH_IMG_ORDER(col2im_kernel_k3, "col2im", static_cast<int64_t>(h) * w, al, true, col, in_deltas);
+    BSHIP_LAUNCH_IMG_ORDER(col2im_kernel, "col2im", static_cast<int64_t>(h) * w, al, true, col, in_deltas);
 }
 
 int bship_maxpool_fwd_nhwc_f32(const float* in, float* out, float* argmax, int64_t n, int h, int w,
