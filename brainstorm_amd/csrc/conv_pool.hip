@@ -1180,17 +1180,20 @@ using namespace bship;
 // caller's local variables in_pitch, out_pitch and aux_pitch; through_out, another local, says whether
 // the kernel stores its result write-through (ImgPlan::through).
 #define BSHIP_LAUNCH_IMG(kernel, name, positions, aligned, ...) \
-    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, kImagesPerWorkgroup, false, __VA_ARGS__)
+    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, kImagesPerWorkgroup, false, true, __VA_ARGS__)
 // in_order: tiles in dispatch order instead of one run per XCD (img_block)
 #define BSHIP_LAUNCH_IMG_ORDER(kernel, name, positions, aligned, order_, ...) \
-    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, kImagesPerWorkgroup, order_, __VA_ARGS__)
+    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, kImagesPerWorkgroup, order_, true, __VA_ARGS__)
 #define BSHIP_LAUNCH_IMG_N(kernel, name, positions, aligned, images_per_wg, ...) \
-    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, images_per_wg, false, __VA_ARGS__)
+    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, images_per_wg, false, true, __VA_ARGS__)
+// for kernels that take exactly kImagesPerWorkgroup images at a time (im2col_body)
+#define BSHIP_LAUNCH_IMG_EXACT(kernel, name, positions, aligned, ...) \
+    BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, kImagesPerWorkgroup, false, false, __VA_ARGS__)
 // images_per_wg: how many images a workgroup walks through, one after the other (kernels whose image
 // loop is `img = group; img += groups`; im2col_body needs kImagesPerWorkgroup). Measured at batch 2048:
 // the pooling backward kernels (read-modify-write of in_deltas) want 1 (max 32x32x32: 0.75 -> 0.89 of
 // peak, avg 0.71 -> 0.80), max pooling forward 4 (0.90 against 0.82 with 1).
-#define BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, images_per_wg, order_, ...)             \
+#define BSHIP_LAUNCH_IMG_FULL(kernel, name, positions, aligned, images_per_wg, order_, few_ok_, ...)    \
     do {                                                                                                \
         const bool vec4_ = (g.c % 4 == 0);                                                              \
         const int cv_ = vec4_ ? g.c / 4 : g.c;                                                          \
@@ -1211,8 +1214,11 @@ using namespace bship;
         pl_.in_pitch = in_pitch;                                                                        \
         pl_.out_pitch = out_pitch;                                                                      \
         pl_.aux_pitch = aux_pitch;                                                                      \
-        const int64_t gy_ = ceil_div(n, images_per_wg);                                                 \
         pl_.tiles = static_cast<uint32_t>(ceil_div(lanes_, kBlock));                                    \
+        /* a small batch: one image per workgroup when several would leave compute units without work */ \
+        const int64_t ipw_ = ((few_ok_) && static_cast<int64_t>(pl_.tiles) * ceil_div(n, images_per_wg) <  \
+                                               4 * static_cast<int64_t>(ctx().num_cus)) ? 1 : (images_per_wg); \
+        const int64_t gy_ = ceil_div(n, ipw_);                                                          \
         pl_.groups = static_cast<uint32_t>(gy_ < 65535 ? gy_ : 65535);                                  \
         if (static_cast<int64_t>(pl_.tiles) * pl_.groups > 0x7ffffff0)                                  \
             pl_.groups = static_cast<uint32_t>(imax(1, static_cast<int>(0x7ffffff0 / pl_.tiles)));      \
@@ -1307,8 +1313,8 @@ int bship_im2col_nhwc_pitched_f32(const float* in, int64_t in_pitch, float* col,
     }
     const bool al = aligned16(in) && aligned16(col) && in_pitch % 4 == 0;
     if (write_through)
-        BSHIP_LAUNCH_IMG(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
-    BSHIP_LAUNCH_IMG(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
+        BSHIP_LAUNCH_IMG_EXACT(im2col_wt, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
+    BSHIP_LAUNCH_IMG_EXACT(im2col_cached, "im2col", static_cast<int64_t>(g.oh) * g.ow * kh * kw, al, in, col);
 }
 
 int bship_col2im_nhwc_f32(const float* col, float* in_deltas, int64_t n, int h, int w, int c,
