@@ -33,6 +33,7 @@ struct Context {
     size_t store_through_min = size_t(1) << 18, store_through_max = size_t(1) << 26;
     size_t softmax_run_bytes = size_t(512) << 10;  // softmax rows a multiple of 64 KiB apart: bytes of adjacent rows that an XCD takes in one run (BSHIP_SM_CHUNK_KB)
     size_t ew_run_bytes = size_t(512) << 10;      // elementwise kernels with two inputs: bytes per stream that an XCD takes in one run (BSHIP_EW_RUN_KB)
+    int64_t col2im_stream_min_images_per_cu = 1;  // col2im: the streaming kernel takes batches of at least this many images per compute unit, 0: never (BSHIP_COL2IM_STREAM_MIN)
     char name[256] = {0};
 };
 

@@ -96,6 +96,8 @@ int bship_init(int device) {
     if (smk && smk[0]) g_ctx.softmax_run_bytes = static_cast<size_t>(strtoull(smk, nullptr, 10)) << 10;
     const char* erk = getenv("BSHIP_EW_RUN_KB");
     if (erk && erk[0]) g_ctx.ew_run_bytes = static_cast<size_t>(strtoull(erk, nullptr, 10)) << 10;
+    const char* csm = getenv("BSHIP_COL2IM_STREAM_MIN");
+    if (csm && csm[0]) g_ctx.col2im_stream_min_images_per_cu = static_cast<int64_t>(strtoll(csm, nullptr, 10));
     g_ctx.device = device;
     g_ctx.inited = true;
     return 0;

@@ -14,6 +14,8 @@
 #pragma clang fp contract(off)
 
 #include <cfloat>
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 
@@ -646,6 +648,209 @@ __global__ __launch_bounds__(kCol2imThreads) void col2im_band(const float* __res
     }
 }
 
+// col2im for narrow channel counts and many images (KS x KS windows, stride 1, C channels, both known
+// at compile time). The col matrix streams from memory straight into LDS (128-bit global loads with
+// an LDS destination: no registers in between) and every col row is used up in the one phase after
+// its arrival, so most of LDS holds data in flight.
+//
+// A workgroup takes whole images one after the other (image = workgroup index + i * workgroups). A
+// phase is R consecutive col rows oy0 .. oy0+R-1 of one image. Their terms belong to the M = KS+R-1
+// image rows oy0-pad .. oy0-pad+M-1; lane (s, ch, x) of the first M*w*C lanes owns, during a phase,
+// the element (y, x, ch) of the one row with y = s (mod M) among them, and keeps its sum in a
+// register from the phase with the row's first col row (where it starts from the old value:
+// in_deltas is added to) to the phase with its last one (where it is stored). For each col row of
+// the phase in turn, the lane adds the KS terms of its window row ky = y + pad - oy, kx descending:
+// an element receives its terms with oy ascending, then ox ascending - the order of the serial loops.
+//
+// The other wavefronts request data: the col rows of a phase and the image rows that start in it go
+// to the next slots of two rings in LDS, DEPTH phases before they are needed, as pieces of 1 KiB
+// (one load instruction: 64 lanes x 16 bytes, LDS address = the wavefront's base + 16 * lane).
+// Every requesting wavefront issues exactly PER load instructions per phase (pieces it has no use
+// for become a 16-byte load into a spare slot). Loads complete in order, so when at most
+// (DEPTH-1)*PER are outstanding, the wavefront's pieces of the current phase have arrived; then the
+// workgroup's barrier. One barrier per phase; the slots that phase t + DEPTH fills are the ones
+// phase t - 1 read.
+// (A wavefront issues an instruction every four cycles at best and a phase lasts as long as its
+// longest instruction stream, which is why requesting and adding run side by side in different
+// wavefronts, and why the bookkeeping is additions on running counters.)
+// Terms beyond the left and right image border are read from wherever their address falls (the
+// ring has a guard in front and the old values behind) and not added.
+// Needs ow*KS*KS*C and w*C to be multiples of 4, both operands 16-byte aligned, in_pitch % 4 == 0.
+constexpr int kPieceFloats = 256;         // floats per load instruction of a wavefront
+
+struct Col2imStreamPlan {
+    int h, w, oh, ow, pad;
+    int phases;            // phases per image
+    int add_waves;         // adding wavefronts; the others request data
+    int old_ring;          // image rows of old values held in LDS
+    int old_image_step;    // what the ring position of image row "oy0 - pad" moves by from the last phase of an image to the first of the next, less R, modulo old_ring
+    int guard;             // floats in front of the col ring
+    int owk;               // ow*KS*KS*C : floats per col row
+    int64_t in_pitch;      // elements from one image of in_deltas to the next
+    FastDiv d_wc, d_w;
+};
+
+// Waits until at most N of this wavefront's vector memory operations are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_until_outstanding() {
+    static_assert(N >= 0 && N < 64, "the counter has 6 bits");
+    // vmcnt: bits 3:0 and 15:14; expcnt (6:4) and lgkmcnt (11:8) at their maximum: not waited for
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+    asm volatile("" ::: "memory");
+}
+
+template <int KS, int C, int R, int THREADS, int DEPTH, int PER>
+__global__ __launch_bounds__(THREADS) void col2im_stream(const float* __restrict__ col,
+                                                         float* __restrict__ in_deltas, int64_t n,
+                                                         Col2imStreamPlan pl) {
+    extern __shared__ float stream_lds[];
+    constexpr int kWaves = THREADS / kWave;
+    constexpr int KC = KS * KS * C;
+    constexpr int M = KS + R - 1;                           // image rows a phase adds to
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWave);
+    const int lane = static_cast<int>(threadIdx.x) & (kWave - 1);
+    const int wc = pl.w * C, pitch = pl.owk;
+    float* const tile = stream_lds + pl.guard;
+    float* const old_area = tile + (DEPTH + 1) * R * pitch;
+    const int my_images = static_cast<int>((n - blockIdx.x + gridDim.x - 1) / gridDim.x);
+    const int total = my_images * pl.phases;                // the launcher keeps this below 2^31
+    const int64_t col_image = static_cast<int64_t>(pl.oh) * pitch;
+    const int64_t col_step = static_cast<int64_t>(gridDim.x) * col_image;
+    const int64_t old_step = static_cast<int64_t>(gridDim.x) * pl.in_pitch;
+    const int add_waves = pl.add_waves;
+
+    if (wave >= add_waves) {
+        // ---------------- requests ----------------
+        const int req_wave = wave - add_waves, req_waves = kWaves - add_waves;
+        const int row_pieces = (wc + kPieceFloats - 1) / kPieceFloats;
+        float* const spare = old_area + pl.old_ring * wc;
+        int req_phase = 0, req_slot = 0, req_old_slot = 0;
+        const float* req_col = col + static_cast<int64_t>(blockIdx.x) * col_image;          // the image's col matrix
+        const float* req_img = in_deltas + static_cast<int64_t>(blockIdx.x) * pl.in_pitch;  // the image's old values
+        auto request = [&](bool real) {
+            const int oy0 = req_phase * R;
+            const int col_floats = imin(R, pl.oh - oy0) * pitch;
+            const int col_pieces = (col_floats + kPieceFloats - 1) / kPieceFloats;
+            // image rows whose first col row is in this phase
+            const int y0 = oy0 == 0 ? 0 : oy0 + KS - 1 - pl.pad;
+            const int rows = imax(imin(oy0 + R + KS - 1 - pl.pad, pl.h) - y0, 0);
+            const int pieces = real ? col_pieces + rows * row_pieces : 0;
+#pragma unroll
+            for (int k = 0; k < PER; ++k) {
+                const int p = req_wave + k * req_waves;
+                const float* src = col;
+                float* dst = spare;
+                int valid = 4;                 // floats left from this piece's start
+                if (p < col_pieces && p < pieces) {
+                    src = req_col + static_cast<int64_t>(oy0) * pitch + p * kPieceFloats;
+                    dst = tile + req_slot * (R * pitch) + p * kPieceFloats;
+                    valid = col_floats - p * kPieceFloats;
+                } else if (p < pieces) {
+                    const int q = p - col_pieces;
+                    const int r = q / row_pieces, m = q - r * row_pieces;
+                    int slot = req_old_slot + r;
+                    if (slot >= pl.old_ring) slot -= pl.old_ring;
+                    src = req_img + static_cast<int64_t>(y0 + r) * wc + m * kPieceFloats;
+                    dst = old_area + slot * wc + m * kPieceFloats;
+                    valid = wc - m * kPieceFloats;
+                }
+                if (lane * 4 < valid) __builtin_amdgcn_global_load_lds(src + lane * 4, dst, 16, 0, 2 /* non-temporal */);
+            }
+            if (!real) return;
+            req_slot = req_slot == DEPTH ? 0 : req_slot + 1;
+            req_old_slot += rows;
+            if (req_old_slot >= pl.old_ring) req_old_slot -= pl.old_ring;
+            if (++req_phase == pl.phases) {
+                req_phase = 0;
+                req_col += col_step;
+                req_img += old_step;
+            }
+        };
+        for (int d = 0; d < DEPTH; ++d) request(d < total);
+        for (int t = 0; t < total; ++t) {
+            wait_until_outstanding<(DEPTH - 1) * PER>();   // this wavefront's pieces of phase t are in LDS
+            asm volatile("s_barrier" ::: "memory");        // everyone's are, and the adding wavefronts have left phase t - 1
+            request(t + DEPTH < total);
+        }
+        wait_until_outstanding<0>();
+        return;
+    }
+
+    // ---------------- additions ----------------
+    // lane -> (s, ch, x): channel before x, so that neighbouring lanes read LDS words KS*KS*C apart
+    // (an odd stride for RGB images)
+    uint32_t s_u, rem, ch_u, xx_u;
+    pl.d_wc.divmod(static_cast<uint32_t>(threadIdx.x), s_u, rem);
+    pl.d_w.divmod(rem, ch_u, xx_u);
+    const int s = static_cast<int>(s_u), ch = static_cast<int>(ch_u), xx = static_cast<int>(xx_u);
+    const bool owner = s < M;
+    const int eoff = xx * C + ch;                          // within an image row
+    // term (ky, kx) of element (y, x, ch) sits at  slot(oy)*pitch + (x+pad-kx)*KC + (ky*KS+kx)*C + ch
+    //   = slot(oy)*pitch + ebase + ky*KS*C + (KS-1-kx)*(KC-C)
+    const int ebase = (xx + pl.pad) * KC + ch - (KS - 1) * (KC - C);
+    bool xok[KS];                                          // the term with kx = KS-1-b exists
+#pragma unroll
+    for (int b = 0; b < KS; ++b) {
+        const int ox = xx + pl.pad - (KS - 1 - b);
+        xok[b] = ox >= 0 && ox < pl.ow;
+    }
+    const int m_start = (M - pl.pad % M) % M;
+    float acc = 0.0f;
+    int phase = 0, slot = 0;
+    int mm = m_start;                      // (oy0 - pad) modulo M
+    int old_pos = pl.old_ring - pl.pad;    // ring position of image row oy0 - pad (rows before the image have one too)
+    float* img = in_deltas + static_cast<int64_t>(blockIdx.x) * pl.in_pitch;
+    for (int t = 0; t < total; ++t) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // done reading phase t - 1
+        asm volatile("s_barrier" ::: "memory");              // phase t is complete in LDS
+        const int oy0 = phase * R;
+        int d = s - mm;                                      // the lane's row is oy0 - pad + d
+        if (d < 0) d += M;
+        const int y = oy0 - pl.pad + d;
+        const bool mine = owner && y >= 0 && y < pl.h;
+        {
+            // Everything below is selects rather than branches: a branch on a per-lane condition costs
+            // several scalar instructions, and the scalar unit is shared by the whole compute unit.
+            int pos = old_pos + d;
+            if (pos >= pl.old_ring) pos -= pl.old_ring;
+            const float old_value = old_area[pos * wc + eoff];    // meaningful in the row's first phase
+            const float* tphase = tile + slot * (R * pitch) + ebase;
+            float v[R][KS];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int ky = imin(imax(d - r, 0), KS - 1);      // clamped: the terms of a row without one are not added
+                const float* trow = tphase + r * pitch + ky * (KS * C);
+#pragma unroll
+                for (int b = 0; b < KS; ++b) v[r][b] = trow[b * (KC - C)];
+            }
+            bool store = false;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int ky = d - r, oy = oy0 + r;
+                const bool valid = mine && ky >= 0 && ky < KS && oy < pl.oh;
+                float sum = (ky == KS - 1 || oy == 0) ? old_value : acc;   // the row's first col row starts from the old value
+#pragma unroll
+                for (int b = 0; b < KS; ++b) sum = xok[b] ? sum + v[r][b] : sum;
+                acc = valid ? sum : acc;
+                store = store || (valid && (ky == 0 || oy == pl.oh - 1));       // its last one
+            }
+            if (store) img[static_cast<int64_t>(y) * wc + eoff] = acc;
+        }
+        slot = slot == DEPTH ? 0 : slot + 1;
+        mm += R % M;
+        if (mm >= M) mm -= M;
+        old_pos += R;
+        if (old_pos >= pl.old_ring) old_pos -= pl.old_ring;
+        if (++phase == pl.phases) {
+            phase = 0;
+            img += old_step;
+            mm = m_start;
+            old_pos += pl.old_image_step;
+            if (old_pos >= pl.old_ring) old_pos -= pl.old_ring;
+        }
+    }
+}
+
 // _cpuop 57-80: strict '>' from -FLT_MAX, so the first maximum in (y, x) scan
 // order wins and NaN never does; empty windows give output 0 and argmax -1.
 // One lane per W channels of one output position; lanes_per_image = oh*ow*cv.
@@ -1153,6 +1358,46 @@ static bool plan_col2im_band(const ImgGeom& g, int64_t n, Col2imBandPlan* out, s
     return true;
 }
 
+// col2im_stream with `rows` col rows per phase, requests `depth` phases ahead and `per` loads per phase
+// and requesting wavefront.
+static bool plan_col2im_stream(const ImgGeom& g, int rows, int depth, int threads, int per, Col2imStreamPlan* out,
+                               size_t* lds_bytes) {
+    if (g.kh != g.kw || g.sh != 1 || g.sw != 1 || g.pad > g.kh - 1 || g.c >= 16) return false;
+    if (g.h == 0 || g.w == 0 || g.c == 0 || g.oh == 0 || g.ow == 0 || rows < 1 || depth < 1) return false;
+    const int kc = g.kh * g.kw * g.c;
+    const int64_t owk = static_cast<int64_t>(g.ow) * kc;
+    const int64_t wc = static_cast<int64_t>(g.w) * g.c;
+    if (owk % 4 != 0 || wc % 4 != 0 || owk * g.oh > 0x7fffffff) return false;
+    const int m = g.kh + rows - 1;                      // image rows a phase adds to
+    // one lane per element of those rows, and wavefronts left to request a phase's data with `per` loads each
+    const int64_t add_waves = (m * wc + kWave - 1) / kWave;
+    const int64_t req_waves = threads / kWave - add_waves;
+    const int64_t pieces = (rows * owk + kPieceFloats - 1) / kPieceFloats +
+                           imin(m - g.pad, g.h) * ((wc + kPieceFloats - 1) / kPieceFloats);
+    if (req_waves < 1 || per * req_waves < pieces || (depth - 1) * per > 63) return false;
+    const int old_ring = (depth + 1) * rows + g.kh;
+    if (g.pad >= old_ring) return false;
+    // reads of terms beyond the left and right image borders fall this far outside a col row
+    const int guard = ((g.kh - 1) * (kc - g.c) + 3) / 4 * 4;
+    const int back = imax((g.kh - 1) * kc, 4);
+    const size_t bytes = (static_cast<size_t>(guard) + static_cast<size_t>(depth + 1) * rows * owk +
+                          static_cast<size_t>(old_ring) * wc + back) * sizeof(float);
+    if (bytes > 160 * 1024) return false;
+    out->h = g.h; out->w = g.w; out->oh = g.oh; out->ow = g.ow; out->pad = g.pad;
+    out->phases = (g.oh + rows - 1) / rows;
+    out->add_waves = static_cast<int>(add_waves);
+    out->old_ring = old_ring;
+    // image row "oy0 - pad" of an image's last phase is row (phases-1)*rows - pad; of the next image's first
+    // phase it is row -pad, h rows further on in the sequence of all image rows; every phase steps by `rows`
+    out->old_image_step = ((g.h - out->phases * rows) % old_ring + old_ring) % old_ring;
+    out->guard = guard;
+    out->owk = static_cast<int>(owk);
+    out->d_wc = FastDiv(static_cast<uint32_t>(wc));
+    out->d_w = FastDiv(static_cast<uint32_t>(g.w));
+    *lds_bytes = bytes;
+    return true;
+}
+
 // Lets `kernel` use `bytes` of dynamic LDS (more than the default limit has to be asked for);
 // remembers what each kernel was granted.
 static bool allow_dynamic_lds_impl(const void* kernel, size_t bytes) {
@@ -1169,6 +1414,47 @@ static bool allow_dynamic_lds_impl(const void* kernel, size_t bytes) {
 template <typename K>
 static bool allow_dynamic_lds(K kernel, size_t bytes) {
     return allow_dynamic_lds_impl(reinterpret_cast<const void*>(kernel), bytes);
+}
+
+// col2im_stream for 5x5 windows with stride 1 on 1 or 3 channels. A phase costs about 0.4 us
+// whatever it carries, so the kernel is used where a phase's col rows are at least kStreamMinPhaseBytes
+// (32x32x3 images under a 5x5 window: 19 KB; there, at batch 2048, 120 us against the banded kernel's
+// 135, and 18 against 24 at batch 256; with 6-11 KB per phase it takes twice the banded kernel's time),
+// and for at least one image per workgroup. *launched says whether it ran.
+constexpr size_t kStreamMinPhaseBytes = 16 * 1024;
+constexpr int kStreamRows = 2, kStreamDepth = 4, kStreamThreads = 1024;
+static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_deltas, int64_t in_pitch, int64_t n,
+                             int* launched) {
+    *launched = 0;
+    const Context& c = ctx();
+    const int64_t min_per_cu = c.col2im_stream_min_images_per_cu;
+    if (min_per_cu <= 0 || n < min_per_cu * c.num_cus || !aligned16(col) || !aligned16(in_deltas) || in_pitch % 4 != 0)
+        return 0;
+    if (g.kh != 5 || !(g.c == 1 || g.c == 3)) return 0;   // col rows of 3x3 windows that are long enough need more lanes than a workgroup has
+    if (static_cast<size_t>(kStreamRows) * g.ow * g.kh * g.kw * g.c * sizeof(float) < kStreamMinPhaseBytes) return 0;
+    if ((n / c.num_cus + 1) * g.oh > 0x7fffffff) return 0;
+    Col2imStreamPlan sp;
+    size_t lds = 0;
+    int per = 0;
+    for (int p : {4, 8, 12})
+        if (per == 0 && plan_col2im_stream(g, kStreamRows, kStreamDepth, kStreamThreads, p, &sp, &lds)) per = p;
+    if (per == 0) return 0;
+    sp.in_pitch = in_pitch;
+    const dim3 grid(static_cast<unsigned>(c.num_cus));      // one workgroup per compute unit: it takes most of the LDS
+#define BSHIP_COL2IM_STREAM(KS_, C_, P_)                                                                          \
+    if (g.kh == KS_ && g.c == C_ && per == P_) {                                                                  \
+        auto kernel = col2im_stream<KS_, C_, kStreamRows, kStreamThreads, kStreamDepth, P_>;                      \
+        if (!allow_dynamic_lds(kernel, lds)) { (void)hipGetLastError(); return 0; }                               \
+        hipLaunchKernelGGL(kernel, grid, dim3(kStreamThreads), lds, c.stream, col, in_deltas, n, sp);             \
+        *launched = 1;                                                                                            \
+        return check_launch("col2im");                                                                            \
+    }
+#define BSHIP_COL2IM_STREAM_PER(KS_, C_) BSHIP_COL2IM_STREAM(KS_, C_, 4) BSHIP_COL2IM_STREAM(KS_, C_, 8) BSHIP_COL2IM_STREAM(KS_, C_, 12)
+    BSHIP_COL2IM_STREAM_PER(5, 3)
+    BSHIP_COL2IM_STREAM_PER(5, 1)
+#undef BSHIP_COL2IM_STREAM_PER
+#undef BSHIP_COL2IM_STREAM
+    return 0;
 }
 
 }  // namespace bship
@@ -1340,6 +1626,11 @@ int bship_col2im_nhwc_pitched_f32(const float* col, float* in_deltas, int64_t in
     BSHIP_REQUIRE_F32_ALIGNED(col);
     BSHIP_REQUIRE_F32_ALIGNED(in_deltas);
     const int64_t out_pitch = 0, aux_pitch = 0;
+    {
+        int launched = 0;
+        st = try_col2im_stream(g, col, in_deltas, in_pitch, n, &launched);
+        if (launched) return st;
+    }
     Col2imBandPlan bp;
     size_t lds = 0;
     if (plan_col2im_band(g, n, &bp, &lds)) {

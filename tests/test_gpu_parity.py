@@ -958,6 +958,42 @@ def test_im2col_col2im_banded_exact(hip, ref):
         assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, kh, kw, pad, stride),))
 
 
+# Geometries for the streaming col2im kernel (5x5 windows, stride 1, 1 or 3 channels, col rows of at least
+# 8 KB, one image or more per compute unit): an odd number of col rows (the last phase holds one), padding
+# of 0 and of the kernel size minus one, images of a single phase, more images than workgroups by a
+# remainder, exactly one image per workgroup; the last one stays with the banded kernel (col rows too short).
+STREAM_CASES = [(300, 9, 32, 3, 5, 4), (257, 6, 88, 1, 5, 0), (530, 12, 32, 3, 5, 2), (260, 7, 100, 1, 5, 2),
+                (256, 20, 84, 1, 5, 2), (300, 12, 12, 3, 5, 2)]
+
+
+def test_col2im_streaming_exact(hip, ref):
+    rng = np.random.RandomState(128)
+    lib = hip._lib
+    for n, h, w, c, k, pad in STREAM_CASES:
+        oh, ow = _out_size(h, k, pad, 1), _out_size(w, k, pad, 1)
+        cols = rand(rng, (n, oh * ow, k * k * c))
+        din = rand(rng, (n, h, w, c))
+        din[0, 0, :3, 0] = [-0.0, np.inf, np.nan]          # adding nothing must leave -0.0 alone
+        cols[0, :2] = 0.0
+        cols[0, :2, ::2] = -0.0
+        want = din.copy()
+        for i in range(n):
+            ref._col2im(cols[i], k, k, pad, (1, 1), want[i])
+        colsd = hip.create_from_numpy(cols)
+        dind = hip.create_from_numpy(din)
+        hip._call(lib.bship_col2im_nhwc_f32(colsd.ptr, dind.ptr, n, h, w, c, k, k, pad, 1, 1))
+        assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, k, pad),))
+        # the same images a pitch apart (every image followed by 8 floats that must stay as they are)
+        image = h * w * c
+        wide = np.full((n, image + 8), 5.0, F32)
+        wide[:, :image] = din.reshape(n, image)
+        wided = hip.create_from_numpy(wide)
+        hip._call(lib.bship_col2im_nhwc_pitched_f32(colsd.ptr, wided.ptr, image + 8, n, h, w, c, k, k, pad, 1, 1))
+        got = wided.get()
+        assert_bit_equal(got[:, :image].reshape(din.shape), want, "pitched col2im %r" % ((n, h, w, c, k, pad),))
+        assert (got[:, image:] == 5.0).all()
+
+
 def test_im2col_col2im_random_geometries(hip, ref):
     # the banded kernels choose band sizes, LDS rings and phases from the geometry: many random
     # geometries (non-square kernels, strides up to 3, padding up to the kernel size minus one,
