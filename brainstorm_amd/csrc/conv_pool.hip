@@ -655,11 +655,11 @@ __global__ __launch_bounds__(kCol2imThreads) void col2im_band(const float* __res
 //
 // A workgroup takes whole images one after the other (image = workgroup index + i * workgroups). A
 // phase is R consecutive col rows oy0 .. oy0+R-1 of one image. Their terms belong to the M = KS+R-1
-// image rows oy0-pad .. oy0-pad+M-1; lane (s, ch, x) of the first M*w*C lanes owns, during a phase,
-// the element (y, x, ch) of the one row with y = s (mod M) among them, and keeps its sum in a
-// register from the phase with the row's first col row (where it starts from the old value:
-// in_deltas is added to) to the phase with its last one (where it is stored). For each col row of
-// the phase in turn, the lane adds the KS terms of its window row ky = y + pad - oy, kx descending:
+// image rows oy0-pad .. oy0-pad+M-1; lane (s, x) of the first M*w lanes owns, during a phase, the
+// pixel (y, x) of the one row with y = s (mod M) among them, and keeps the sums of its C channels in
+// registers from the phase with the row's first col row (where they start from the old values:
+// in_deltas is added to) to the phase with its last one (where they are stored). For each col row
+// of the phase in turn, the lane adds the KS terms of its window row ky = y + pad - oy, kx descending:
 // an element receives its terms with oy ascending, then ox ascending - the order of the serial loops.
 //
 // The other wavefronts request data: the col rows of a phase and the image rows that start in it go
@@ -687,7 +687,7 @@ struct Col2imStreamPlan {
     int guard;             // floats in front of the col ring
     int owk;               // ow*KS*KS*C : floats per col row
     int64_t in_pitch;      // elements from one image of in_deltas to the next
-    FastDiv d_wc, d_w;
+    FastDiv d_w;
 };
 
 // Waits until at most N of this wavefront's vector memory operations are outstanding.
@@ -777,25 +777,27 @@ __global__ __launch_bounds__(THREADS) void col2im_stream(const float* __restrict
     }
 
     // ---------------- additions ----------------
-    // lane -> (s, ch, x): channel before x, so that neighbouring lanes read LDS words KS*KS*C apart
-    // (an odd stride for RGB images)
-    uint32_t s_u, rem, ch_u, xx_u;
-    pl.d_wc.divmod(static_cast<uint32_t>(threadIdx.x), s_u, rem);
-    pl.d_w.divmod(rem, ch_u, xx_u);
-    const int s = static_cast<int>(s_u), ch = static_cast<int>(ch_u), xx = static_cast<int>(xx_u);
+    // lane -> (s, x): the lane owns all C channels of its pixel (what it decides per window row - which
+    // row, whether it has terms, first, last - it decides once for C sums); neighbouring lanes read LDS
+    // words KS*KS*C apart (an odd stride for RGB images)
+    uint32_t s_u, xx_u;
+    pl.d_w.divmod(static_cast<uint32_t>(threadIdx.x), s_u, xx_u);
+    const int s = static_cast<int>(s_u), xx = static_cast<int>(xx_u);
     const bool owner = s < M;
-    const int eoff = xx * C + ch;                          // within an image row
+    const int eoff = xx * C;                               // within an image row
     // term (ky, kx) of element (y, x, ch) sits at  slot(oy)*pitch + (x+pad-kx)*KC + (ky*KS+kx)*C + ch
-    //   = slot(oy)*pitch + ebase + ky*KS*C + (KS-1-kx)*(KC-C)
-    const int ebase = (xx + pl.pad) * KC + ch - (KS - 1) * (KC - C);
-    bool xok[KS];                                          // the term with kx = KS-1-b exists
+    //   = slot(oy)*pitch + ebase + ch + ky*KS*C + (KS-1-kx)*(KC-C)
+    const int ebase = (xx + pl.pad) * KC - (KS - 1) * (KC - C);
+    bool xok[KS];                                          // the terms with kx = KS-1-b exist
 #pragma unroll
     for (int b = 0; b < KS; ++b) {
         const int ox = xx + pl.pad - (KS - 1 - b);
         xok[b] = ox >= 0 && ox < pl.ow;
     }
     const int m_start = (M - pl.pad % M) % M;
-    float acc = 0.0f;
+    float acc[C];
+#pragma unroll
+    for (int k = 0; k < C; ++k) acc[k] = 0.0f;
     int phase = 0, slot = 0;
     int mm = m_start;                      // (oy0 - pad) modulo M
     int old_pos = pl.old_ring - pl.pad;    // ring position of image row oy0 - pad (rows before the image have one too)
@@ -813,28 +815,40 @@ __global__ __launch_bounds__(THREADS) void col2im_stream(const float* __restrict
             // several scalar instructions, and the scalar unit is shared by the whole compute unit.
             int pos = old_pos + d;
             if (pos >= pl.old_ring) pos -= pl.old_ring;
-            const float old_value = old_area[pos * wc + eoff];    // meaningful in the row's first phase
+            float old_value[C];                                   // meaningful in the row's first phase
+#pragma unroll
+            for (int k = 0; k < C; ++k) old_value[k] = old_area[pos * wc + eoff + k];
             const float* tphase = tile + slot * (R * pitch) + ebase;
-            float v[R][KS];
+            float v[R][KS][C];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int ky = imin(imax(d - r, 0), KS - 1);      // clamped: the terms of a row without one are not added
                 const float* trow = tphase + r * pitch + ky * (KS * C);
 #pragma unroll
-                for (int b = 0; b < KS; ++b) v[r][b] = trow[b * (KC - C)];
+                for (int b = 0; b < KS; ++b)
+#pragma unroll
+                    for (int k = 0; k < C; ++k) v[r][b][k] = trow[b * (KC - C) + k];
             }
             bool store = false;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int ky = d - r, oy = oy0 + r;
                 const bool valid = mine && ky >= 0 && ky < KS && oy < pl.oh;
-                float sum = (ky == KS - 1 || oy == 0) ? old_value : acc;   // the row's first col row starts from the old value
+                const bool first = ky == KS - 1 || oy == 0;       // the row's first col row starts from the old value
 #pragma unroll
-                for (int b = 0; b < KS; ++b) sum = xok[b] ? sum + v[r][b] : sum;
-                acc = valid ? sum : acc;
+                for (int k = 0; k < C; ++k) {
+                    float sum = first ? old_value[k] : acc[k];
+#pragma unroll
+                    for (int b = 0; b < KS; ++b) sum = xok[b] ? sum + v[r][b][k] : sum;
+                    acc[k] = valid ? sum : acc[k];
+                }
                 store = store || (valid && (ky == 0 || oy == pl.oh - 1));       // its last one
             }
-            if (store) img[static_cast<int64_t>(y) * wc + eoff] = acc;
+            if (store) {
+                float* q = img + static_cast<int64_t>(y) * wc + eoff;
+#pragma unroll
+                for (int k = 0; k < C; ++k) q[k] = acc[k];
+            }
         }
         slot = slot == DEPTH ? 0 : slot + 1;
         mm += R % M;
@@ -1369,8 +1383,8 @@ static bool plan_col2im_stream(const ImgGeom& g, int rows, int depth, int thread
     const int64_t wc = static_cast<int64_t>(g.w) * g.c;
     if (owk % 4 != 0 || wc % 4 != 0 || owk * g.oh > 0x7fffffff) return false;
     const int m = g.kh + rows - 1;                      // image rows a phase adds to
-    // one lane per element of those rows, and wavefronts left to request a phase's data with `per` loads each
-    const int64_t add_waves = (m * wc + kWave - 1) / kWave;
+    // wavefronts left to request a phase's data with `per` loads each
+    const int64_t add_waves = (static_cast<int64_t>(m) * g.w + kWave - 1) / kWave;   // one lane per pixel of those rows
     const int64_t req_waves = threads / kWave - add_waves;
     const int64_t pieces = (rows * owk + kPieceFloats - 1) / kPieceFloats +
                            imin(m - g.pad, g.h) * ((wc + kPieceFloats - 1) / kPieceFloats);
@@ -1392,7 +1406,6 @@ static bool plan_col2im_stream(const ImgGeom& g, int rows, int depth, int thread
     out->old_image_step = ((g.h - out->phases * rows) % old_ring + old_ring) % old_ring;
     out->guard = guard;
     out->owk = static_cast<int>(owk);
-    out->d_wc = FastDiv(static_cast<uint32_t>(wc));
     out->d_w = FastDiv(static_cast<uint32_t>(g.w));
     *lds_bytes = bytes;
     return true;
@@ -1436,7 +1449,7 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
     Col2imStreamPlan sp;
     size_t lds = 0;
     int per = 0;
-    for (int p : {4, 8, 12})
+    for (int p : {2, 4, 8, 12})
         if (per == 0 && plan_col2im_stream(g, kStreamRows, kStreamDepth, kStreamThreads, p, &sp, &lds)) per = p;
     if (per == 0) return 0;
     sp.in_pitch = in_pitch;
@@ -1449,7 +1462,8 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
         *launched = 1;                                                                                            \
         return check_launch("col2im");                                                                            \
     }
-#define BSHIP_COL2IM_STREAM_PER(KS_, C_) BSHIP_COL2IM_STREAM(KS_, C_, 4) BSHIP_COL2IM_STREAM(KS_, C_, 8) BSHIP_COL2IM_STREAM(KS_, C_, 12)
+#define BSHIP_COL2IM_STREAM_PER(KS_, C_) \
+    BSHIP_COL2IM_STREAM(KS_, C_, 2) BSHIP_COL2IM_STREAM(KS_, C_, 4) BSHIP_COL2IM_STREAM(KS_, C_, 8) BSHIP_COL2IM_STREAM(KS_, C_, 12)
     BSHIP_COL2IM_STREAM_PER(5, 3)
     BSHIP_COL2IM_STREAM_PER(5, 1)
 #undef BSHIP_COL2IM_STREAM_PER
