@@ -233,6 +233,16 @@ struct FastDiv {
     }
 };
 
+// ---- loads that complete in order: waiting by count ----
+// Waits until at most N of this wavefront's vector memory operations are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_until_outstanding() {
+    static_assert(N >= 0 && N < 64, "the counter has 6 bits");
+    // vmcnt: bits 3:0 and 15:14; expcnt (6:4) and lgkmcnt (11:8) at their maximum: not waited for
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+    asm volatile("" ::: "memory");
+}
+
 // ---- integer labels stored as float32 (device) ----
 // Column selected by label v in a row of K columns: truncated toward zero like astype(int32);
 // labels in [-K, -1] count from the end, as NumPy's indexing does (numpy_handler.py:101, 203).

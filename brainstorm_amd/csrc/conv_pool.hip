@@ -690,15 +690,6 @@ struct Col2imStreamPlan {
     FastDiv d_w;
 };
 
-// Waits until at most N of this wavefront's vector memory operations are outstanding.
-template <int N>
-__device__ __forceinline__ void wait_until_outstanding() {
-    static_assert(N >= 0 && N < 64, "the counter has 6 bits");
-    // vmcnt: bits 3:0 and 15:14; expcnt (6:4) and lgkmcnt (11:8) at their maximum: not waited for
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
-    asm volatile("" ::: "memory");
-}
-
 template <int KS, int C, int R, int THREADS, int DEPTH, int PER>
 __global__ __launch_bounds__(THREADS) void col2im_stream(const float* __restrict__ col,
                                                          float* __restrict__ in_deltas, int64_t n,
@@ -808,6 +799,7 @@ __global__ __launch_bounds__(THREADS) void col2im_stream(const float* __restrict
         const int oy0 = phase * R;
         int d = s - mm;                                      // the lane's row is oy0 - pad + d
         if (d < 0) d += M;
+        if (!owner) d = 0;                                   // lanes past the last pixel read where lane 0's row reads, and add nothing
         const int y = oy0 - pl.pad + d;
         const bool mine = owner && y >= 0 && y < pl.h;
         {

@@ -452,7 +452,9 @@ def test_softmax_m(hip, ref):
                                (3, 16384), (2, 70001), (2, 70000), (300, 256), (9, 1024), (9, 1025),
                                # rows 64 KiB or 128 KiB apart: workgroups take the rows in another order,
                                # all of them, some of them and (3 rows) none
-                               (64, 16384), (100, 16384), (70, 32768))
+                               (64, 16384), (100, 16384), (70, 32768),
+                               # more rows than the device holds workgroups at once
+                               (1100, 16384), (1030, 12288))
     for shape in shapes:
         for scale in (1.0, 20.0):
             m = (rand(rng, shape) * scale).astype(F32)
@@ -961,9 +963,10 @@ def test_im2col_col2im_banded_exact(hip, ref):
 # Geometries for the streaming col2im kernel (5x5 windows, stride 1, 1 or 3 channels, col rows of at least
 # 8 KB, one image or more per compute unit): an odd number of col rows (the last phase holds one), padding
 # of 0 and of the kernel size minus one, images of a single phase, more images than workgroups by a
-# remainder, exactly one image per workgroup; the last one stays with the banded kernel (col rows too short).
+# remainder, exactly one image per workgroup, a single col row with lanes left over in the last adding
+# wavefront; the last one stays with the banded kernel (col rows too short).
 STREAM_CASES = [(300, 9, 32, 3, 5, 4), (257, 6, 88, 1, 5, 0), (530, 12, 32, 3, 5, 2), (260, 7, 100, 1, 5, 2),
-                (256, 20, 84, 1, 5, 2), (300, 12, 12, 3, 5, 2)]
+                (256, 20, 84, 1, 5, 2), (256, 5, 100, 1, 5, 0), (300, 12, 12, 3, 5, 2)]
 
 
 def test_col2im_streaming_exact(hip, ref):
@@ -1149,6 +1152,11 @@ m = rng.standard_normal((72, 16384)).astype(np.float32)
 md, sd = h.create_from_numpy(m), h.allocate(m.shape)
 h.softmax_m(md, sd)
 print("SOFTMAX", hashlib.sha256(sd.get().tobytes()).hexdigest())
+for name, shape in (("SOFTMAX_LONG", (1100, 16384)),):
+    m = (rng.standard_normal(shape) * 3).astype(np.float32)
+    md, sd = h.create_from_numpy(m), h.allocate(m.shape)
+    h.softmax_m(md, sd)
+    print(name, hashlib.sha256(sd.get().tobytes()).hexdigest())
 x = rng.standard_normal((100, 4003)).astype(np.float32)
 w = rng.standard_normal((4003, 1001)).astype(np.float32)
 out = h.allocate((100, 1001))
@@ -1186,7 +1194,7 @@ def test_launch_order_switches_leave_the_results_alone():
     # change the summation order, so products are held to the float64 value with either setting
     default, _ = _run_with({})
     plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_STORE_THROUGH_MIN": str(2 ** 40)})
-    for key in ("ADD", "MULTADD", "SOFTMAX"):
+    for key in ("ADD", "MULTADD", "SOFTMAX", "SOFTMAX_LONG"):
         assert default[key] == plain[key], key
     for res in (default, plain):
         assert res["DOT_OK"] == "True" and res["DOTADD_OK"] == "True"
