@@ -1422,12 +1422,12 @@ static bool allow_dynamic_lds(K kernel, size_t bytes) {
 }
 
 // col2im_stream for 5x5 windows with stride 1 on 1 or 3 channels. A phase costs about 0.4 us
-// whatever it carries, so the kernel is used where a phase's col rows are at least kStreamMinPhaseBytes
-// (32x32x3 images under a 5x5 window: 19 KB; there, at batch 2048, 120 us against the banded kernel's
-// 135, and 18 against 24 at batch 256; with 6-11 KB per phase it takes twice the banded kernel's time),
-// and for at least one image per workgroup. *launched says whether it ran.
-constexpr size_t kStreamMinPhaseBytes = 16 * 1024;
-constexpr int kStreamRows = 2, kStreamDepth = 4, kStreamThreads = 1024;
+// whatever it carries, so the kernel is used where a col row is at least kStreamMinColRowBytes
+// (32x32x3 images under a 5x5 window: 9.6 KB; there, at batch 2048, 118-120 us against the banded
+// kernel's 135, and 16 against 24 at batch 256; with col rows of 3-5 KB it takes twice the banded
+// kernel's time), and for at least one image per workgroup. *launched says whether it ran.
+constexpr size_t kStreamMinColRowBytes = 8 * 1024;
+constexpr int kStreamThreads = 1024;
 static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_deltas, int64_t in_pitch, int64_t n,
                              int* launched) {
     *launched = 0;
@@ -1436,28 +1436,33 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
     if (min_per_cu <= 0 || n < min_per_cu * c.num_cus || !aligned16(col) || !aligned16(in_deltas) || in_pitch % 4 != 0)
         return 0;
     if (g.kh != 5 || !(g.c == 1 || g.c == 3)) return 0;   // col rows of 3x3 windows that are long enough need more lanes than a workgroup has
-    if (static_cast<size_t>(kStreamRows) * g.ow * g.kh * g.kw * g.c * sizeof(float) < kStreamMinPhaseBytes) return 0;
+    if (static_cast<size_t>(g.ow) * g.kh * g.kw * g.c * sizeof(float) < kStreamMinColRowBytes) return 0;
     if ((n / c.num_cus + 1) * g.oh > 0x7fffffff) return 0;
+    // four col rows per phase and two phases in flight where the lanes and the LDS allow it (32x32x3 at batch
+    // 2048: 117.5-118 us against 119-119.5 for two rows and four phases), else two rows and four phases
     Col2imStreamPlan sp;
     size_t lds = 0;
-    int per = 0;
-    for (int p : {2, 4, 8, 12})
-        if (per == 0 && plan_col2im_stream(g, kStreamRows, kStreamDepth, kStreamThreads, p, &sp, &lds)) per = p;
+    int rows = 0, per = 0;
+    for (int r : {4, 2})
+        for (int p : {2, 4, 8, 12})
+            if (per == 0 && plan_col2im_stream(g, r, r == 4 ? 2 : 4, kStreamThreads, p, &sp, &lds)) { rows = r; per = p; }
     if (per == 0) return 0;
     sp.in_pitch = in_pitch;
     const dim3 grid(static_cast<unsigned>(c.num_cus));      // one workgroup per compute unit: it takes most of the LDS
-#define BSHIP_COL2IM_STREAM(KS_, C_, P_)                                                                          \
-    if (g.kh == KS_ && g.c == C_ && per == P_) {                                                                  \
-        auto kernel = col2im_stream<KS_, C_, kStreamRows, kStreamThreads, kStreamDepth, P_>;                      \
+#define BSHIP_COL2IM_STREAM(C_, R_, D_, P_)                                                                       \
+    if (g.c == C_ && rows == R_ && per == P_) {                                                                   \
+        auto kernel = col2im_stream<5, C_, R_, kStreamThreads, D_, P_>;                                           \
         if (!allow_dynamic_lds(kernel, lds)) { (void)hipGetLastError(); return 0; }                               \
         hipLaunchKernelGGL(kernel, grid, dim3(kStreamThreads), lds, c.stream, col, in_deltas, n, sp);             \
         *launched = 1;                                                                                            \
         return check_launch("col2im");                                                                            \
     }
-#define BSHIP_COL2IM_STREAM_PER(KS_, C_) \
-    BSHIP_COL2IM_STREAM(KS_, C_, 2) BSHIP_COL2IM_STREAM(KS_, C_, 4) BSHIP_COL2IM_STREAM(KS_, C_, 8) BSHIP_COL2IM_STREAM(KS_, C_, 12)
-    BSHIP_COL2IM_STREAM_PER(5, 3)
-    BSHIP_COL2IM_STREAM_PER(5, 1)
+#define BSHIP_COL2IM_STREAM_PER(C_, R_, D_) \
+    BSHIP_COL2IM_STREAM(C_, R_, D_, 2) BSHIP_COL2IM_STREAM(C_, R_, D_, 4) BSHIP_COL2IM_STREAM(C_, R_, D_, 8) BSHIP_COL2IM_STREAM(C_, R_, D_, 12)
+    BSHIP_COL2IM_STREAM_PER(3, 4, 2)
+    BSHIP_COL2IM_STREAM_PER(3, 2, 4)
+    BSHIP_COL2IM_STREAM_PER(1, 4, 2)
+    BSHIP_COL2IM_STREAM_PER(1, 2, 4)
 #undef BSHIP_COL2IM_STREAM_PER
 #undef BSHIP_COL2IM_STREAM
     return 0;
