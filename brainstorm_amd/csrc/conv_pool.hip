@@ -660,7 +660,8 @@ __global__ __launch_bounds__(kCol2imThreads) void col2im_band(const float* __res
 // registers from the phase with the row's first col row (where they start from the old values:
 // in_deltas is added to) to the phase with its last one (where they are stored). For each col row
 // of the phase in turn, the lane adds the KS terms of its window row ky = y + pad - oy, kx descending:
-// an element receives its terms with oy ascending, then ox ascending - the order of the serial loops.
+// an element receives its terms with oy ascending, then ox ascending - the order of the serial loops
+// (_cpuop 295-309).
 //
 // The other wavefronts request data: the col rows of a phase and the image rows that start in it go
 // to the next slots of two rings in LDS, DEPTH phases before they are needed, as pieces of 1 KiB
