@@ -1422,12 +1422,13 @@ static bool allow_dynamic_lds(K kernel, size_t bytes) {
     return allow_dynamic_lds_impl(reinterpret_cast<const void*>(kernel), bytes);
 }
 
-// col2im_stream for 5x5 windows with stride 1 on 1 or 3 channels. A phase costs about 0.4 us
-// whatever it carries, so the kernel is used where a col row is at least kStreamMinColRowBytes
-// (32x32x3 images under a 5x5 window: 9.6 KB; there, at batch 2048, 118-120 us against the banded
-// kernel's 135, and 16 against 24 at batch 256; with col rows of 3-5 KB it takes twice the banded
-// kernel's time), and for at least one image per workgroup. *launched says whether it ran.
-constexpr size_t kStreamMinColRowBytes = 8 * 1024;
+// col2im_stream for 5x5 windows with stride 1 on 1 or 3 channels. A phase costs about 0.4 us whatever it
+// carries, so the kernel is used where a phase of four (or two) col rows holds at least kStreamMinPhaseBytes.
+// Measured at batch 2048 against the banded kernel: 32x32x3 (col rows of 9.6 KB) 118 us against 138, and 16
+// against 24 at batch 256; 24x24x3 (7.2 KB) 66 against 79; 64x64x1 at batch 1024 (6.4 KB) 76 against 88;
+// 16x16x3 and 48x48x1 (4.8 KB) 7 % ahead; col rows of 4.0 KB 6 % behind, 28x28x1 (2.8 KB, eight rows per
+// phase) 20 % behind. Needs at least one image per workgroup. *launched says whether it ran.
+constexpr size_t kStreamMinPhaseBytes = 18 * 1024;
 constexpr int kStreamThreads = 1024;
 static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_deltas, int64_t in_pitch, int64_t n,
                              int* launched) {
@@ -1437,16 +1438,18 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
     if (min_per_cu <= 0 || n < min_per_cu * c.num_cus || !aligned16(col) || !aligned16(in_deltas) || in_pitch % 4 != 0)
         return 0;
     if (g.kh != 5 || !(g.c == 1 || g.c == 3)) return 0;   // col rows of 3x3 windows that are long enough need more lanes than a workgroup has
-    if (static_cast<size_t>(g.ow) * g.kh * g.kw * g.c * sizeof(float) < kStreamMinColRowBytes) return 0;
+    const size_t col_row_bytes = static_cast<size_t>(g.ow) * g.kh * g.kw * g.c * sizeof(float);
     if ((n / c.num_cus + 1) * g.oh > 0x7fffffff) return 0;
     // four col rows per phase and two phases in flight where the lanes and the LDS allow it (32x32x3 at batch
     // 2048: 117.5-118 us against 119-119.5 for two rows and four phases), else two rows and four phases
     Col2imStreamPlan sp;
     size_t lds = 0;
     int rows = 0, per = 0;
-    for (int r : {4, 2})
+    for (int r : {4, 2}) {
+        if (r * col_row_bytes < kStreamMinPhaseBytes) continue;
         for (int p : {2, 4, 8, 12})
-            if (per == 0 && plan_col2im_stream(g, r, r == 4 ? 2 : 4, kStreamThreads, p, &sp, &lds)) { rows = r; per = p; }
+            if (per == 0 && plan_col2im_stream(g, r, r == 2 ? 4 : 2, kStreamThreads, p, &sp, &lds)) { rows = r; per = p; }
+    }
     if (per == 0) return 0;
     sp.in_pitch = in_pitch;
     const dim3 grid(static_cast<unsigned>(c.num_cus));      // one workgroup per compute unit: it takes most of the LDS
