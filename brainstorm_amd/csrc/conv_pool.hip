@@ -1422,14 +1422,15 @@ static bool allow_dynamic_lds(K kernel, size_t bytes) {
     return allow_dynamic_lds_impl(reinterpret_cast<const void*>(kernel), bytes);
 }
 
-// col2im_stream for 5x5 windows with stride 1 on 1 or 3 channels. A phase costs about 0.4 us whatever it
-// carries, so the kernel is used where a phase of four (or two) col rows holds at least kStreamMinPhaseBytes.
-// Measured at batch 2048 against the banded kernel: 32x32x3 (col rows of 9.6 KB) 118 us against 138, and 16
-// against 24 at batch 256; 24x24x3 (7.2 KB) 66 against 79; 64x64x1 at batch 1024 (6.4 KB) 76 against 88;
-// 16x16x3 and 48x48x1 (4.8 KB) 7 % ahead; col rows of 4.0 KB 6 % behind, 28x28x1 (2.8 KB, eight rows per
-// phase) 20 % behind. Needs at least one image per workgroup. *launched says whether it ran.
+// col2im_stream for 5x5 windows on 1 or 3 channels and 3x3 windows on 3, stride 1. A phase costs about 0.4 us whatever
+// it carries, so the kernel is used where a phase of four (or two) col rows holds at least kStreamMinPhaseBytes.
+// Measured at batch 2048 against the banded kernel: 32x32x3 under 5x5 (col rows of 9.6 KB) 118 us against 138,
+// and 16 against 24 at batch 256; 24x24x3 (7.2 KB) 66 against 79; 64x64x1 at batch 1024 (6.4 KB) 76 against 88;
+// 64x64x3 under 3x3 (6.9 KB) 195 against 213, 96x96x3 at batch 1024 221 against 256; 16x16x3 and 48x48x1
+// (4.8 KB) 7 % ahead; col rows of 4.0 KB 6 % behind, 28x28x1 (2.8 KB, eight rows per phase) 20 % behind.
+// Needs at least one image per workgroup. *launched says whether it ran.
 constexpr size_t kStreamMinPhaseBytes = 18 * 1024;
-constexpr int kStreamThreads = 1024;
+constexpr int kStreamThreads = 1024, kStreamMinRequesters = 6;
 static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_deltas, int64_t in_pitch, int64_t n,
                              int* launched) {
     *launched = 0;
@@ -1437,7 +1438,8 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
     const int64_t min_per_cu = c.col2im_stream_min_images_per_cu;
     if (min_per_cu <= 0 || n < min_per_cu * c.num_cus || !aligned16(col) || !aligned16(in_deltas) || in_pitch % 4 != 0)
         return 0;
-    if (g.kh != 5 || !(g.c == 1 || g.c == 3)) return 0;   // col rows of 3x3 windows that are long enough need more lanes than a workgroup has
+    // (3x3 windows on one channel: col rows long enough would need more adding wavefronts than the rules below allow)
+    if (!((g.kh == 5 && (g.c == 1 || g.c == 3)) || (g.kh == 3 && g.c == 3))) return 0;
     const size_t col_row_bytes = static_cast<size_t>(g.ow) * g.kh * g.kw * g.c * sizeof(float);
     if ((n / c.num_cus + 1) * g.oh > 0x7fffffff) return 0;
     // four col rows per phase and two phases in flight where the lanes and the LDS allow it (32x32x3 at batch
@@ -1447,26 +1449,35 @@ static int try_col2im_stream(const ImgGeom& g, const float* col, float* in_delta
     int rows = 0, per = 0;
     for (int r : {4, 2}) {
         if (r * col_row_bytes < kStreamMinPhaseBytes) continue;
-        for (int p : {2, 4, 8, 12})
-            if (per == 0 && plan_col2im_stream(g, r, r == 2 ? 4 : 2, kStreamThreads, p, &sp, &lds)) { rows = r; per = p; }
+        for (int p : {2, 4, 8, 12}) {
+            Col2imStreamPlan candidate;
+            if (per != 0 || !plan_col2im_stream(g, r, r == 2 ? 4 : 2, kStreamThreads, p, &candidate, &lds)) continue;
+            // with fewer requesting wavefronts the kernel falls behind the banded one (128x128x1 under 3x3:
+            // 12 adding and 4 requesting wavefronts, 166 us against 140)
+            if (kStreamThreads / kWave - candidate.add_waves < kStreamMinRequesters) continue;
+            sp = candidate; rows = r; per = p;
+        }
     }
     if (per == 0) return 0;
     sp.in_pitch = in_pitch;
     const dim3 grid(static_cast<unsigned>(c.num_cus));      // one workgroup per compute unit: it takes most of the LDS
-#define BSHIP_COL2IM_STREAM(C_, R_, D_, P_)                                                                       \
-    if (g.c == C_ && rows == R_ && per == P_) {                                                                   \
-        auto kernel = col2im_stream<5, C_, R_, kStreamThreads, D_, P_>;                                           \
+#define BSHIP_COL2IM_STREAM(KS_, C_, R_, D_, P_)                                                                  \
+    if (g.kh == KS_ && g.c == C_ && rows == R_ && per == P_) {                                                    \
+        auto kernel = col2im_stream<KS_, C_, R_, kStreamThreads, D_, P_>;                                         \
         if (!allow_dynamic_lds(kernel, lds)) { (void)hipGetLastError(); return 0; }                               \
         hipLaunchKernelGGL(kernel, grid, dim3(kStreamThreads), lds, c.stream, col, in_deltas, n, sp);             \
         *launched = 1;                                                                                            \
         return check_launch("col2im");                                                                            \
     }
-#define BSHIP_COL2IM_STREAM_PER(C_, R_, D_) \
-    BSHIP_COL2IM_STREAM(C_, R_, D_, 2) BSHIP_COL2IM_STREAM(C_, R_, D_, 4) BSHIP_COL2IM_STREAM(C_, R_, D_, 8) BSHIP_COL2IM_STREAM(C_, R_, D_, 12)
-    BSHIP_COL2IM_STREAM_PER(3, 4, 2)
-    BSHIP_COL2IM_STREAM_PER(3, 2, 4)
-    BSHIP_COL2IM_STREAM_PER(1, 4, 2)
-    BSHIP_COL2IM_STREAM_PER(1, 2, 4)
+#define BSHIP_COL2IM_STREAM_PER(KS_, C_, R_, D_)                                                 \
+    BSHIP_COL2IM_STREAM(KS_, C_, R_, D_, 2) BSHIP_COL2IM_STREAM(KS_, C_, R_, D_, 4)             \
+    BSHIP_COL2IM_STREAM(KS_, C_, R_, D_, 8) BSHIP_COL2IM_STREAM(KS_, C_, R_, D_, 12)
+    BSHIP_COL2IM_STREAM_PER(5, 3, 4, 2)
+    BSHIP_COL2IM_STREAM_PER(5, 3, 2, 4)
+    BSHIP_COL2IM_STREAM_PER(5, 1, 4, 2)
+    BSHIP_COL2IM_STREAM_PER(5, 1, 2, 4)
+    BSHIP_COL2IM_STREAM_PER(3, 3, 4, 2)
+    BSHIP_COL2IM_STREAM_PER(3, 3, 2, 4)
 #undef BSHIP_COL2IM_STREAM_PER
 #undef BSHIP_COL2IM_STREAM
     return 0;

@@ -960,13 +960,14 @@ def test_im2col_col2im_banded_exact(hip, ref):
         assert_bit_equal(dind.get(), want, "col2im %r" % ((n, h, w, c, kh, kw, pad, stride),))
 
 
-# Geometries for the streaming col2im kernel (5x5 windows, stride 1, 1 or 3 channels, col rows of at least
-# 4.5 KB, one image or more per compute unit): an odd number of col rows (the last phase holds one), padding
+# Geometries for the streaming col2im kernel (3x3 and 5x5 windows, stride 1, 1 or 3 channels, col rows of at
+# least 4.5 KB, one image or more per compute unit): an odd number of col rows (the last phase holds one), padding
 # of 0 and of the kernel size minus one, images of a single phase, more images than workgroups by a
 # remainder, exactly one image per workgroup, a single col row with lanes left over in the last adding
 # wavefront; the last one stays with the banded kernel (col rows too short).
 STREAM_CASES = [(300, 9, 32, 3, 5, 4), (257, 6, 88, 1, 5, 0), (530, 12, 32, 3, 5, 2), (260, 7, 100, 1, 5, 2),
-                (256, 20, 84, 1, 5, 2), (256, 5, 100, 1, 5, 0), (290, 11, 16, 3, 5, 2), (300, 12, 12, 3, 5, 2)]
+                (256, 20, 84, 1, 5, 2), (256, 5, 100, 1, 5, 0), (290, 11, 16, 3, 5, 2), (270, 9, 64, 3, 3, 1),
+                (260, 5, 104, 3, 3, 1), (300, 12, 12, 3, 5, 2)]
 
 
 def test_col2im_streaming_exact(hip, ref):
