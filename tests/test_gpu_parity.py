@@ -1158,6 +1158,11 @@ for name, shape in (("SOFTMAX_LONG", (1100, 16384)),):
     md, sd = h.create_from_numpy(m), h.allocate(m.shape)
     h.softmax_m(md, sd)
     print(name, hashlib.sha256(sd.get().tobytes()).hexdigest())
+cols = rng.standard_normal((260, 12 * 32, 75)).astype(np.float32)
+dimg = rng.standard_normal((260, 12, 32, 3)).astype(np.float32)
+cd, dd = h.create_from_numpy(cols), h.create_from_numpy(dimg)
+h._call(h._lib.bship_col2im_nhwc_f32(cd.ptr, dd.ptr, 260, 12, 32, 3, 5, 5, 2, 1, 1))
+print("COL2IM", hashlib.sha256(dd.get().tobytes()).hexdigest())
 x = rng.standard_normal((100, 4003)).astype(np.float32)
 w = rng.standard_normal((4003, 1001)).astype(np.float32)
 out = h.allocate((100, 1001))
@@ -1191,11 +1196,13 @@ def _run_with(env_extra):
 def test_launch_order_switches_leave_the_results_alone():
     # the order in which tiles and rows are dealt to the XCDs and the kind of store (write-through for
     # outputs of 2^18 to 2^26 elements, as the three here) are a matter of speed only: elementwise results
-    # and softmax rows are the same bits with and without them; the product's kernel choice may
+    # and softmax rows are the same bits with and without them, col2im with either of its kernels for
+    # 3-channel images as well; the product's kernel choice may
     # change the summation order, so products are held to the float64 value with either setting
     default, _ = _run_with({})
-    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_STORE_THROUGH_MIN": str(2 ** 40)})
-    for key in ("ADD", "MULTADD", "SOFTMAX", "SOFTMAX_LONG"):
+    plain, _ = _run_with({"BSHIP_EW_RUN_KB": "0", "BSHIP_SM_CHUNK_KB": "0", "BSHIP_STORE_THROUGH_MIN": str(2 ** 40),
+                          "BSHIP_COL2IM_STREAM_MIN": "0"})
+    for key in ("ADD", "MULTADD", "SOFTMAX", "SOFTMAX_LONG", "COL2IM"):
         assert default[key] == plain[key], key
     for res in (default, plain):
         assert res["DOT_OK"] == "True" and res["DOTADD_OK"] == "True"
