@@ -371,6 +371,8 @@ def run_nets_gpu(hip):
                                                                   hip.synchronize, fused="sequence"),
         # the convolutional workload (conv 5x5x32, max pool 3x3/2, conv 5x5x64, max pool, 1000, 10)
         "cnn_32x32x3_batch100": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize),
+        # same network and bits, the step recorded into a HIP graph and replayed
+        "cnn_32x32x3_batch100_recorded": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize, recorded=True),
         # the bandwidth-stress workload: 50 Highway + batch normalisation blocks of width 4096
         "highway_bn_50x4096_batch2048": time_net(hip, configs.build_highway, 3, 1, hip.synchronize),
         "highway_bn_50x4096_batch2048_fused": time_net(hip, configs.build_highway, 3, 1, hip.synchronize,

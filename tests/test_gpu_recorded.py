@@ -208,9 +208,9 @@ def test_recorded_training_steps_equal_eager_ones():
     from brainstorm_amd.drivers import configs
     from brainstorm_amd.drivers.net import MomentumStepper
 
-    def train(recorded, fused):
+    def train(recorded, fused, builder=configs.build_mlp):
         h = HipHandler(seed=77)
-        net, data = configs.build_mlp(h, fused=fused)
+        net, data = builder(h, fused=fused)
         net.provide_external_data(data)
         stepper = MomentumStepper(0.1, 0.9, fused=fused)
         stepper.start(net)
@@ -231,6 +231,11 @@ def test_recorded_training_steps_equal_eager_ones():
         got_losses, got_params = train(True, fused)
         assert got_losses == want_losses, (fused, got_losses, want_losses)
         assert_bit_equal(got_params, want_params, "parameters after recorded steps (fused=%r)" % fused)
+    # the convolutional workload: im2col / col2im, pooling and products with a bias epilogue inside the recording
+    want_losses, want_params = train(False, False, configs.build_cnn)
+    got_losses, got_params = train(True, False, configs.build_cnn)
+    assert got_losses == want_losses, (got_losses, want_losses)
+    assert_bit_equal(got_params, want_params, "parameters after recorded steps of the convolutional workload")
 
 
 def test_graph_entry_points_report_misuse(hip):
