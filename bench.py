@@ -373,6 +373,10 @@ def run_nets_gpu(hip):
         "cnn_32x32x3_batch100": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize),
         # same network and bits, the step recorded into a HIP graph and replayed
         "cnn_32x32x3_batch100_recorded": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize, recorded=True),
+        # ... with the fused entry points (bias + activation, softmax cross entropy, momentum update; same bits)
+        "cnn_32x32x3_batch100_fused": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize, fused=True),
+        "cnn_32x32x3_batch100_fused_recorded": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize,
+                                                        recorded=True, fused=True),
         # the bandwidth-stress workload: 50 Highway + batch normalisation blocks of width 4096
         "highway_bn_50x4096_batch2048": time_net(hip, configs.build_highway, 3, 1, hip.synchronize),
         "highway_bn_50x4096_batch2048_fused": time_net(hip, configs.build_highway, 3, 1, hip.synchronize,
