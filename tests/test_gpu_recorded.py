@@ -232,10 +232,12 @@ def test_recorded_training_steps_equal_eager_ones():
         assert got_losses == want_losses, (fused, got_losses, want_losses)
         assert_bit_equal(got_params, want_params, "parameters after recorded steps (fused=%r)" % fused)
     # the convolutional workload: im2col / col2im, pooling and products with a bias epilogue inside the recording
-    want_losses, want_params = train(False, False, configs.build_cnn)
-    got_losses, got_params = train(True, False, configs.build_cnn)
-    assert got_losses == want_losses, (got_losses, want_losses)
-    assert_bit_equal(got_params, want_params, "parameters after recorded steps of the convolutional workload")
+    for fused in (False, True):
+        want_losses, want_params = train(False, fused, configs.build_cnn)
+        got_losses, got_params = train(True, fused, configs.build_cnn)
+        assert got_losses == want_losses, (fused, got_losses, want_losses)
+        assert_bit_equal(got_params, want_params,
+                         "parameters after recorded steps of the convolutional workload (fused=%r)" % fused)
 
 
 def test_graph_entry_points_report_misuse(hip):
