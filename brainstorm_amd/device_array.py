@@ -59,6 +59,18 @@ class DeviceArray:
         self._owner = owner         # keeps the pool block alive
         self._handler = handler     # for get()
 
+    @classmethod
+    def _view_of(cls, parent, ptr, shape, size):
+        """A dense view into ``parent``'s memory whose size is known (the views of the recurrent
+        layers' inner loops are made thousands of times per step: no product over the shape)."""
+        v = cls.__new__(cls)
+        v.ptr = ptr
+        v.shape = shape
+        v.size = size
+        v._owner = parent._owner
+        v._handler = parent._handler
+        return v
+
     # ---------------------------------------------------------------- basics
     @property
     def ndim(self):
@@ -171,10 +183,8 @@ class DeviceArray:
                 key += n
             if not 0 <= key < n:
                 raise IndexError("index out of bounds for axis 0 with size %d" % n)
-            rest = shape[1:]
             inner = self.size // n
-            return DeviceArray(self.ptr + key * inner * ITEMSIZE if self.ptr else 0, rest,
-                               self._owner, self._handler)
+            return DeviceArray._view_of(self, self.ptr + key * inner * ITEMSIZE if self.ptr else 0, shape[1:], inner)
         if type(key) is slice:
             if not shape:
                 raise IndexError("too many indices for a 0-d array")
@@ -184,8 +194,8 @@ class DeviceArray:
             start, stop, _ = key.indices(n)
             length = max(0, stop - start)
             inner = self.size // n if n else _prod(shape[1:])
-            return DeviceArray(self.ptr + start * inner * ITEMSIZE if self.ptr else 0,
-                               (length,) + shape[1:], self._owner, self._handler)
+            return DeviceArray._view_of(self, self.ptr + start * inner * ITEMSIZE if self.ptr else 0,
+                                        (length,) + shape[1:], length * inner)
         return self._getitem_general(key)
 
     def _getitem_general(self, key):
