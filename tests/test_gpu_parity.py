@@ -867,7 +867,9 @@ CONV_CASES = [(2, 5, 4, 3, 2, 3, 3, 0, (1, 1)), (2, 5, 4, 3, 2, 3, 3, 1, (2, 1))
               (2, 6, 6, 3, 4, 2, 2, 1, (2, 2)), (5, 8, 4, 2, 3, 3, 3, 1, (1, 1)), (9, 6, 6, 1, 2, 3, 3, 1, (1, 1)),
               # 3x3 and 5x5 windows with stride 1 and 16 or more channels (col2im with all terms of an element
               # loaded together): no padding, the usual padding, and a padding as wide as the window allows
-              (3, 7, 6, 16, 4, 3, 3, 1, (1, 1)), (2, 9, 8, 20, 4, 5, 5, 0, (1, 1)), (2, 6, 7, 16, 4, 5, 5, 4, (1, 1))]
+              (3, 7, 6, 16, 4, 3, 3, 1, (1, 1)), (2, 9, 8, 20, 4, 5, 5, 0, (1, 1)), (2, 6, 7, 16, 4, 5, 5, 4, (1, 1)),
+              # an image per compute unit and col rows of 9.6 KB: the backward pass's col2im streams the col matrix into LDS
+              (256, 10, 32, 3, 4, 5, 5, 2, (1, 1))]
 
 
 def test_conv2d_forward_backward(hip, ref):
