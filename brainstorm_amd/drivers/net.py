@@ -170,20 +170,18 @@ class Net:
         self.apply_gradient_modifiers()                    # network.py:445
 
     def apply_weight_modifiers(self):
-        """network.py:490-495; ``weight_modifiers`` maps (layer, parameter) to a list of modifiers."""
-        for (layer, view), mods in getattr(self, "weight_modifiers", {}).items():
-            for mod in mods:
-                mod(self.handler, self.buffers[layer].parameters[view])
+        """After every update (network.py:490-495): ``weight_modifiers`` maps (layer, parameter) to a list of
+        callables ``hook(handler, view)``."""
+        for (layer, view), hooks in getattr(self, "weight_modifiers", {}).items():
+            for hook in hooks:
+                hook(self.handler, self.buffers[layer].parameters[view])
 
     def apply_gradient_modifiers(self):
-        """network.py:497-509: GradientModifiers get (parameters, gradients), others the gradients."""
-        from .modifiers import GradientModifier
-        for (layer, view), mods in getattr(self, "gradient_modifiers", {}).items():
-            for mod in mods:
-                if isinstance(mod, GradientModifier):
-                    mod(self.handler, self.buffers[layer].parameters[view], self.buffers[layer].gradients[view])
-                else:
-                    mod(self.handler, self.buffers[layer].gradients[view])
+        """At the end of the backward pass (network.py:497-509): ``gradient_modifiers`` maps (layer, parameter)
+        to a list of callables ``hook(handler, parameters, gradients)``."""
+        for (layer, view), hooks in getattr(self, "gradient_modifiers", {}).items():
+            for hook in hooks:
+                hook(self.handler, self.buffers[layer].parameters[view], self.buffers[layer].gradients[view])
 
     def get(self, layer, group, name):
         return self.handler.get_numpy_copy(getattr(self.buffers[layer], group)[name])

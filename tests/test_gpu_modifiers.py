@@ -1,10 +1,11 @@
-"""GPU: arithmetic operators of DeviceArray, the value/gradient modifiers that use them, and the
-contract-checking wrapper around HipHandler, each against the CPU oracle on the same inputs."""
+"""GPU: arithmetic operators of DeviceArray, the modifier-like op sequences that use them (modifier_ops.py),
+and the contract-checking wrapper around HipHandler, each against the CPU oracle on the same inputs."""
 import numpy as np
 import pytest
 
 from brainstorm_amd.checked_handler import CheckedHandler, ContractError
-from brainstorm_amd.drivers import configs, modifiers
+import modifier_ops
+from brainstorm_amd.drivers import configs
 from brainstorm_amd.drivers.net import MomentumStepper
 from oracle.numpy_ref_handler import NumpyRefHandler
 from util import assert_bit_equal
@@ -43,7 +44,7 @@ def test_modifiers_match_the_oracle(hip):
     g = rng.standard_normal(w.shape).astype(F32)
     mask = (rng.uniform(size=w.shape) < 0.5).astype(F32)
 
-    def both(make, exact=True, with_grad=False):
+    def both(what, make, exact=True, with_grad=False):
         outs = []
         for h in (hip, ref):
             view = h.create_from_numpy(w.copy())
@@ -56,28 +57,29 @@ def test_modifiers_match_the_oracle(hip):
                 mod(h, view)
                 outs.append(h.get_numpy_copy(view))
         if exact:
-            assert_bit_equal(outs[0], outs[1], make().__class__.__name__)
+            assert_bit_equal(outs[0], outs[1], what)
         return outs
 
-    got, want = both(lambda: modifiers.ConstrainL2Norm(2.0), exact=False)
-    np.testing.assert_allclose(got, want, rtol=1e-5)             # row sums of squares: 1e-5 relative
-    assert np.sqrt((got.reshape(300, -1).astype(np.float64) ** 2).sum(axis=1)).max() <= 2.0 * (1 + 1e-5)
-    both(lambda: modifiers.ClipValues(-0.5, 0.25))
-    both(lambda: modifiers.MaskValues(mask))
-    both(lambda: modifiers.FreezeValues(weights=g))
-    both(lambda: modifiers.L1Decay(0.01), with_grad=True)
-    both(lambda: modifiers.L2Decay(0.01), with_grad=True)
+    for with_operators in (True, False):
+        got, want = both("cap_row_norms", lambda: modifier_ops.cap_row_norms(2.0, with_operators), exact=False)
+        np.testing.assert_allclose(got, want, rtol=1e-5)         # row sums of squares: 1e-5 relative
+        assert np.sqrt((got.reshape(300, -1).astype(np.float64) ** 2).sum(axis=1)).max() <= 2.0 * (1 + 1e-5)
+    both("clamp", lambda: modifier_ops.clamp(-0.5, 0.25))
+    both("keep_where", lambda: modifier_ops.keep_where(mask))
+    both("hold_values", lambda: modifier_ops.hold_values(g))
+    both("shrink_l1", lambda: modifier_ops.shrink_l1(0.01), with_grad=True)
+    both("shrink_l2", lambda: modifier_ops.shrink_l2(0.01), with_grad=True)
 
 
 def test_mlp_with_norm_constraint_trains_like_the_oracle(hip):
-    # the shape of examples/mnist_pi.py including its ConstrainL2Norm weight modifiers
+    # the shape of examples/mnist_pi.py including a row-norm cap on every weight matrix after each update
     nets = []
     for h in (hip, NumpyRefHandler(F32, seed=9)):
         if h is hip:
             hip.rnd.seed(9)
         net, data = configs.build_mlp(h, batch=50, in_size=64, hidden=96)
         net.provide_external_data(data)
-        net.weight_modifiers = {(name, "W"): [modifiers.ConstrainL2Norm(0.3)] for name in ("fc1", "fc2", "out")}
+        net.weight_modifiers = {(name, "W"): [modifier_ops.cap_row_norms(0.3)] for name in ("fc1", "fc2", "out")}
         stepper = MomentumStepper(0.1, 0.9)
         stepper.start(net)
         for _ in range(10):
