@@ -87,6 +87,20 @@ SIGNATURES = {
     "bship_prob_mask_fast_f32": [_P, c_size_t, c_double],
     "bship_dropout_fwd_fast_f32": [_P, _P, _P, c_size_t, c_double, c_float],
     "bship_rng_get_state": [POINTER(c_uint32), POINTER(c_int), POINTER(c_int), POINTER(c_double)],
+    "bship_rng_seed_on": [c_int, c_uint32],
+    "bship_rng_get_state_on": [c_int, POINTER(c_uint32), POINTER(c_int), POINTER(c_int), POINTER(c_double)],
+    "bship_prob_mask_on_f32": [c_int, _P, c_size_t, c_double],
+    "bship_prob_mask_pitched_on_f32": [c_int, _P, _I64, _I64, _I64, c_double],
+    "bship_fill_gaussian_on_f32": [c_int, _P, c_size_t, c_double, c_double],
+    "bship_dropout_fwd_on_f32": [c_int, _P, _P, _P, c_size_t, c_double, c_float],
+    "bship_fast_rng_seed_on": [c_int, ctypes.c_ulonglong],
+    "bship_fast_rng_get_state_on": [c_int, POINTER(ctypes.c_ulonglong), POINTER(ctypes.c_ulonglong)],
+    "bship_prob_mask_fast_on_f32": [c_int, _P, c_size_t, c_double],
+    "bship_dropout_fwd_fast_on_f32": [c_int, _P, _P, _P, c_size_t, c_double, c_float],
+    "bship_fusing_set": [c_int],
+    "bship_fusing_get": [POINTER(c_int)],
+    "bship_fusing_flush": [],
+    "bship_fusing_stats": [POINTER(ctypes.c_ulonglong)] * 5 + [c_int],
     "bship_gemm_f32": [c_int, c_int, _I64, _I64, _I64, c_float, _P, _I64, _P, _I64, c_float, _P, _I64],
     "bship_gemm_bias_f32": [c_int, c_int, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P, _I64],
     "bship_im2col_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,

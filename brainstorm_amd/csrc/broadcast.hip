@@ -5,6 +5,7 @@
 #pragma clang fp contract(off)
 
 #include "common.h"
+#include "window.h"
 
 namespace bship {
 
@@ -171,7 +172,7 @@ extern "C" {
 
 int bship_mv_f32(int op, const float* m, const float* v, float* out, int64_t M, int64_t N,
                  int v_is_col, int accumulate) {
-    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
     BSHIP_REQUIRE_DIM(M >= 0 && N >= 0);
     if (M == 0 || N == 0) return 0;
     BSHIP_REQUIRE_PTR(m);
@@ -180,6 +181,10 @@ int bship_mv_f32(int op, const float* m, const float* v, float* out, int64_t M, 
     BSHIP_REQUIRE_F32_ALIGNED(m);
     BSHIP_REQUIRE_F32_ALIGNED(v);
     BSHIP_REQUIRE_F32_ALIGNED(out);
+    if (op < BSHIP_ADD || op > BSHIP_DIV) return set_error(BSHIP_ERR_BAD_OP, "bship_mv_f32: unknown op %d", op);
+    // matrix-vector operations open and fill most of the layers' sequences: through the fusing window
+    if (window_takes()) return window_push(window::rec_mv(op, m, v, out, M, N, v_is_col != 0, accumulate != 0));
+    BSHIP_FLUSH_PENDING();
     if (accumulate) {
         switch (op) {
             case BSHIP_ADD: return launch_mv<true>("add_mv(acc)", MvAdd<true>{}, m, v, out, M, N, v_is_col);

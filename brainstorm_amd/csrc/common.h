@@ -66,6 +66,19 @@ int check_launch(const char* what);
 int flush_deferred_fills();
 extern std::atomic<int> g_deferred_fill_count;   // read without the list's lock: 0 means nothing to do
 
+// The fusing window (window.hip, window_core.h) holds back operations that may turn out to be the
+// beginning of a layer's sequence. Entry points that take part hand their call to window_push()
+// while window_takes(); every other entry point first enqueues what is held (BSHIP_REQUIRE_INIT),
+// so the order of effects stays the order of the calls. While the window itself enqueues kernels
+// through the public entry points, t_window_emitting keeps them from coming back to it.
+extern std::atomic<int> g_window_on;       // bship_fusing_set
+extern std::atomic<int> g_window_held;     // operations held right now
+extern thread_local bool t_window_emitting;
+int window_flush();
+static inline bool window_takes() {
+    return g_window_on.load(std::memory_order_relaxed) != 0 && !t_window_emitting;
+}
+
 #define BSHIP_REQUIRE_INIT_NO_FLUSH()                                            \
     do {                                                                         \
         if (!::bship::ctx().inited)                                              \
@@ -74,13 +87,27 @@ extern std::atomic<int> g_deferred_fill_count;   // read without the list's lock
                                       __func__);                                 \
     } while (0)
 
-#define BSHIP_REQUIRE_INIT()                                                     \
+// What earlier calls left behind goes first. Noted fills are older than anything the window holds
+// (with the window on, a fill is noted only when the window lets it go), and the entry points
+// through which the window enqueues held operations start with this same macro, so the fills
+// still go first.
+#define BSHIP_FLUSH_PENDING()                                                    \
     do {                                                                         \
-        BSHIP_REQUIRE_INIT_NO_FLUSH();                                           \
+        if (::bship::g_window_held.load(std::memory_order_relaxed) != 0 &&       \
+            !::bship::t_window_emitting) {                                       \
+            int flush_st_ = ::bship::window_flush();                             \
+            if (flush_st_ != 0) return flush_st_;                                \
+        }                                                                        \
         if (::bship::g_deferred_fill_count.load(std::memory_order_relaxed) != 0) { \
             int flush_st_ = ::bship::flush_deferred_fills();                     \
             if (flush_st_ != 0) return flush_st_;                                \
         }                                                                        \
+    } while (0)
+
+#define BSHIP_REQUIRE_INIT()                                                     \
+    do {                                                                         \
+        BSHIP_REQUIRE_INIT_NO_FLUSH();                                           \
+        BSHIP_FLUSH_PENDING();                                                   \
     } while (0)
 
 #define BSHIP_REQUIRE_PTR(p)                                                     \

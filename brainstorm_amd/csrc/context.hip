@@ -106,7 +106,9 @@ int bship_init(int device) {
 int bship_shutdown(void) {
     std::lock_guard<std::mutex> lock(g_ctx_mutex);
     if (!g_ctx.inited) return 0;
+    (void)window_flush();
     (void)flush_deferred_fills();
+    g_window_on.store(0);
     graph_release_all();
     (void)hipStreamSynchronize(g_ctx.stream);
     gemm_release();

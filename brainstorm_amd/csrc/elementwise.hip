@@ -11,6 +11,7 @@
 #pragma clang fp contract(off)
 
 #include "common.h"
+#include "window.h"
 #include "functors.h"
 
 namespace bship {
@@ -88,13 +89,23 @@ int launch_ew(const char* name, F f, const float* p0, const float* p1, const flo
 
 using namespace bship;
 
+// The elementwise entry points go through the fusing window: the checks first, then either the
+// window takes the call (BSHIP_EW_WINDOW) or what earlier calls left behind is enqueued and the
+// kernel launched.
 #define BSHIP_EW_PROLOGUE(first, outp)        \
-    BSHIP_REQUIRE_INIT();                     \
+    BSHIP_REQUIRE_INIT_NO_FLUSH();            \
     if (n == 0) return 0;                     \
     BSHIP_REQUIRE_PTR(first);                 \
     BSHIP_REQUIRE_PTR(outp);                  \
     BSHIP_REQUIRE_F32_ALIGNED(first);         \
     BSHIP_REQUIRE_F32_ALIGNED(outp)
+
+#define BSHIP_EW_WINDOW(op_ok, what, record)                                                     \
+    do {                                                                                         \
+        if (!(op_ok)) return set_error(BSHIP_ERR_BAD_OP, "%s: unknown op %d", __func__, what);   \
+        if (window_takes()) return window_push(record);                                          \
+        BSHIP_FLUSH_PENDING();                                                                   \
+    } while (0)
 
 extern "C" {
 
@@ -102,6 +113,7 @@ int bship_binary_f32(int op, const float* a, const float* b, float* out, size_t 
     BSHIP_EW_PROLOGUE(a, out);
     BSHIP_REQUIRE_PTR(b);
     BSHIP_REQUIRE_F32_ALIGNED(b);
+    BSHIP_EW_WINDOW(op >= BSHIP_ADD && op <= BSHIP_FMOD, op, window::rec_binary(op, a, b, out, n));
     switch (op) {
         case BSHIP_ADD:  return launch_ew<2>("add_tt", AddOp{}, a, b, nullptr, out, n);
         case BSHIP_SUB:  return launch_ew<2>("subtract_tt", SubOp{}, a, b, nullptr, out, n);
@@ -116,11 +128,13 @@ int bship_mult_add_tt_f32(const float* a, const float* b, float* out, size_t n) 
     BSHIP_EW_PROLOGUE(a, out);
     BSHIP_REQUIRE_PTR(b);
     BSHIP_REQUIRE_F32_ALIGNED(b);
+    BSHIP_EW_WINDOW(true, 0, window::rec_mult_add_tt(a, b, out, n));
     return launch_ew<3>("mult_add_tt", MultAddOp{}, a, b, out, out, n);
 }
 
 int bship_scalar_f32(int op, float s, const float* t, float* out, size_t n) {
     BSHIP_EW_PROLOGUE(t, out);
+    BSHIP_EW_WINDOW(op >= BSHIP_ADD_ST && op <= BSHIP_MULT_ADD_ST, op, window::rec_scalar(op, s, t, out, n));
     switch (op) {
         case BSHIP_ADD_ST:      return launch_ew<1>("add_st", AddStOp{s}, t, nullptr, nullptr, out, n);
         case BSHIP_MULT_ST:     return launch_ew<1>("mult_st", MultStOp{s}, t, nullptr, nullptr, out, n);
@@ -131,6 +145,7 @@ int bship_scalar_f32(int op, float s, const float* t, float* out, size_t n) {
 
 int bship_unary_f32(int op, const float* x, float* y, size_t n) {
     BSHIP_EW_PROLOGUE(x, y);
+    BSHIP_EW_WINDOW(op >= BSHIP_ABS && op <= BSHIP_EL, op, window::rec_unary(op, x, y, n));
     switch (op) {
         case BSHIP_ABS:     return launch_ew<1>("abs_t", AbsOp{}, x, nullptr, nullptr, y, n);
         case BSHIP_SIGN:    return launch_ew<1>("sign_t", SignOp{}, x, nullptr, nullptr, y, n);
@@ -148,6 +163,7 @@ int bship_deriv_f32(int op, const float* y, const float* dy, float* dx, size_t n
     BSHIP_EW_PROLOGUE(y, dx);
     BSHIP_REQUIRE_PTR(dy);
     BSHIP_REQUIRE_F32_ALIGNED(dy);
+    BSHIP_EW_WINDOW(op >= BSHIP_SIGMOID_DERIV && op <= BSHIP_EL_DERIV, op, window::rec_deriv(op, y, dy, dx, n));
     switch (op) {
         case BSHIP_SIGMOID_DERIV: return launch_ew<2>("sigmoid_deriv", SigmoidDerivOp{}, y, dy, nullptr, dx, n);
         case BSHIP_TANH_DERIV:    return launch_ew<2>("tanh_deriv", TanhDerivOp{}, y, dy, nullptr, dx, n);
@@ -159,12 +175,14 @@ int bship_deriv_f32(int op, const float* y, const float* dy, float* dx, size_t n
 
 int bship_clip_f32(const float* a, float lo, float hi, float* out, size_t n) {
     BSHIP_EW_PROLOGUE(a, out);
+    BSHIP_EW_WINDOW(true, 0, window::rec_clip(a, lo, hi, out, n));
     return launch_ew<1>("clip_t", ClipOp{lo, hi}, a, nullptr, nullptr, out, n);
 }
 
 int bship_cond_f32(int op, const float* a, float val, float* out, const float* cond, size_t n) {
     BSHIP_EW_PROLOGUE(cond, out);
     BSHIP_REQUIRE_F32_ALIGNED(a);
+    BSHIP_FLUSH_PENDING();          // the conditional operations belong to no layer's sequence
     switch (op) {
         case BSHIP_COPY_IF:
             BSHIP_REQUIRE_PTR(a);

@@ -8,6 +8,7 @@
 
 #include "colsum.h"
 #include "common.h"
+#include "window.h"
 #include "functors.h"
 #include "lstm_cell.h"
 
@@ -563,6 +564,7 @@ int check_step_args(const char* fn, int act, int64_t batch, int64_t n, const voi
                     int count) {
     if (!ctx().inited)
         return set_error(BSHIP_ERR_NOT_INITIALIZED, "%s: bship_init() has not been called", fn);
+    BSHIP_FLUSH_PENDING();
     if (batch < 0 || n < 0 || n > 0x3fffffff)
         return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: bad dimensions batch=%lld n=%lld", fn,
                          (long long)batch, (long long)n);
@@ -613,6 +615,34 @@ int lstm_bwd_launch(const char* fn, bool packed, int act, int64_t batch, int64_t
 }
 
 }  // namespace
+
+// batch_normalization_layer.py:68-105 for a training pass; the scalars are the ones the layer's calls carry
+// (mult_st(-1/m), mult_st(decay), mult_add_st(1-decay) for the mean; mult_st(1/m), add_st(eps), mult_st(decay),
+// mult_add_st(1-decay) for the deviation).
+int batchnorm_fwd_train_launch(const float* inputs, const float* gamma, const float* beta, float* mu, float* sigma,
+                               float* sigma_b, float* centered, float* x_hat, float* out, int64_t M, int64_t N,
+                               float neg_inv_m, float decay_mu, float rest_mu, float inv_m, float eps,
+                               float decay_sigma, float rest_sigma) {
+    if (N == 0) return 0;
+    if (M < 1) return set_error(BSHIP_ERR_BAD_DIMENSION, "batchnorm_forward: no rows");
+    const dim3 vgrid(static_cast<unsigned>(ceil_div(N, kBlock))), blk(kBlock);
+    hipStream_t s = ctx().stream;
+    // negative batch mean into sigma_b (the layer uses that buffer as scratch), running mean
+    int st = M == 1 ? bship_d2d(sigma_b, inputs, static_cast<size_t>(N) * 4)
+                    : launch_colsum(PlainSrc{inputs}, sigma_b, M, N);
+    if (st != 0) return st;
+    hipLaunchKernelGGL(bn_mean_update_kernel, vgrid, blk, 0, s, sigma_b, mu, neg_inv_m, decay_mu, rest_mu, N);
+    if ((st = check_launch("batchnorm mean")) != 0) return st;
+    // centered = inputs + mu_b while summing centered^2 down the columns
+    st = launch_colsum(CenterSquareSrc{inputs, sigma_b, centered,
+                                       store_through(static_cast<size_t>(M) * static_cast<size_t>(N))}, sigma_b, M, N);
+    if (st != 0) return st;
+    hipLaunchKernelGGL(bn_sigma_update_kernel, vgrid, blk, 0, s, sigma_b, sigma, inv_m, eps, decay_sigma, rest_sigma, N);
+    if ((st = check_launch("batchnorm deviation")) != 0) return st;
+    BnNormBody b{{sigma_b, gamma, beta}, {centered}, {x_hat, out}};
+    return launch_rowvec_fused("batchnorm_forward", b, M, N);
+}
+
 }  // namespace bship
 
 using namespace bship;
@@ -738,7 +768,7 @@ int bship_softmax_ce_fwd_f32(const float* inputs, const float* targets, float* p
     int st = check_pointers(__func__, ptrs, 4);
     if (st != 0) return st;
     BSHIP_REQUIRE_DIM(M <= 0x7fffffff);
-    st = bship_softmax_rows_f32(inputs, probs, M, K);
+    st = bship_softmax_rows_pitched_f32(inputs, K, probs, K, M, K);     // not through the fusing window
     if (st != 0) return st;
     hipLaunchKernelGGL(softmax_ce_loss_kernel, dim3(static_cast<unsigned>(ceil_div(M, kBlock))), dim3(kBlock), 0,
                        ctx().stream, probs, targets, loss, M, K);
@@ -798,22 +828,8 @@ int bship_batchnorm_fwd_f32(int training, const float* inputs, const float* gamm
     const float dec = static_cast<float>(decay);
     const float omd = static_cast<float>(1.0 - decay);
     const float eps = static_cast<float>(epsilon);
-    const dim3 vgrid(static_cast<unsigned>(ceil_div(N, kBlock))), blk(kBlock);
-    hipStream_t s = ctx().stream;
-    // negative batch mean into sigma_b (the layer uses that buffer as scratch), running mean
-    st = M == 1 ? bship_d2d(sigma_b, inputs, static_cast<size_t>(N) * 4)
-                : launch_colsum(PlainSrc{inputs}, sigma_b, M, N);
-    if (st != 0) return st;
-    hipLaunchKernelGGL(bn_mean_update_kernel, vgrid, blk, 0, s, sigma_b, mu, neg_inv_m, dec, omd, N);
-    if ((st = check_launch("batchnorm mean")) != 0) return st;
-    // centered = inputs + mu_b while summing centered^2 down the columns
-    st = launch_colsum(CenterSquareSrc{inputs, sigma_b, centered,
-                                       store_through(static_cast<size_t>(M) * static_cast<size_t>(N))}, sigma_b, M, N);
-    if (st != 0) return st;
-    hipLaunchKernelGGL(bn_sigma_update_kernel, vgrid, blk, 0, s, sigma_b, sigma, inv_m, eps, dec, omd, N);
-    if ((st = check_launch("batchnorm deviation")) != 0) return st;
-    BnNormBody b{{sigma_b, gamma, beta}, {centered}, {x_hat, out}};
-    return launch_rowvec_fused("batchnorm_forward", b, M, N);
+    return batchnorm_fwd_train_launch(inputs, gamma, beta, mu, sigma, sigma_b, centered, x_hat, out, M, N,
+                                      neg_inv_m, dec, omd, inv_m, eps, dec, omd);
 }
 
 int bship_batchnorm_bwd_f32(const float* out_deltas, const float* x_hat, const float* gamma,

@@ -23,6 +23,7 @@
 #include <tuple>
 
 #include "common.h"
+#include "window.h"
 
 namespace bship {
 
@@ -236,12 +237,13 @@ static int gemm_impl(int transa, int transb, int64_t M, int64_t N, int64_t K, fl
 extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int64_t K, float alpha,
                               const float* A, int64_t lda, const float* B, int64_t ldb, float beta,
                               float* C, int64_t ldc) {
-    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
     BSHIP_REQUIRE_DIM(M >= 0 && N >= 0 && K >= 0);
     if (M == 0 || N == 0) return 0;
     BSHIP_REQUIRE_PTR(C);
     BSHIP_REQUIRE_DIM(ldc >= N);
     if (K == 0) {
+        BSHIP_FLUSH_PENDING();
         // empty inner dimension: C = beta * C
         if (beta == 1.0f) return 0;
         if (ldc != N) return set_error(BSHIP_ERR_UNSUPPORTED, "bship_gemm_f32: K == 0 needs a dense C");
@@ -252,6 +254,23 @@ extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int6
     BSHIP_REQUIRE_PTR(B);
     BSHIP_REQUIRE_DIM(lda >= (transa ? M : K));
     BSHIP_REQUIRE_DIM(ldb >= (transb ? K : N));
+    if (g_window_held.load(std::memory_order_relaxed) != 0 && !t_window_emitting) {
+        // A layer's products lie between its elementwise calls (lstm_layer.py:121-145). The product goes
+        // ahead of the operations the fusing window holds when it shares no operand with them that either
+        // side writes; otherwise they are enqueued first.
+        const int64_t a_rows = transa ? K : M, a_cols = transa ? M : K, b_rows = transb ? N : K, b_cols = transb ? K : N;
+        const void* rd[3] = {A, B, C};
+        const size_t rd_len[3] = {static_cast<size_t>((a_rows - 1) * lda + a_cols) * 4,
+                                  static_cast<size_t>((b_rows - 1) * ldb + b_cols) * 4,
+                                  static_cast<size_t>((M - 1) * ldc + N) * 4};
+        const void* wr[1] = {C};
+        int st = window_before_product(rd, rd_len, beta != 0.0f ? 3 : 2, wr, rd_len + 2, 1);
+        if (st != 0) return st;
+    }
+    if (g_deferred_fill_count.load(std::memory_order_relaxed) != 0) {
+        int st = flush_deferred_fills();
+        if (st != 0) return st;
+    }
     return gemm_impl(transa, transb, M, N, K, alpha, A, lda, B, ldb, beta, nullptr, C, ldc);
 }
 

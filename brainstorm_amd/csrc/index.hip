@@ -3,6 +3,7 @@
 // like NumPy's astype(int32); negative labels count from the last column, as
 // NumPy's indexing does (label_column in common.h).
 #include "common.h"
+#include "window.h"
 
 namespace bship {
 
@@ -58,6 +59,12 @@ using namespace bship;
 extern "C" {
 
 int bship_binarize_f32(const float* v, float* out, int64_t M, int64_t K) {
+    // the first call of the softmax cross-entropy layer's backward sequence: through the fusing window
+    if (window_takes() && M >= 1 && K >= 1 && v && out &&
+        ((reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 3u) == 0) {
+        BSHIP_REQUIRE_INIT_NO_FLUSH();
+        return window_push(window::rec_binarize(v, out, M, K));
+    }
     return bship_binarize_pitched_f32(v, 1, out, K, M, K);
 }
 
@@ -100,6 +107,10 @@ int bship_binarize_pitched_f32(const float* v, int64_t ld_v, float* out, int64_t
 }
 
 int bship_index_m_by_v_f32(const float* m, const float* v, float* out, int64_t M, int64_t K) {
+    if (window_takes() && M >= 1 && K >= 0 && m && v && out) {      // part of the softmax cross-entropy forward sequence
+        BSHIP_REQUIRE_INIT_NO_FLUSH();
+        return window_push(window::rec_index(m, v, out, M, K));
+    }
     return bship_index_m_by_v_pitched_f32(m, K, v, 1, out, 1, M, K);
 }
 

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "common.h"
+#include "window.h"
 
 namespace bship {
 
@@ -314,8 +315,12 @@ int bship_malloc(size_t nbytes, void** out) {
     BSHIP_REQUIRE_PTR(out);
     int st = pool_alloc_raw(nbytes, out);
     if (st != 0 || *out == nullptr) return st;
-    // Blocks are rounded to a multiple of 256 bytes, so clearing whole floats covers nbytes.
-    return launch_fill(static_cast<float*>(*out), 0.0f, (nbytes + 3) / 4);
+    // Blocks are rounded to a multiple of 256 bytes, so clearing whole floats covers nbytes. Small
+    // blocks (a layer's vector-sized temporaries) are cleared with the noted fills: every launch
+    // enqueues those first.
+    const size_t n = (nbytes + 3) / 4;
+    if (n <= kDeferredFillMax) return defer_fill(static_cast<float*>(*out), 0.0f, n);
+    return launch_fill(static_cast<float*>(*out), 0.0f, n);
 }
 
 int bship_malloc_scratch(size_t nbytes, void** out) {
@@ -325,7 +330,22 @@ int bship_malloc_scratch(size_t nbytes, void** out) {
 }
 
 int bship_free(void* p) {
-    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
+    // Operations that the fusing window holds may still name this block: they are enqueued before
+    // anything a later owner does (bship_malloc enqueues what is held first), and a layer's
+    // sequence that only waits for its temporaries to be dropped is completed by this very call.
+    if (p && g_window_held.load(std::memory_order_relaxed) != 0 && !t_window_emitting) {
+        size_t bytes = 0;
+        {
+            std::lock_guard<std::mutex> lock(g_pool_mutex);
+            auto it = g_live.find(p);
+            if (it != g_live.end()) bytes = it->second;
+        }
+        if (bytes) {
+            int st = window_note_free(p, bytes);
+            if (st != 0) { (void)pool_free_raw(p); return st; }
+        }
+    }
     return pool_free_raw(p);
 }
 
@@ -490,6 +510,9 @@ int bship_fill_f32(float* mem, float val, size_t n) {
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(mem);
     BSHIP_REQUIRE_F32_ALIGNED(mem);
+    // fills are part of layers' sequences (highway_layer.py:64, softmax_ce_layer.py:83): with the
+    // fusing window on they pass through it and come back here when it lets them go
+    if (window_takes()) return window_push(window::rec_fill(mem, val, n));
     if (n <= kDeferredFillMax) return defer_fill(mem, val, n);
     int st = flush_deferred_fills();
     return st != 0 ? st : launch_fill(mem, val, n);

@@ -5,6 +5,7 @@
 #pragma clang fp contract(off)
 
 #include "common.h"
+#include "window.h"
 #include "colsum.h"
 
 namespace bship {
@@ -420,7 +421,13 @@ int bship_sum_noalloc_f32(const float* a, float* out, int64_t M, int64_t N, int 
 }
 
 int bship_sum_f32(const float* a, float* out, int64_t M, int64_t N, int axis) {
-    return bship_sum_pitched_f32(a, N, out, M, N, axis);
+    // column sums are part of the batch normalisation sequences: a dense sum goes through the fusing window
+    if (window_takes() && M >= 1 && N >= 1 && M <= 0x7fffffff && (axis == 0 || axis == 1 || axis == -1) && a && out &&
+        a != out && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(out)) & 3u) == 0) {
+        BSHIP_REQUIRE_INIT_NO_FLUSH();
+        return window_push(window::rec_sum(a, out, M, N, axis));
+    }
+    return bship_sum_pitched_f32(a, N, out, M, N, axis);       // reports what is wrong with the arguments, too
 }
 
 int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, int64_t N, int axis) {
@@ -451,6 +458,12 @@ int bship_sum_pitched_f32(const float* a, int64_t ld_a, float* out, int64_t M, i
 }
 
 int bship_softmax_rows_f32(const float* m, float* out, int64_t M, int64_t N) {
+    // the first call of the softmax cross-entropy layer's forward sequence: through the fusing window
+    if (window_takes() && M >= 1 && N >= 1 && M <= 0x7fffffff && m && out &&
+        ((reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(out)) & 3u) == 0) {
+        BSHIP_REQUIRE_INIT_NO_FLUSH();
+        return window_push(window::rec_softmax(m, out, M, N));
+    }
     return bship_softmax_rows_pitched_f32(m, N, out, N, M, N);
 }
 

@@ -40,6 +40,7 @@
 #include <vector>
 
 #include "common.h"
+#include "window.h"
 #include "mt_jump.h"
 
 namespace bship {
@@ -1135,45 +1136,17 @@ void rng_release() {
 
 using namespace bship;
 
-extern "C" {
-
-int bship_rng_create(int* generator_id) {
-    BSHIP_REQUIRE_INIT();
-    BSHIP_REQUIRE_PTR(generator_id);
-    std::lock_guard<std::mutex> lock(g_rng_mutex);
-    *generator_id = g_next_generator++;
-    g_generators[*generator_id] = Generator();
-    return 0;
-}
-
-int bship_rng_select(int generator_id) {
-    BSHIP_REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_rng_mutex);
-    return select_generator_locked(generator_id);
-}
-
-int bship_rng_destroy(int generator_id) {
-    BSHIP_REQUIRE_INIT();
-    std::lock_guard<std::mutex> lock(g_rng_mutex);
-    if (generator_id == 0) return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator 0 is the library's own");
-    if (g_generators.find(generator_id) == g_generators.end())
-        return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator %d does not exist", generator_id);
-    if (generator_id == g_current_generator) {
-        int st = select_generator_locked(0);
-        if (st != 0) return st;
-    }
-    // the blocks' next owners run on the library's stream, behind every kernel that used them
-    const Generator g = g_generators[generator_id];
-    if (g.state) pool_free_raw(g.state);
-    if (g.fast) pool_free_raw(g.fast);
-    g_generators.erase(generator_id);
-    return 0;
-}
-
-int bship_rng_seed(uint32_t seed) {
+// The drawing and state operations. generator >= 0: that generator is selected first, under the same
+// lock as the operation itself, so that two handlers used from two threads cannot come between
+// another handler's selection and its draw; generator < 0: the generator selected last.
+static int rng_seed_impl(int generator, uint32_t seed) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     int st = rng_ensure_state();
     if (st == 0) st = prefetch_flush(false);
     if (st == 0) st = graph_masks_unprime();
@@ -1189,10 +1162,14 @@ int bship_rng_seed(uint32_t seed) {
     return bship_h2d(g_state, &h, sizeof(RngState));
 }
 
-int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) {
+static int rng_get_state_impl(int generator, uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_rng_get_state: bship_rng_seed() has not been called");
     RngState h;
     int st = prefetch_flush(true);
@@ -1206,11 +1183,7 @@ int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, 
     return 0;
 }
 
-int bship_prob_mask_f32(float* mask, size_t n, double p) {
-    return bship_prob_mask_pitched_f32(mask, static_cast<int64_t>(n), 1, static_cast<int64_t>(n), p);
-}
-
-int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p) {
+static int prob_mask_pitched_f32_impl(int generator, float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_DIM(rows >= 0 && cols >= 0 && ld_mask >= cols);
     const size_t n = static_cast<size_t>(rows) * static_cast<size_t>(cols);
@@ -1218,7 +1191,11 @@ int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int6
     BSHIP_REQUIRE_PTR(mask);
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
-    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "%s: bship_rng_seed() has not been called", __func__);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
+    if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "%s: bship_rng_seed() has not been called", "bship_prob_mask_pitched_f32");
     MaskPrefetch hit;
     bool is_hit = false;
     int st = mask_begin(mask, n, p, &hit, &is_hit, static_cast<size_t>(cols), static_cast<size_t>(ld_mask));
@@ -1228,7 +1205,7 @@ int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int6
     return mask_end(hit);
 }
 
-int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, double keep_probability,
+static int dropout_fwd_f32_impl(int generator, const float* in, float* mask, float* out, size_t n, double keep_probability,
                           float scale) {
     BSHIP_REQUIRE_INIT();
     if (n == 0) return 0;
@@ -1239,8 +1216,12 @@ int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, do
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     const size_t tiles = (n + static_cast<size_t>(kBlock) * 4 - 1) / (static_cast<size_t>(kBlock) * 4);
-    if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", __func__, n);
+    if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", "bship_dropout_fwd_f32", n);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_dropout_fwd_f32: bship_rng_seed() has not been called");
     MaskPrefetch hit;
     bool is_hit = false;
@@ -1260,13 +1241,17 @@ int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, do
     return st;
 }
 
-int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
+static int fill_gaussian_f32_impl(int generator, float* out, size_t n, double mean, double stdv) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_fill_gaussian_f32: bship_rng_seed() has not been called");
     hipStream_t s = ctx().stream;
     int st = prefetch_flush(true);
@@ -1327,10 +1312,14 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) {
     return st;
 }
 
-int bship_fast_rng_seed(unsigned long long seed) {
+static int fast_rng_seed_impl(int generator, unsigned long long seed) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_fast_state) {
         void* p = nullptr;
         int st = pool_alloc_raw(sizeof(FastRngState), &p);
@@ -1341,10 +1330,14 @@ int bship_fast_rng_seed(unsigned long long seed) {
     return bship_h2d(g_fast_state, &h, sizeof(h));
 }
 
-int bship_fast_rng_get_state(unsigned long long* seed_host, unsigned long long* next_block_host) {
+static int fast_rng_get_state_impl(int generator, unsigned long long* seed_host, unsigned long long* next_block_host) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_fast_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_fast_rng_get_state: bship_fast_rng_seed() has not been called");
     FastRngState h;
     int st = bship_d2h(&h, g_fast_state, sizeof(h));
@@ -1354,17 +1347,21 @@ int bship_fast_rng_get_state(unsigned long long* seed_host, unsigned long long* 
     return 0;
 }
 
-int bship_prob_mask_fast_f32(float* mask, size_t n, double p) {
+static int prob_mask_fast_f32_impl(int generator, float* mask, size_t n, double p) {
     BSHIP_REQUIRE_INIT();
     if (n == 0) return 0;
     BSHIP_REQUIRE_PTR(mask);
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_fast_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_prob_mask_fast_f32: bship_fast_rng_seed() has not been called");
     return launch_fast_mask(nullptr, mask, nullptr, n, p, 1.0f);
 }
 
-int bship_dropout_fwd_fast_f32(const float* in, float* mask, float* out, size_t n, double keep_probability,
+static int dropout_fwd_fast_f32_impl(int generator, const float* in, float* mask, float* out, size_t n, double keep_probability,
                                float scale) {
     BSHIP_REQUIRE_INIT();
     if (n == 0) return 0;
@@ -1375,8 +1372,141 @@ int bship_dropout_fwd_fast_f32(const float* in, float* mask, float* out, size_t 
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator >= 0) {
+        int sel_st = select_generator_locked(generator);
+        if (sel_st != 0) return sel_st;
+    }
     if (!g_fast_state) return set_error(BSHIP_ERR_NOT_INITIALIZED, "bship_dropout_fwd_fast_f32: bship_fast_rng_seed() has not been called");
     return launch_fast_mask(in, mask, out, n, keep_probability, scale);
+}
+
+extern "C" {
+
+int bship_rng_create(int* generator_id) {
+    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_PTR(generator_id);
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    *generator_id = g_next_generator++;
+    g_generators[*generator_id] = Generator();
+    return 0;
+}
+
+int bship_rng_select(int generator_id) {
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
+    {
+        std::lock_guard<std::mutex> lock(g_rng_mutex);
+        if (generator_id == g_current_generator) return 0;
+    }
+    BSHIP_FLUSH_PENDING();       // masks that the fusing window holds are drawn from the generator selected so far
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    return select_generator_locked(generator_id);
+}
+
+int bship_rng_destroy(int generator_id) {
+    BSHIP_REQUIRE_INIT();
+    std::lock_guard<std::mutex> lock(g_rng_mutex);
+    if (generator_id == 0) return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator 0 is the library's own");
+    if (g_generators.find(generator_id) == g_generators.end())
+        return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator %d does not exist", generator_id);
+    if (generator_id == g_current_generator) {
+        int st = select_generator_locked(0);
+        if (st != 0) return st;
+    }
+    // the blocks' next owners run on the library's stream, behind every kernel that used them
+    const Generator g = g_generators[generator_id];
+    if (g.state) pool_free_raw(g.state);
+    if (g.fast) pool_free_raw(g.fast);
+    g_generators.erase(generator_id);
+    return 0;
+}
+
+int bship_rng_seed(uint32_t seed) { return rng_seed_impl(-1, seed); }
+
+int bship_rng_seed_on(int generator, uint32_t seed) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return rng_seed_impl(generator, seed);
+}
+
+int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) { return rng_get_state_impl(-1, key_host, pos_host, has_gauss_host, gauss_host); }
+
+int bship_rng_get_state_on(int generator, uint32_t* key_host, int* pos_host, int* has_gauss_host, double* gauss_host) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return rng_get_state_impl(generator, key_host, pos_host, has_gauss_host, gauss_host);
+}
+
+// A dense mask may be the first call of a dropout layer's sequence (dropout_layer.py:41-45): it goes
+// through the fusing window. generator < 0: the generator selected when the mask is drawn
+// (bship_rng_select enqueues what the window holds before it selects another one).
+static int dense_mask(int generator, float* mask, size_t n, double p, bool fast) {
+    if (window_takes()) {
+        BSHIP_REQUIRE_INIT_NO_FLUSH();
+        if (n == 0) return 0;
+        BSHIP_REQUIRE_PTR(mask);
+        BSHIP_REQUIRE_F32_ALIGNED(mask);
+        return window_push(window::rec_mask(mask, n, p, generator, fast));
+    }
+    if (fast) return prob_mask_fast_f32_impl(generator, mask, n, p);
+    return prob_mask_pitched_f32_impl(generator, mask, static_cast<int64_t>(n), 1, static_cast<int64_t>(n), p);
+}
+
+int bship_prob_mask_f32(float* mask, size_t n, double p) { return dense_mask(-1, mask, n, p, false); }
+
+int bship_prob_mask_on_f32(int generator, float* mask, size_t n, double p) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return dense_mask(generator, mask, n, p, false);
+}
+
+int bship_prob_mask_pitched_f32(float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p) { return prob_mask_pitched_f32_impl(-1, mask, ld_mask, rows, cols, p); }
+
+int bship_prob_mask_pitched_on_f32(int generator, float* mask, int64_t ld_mask, int64_t rows, int64_t cols, double p) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return prob_mask_pitched_f32_impl(generator, mask, ld_mask, rows, cols, p);
+}
+
+int bship_dropout_fwd_f32(const float* in, float* mask, float* out, size_t n, double keep_probability,
+                          float scale) { return dropout_fwd_f32_impl(-1, in, mask, out, n, keep_probability, scale); }
+
+int bship_dropout_fwd_on_f32(int generator, const float* in, float* mask, float* out, size_t n, double keep_probability,
+                          float scale) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return dropout_fwd_f32_impl(generator, in, mask, out, n, keep_probability, scale);
+}
+
+int bship_fill_gaussian_f32(float* out, size_t n, double mean, double stdv) { return fill_gaussian_f32_impl(-1, out, n, mean, stdv); }
+
+int bship_fill_gaussian_on_f32(int generator, float* out, size_t n, double mean, double stdv) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return fill_gaussian_f32_impl(generator, out, n, mean, stdv);
+}
+
+int bship_fast_rng_seed(unsigned long long seed) { return fast_rng_seed_impl(-1, seed); }
+
+int bship_fast_rng_seed_on(int generator, unsigned long long seed) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return fast_rng_seed_impl(generator, seed);
+}
+
+int bship_fast_rng_get_state(unsigned long long* seed_host, unsigned long long* next_block_host) { return fast_rng_get_state_impl(-1, seed_host, next_block_host); }
+
+int bship_fast_rng_get_state_on(int generator, unsigned long long* seed_host, unsigned long long* next_block_host) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return fast_rng_get_state_impl(generator, seed_host, next_block_host);
+}
+
+int bship_prob_mask_fast_f32(float* mask, size_t n, double p) { return dense_mask(-1, mask, n, p, true); }
+
+int bship_prob_mask_fast_on_f32(int generator, float* mask, size_t n, double p) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return dense_mask(generator, mask, n, p, true);
+}
+
+int bship_dropout_fwd_fast_f32(const float* in, float* mask, float* out, size_t n, double keep_probability,
+                               float scale) { return dropout_fwd_fast_f32_impl(-1, in, mask, out, n, keep_probability, scale); }
+
+int bship_dropout_fwd_fast_on_f32(int generator, const float* in, float* mask, float* out, size_t n, double keep_probability,
+                               float scale) {
+    BSHIP_REQUIRE_DIM(generator >= 0);
+    return dropout_fwd_fast_f32_impl(generator, in, mask, out, n, keep_probability, scale);
 }
 
 }  // extern "C"

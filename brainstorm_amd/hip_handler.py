@@ -37,8 +37,8 @@ class HipRandomState:
 
     Every instance is a generator of its own in the library (bship_rng_create), as every
     reference handler has its own ``self.rnd`` (numpy_handler.py:21): handlers that are alive
-    together do not disturb each other's streams. ``select()`` makes this generator the one the
-    library's random calls use; the handler calls it in front of each of them.
+    together do not disturb each other's streams. Every random call names its generator, so the
+    library selects and draws under one lock (handlers may be driven from different threads).
     """
 
     def __init__(self, handler, seed=None):
@@ -52,6 +52,7 @@ class HipRandomState:
         self.seed(seed)
 
     def select(self):
+        """Makes this generator the one that the library's unnamed random calls and recordings use."""
         st = self._lib.bship_rng_select(self._id)
         if st:
             self._handler._call(st)
@@ -70,10 +71,9 @@ class HipRandomState:
         seed = int(seed)
         if not 0 <= seed < 2 ** 32:
             raise ValueError("seed must be between 0 and 2**32 - 1")
-        self.select()
-        self._handler._call(self._handler._lib.bship_rng_seed(seed))
+        self._handler._call(self._lib.bship_rng_seed_on(self._id, seed))
         if self._handler.fast_masks:               # the optional mask stream restarts with it
-            self._handler._call(self._handler._lib.bship_fast_rng_seed(seed))
+            self._handler._call(self._lib.bship_fast_rng_seed_on(self._id, seed))
         self._seed = seed
 
     def get_seed(self):
@@ -90,9 +90,8 @@ class HipRandomState:
         key = (ctypes.c_uint32 * 624)()
         pos, has_gauss, gauss = ctypes.c_int(), ctypes.c_int(), ctypes.c_double()
         h = self._handler
-        self.select()
-        h._call(h._lib.bship_rng_get_state(key, ctypes.byref(pos), ctypes.byref(has_gauss),
-                                           ctypes.byref(gauss)))
+        h._call(h._lib.bship_rng_get_state_on(self._id, key, ctypes.byref(pos), ctypes.byref(has_gauss),
+                                              ctypes.byref(gauss)))
         return ('MT19937', np.frombuffer(key, dtype=np.uint32).copy(), pos.value,
                 has_gauss.value, gauss.value)
 
@@ -187,7 +186,13 @@ class HipHandler(Handler):
 
     array_type = DeviceArray
 
-    def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False):
+    def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False, fusing=True):
+        # fusing: the library's fusing window. brainstorm's layers issue primitive operations only; with
+        # the window on, the library recognises the layers' call sequences (an LSTM time step, a batch
+        # normalisation pass, bias + activation, dropout, softmax cross entropy, Highway, the momentum
+        # update) and runs each as one fused kernel with the same float32 operations in the same order,
+        # so results are the same bits as with fusing=False. The switch is the library's: it holds for
+        # every handler of the process (the last handler created decides).
         # fast_masks: dropout masks from a counter-based generator (Philox4x32-10) instead of
         # NumPy's MT19937 stream. One parallel launch per mask instead of a sequential walk, but
         # NOT the masks NumpyHandler draws for the same seed (the reference's own GPU handler does
@@ -209,18 +214,21 @@ class HipHandler(Handler):
         self._free = self._lib.bship_free
         self.EMPTY = DeviceArray(0, (0,), None, self)
         self.fast_masks = bool(fast_masks)
+        self.fusing = bool(fusing)
+        self._call(self._lib.bship_fusing_set(int(self.fusing)))
         self.rnd = HipRandomState(self, seed)
 
     def __describe__(self):
         # the constructor's settings travel with a saved network description, as NumpyHandler's
         # dtype does (numpy_handler.py:25-33); the seed does not (the reference's does not either)
         return {'@type': self.__class__.__name__, 'device': self.device,
-                'pitched_views': self.pitched_views, 'fast_masks': self.fast_masks}
+                'pitched_views': self.pitched_views, 'fast_masks': self.fast_masks, 'fusing': self.fusing}
 
     def __init_from_description__(self, description):
         self.__init__(device=int(description.get('device', 0)),
                       pitched_views=bool(description.get('pitched_views', False)),
-                      fast_masks=bool(description.get('fast_masks', False)))
+                      fast_masks=bool(description.get('fast_masks', False)),
+                      fusing=bool(description.get('fusing', True)))
 
     # ------------------------------------------------------------- plumbing
     # parameters an operation writes (everything else is only read); operations that are not
@@ -367,8 +375,8 @@ class HipHandler(Handler):
     def _pitched_mask(self, mask, probability):
         if self.fast_masks or type(mask) is not PitchedDeviceArray:
             raise _NoNativePath()
-        self.rnd.select()
-        self._call(self._lib.bship_prob_mask_pitched_f32(mask._base, mask.pitch, mask.rows, mask.run, probability))
+        self._call(self._lib.bship_prob_mask_pitched_on_f32(self.rnd._id, mask._base, mask.pitch, mask.rows, mask.run,
+                                                            probability))
 
     @staticmethod
     def _runs(a):
@@ -520,6 +528,19 @@ class HipHandler(Handler):
     def synchronize(self):
         """Waits until every operation issued so far has finished."""
         self._call(self._lib.bship_sync())
+
+    def set_fusing(self, on):
+        """Switches the library's fusing window on or off (what it holds is enqueued first)."""
+        self.fusing = bool(on)
+        self._call(self._lib.bship_fusing_set(int(self.fusing)))
+
+    def fusing_stats(self, reset=False):
+        """Counters of the fusing window since the last reset: operations that entered it, operations
+        enqueued as they were, operations replaced by fused launches, fused launches, matrix products
+        that overtook held operations."""
+        vals = [ctypes.c_ulonglong() for _ in range(5)]
+        self._call(self._lib.bship_fusing_stats(*[ctypes.byref(v) for v in vals], int(bool(reset))))
+        return dict(zip(("calls", "unfused", "fused_calls", "fused_launches", "overtaken"), (v.value for v in vals)))
 
     # --------------------------------------------------- recorded steps
     def record(self, fn):
@@ -803,21 +824,18 @@ class HipHandler(Handler):
 
     # ------------------------------------------------------------------- RNG
     def fill_gaussian(self, mean, std, out):
-        self.rnd.select()
-        self._call(self._lib.bship_fill_gaussian_f32(out.ptr, out.size, mean, std))
+        self._call(self._lib.bship_fill_gaussian_on_f32(self.rnd._id, out.ptr, out.size, mean, std))
 
     def generate_probability_mask(self, mask, probability):
-        self.rnd.select()
         if self.fast_masks:
-            self._call(self._lib.bship_prob_mask_fast_f32(mask.ptr, mask.size, probability))
+            self._call(self._lib.bship_prob_mask_fast_on_f32(self.rnd._id, mask.ptr, mask.size, probability))
         else:
-            self._call(self._lib.bship_prob_mask_f32(mask.ptr, mask.size, probability))
+            self._call(self._lib.bship_prob_mask_on_f32(self.rnd._id, mask.ptr, mask.size, probability))
 
     def fast_mask_state(self):
         """(seed, next block) of the fast mask generator (fast_masks=True)."""
         seed, block = ctypes.c_ulonglong(), ctypes.c_ulonglong()
-        self.rnd.select()
-        self._call(self._lib.bship_fast_rng_get_state(ctypes.byref(seed), ctypes.byref(block)))
+        self._call(self._lib.bship_fast_rng_get_state_on(self.rnd._id, ctypes.byref(seed), ctypes.byref(block)))
         return seed.value, block.value
 
     # ------------------------------------------------------- dense products
@@ -1147,6 +1165,5 @@ class HipHandler(Handler):
         out = scale * out (dropout_layer.py:41-45) with one pass behind the mask."""
         if not (inputs.shape == mask.shape == out.shape):
             raise ValueError("dropout_forward: inconsistent shapes")
-        self.rnd.select()
-        fn = self._lib.bship_dropout_fwd_fast_f32 if self.fast_masks else self._lib.bship_dropout_fwd_f32
-        self._call(fn(inputs.ptr, mask.ptr, out.ptr, out.size, float(keep_probability), float(scale)))
+        fn = self._lib.bship_dropout_fwd_fast_on_f32 if self.fast_masks else self._lib.bship_dropout_fwd_on_f32
+        self._call(fn(self.rnd._id, inputs.ptr, mask.ptr, out.ptr, out.size, float(keep_probability), float(scale)))

@@ -326,6 +326,17 @@ int bship_fill_gaussian_f32(float* out, size_t n, double mean, double std);
  * the host (for tests and for saving the stream position). Blocks. */
 int bship_rng_get_state(uint32_t* key_host, int* pos_host, int* has_gauss_host,
                         double* gauss_host);
+/* The same operations on a named generator: what `handler.rnd` is to one handler object
+ * (numpy 21, 193-200; randomness.py 66-80). The generator is selected and used under one lock,
+ * so handlers that are driven from different threads cannot come between each other's selection
+ * and draw. */
+int bship_rng_seed_on(int generator, uint32_t seed);
+int bship_rng_get_state_on(int generator, uint32_t* key_host, int* pos_host, int* has_gauss_host,
+                           double* gauss_host);
+int bship_prob_mask_on_f32(int generator, float* mask, size_t n, double p);
+int bship_prob_mask_pitched_on_f32(int generator, float* mask, int64_t ld_mask, int64_t rows, int64_t cols,
+                                   double p);
+int bship_fill_gaussian_on_f32(int generator, float* out, size_t n, double mean, double std);
 
 /* -------------------------------- dense ---------------------------------- */
 
@@ -589,6 +600,15 @@ int bship_fast_rng_get_state(unsigned long long* seed_host, unsigned long long* 
 int bship_prob_mask_fast_f32(float* mask, size_t n, double p);
 int bship_dropout_fwd_fast_f32(const float* in, float* mask, float* out, size_t n,
                                double keep_probability, float scale);
+/* The dropout pass and the fast stream's calls on a named generator (see bship_rng_seed_on). */
+int bship_dropout_fwd_on_f32(int generator, const float* in, float* mask, float* out, size_t n,
+                             double keep_probability, float scale);
+int bship_fast_rng_seed_on(int generator, unsigned long long seed);
+int bship_fast_rng_get_state_on(int generator, unsigned long long* seed_host,
+                                unsigned long long* next_block_host);
+int bship_prob_mask_fast_on_f32(int generator, float* mask, size_t n, double p);
+int bship_dropout_fwd_fast_on_f32(int generator, const float* in, float* mask, float* out, size_t n,
+                                  double keep_probability, float scale);
 /* BatchNormLayerImpl.forward_pass (batch_normalization_layer.py 54-105) on
  * (M,N) matrices and N-element vectors. training != 0: batch statistics (the
  * negative batch mean and then the deviation go through sigma_b as in the
@@ -611,6 +631,35 @@ int bship_batchnorm_bwd_f32(const float* out_deltas, const float* x_hat,
                             const float* gamma, const float* sigma_b,
                             float* dgamma, float* dbeta, float* in_deltas,
                             int64_t M, int64_t N);
+
+/* ---------------------------- the fusing window --------------------------- */
+
+/* brainstorm's layers know the primitive operations only: an LSTM time step is 19 handler calls
+ * (lstm_layer.py 117-145), a batch normalisation pass 15 (batch_normalization_layer.py 68-105).
+ * With the fusing window on, the entry points of the elementwise, matrix-vector, fill, dense sum,
+ * softmax, one-hot, gather and dense mask operations do not launch at once: a call is held back
+ * while the calls so far are the beginning of one of the layers' sequences (LSTM forward and
+ * backward step, bias + activation, dropout, softmax cross entropy forward and backward, momentum
+ * update, Highway forward and backward, batch normalisation forward, inference and backward:
+ * same operations, same operand identities), a complete sequence is enqueued as the fused entry
+ * point that computes it (same float32 operations in the same order: same bits in every array the
+ * sequence writes), and everything else is enqueued as it was called, in call order. Arrays that
+ * a sequence only uses as temporaries (highway_layer.py 48 and 64, batch_normalization_layer.py
+ * 119-120) are not written by the fused kernels: such a sequence is fused only when bship_free
+ * of the temporaries follows its last call directly, as it does when the layer drops them.
+ * Matrix products are never held; they overtake held calls that share no operand with them which
+ * either side writes. Every other entry point (copies to the host, bship_sync, allocation,
+ * recording, ...) first enqueues what is held. Errors of a held call are reported by the call that
+ * causes it to be enqueued. The switch belongs to the library, not to a handler object. */
+int bship_fusing_set(int on);
+int bship_fusing_get(int* on_host);
+/* Enqueues what the window holds. */
+int bship_fusing_flush(void);
+/* Counters since the last reset: operations that entered the window, those enqueued as they were,
+ * those replaced by fused launches, fused launches, matrix products that overtook held calls. */
+int bship_fusing_stats(unsigned long long* calls, unsigned long long* unfused,
+                       unsigned long long* fused_calls, unsigned long long* fused_launches,
+                       unsigned long long* overtaken, int reset);
 
 #ifdef __cplusplus
 }

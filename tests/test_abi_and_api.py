@@ -112,17 +112,17 @@ def test_description_round_trips_the_constructor_settings():
     # the constructor is replaced by a recorder.
     from brainstorm_amd.hip_handler import HipHandler
     h = object.__new__(HipHandler)
-    h.device, h.pitched_views, h.fast_masks = 2, True, True
+    h.device, h.pitched_views, h.fast_masks, h.fusing = 2, True, True, False
     desc = h.__describe__()
-    assert desc == {"@type": "HipHandler", "device": 2, "pitched_views": True, "fast_masks": True}
+    assert desc == {"@type": "HipHandler", "device": 2, "pitched_views": True, "fast_masks": True, "fusing": False}
     seen = {}
 
     class Recorder(HipHandler):
-        def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False):
-            seen.update(seed=seed, device=device, pitched_views=pitched_views, fast_masks=fast_masks)
+        def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False, fusing=True):
+            seen.update(seed=seed, device=device, pitched_views=pitched_views, fast_masks=fast_masks, fusing=fusing)
 
     r = object.__new__(Recorder)
     r.__init_from_description__(desc)
-    assert seen == {"seed": None, "device": 2, "pitched_views": True, "fast_masks": True}
+    assert seen == {"seed": None, "device": 2, "pitched_views": True, "fast_masks": True, "fusing": False}
     r.__init_from_description__({"@type": "HipHandler"})                  # descriptions written before
-    assert seen == {"seed": None, "device": 0, "pitched_views": False, "fast_masks": False}
+    assert seen == {"seed": None, "device": 0, "pitched_views": False, "fast_masks": False, "fusing": True}

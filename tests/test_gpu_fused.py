@@ -13,6 +13,16 @@ pytestmark = pytest.mark.gpu
 F32 = np.float32
 
 
+@pytest.fixture(autouse=True)
+def single_operations_stay_single(hip):
+    # the comparison is against the primitive launches: the fusing window would turn them into the
+    # very kernels under test
+    before = hip.fusing
+    hip.set_fusing(False)
+    yield
+    hip.set_fusing(before)
+
+
 def run_lstm(hip, fused, **kw):
     hip.rnd.seed(5)
     net, data = configs.build_lstm(hip, fused=fused, **kw)

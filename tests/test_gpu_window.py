@@ -1,0 +1,187 @@
+"""GPU: the fusing window. A caller that issues the reference layers' primitive operations only
+(fused=False drivers) must get, with the window on, the same bits in every buffer as with the
+window off - on all four network workloads, over several training steps, with in-place and
+aliased calls, and when a sequence is cut short by a read-back. The window-off runs are what
+test_gpu_configs.py holds to the CPU oracle."""
+import numpy as np
+import pytest
+
+from brainstorm_amd.drivers import configs
+from brainstorm_amd.drivers.net import MomentumStepper
+from util import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F32 = np.float32
+
+
+@pytest.fixture(autouse=True)
+def restore_fusing(hip):
+    before = hip.fusing
+    yield
+    hip.set_fusing(before)
+
+
+def train(hip, builder, fusing, steps, seed=11, **kw):
+    hip.set_fusing(fusing)
+    hip.rnd.seed(seed)
+    net, data = builder(hip, **kw)
+    net.provide_external_data(data)
+    stepper = MomentumStepper(0.05, 0.9)
+    stepper.start(net)
+    hip.fusing_stats(reset=True)
+    losses = []
+    for _ in range(steps):
+        stepper.run()
+        losses.append(net.get("loss", "outputs", "loss").copy())
+    stats = hip.fusing_stats()
+    everything = hip.get_numpy_copy(net.full_buffer)
+    velocity = hip.get_numpy_copy(stepper.velocity)
+    return everything, velocity, np.concatenate([l.ravel() for l in losses]), stats
+
+
+WORKLOADS = [
+    ("mlp", configs.build_mlp, dict(batch=23, in_size=37, hidden=41), 4,
+     dict(fused_launches=4 * (3 + 2 + 1 + 1 + 1))),
+    ("mlp_full", configs.build_mlp, dict(), 3, dict(fused_launches=3 * 8)),
+    ("lstm", configs.build_lstm, dict(time_steps=9, batch=7, symbols=11, hidden=13), 3,
+     dict(fused_launches=3 * (9 + 9 + 1 + 1 + 1))),
+    ("lstm_wide", configs.build_lstm, dict(time_steps=12, batch=33, symbols=50, hidden=257), 2,
+     dict(fused_launches=2 * (12 + 12 + 1 + 1 + 1))),
+    ("highway", configs.build_highway, dict(blocks=3, batch=37, width=129), 3,
+     dict(fused_launches=3 * (3 * (2 + 2 + 2) + 1 + 1 + 1))),
+    ("cnn", configs.build_cnn, dict(batch=6, size=16), 3, dict(fused_launches=3 * (1 + 1 + 1 + 1))),
+]
+
+
+@pytest.mark.parametrize("name,builder,kw,steps,expect", WORKLOADS, ids=[w[0] for w in WORKLOADS])
+def test_unchanged_callers_get_the_same_bits(hip, name, builder, kw, steps, expect):
+    plain = train(hip, builder, False, steps, **kw)
+    fused = train(hip, builder, True, steps, **kw)
+    assert plain[3]["calls"] == 0                      # nothing went through the window when it was off
+    assert fused[3]["fused_launches"] == expect["fused_launches"], fused[3]
+    assert_bit_equal(fused[2], plain[2], name + ": losses")
+    assert_bit_equal(fused[0], plain[0], name + ": parameters, gradients and every buffer")
+    assert_bit_equal(fused[1], plain[1], name + ": velocity")
+
+
+def test_lstm_full_size_through_the_window(hip):
+    # the char-LSTM workload at its full size: T=100, batch 100, 1000 units, one forward and backward pass
+    results = []
+    for fusing in (False, True):
+        hip.set_fusing(fusing)
+        hip.rnd.seed(2)
+        net, data = configs.build_lstm(hip)
+        net.provide_external_data(data)
+        hip.fusing_stats(reset=True)
+        net.forward_pass(training_pass=True)
+        net.backward_pass()
+        stats = hip.fusing_stats()
+        results.append((hip.get_numpy_copy(net.gradients), net.get("lstm", "outputs", "default"),
+                        net.get("lstm", "internals", "dZa"), net.get("loss", "outputs", "loss"), stats))
+        del net
+    plain, fused = results
+    assert fused[4]["fused_launches"] == 100 + 100 + 1 + 1
+    assert fused[4]["overtaken"] >= 300           # the input-, forget- and output-gate products of every forward step
+    for k, what in enumerate(("gradients", "outputs", "dZa", "loss")):
+        assert_bit_equal(fused[k], plain[k], what)
+
+
+def test_a_sequence_cut_by_a_read_back(hip):
+    rng = np.random.RandomState(3)
+    batch, n = 19, 67
+    x = rng.standard_normal((batch, n)).astype(F32)
+    b = rng.standard_normal((1, n)).astype(F32)
+    p = rng.standard_normal((1, n)).astype(F32)
+    c = rng.standard_normal((batch, n)).astype(F32)
+
+    def run(fusing, cut):
+        hip.set_fusing(fusing)
+        Za, Ia, Cp = hip.create_from_numpy(x), hip.create_from_numpy(x * 0.5), hip.create_from_numpy(c)
+        bias, peep = hip.create_from_numpy(b), hip.create_from_numpy(p)
+        Zb, Ib = hip.allocate((batch, n)), hip.allocate((batch, n))
+        seen = []
+        # the first five calls of an LSTM time step (lstm_layer.py:122-128) ...
+        hip.add_mv(Za, bias, Za)
+        hip.tanh(Za, Zb)
+        if cut:
+            seen.append(hip.get_numpy_copy(Zb))       # ... read back in the middle
+        hip.mult_add_mv(Cp, peep, Ia)
+        hip.add_mv(Ia, bias, Ia)
+        hip.sigmoid(Ia, Ib)
+        # ... and then something else
+        hip.mult_tt(Ib, Zb, Za)
+        return [hip.get_numpy_copy(a) for a in (Za, Zb, Ia, Ib)] + seen
+
+    want = run(False, True)
+    for cut in (True, False):
+        got = run(True, cut)
+        for k, (g, w) in enumerate(zip(got, want)):
+            assert_bit_equal(g, w, "array %d (cut=%r)" % (k, cut))
+
+
+def test_in_place_and_aliased_calls(hip):
+    rng = np.random.RandomState(4)
+    m, n = 29, 131
+    x = rng.standard_normal((m, n)).astype(F32)
+    v = rng.standard_normal((1, n)).astype(F32)
+
+    def run(fusing):
+        hip.set_fusing(fusing)
+        out = []
+        # bias + activation in place and out of place
+        a, bias = hip.create_from_numpy(x), hip.create_from_numpy(v)
+        hip.add_mv(a, bias, a)
+        hip.sigmoid(a, a)
+        out.append(hip.get_numpy_copy(a))
+        a, t = hip.create_from_numpy(x), hip.allocate((m, n))
+        hip.add_mv(a, bias, t)
+        hip.rel(t, t)
+        out += [hip.get_numpy_copy(a), hip.get_numpy_copy(t)]
+        # the momentum update's three calls on ONE array (velocity = gradients = parameters): not the fused form
+        w = hip.create_from_numpy(x)
+        hip.mult_st(0.9, w, w)
+        hip.mult_add_st(-0.1, w, w)
+        hip.add_tt(w, w, w)
+        out.append(hip.get_numpy_copy(w))
+        # Highway's forward calls with H = x (reads may alias) and with y = the temporary (must not fuse)
+        H, T = hip.create_from_numpy(x), hip.create_from_numpy(np.abs(x) % 1)
+        y = hip.allocate((m, n))
+        tmp = hip.zeros((m, n))
+        hip.subtract_tt(H, H, tmp)
+        hip.mult_tt(T, tmp, tmp)
+        hip.add_tt(tmp, H, y)
+        del tmp
+        out.append(hip.get_numpy_copy(y))
+        tmp = hip.zeros((m, n))
+        hip.subtract_tt(H, T, tmp)
+        hip.mult_tt(T, tmp, tmp)
+        hip.add_tt(tmp, T, tmp)
+        out.append(hip.get_numpy_copy(tmp))
+        # softmax cross entropy backward with the deltas aliasing the one-hot buffer
+        probs = hip.create_from_numpy(np.abs(x))
+        labels = hip.create_from_numpy(rng.randint(0, n, (m, 1)).astype(F32))
+        dloss = hip.create_from_numpy(rng.standard_normal((m, 1)).astype(F32))
+        tb = hip.allocate((m, n))
+        hip.binarize_v(labels, tb)
+        hip.mult_st(-1, tb, tb)
+        hip.add_tt(tb, probs, tb)
+        hip.mult_mv(tb, dloss, tb)
+        hip.add_tt(tb, tb, tb)
+        out.append(hip.get_numpy_copy(tb))
+        return out
+
+    rng_state = rng.get_state()
+    want = run(False)
+    rng.set_state(rng_state)
+    got = run(True)
+    for k, (g, w) in enumerate(zip(got, want)):
+        assert_bit_equal(g, w, "result %d" % k)
+
+
+def test_errors_of_held_calls_surface(hip):
+    hip.set_fusing(True)
+    a, v = hip.allocate((4, 6)), hip.allocate((1, 6))
+    hip.add_mv(a, v, a)                          # held
+    assert hip.fusing_stats()["calls"] >= 1
+    hip.synchronize()                            # enqueues it; nothing to report
+    assert np.array_equal(hip.get_numpy_copy(a), np.zeros((4, 6), F32))
