@@ -489,15 +489,16 @@ int bship_isfinite_f32(const float* a, size_t n, int* result_host) {
     BSHIP_REQUIRE_PTR(a);
     BSHIP_REQUIRE_F32_ALIGNED(a);
     void* p = nullptr;
-    int st = bship_malloc(sizeof(int), &p);     // zero-filled
-    if (st != 0) return st;
+    int st = pool_alloc_raw(sizeof(int), &p);
+    if (st == 0) st = launch_fill(static_cast<float*>(p), 0.0f, 1);     // the flag starts at zero
+    if (st != 0) { pool_free_raw(p); return st; }
     hipLaunchKernelGGL(nonfinite_kernel,
                        dim3(stream_grid(ceil_div(static_cast<int64_t>(n), kBlock * 4))),
                        dim3(kBlock), 0, ctx().stream, a, n, static_cast<int*>(p));
     st = check_launch("is_fully_finite");
     int flag = 0;
     if (st == 0) st = bship_d2h(&flag, p, sizeof(int));
-    bship_free(p);
+    pool_free_raw(p);
     if (st == 0) *result_host = flag ? 0 : 1;
     return st;
 }

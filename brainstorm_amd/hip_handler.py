@@ -122,6 +122,14 @@ class RecordedStep(object):
             pass
 
 
+def _mismatch(op, *arrays):
+    """NumPy raises ValueError when the operands of `out[:] = a + b` cannot be combined
+    (numpy_handler.py:86-87); the kernels take one element count and raw addresses, so operands
+    of different sizes are refused here, before anything reaches the device."""
+    return ValueError("%s: operands with shapes %s do not match"
+                      % (op, ", ".join(repr(tuple(a.shape)) for a in arrays)))
+
+
 class _NoNativePath(Exception):
     """The operands of a call on row-pitched views do not fit the row-pitched kernels."""
 
@@ -434,6 +442,7 @@ class HipHandler(Handler):
 
     def _pitched_maxpool_fwd(self, inputs, window, outputs, padding, stride, argmax, **_):
         n, h, w, c = inputs.shape
+        self._window_geometry("maxpool2d_forward_batch", inputs, window, outputs, padding, stride, c)
         (pi, li), (po, lo), (pa, la) = self._images(inputs), self._images(outputs), self._images(argmax)
         self._call(self._lib.bship_maxpool_fwd_nhwc_pitched_f32(
             pi, li, po, lo, pa, la, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
@@ -441,6 +450,7 @@ class HipHandler(Handler):
 
     def _pitched_maxpool_bwd(self, inputs, window, outputs, padding, stride, argmax, in_deltas, out_deltas, **_):
         n, h, w, c = inputs.shape
+        self._window_geometry("maxpool2d_backward_batch", inputs, window, outputs, padding, stride, c)
         (pa, la), (pd, ld), (pi, li) = self._images(argmax), self._images(out_deltas), self._images(in_deltas)
         self._call(self._lib.bship_maxpool_bwd_nhwc_pitched_f32(
             pa, la, pd, ld, pi, li, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
@@ -448,6 +458,7 @@ class HipHandler(Handler):
 
     def _pitched_avgpool_fwd(self, inputs, window, outputs, padding, stride, **_):
         n, h, w, c = inputs.shape
+        self._window_geometry("avgpool2d_forward_batch", inputs, window, outputs, padding, stride, c)
         (pi, li), (po, lo) = self._images(inputs), self._images(outputs)
         self._call(self._lib.bship_avgpool_fwd_nhwc_pitched_f32(
             pi, li, po, lo, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
@@ -455,6 +466,7 @@ class HipHandler(Handler):
 
     def _pitched_avgpool_bwd(self, inputs, window, outputs, padding, stride, in_deltas, out_deltas, **_):
         n, h, w, c = inputs.shape
+        self._window_geometry("avgpool2d_backward_batch", inputs, window, outputs, padding, stride, c)
         (pd, ld), (pi, li) = self._images(out_deltas), self._images(in_deltas)
         self._call(self._lib.bship_avgpool_bwd_nhwc_pitched_f32(
             pd, ld, pi, li, n, h, w, c, outputs.shape[1], outputs.shape[2], window[0], window[1],
@@ -613,29 +625,40 @@ class HipHandler(Handler):
 
     # --------------------------------------------------------- copy and fill
     def copy_to(self, src, dest):
-        # numpy 47-52 / pycuda 83-85
-        # np.copyto broadcasts src to dest's shape: a scalar, a row for every row, a column for every
-        # column ... Served when the axes that repeat are neighbours (one broadcast_t), which covers those.
-        if src.shape == dest.shape or (src.size == dest.size and src.ndim <= 1):
+        # numpy 47-52 / pycuda 83-85: np.copyto broadcasts src to dest's shape (a scalar, a row for every
+        # row, a column for every column, ...). Every run of neighbouring axes that repeat is one broadcast_t.
+        if src.shape == dest.shape:
             self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
             return
         if src.ndim > dest.ndim:
             raise ValueError("copy_to: could not broadcast %r into %r" % (src.shape, dest.shape))
-        padded = (1,) * (dest.ndim - src.ndim) + tuple(src.shape)
-        repeat = [k for k, (s, d) in enumerate(zip(padded, dest.shape)) if s != d]
-        if any(padded[k] != 1 for k in repeat):
+        shape = (1,) * (dest.ndim - src.ndim) + tuple(src.shape)
+        repeat = [k for k, (s, d) in enumerate(zip(shape, dest.shape)) if s != d]
+        if any(shape[k] != 1 for k in repeat):
             raise ValueError("copy_to: could not broadcast %r into %r" % (src.shape, dest.shape))
         if dest.size == 0:
             return
-        if repeat[-1] - repeat[0] + 1 != len(repeat):
-            raise NotImplementedError("copy_to: broadcasting %r into %r repeats axes that are not neighbours"
-                                      % (src.shape, dest.shape))
-        outer = _prod(dest.shape[:repeat[0]])
-        inner = _prod(dest.shape[repeat[-1] + 1:])
-        times = _prod(dest.shape[repeat[0]:repeat[-1] + 1])
-        self._call(self._lib.bship_broadcast_f32(src.ptr, dest.ptr, outer, times, inner))
+        if not repeat:                       # only leading axes of length 1 differ
+            self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
+            return
+        runs = [[repeat[0], repeat[0]]]
+        for k in repeat[1:]:
+            if k == runs[-1][1] + 1:
+                runs[-1][1] = k
+            else:
+                runs.append([k, k])
+        current, shape = src, list(shape)
+        for first, last in reversed(runs):   # innermost run first: the intermediate arrays stay small
+            outer, inner = _prod(shape[:first]), _prod(shape[last + 1:])
+            times = _prod(dest.shape[first:last + 1])
+            shape[first:last + 1] = dest.shape[first:last + 1]
+            out = dest if [first, last] == runs[0] else self._scratch(tuple(shape))
+            self._call(self._lib.bship_broadcast_f32(current.ptr, out.ptr, outer, times, inner))
+            current = out
 
     def copy_to_if(self, src, dest, cond):
+        if src.size != dest.size or cond.size != dest.size:
+            raise _mismatch("copy_to_if", src, dest, cond)
         self._call(self._lib.bship_cond_f32(COPY_IF, src.ptr, 0.0, dest.ptr, cond.ptr, dest.size))
 
     def create_from_numpy(self, arr):
@@ -649,6 +672,8 @@ class HipHandler(Handler):
         self._call(self._lib.bship_fill_f32(mem.ptr, val, mem.size))
 
     def fill_if(self, mem, val, cond):
+        if cond.size != mem.size:
+            raise _mismatch("fill_if", mem, cond)
         self._call(self._lib.bship_cond_f32(FILL_IF, None, val, mem.ptr, cond.ptr, mem.size))
 
     def get_numpy_copy(self, mem):
@@ -675,54 +700,86 @@ class HipHandler(Handler):
 
     # ------------------------------------------------ elementwise operations
     def abs_t(self, a, out):
+        if a.size != out.size:
+            raise _mismatch("abs_t", a, out)
         self._call(self._lib.bship_unary_f32(ABS, a.ptr, out.ptr, out.size))
 
     def add_into_if(self, a, out, cond):
+        if a.size != out.size or cond.size != out.size:
+            raise _mismatch("add_into_if", a, out, cond)
         self._call(self._lib.bship_cond_f32(ADD_IF, a.ptr, 0.0, out.ptr, cond.ptr, out.size))
 
     def add_st(self, s, t, out):
+        if t.size != out.size:
+            raise _mismatch("add_st", t, out)
         self._call(self._lib.bship_scalar_f32(ADD_ST, s, t.ptr, out.ptr, out.size))
 
     def add_tt(self, a, b, out):
+        if a.size != out.size or b.size != out.size:
+            raise _mismatch("add_tt", a, b, out)
         self._call(self._lib.bship_binary_f32(ADD, a.ptr, b.ptr, out.ptr, out.size))
 
     def clip_t(self, a, a_min, a_max, out):
+        if a.size != out.size:
+            raise _mismatch("clip_t", a, out)
         self._call(self._lib.bship_clip_f32(a.ptr, a_min, a_max, out.ptr, out.size))
 
     def divide_tt(self, a, b, out):
+        if a.size != out.size or b.size != out.size:
+            raise _mismatch("divide_tt", a, b, out)
         self._call(self._lib.bship_binary_f32(DIV, a.ptr, b.ptr, out.ptr, out.size))
 
     def log_t(self, a, out):
+        if a.size != out.size:
+            raise _mismatch("log_t", a, out)
         self._call(self._lib.bship_unary_f32(LOG, a.ptr, out.ptr, out.size))
 
     def modulo_tt(self, a, b, out):
+        if a.size != out.size or b.size != out.size:
+            raise _mismatch("modulo_tt", a, b, out)
         self._call(self._lib.bship_binary_f32(FMOD, a.ptr, b.ptr, out.ptr, out.size))
 
     def mult_add_st(self, s, t, out):
+        if t.size != out.size:
+            raise _mismatch("mult_add_st", t, out)
         self._call(self._lib.bship_scalar_f32(MULT_ADD_ST, s, t.ptr, out.ptr, out.size))
 
     def mult_add_tt(self, a, b, out):
+        if a.size != out.size or b.size != out.size:
+            raise _mismatch("mult_add_tt", a, b, out)
         self._call(self._lib.bship_mult_add_tt_f32(a.ptr, b.ptr, out.ptr, out.size))
 
     def mult_st(self, s, t, out):
+        if t.size != out.size:
+            raise _mismatch("mult_st", t, out)
         self._call(self._lib.bship_scalar_f32(MULT_ST, s, t.ptr, out.ptr, out.size))
 
     def mult_tt(self, a, b, out):
+        if a.size != out.size or b.size != out.size:
+            raise _mismatch("mult_tt", a, b, out)
         self._call(self._lib.bship_binary_f32(MUL, a.ptr, b.ptr, out.ptr, out.size))
 
     def sign_t(self, a, out):
+        if a.size != out.size:
+            raise _mismatch("sign_t", a, out)
         self._call(self._lib.bship_unary_f32(SIGN, a.ptr, out.ptr, out.size))
 
     def sqrt_t(self, a, out):
+        if a.size != out.size:
+            raise _mismatch("sqrt_t", a, out)
         self._call(self._lib.bship_unary_f32(SQRT, a.ptr, out.ptr, out.size))
 
     def subtract_tt(self, a, b, out):
         assert a.shape == b.shape == out.shape     # numpy 265
+        if a.size != out.size or b.size != out.size:     # also when assertions are switched off
+            raise _mismatch("subtract_tt", a, b, out)
         self._call(self._lib.bship_binary_f32(SUB, a.ptr, b.ptr, out.ptr, out.size))
 
     # -------------------------------------------------- broadcast operations
     def _mv(self, op, m, v, out, accumulate):
         """out (+)= m (op) v with v a row vector (1,N)/(N,) or a column vector (M,1)."""
+        if out.size != m.size:
+            raise _mismatch("matrix-vector operation", m, v, out)
         if v.shape == m.shape:
             if accumulate:
                 assert op == MUL
@@ -760,6 +817,8 @@ class HipHandler(Handler):
     def broadcast_t(self, a, axis, out):
         # numpy 103-105
         assert (out.shape[:axis] + (1,) + out.shape[axis + 1:]) == a.shape
+        if a.size * out.shape[axis] != out.size:
+            raise _mismatch("broadcast_t", a, out)
         outer = _prod(out.shape[:axis])
         inner = _prod(out.shape[axis + 1:])
         self._call(self._lib.bship_broadcast_f32(a.ptr, out.ptr, outer, out.shape[axis], inner))
@@ -769,6 +828,8 @@ class HipHandler(Handler):
         na, nb = a.shape[-1], b.shape[-1]
         assert na + nb == out.shape[-1]
         rows = out.size // out.shape[-1] if out.shape[-1] else 0
+        if na + nb != out.shape[-1] or a.size != rows * na or b.size != rows * nb:
+            raise _mismatch("merge_tt", a, b, out)
         self._call(self._lib.bship_merge_f32(a.ptr, b.ptr, out.ptr, rows, na, nb))
 
     def split_add_tt(self, x, out_a, out_b):
@@ -776,12 +837,16 @@ class HipHandler(Handler):
         na, nb = out_a.shape[-1], out_b.shape[-1]
         assert na + nb == x.shape[-1]
         rows = x.size // x.shape[-1] if x.shape[-1] else 0
+        if na + nb != x.shape[-1] or out_a.size != rows * na or out_b.size != rows * nb:
+            raise _mismatch("split_add_tt", x, out_a, out_b)
         self._call(self._lib.bship_split_add_f32(x.ptr, out_a.ptr, out_b.ptr, rows, na, nb))
 
     # ------------------------------------------------------------ reductions
     def sum_t(self, a, axis, out):
         # numpy 268-273; the shape of `out` decides keepdims, which does not change the layout
         if axis is None or a.ndim <= 1:
+            if out.size != 1:
+                raise _mismatch("sum_t", a, out)
             self._call(self._lib.bship_sum_f32(a.ptr, out.ptr, 1, a.size, -1))
             return
         if not isinstance(axis, (int, np.integer)):
@@ -792,6 +857,8 @@ class HipHandler(Handler):
         # any array is (outer, length of the axis, inner)
         outer, length, inner = _prod(a.shape[:axis]), a.shape[axis], _prod(a.shape[axis + 1:])
         lib = self._lib
+        if out.size != outer * inner:
+            raise _mismatch("sum_t over axis %d" % axis, a, out)
         if outer * inner == 0:
             return
         if inner == 1:
@@ -811,15 +878,21 @@ class HipHandler(Handler):
                                                              a.ptr + k * inner * 4, pitch, 1, out.ptr, inner, outer, inner))
 
     def softmax_m(self, m, out):
+        if out.size != m.size or (out.shape and out.shape[-1] != m.shape[-1]):
+            raise _mismatch("softmax_m", m, out)
         n_cols = m.shape[-1]
         self._call(self._lib.bship_softmax_rows_f32(m.ptr, out.ptr, m.size // n_cols if n_cols else 0,
                                                     n_cols))
 
     # -------------------------------------------------------------- indexing
     def binarize_v(self, v, out):
+        if out.ndim != 2 or v.size != out.shape[0]:
+            raise _mismatch("binarize_v", v, out)
         self._call(self._lib.bship_binarize_f32(v.ptr, out.ptr, out.shape[0], out.shape[1]))
 
     def index_m_by_v(self, m, v, out):
+        if m.ndim != 2 or v.size != m.shape[0] or out.size != m.shape[0]:
+            raise _mismatch("index_m_by_v", m, v, out)
         self._call(self._lib.bship_index_m_by_v_f32(m.ptr, v.ptr, out.ptr, m.shape[0], m.shape[1]))
 
     # ------------------------------------------------------------------- RNG
@@ -889,7 +962,9 @@ class HipHandler(Handler):
         # inputs may be image-pitched (images a hub's full feature count apart); outputs is dense.
         n, h, w, c = inputs.shape
         f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
-        oh, ow = outputs.shape[1], outputs.shape[2]
+        oh, ow = self._window_geometry("conv2d_forward_batch", inputs, (kh, kw), outputs, padding, stride, f)
+        if weights.size != f * kh * kw * c or bias.size != f:
+            raise _mismatch("conv2d_forward_batch", inputs, weights, bias)
         kc = kh * kw * c
         rows = n * oh * ow
         col = self._scratch((rows, kc))       # im2col writes every element
@@ -909,7 +984,10 @@ class HipHandler(Handler):
         # inputs and in_deltas may be image-pitched; everything else is dense.
         n, h, w, c = inputs.shape
         f, kh, kw = weights.shape[0], weights.shape[1], weights.shape[2]
-        oh, ow = out_deltas.shape[1], out_deltas.shape[2]
+        oh, ow = self._window_geometry("conv2d_backward_batch", inputs, (kh, kw), out_deltas, padding, stride, f)
+        if (weights.size != f * kh * kw * c or weight_deltas.size != weights.size or bias_deltas.size != f
+                or in_deltas.size != inputs.size):
+            raise _mismatch("conv2d_backward_batch", inputs, weights, in_deltas, weight_deltas, bias_deltas)
         kc = kh * kw * c
         rows = n * oh * ow
         col = self._scratch((rows, kc))       # im2col writes every element
@@ -924,9 +1002,27 @@ class HipHandler(Handler):
         self._call(self._lib.bship_col2im_nhwc_pitched_f32(col.ptr, p_din, ld_din, n, h, w, c, kh, kw,
                                                            padding, stride[0], stride[1]))
 
+    @staticmethod
+    def _window_geometry(op, inputs, window, outputs, padding, stride, channels_out):
+        """(out_h, out_w) that a window over `inputs` gives, checked against `outputs`: the kernels size
+        their loops from the inputs' geometry, the caller sized `outputs`."""
+        if len(inputs.shape) != 4 or len(outputs.shape) != 4:
+            raise _mismatch(op, inputs, outputs)
+        n, h, w, _ = inputs.shape
+        oh = (h + 2 * padding - window[0]) // stride[0] + 1
+        ow = (w + 2 * padding - window[1]) // stride[1] + 1
+        if tuple(outputs.shape) != (n, oh, ow, channels_out):
+            raise ValueError("%s: inputs %r under a %r window (padding %r, stride %r) give outputs (%d, %d, %d, %d), "
+                             "not %r" % (op, tuple(inputs.shape), tuple(window), padding, tuple(stride), n, oh, ow,
+                                         channels_out, tuple(outputs.shape)))
+        return oh, ow
+
     # --------------------------------------------------------------- pooling
     def maxpool2d_forward_batch(self, inputs, window, outputs, padding, stride, argmax):
         n, h, w, c = inputs.shape
+        self._window_geometry("maxpool2d_forward_batch", inputs, window, outputs, padding, stride, c)
+        if argmax.size != outputs.size:
+            raise _mismatch("maxpool2d_forward_batch", outputs, argmax)
         self._call(self._lib.bship_maxpool_fwd_nhwc_f32(
             inputs.ptr, outputs.ptr, argmax.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
             window[0], window[1], padding, stride[0], stride[1]))
@@ -934,12 +1030,16 @@ class HipHandler(Handler):
     def maxpool2d_backward_batch(self, inputs, window, outputs, padding, stride, argmax,
                                  in_deltas, out_deltas):
         n, h, w, c = inputs.shape
+        self._window_geometry("maxpool2d_backward_batch", inputs, window, outputs, padding, stride, c)
+        if argmax.size != outputs.size or out_deltas.size != outputs.size or in_deltas.size != inputs.size:
+            raise _mismatch("maxpool2d_backward_batch", inputs, outputs, argmax, in_deltas, out_deltas)
         self._call(self._lib.bship_maxpool_bwd_nhwc_f32(
             argmax.ptr, out_deltas.ptr, in_deltas.ptr, n, h, w, c, outputs.shape[1],
             outputs.shape[2], window[0], window[1], padding, stride[0], stride[1]))
 
     def avgpool2d_forward_batch(self, inputs, window, outputs, padding, stride):
         n, h, w, c = inputs.shape
+        self._window_geometry("avgpool2d_forward_batch", inputs, window, outputs, padding, stride, c)
         self._call(self._lib.bship_avgpool_fwd_nhwc_f32(
             inputs.ptr, outputs.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
             window[0], window[1], padding, stride[0], stride[1]))
@@ -947,33 +1047,52 @@ class HipHandler(Handler):
     def avgpool2d_backward_batch(self, inputs, window, outputs, padding, stride, in_deltas,
                                  out_deltas):
         n, h, w, c = inputs.shape
+        self._window_geometry("avgpool2d_backward_batch", inputs, window, outputs, padding, stride, c)
+        if out_deltas.size != outputs.size or in_deltas.size != inputs.size:
+            raise _mismatch("avgpool2d_backward_batch", inputs, outputs, in_deltas, out_deltas)
         self._call(self._lib.bship_avgpool_bwd_nhwc_f32(
             out_deltas.ptr, in_deltas.ptr, n, h, w, c, outputs.shape[1], outputs.shape[2],
             window[0], window[1], padding, stride[0], stride[1]))
 
     # -------------------------------------------------- activation functions
     def rel(self, x, y):
+        if x.size != y.size:
+            raise _mismatch("rel", x, y)
         self._call(self._lib.bship_unary_f32(REL, x.ptr, y.ptr, y.size))
 
     def rel_deriv(self, x, y, dy, dx):
+        if y.size != dx.size or dy.size != dx.size:
+            raise _mismatch("rel_deriv", y, dy, dx)
         self._call(self._lib.bship_deriv_f32(REL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
 
     def sigmoid(self, x, y):
+        if x.size != y.size:
+            raise _mismatch("sigmoid", x, y)
         self._call(self._lib.bship_unary_f32(SIGMOID, x.ptr, y.ptr, y.size))
 
     def sigmoid_deriv(self, x, y, dy, dx):
+        if y.size != dx.size or dy.size != dx.size:
+            raise _mismatch("sigmoid_deriv", y, dy, dx)
         self._call(self._lib.bship_deriv_f32(SIGMOID_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
 
     def tanh(self, x, y):
+        if x.size != y.size:
+            raise _mismatch("tanh", x, y)
         self._call(self._lib.bship_unary_f32(TANH, x.ptr, y.ptr, y.size))
 
     def tanh_deriv(self, x, y, dy, dx):
+        if y.size != dx.size or dy.size != dx.size:
+            raise _mismatch("tanh_deriv", y, dy, dx)
         self._call(self._lib.bship_deriv_f32(TANH_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
 
     def el(self, x, y):
+        if x.size != y.size:
+            raise _mismatch("el", x, y)
         self._call(self._lib.bship_unary_f32(EL, x.ptr, y.ptr, y.size))
 
     def el_deriv(self, x, y, dy, dx):
+        if y.size != dx.size or dy.size != dx.size:
+            raise _mismatch("el_deriv", y, dy, dx)
         self._call(self._lib.bship_deriv_f32(EL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
 
     # ------------------------------------------------ fused layer-level steps

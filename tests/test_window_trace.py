@@ -8,38 +8,8 @@ reference layers' sequences) gets, with the window on, exactly the launches that
 caller asks for (fused=... drivers) with the window off - same entry points, same operands, same
 order - and nothing but reordered matrix products otherwise.
 """
-import ctypes
-import os
-import subprocess
-
 import numpy as np
 import pytest
-
-HERE = os.path.dirname(os.path.abspath(__file__))
-
-
-@pytest.fixture(scope="module")
-def trace(tmp_path_factory):
-    from brainstorm_amd import _lib
-    out = str(tmp_path_factory.mktemp("trace") / "libtrace.so")
-    src = os.path.join(HERE, "window_trace", "trace_lib.cpp")
-    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-shared", "-fPIC", "-o", out, src], check=True)
-    lib = ctypes.CDLL(out)
-    for name, argtypes in _lib.SIGNATURES.items():
-        try:
-            fn = getattr(lib, name)
-        except AttributeError:
-            continue                       # the trace library has only what these tests call
-        fn.argtypes = argtypes
-        fn.restype = ctypes.c_int
-    lib.bship_last_error.restype = ctypes.c_char_p
-    lib.trace_log.restype = ctypes.c_char_p
-    saved = _lib._LIB
-    _lib._LIB = lib
-    try:
-        yield lib
-    finally:
-        _lib._LIB = saved
 
 
 def canonical(log, base, size):

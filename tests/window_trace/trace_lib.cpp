@@ -371,6 +371,32 @@ int bship_maxpool_bwd_nhwc_f32(const float* argmax, const float* dout, float* di
     return 0;
 }
 
+int bship_broadcast_f32(const float* a, float* out, int64_t outer, int64_t bdim, int64_t inner) {
+    flush();
+    logf("broadcast @%lld @%lld %lld %lld %lld", P(a), P(out), (long long)outer, (long long)bdim, (long long)inner);
+    return 0;
+}
+int bship_merge_f32(const float* a, const float* b, float* out, int64_t rows, int64_t na, int64_t nb) {
+    flush();
+    logf("merge @%lld @%lld @%lld %lld %lld %lld", P(a), P(b), P(out), (long long)rows, (long long)na, (long long)nb);
+    return 0;
+}
+int bship_split_add_f32(const float* x, float* oa, float* ob, int64_t rows, int64_t na, int64_t nb) {
+    flush();
+    logf("split_add @%lld @%lld @%lld %lld %lld %lld", P(x), P(oa), P(ob), (long long)rows, (long long)na, (long long)nb);
+    return 0;
+}
+int bship_avgpool_fwd_nhwc_f32(const float* in, float* out, int64_t n, int, int, int, int, int, int, int, int, int, int) {
+    flush();
+    logf("avgpool_fwd @%lld @%lld %lld", P(in), P(out), (long long)n);
+    return 0;
+}
+int bship_avgpool_bwd_nhwc_f32(const float* dout, float* din, int64_t n, int, int, int, int, int, int, int, int, int, int) {
+    flush();
+    logf("avgpool_bwd @%lld @%lld %lld", P(dout), P(din), (long long)n);
+    return 0;
+}
+
 // ---- generators, the switch
 int bship_rng_create(int* id) { static int next = 1; *id = next++; return 0; }
 int bship_rng_select(int) { return flush(); }
