@@ -177,6 +177,24 @@ def load():
     return lib
 
 
+# entry points that the handler calls through brainstorm_amd._fastcall (csrc/fastcall.c)
+FAST_ENTRY_POINTS = ("bship_binary_f32", "bship_mult_add_tt_f32", "bship_scalar_f32", "bship_unary_f32",
+                     "bship_deriv_f32", "bship_clip_f32", "bship_mv_f32", "bship_fill_f32", "bship_gemm_f32",
+                     "bship_d2d", "bship_sum_f32")
+
+
+def entry_point_addresses(lib):
+    """name -> address of the entry points of FAST_ENTRY_POINTS that `lib` exports."""
+    out = {}
+    for name in FAST_ENTRY_POINTS:
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            continue
+        out[name] = ctypes.cast(fn, c_void_p).value
+    return out
+
+
 def raise_for_status(lib, status):
     msg = lib.bship_last_error()
     msg = msg.decode("utf-8", "replace") if msg else ""

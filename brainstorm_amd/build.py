@@ -85,6 +85,31 @@ def build_lib(verbose: bool = False, jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+def fastcall_path() -> str:
+    import sysconfig
+    return os.path.join(HERE, "_fastcall" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_fastcall(verbose: bool = False) -> str:
+    """Compiles csrc/fastcall.c, the CPython extension through which the handler calls the hottest
+    entry points of the C ABI without ctypes' per-argument conversions (plain C, gcc)."""
+    import sysconfig
+    out = fastcall_path()
+    cc = os.environ.get("CC") or shutil.which("gcc") or shutil.which("cc")
+    if not cc:
+        raise RuntimeError("no C compiler found for brainstorm_amd/csrc/fastcall.c")
+    cmd = [cc, "-O2", "-Wall", "-shared", "-fPIC", "-I" + sysconfig.get_paths()["include"],
+           os.path.join(CSRC, "fastcall.c"), "-o", out + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("building the _fastcall extension failed:\n" + res.stdout + res.stderr)
+    os.replace(out + ".tmp", out)
+    return out
+
+
 if __name__ == "__main__":
     path = build_lib(verbose="-v" in sys.argv)
     print("built", path)
+    print("built", build_fastcall(verbose="-v" in sys.argv))

@@ -115,8 +115,11 @@ def _label_count(a):
 
 
 def _labels_in_range(handler, a):
+    """Labels select a column like NumPy's indexing does (numpy_handler.py:101, 203): values in [-K, K),
+    negative ones counted from the last column; NaN and infinities select nothing."""
     labels = handler.get_numpy_copy(a["v"])
-    return labels.size == 0 or (labels.min() >= 0 and int(labels.max()) < _label_count(a))
+    k = _label_count(a)
+    return labels.size == 0 or bool(np.isfinite(labels).all() and -k <= int(labels.min()) and int(labels.max()) < k)
 
 
 _POOL = [shape_tuple("window", 2), shape_tuple("stride", 2), padding_ok]
@@ -217,7 +220,7 @@ def _make_method(name):
         for check in checks:
             if check == "labels":
                 if not _labels_in_range(self.handler, a):
-                    _fail(name, "labels outside [0, %d)" % _label_count(a))
+                    _fail(name, "labels outside [-%d, %d)" % (_label_count(a), _label_count(a)))
             else:
                 check(name, a)
         result = inner(*a.values())           # positionally: handlers differ in some parameter names

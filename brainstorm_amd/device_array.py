@@ -48,7 +48,7 @@ def _prod(shape):
 
 
 class DeviceArray:
-    __slots__ = ("ptr", "shape", "size", "_owner", "_handler")
+    __slots__ = ("ptr", "shape", "size", "_owner", "_handler", "_steps")
 
     dtype = np.dtype(np.float32)
 
@@ -58,6 +58,7 @@ class DeviceArray:
         self.size = _prod(shape)
         self._owner = owner         # keeps the pool block alive
         self._handler = handler     # for get()
+        self._steps = None          # a[i] views handed out so far (see __getitem__)
 
     @classmethod
     def _view_of(cls, parent, ptr, shape, size):
@@ -69,6 +70,7 @@ class DeviceArray:
         v.size = size
         v._owner = parent._owner
         v._handler = parent._handler
+        v._steps = None
         return v
 
     # ---------------------------------------------------------------- basics
@@ -154,6 +156,7 @@ class DeviceArray:
                 raise ValueError("cannot reshape array of size %d into shape %r" % (self.size, new_shape))
             out = DeviceArray.__new__(DeviceArray)
             out.ptr, out.shape, out.size, out._owner, out._handler = self.ptr, new_shape, n, self._owner, self._handler
+            out._steps = None
             return out
         if len(new_shape) == 1 and not isinstance(new_shape[0], (int, np.integer)):
             new_shape = tuple(new_shape[0])
@@ -176,15 +179,26 @@ class DeviceArray:
         shape = self.shape
         # fast paths: a[i] and a[i:j] on the first axis (the recurrent layers' inner loop)
         if type(key) is int:
+            # a[t]: the recurrent layers take the same time-step views of the same buffers in every call of
+            # every step (lstm_layer.py:117-145 indexes Za[t] three times in a row); a view is an immutable
+            # (address, shape) pair, so the ones handed out are kept and handed out again
+            steps = self._steps
+            if steps is not None:
+                v = steps.get(key)
+                if v is not None:
+                    return v
             if not shape:
                 raise IndexError("too many indices for a 0-d array")
             n = shape[0]
-            if key < 0:
-                key += n
-            if not 0 <= key < n:
+            index = key + n if key < 0 else key
+            if not 0 <= index < n:
                 raise IndexError("index out of bounds for axis 0 with size %d" % n)
             inner = self.size // n
-            return DeviceArray._view_of(self, self.ptr + key * inner * ITEMSIZE if self.ptr else 0, shape[1:], inner)
+            v = DeviceArray._view_of(self, self.ptr + index * inner * ITEMSIZE if self.ptr else 0, shape[1:], inner)
+            if steps is None:
+                steps = self._steps = {}
+            steps[key] = v
+            return v
         if type(key) is slice:
             if not shape:
                 raise IndexError("too many indices for a 0-d array")
@@ -284,6 +298,7 @@ class PitchedDeviceArray(DeviceArray):
         self.run = shape[-1] if run is None else run
         self._owner = owner
         self._handler = handler
+        self._steps = None
 
     @property
     def ptr(self):

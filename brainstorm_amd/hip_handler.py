@@ -17,6 +17,10 @@ import ctypes
 import numpy as np
 
 from . import _lib
+try:
+    from . import _fastcall
+except ImportError as exc:          # no fallback: the extension is part of the build
+    raise ImportError("brainstorm_amd._fastcall is not built; run `python -m brainstorm_amd.build` (%s)" % exc)
 from ._lib import (ABS, ADD, ADD_IF, ADD_ST, COPY_IF, DIV, EL, EL_DERIV, FILL_IF, FMOD, LOG, MUL,
                    MULT_ADD_ST, MULT_ST, PITCHED_BINARY, PITCHED_CLIP, PITCHED_COND, PITCHED_DERIV,
                    PITCHED_FILL, PITCHED_MULT_ADD, PITCHED_SCALAR, PITCHED_UNARY, REL, REL_DERIV, SIGMOID,
@@ -216,6 +220,14 @@ class HipHandler(Handler):
         super(HipHandler, self).__init__()
         self._lib = _lib.load()
         self._call(self._lib.bship_init(int(device)))
+        # the operations a network step issues by the thousand are called without ctypes' per-argument
+        # conversions (csrc/fastcall.c); everything else goes through ctypes
+        fast = _fastcall.Calls(_lib.entry_point_addresses(self._lib))
+        self._fast = fast
+        (self._binary, self._mult_add, self._scalar, self._unary, self._deriv, self._clip, self._mv_call,
+         self._fill_call, self._gemm_call, self._d2d, self._sum_call) = (
+            fast.binary, fast.mult_add_tt, fast.scalar, fast.unary, fast.deriv, fast.clip, fast.mv, fast.fill,
+            fast.gemm, fast.d2d, fast.sum)
         self.dtype = np.float32
         self.device = int(device)
         self.context = self._lib
@@ -628,7 +640,9 @@ class HipHandler(Handler):
         # numpy 47-52 / pycuda 83-85: np.copyto broadcasts src to dest's shape (a scalar, a row for every
         # row, a column for every column, ...). Every run of neighbouring axes that repeat is one broadcast_t.
         if src.shape == dest.shape:
-            self._call(self._lib.bship_d2d(dest.ptr, src.ptr, dest.size * 4))
+            st = self._d2d(dest.ptr, src.ptr, dest.size * 4)
+            if st:
+                self._call(st)
             return
         if src.ndim > dest.ndim:
             raise ValueError("copy_to: could not broadcast %r into %r" % (src.shape, dest.shape))
@@ -669,7 +683,9 @@ class HipHandler(Handler):
         return out
 
     def fill(self, mem, val):
-        self._call(self._lib.bship_fill_f32(mem.ptr, val, mem.size))
+        st = self._fill_call(mem.ptr, val, mem.size)
+        if st:
+            self._call(st)
 
     def fill_if(self, mem, val, cond):
         if cond.size != mem.size:
@@ -702,7 +718,9 @@ class HipHandler(Handler):
     def abs_t(self, a, out):
         if a.size != out.size:
             raise _mismatch("abs_t", a, out)
-        self._call(self._lib.bship_unary_f32(ABS, a.ptr, out.ptr, out.size))
+        st = self._unary(ABS, a.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def add_into_if(self, a, out, cond):
         if a.size != out.size or cond.size != out.size:
@@ -712,68 +730,94 @@ class HipHandler(Handler):
     def add_st(self, s, t, out):
         if t.size != out.size:
             raise _mismatch("add_st", t, out)
-        self._call(self._lib.bship_scalar_f32(ADD_ST, s, t.ptr, out.ptr, out.size))
+        st = self._scalar(ADD_ST, s, t.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def add_tt(self, a, b, out):
         if a.size != out.size or b.size != out.size:
             raise _mismatch("add_tt", a, b, out)
-        self._call(self._lib.bship_binary_f32(ADD, a.ptr, b.ptr, out.ptr, out.size))
+        st = self._binary(ADD, a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def clip_t(self, a, a_min, a_max, out):
         if a.size != out.size:
             raise _mismatch("clip_t", a, out)
-        self._call(self._lib.bship_clip_f32(a.ptr, a_min, a_max, out.ptr, out.size))
+        st = self._clip(a.ptr, a_min, a_max, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def divide_tt(self, a, b, out):
         if a.size != out.size or b.size != out.size:
             raise _mismatch("divide_tt", a, b, out)
-        self._call(self._lib.bship_binary_f32(DIV, a.ptr, b.ptr, out.ptr, out.size))
+        st = self._binary(DIV, a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def log_t(self, a, out):
         if a.size != out.size:
             raise _mismatch("log_t", a, out)
-        self._call(self._lib.bship_unary_f32(LOG, a.ptr, out.ptr, out.size))
+        st = self._unary(LOG, a.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def modulo_tt(self, a, b, out):
         if a.size != out.size or b.size != out.size:
             raise _mismatch("modulo_tt", a, b, out)
-        self._call(self._lib.bship_binary_f32(FMOD, a.ptr, b.ptr, out.ptr, out.size))
+        st = self._binary(FMOD, a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def mult_add_st(self, s, t, out):
         if t.size != out.size:
             raise _mismatch("mult_add_st", t, out)
-        self._call(self._lib.bship_scalar_f32(MULT_ADD_ST, s, t.ptr, out.ptr, out.size))
+        st = self._scalar(MULT_ADD_ST, s, t.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def mult_add_tt(self, a, b, out):
         if a.size != out.size or b.size != out.size:
             raise _mismatch("mult_add_tt", a, b, out)
-        self._call(self._lib.bship_mult_add_tt_f32(a.ptr, b.ptr, out.ptr, out.size))
+        st = self._mult_add(a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def mult_st(self, s, t, out):
         if t.size != out.size:
             raise _mismatch("mult_st", t, out)
-        self._call(self._lib.bship_scalar_f32(MULT_ST, s, t.ptr, out.ptr, out.size))
+        st = self._scalar(MULT_ST, s, t.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def mult_tt(self, a, b, out):
         if a.size != out.size or b.size != out.size:
             raise _mismatch("mult_tt", a, b, out)
-        self._call(self._lib.bship_binary_f32(MUL, a.ptr, b.ptr, out.ptr, out.size))
+        st = self._binary(MUL, a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def sign_t(self, a, out):
         if a.size != out.size:
             raise _mismatch("sign_t", a, out)
-        self._call(self._lib.bship_unary_f32(SIGN, a.ptr, out.ptr, out.size))
+        st = self._unary(SIGN, a.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def sqrt_t(self, a, out):
         if a.size != out.size:
             raise _mismatch("sqrt_t", a, out)
-        self._call(self._lib.bship_unary_f32(SQRT, a.ptr, out.ptr, out.size))
+        st = self._unary(SQRT, a.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     def subtract_tt(self, a, b, out):
         assert a.shape == b.shape == out.shape     # numpy 265
         if a.size != out.size or b.size != out.size:     # also when assertions are switched off
             raise _mismatch("subtract_tt", a, b, out)
-        self._call(self._lib.bship_binary_f32(SUB, a.ptr, b.ptr, out.ptr, out.size))
+        st = self._binary(SUB, a.ptr, b.ptr, out.ptr, out.size)
+        if st:
+            self._call(st)
 
     # -------------------------------------------------- broadcast operations
     def _mv(self, op, m, v, out, accumulate):
@@ -783,8 +827,8 @@ class HipHandler(Handler):
         if v.shape == m.shape:
             if accumulate:
                 assert op == MUL
-                return self._call(self._lib.bship_mult_add_tt_f32(m.ptr, v.ptr, out.ptr, out.size))
-            return self._call(self._lib.bship_binary_f32(op, m.ptr, v.ptr, out.ptr, out.size))
+                return self._call(self._mult_add(m.ptr, v.ptr, out.ptr, out.size))
+            return self._call(self._binary(op, m.ptr, v.ptr, out.ptr, out.size))
         n_cols = m.shape[-1] if m.shape else 1
         n_rows = m.size // n_cols if n_cols else 0
         vs = v.shape
@@ -795,8 +839,9 @@ class HipHandler(Handler):
         else:
             raise ValueError("cannot broadcast vector of shape %r against matrix of shape %r"
                              % (vs, m.shape))
-        self._call(self._lib.bship_mv_f32(op, m.ptr, v.ptr, out.ptr, n_rows, n_cols, is_col,
-                                          accumulate))
+        st = self._mv_call(op, m.ptr, v.ptr, out.ptr, n_rows, n_cols, is_col, accumulate)
+        if st:
+            self._call(st)
 
     def add_mv(self, m, v, out):
         self._mv(ADD, m, v, out, 0)
@@ -847,7 +892,9 @@ class HipHandler(Handler):
         if axis is None or a.ndim <= 1:
             if out.size != 1:
                 raise _mismatch("sum_t", a, out)
-            self._call(self._lib.bship_sum_f32(a.ptr, out.ptr, 1, a.size, -1))
+            st = self._sum_call(a.ptr, out.ptr, 1, a.size, -1)
+            if st:
+                self._call(st)
             return
         if not isinstance(axis, (int, np.integer)):
             raise NotImplementedError("sum_t over axes %r" % (axis,))
@@ -862,9 +909,9 @@ class HipHandler(Handler):
         if outer * inner == 0:
             return
         if inner == 1:
-            self._call(lib.bship_sum_f32(a.ptr, out.ptr, outer, length, 1))
+            self._call(self._sum_call(a.ptr, out.ptr, outer, length, 1))
         elif outer == 1:
-            self._call(lib.bship_sum_f32(a.ptr, out.ptr, length, inner, 0))
+            self._call(self._sum_call(a.ptr, out.ptr, length, inner, 0))
         elif outer <= length:
             # a column sum per outer index: slab o is a contiguous (length, inner) matrix
             for o in range(outer):
@@ -924,8 +971,9 @@ class HipHandler(Handler):
         pa, lda = (a._base, a.pitch) if type(a) is PitchedDeviceArray else (a.ptr, a.shape[1])
         pb, ldb = (b._base, b.pitch) if type(b) is PitchedDeviceArray else (b.ptr, b.shape[1])
         pc, ldc = (out._base, out.pitch) if type(out) is PitchedDeviceArray else (out.ptr, n)
-        self._call(self._lib.bship_gemm_f32(int(bool(transa)), int(bool(transb)), m, n, k, 1.0,
-                                            pa, lda, pb, ldb, beta, pc, ldc))
+        st = self._gemm_call(1 if transa else 0, 1 if transb else 0, m, n, k, 1.0, pa, lda, pb, ldb, beta, pc, ldc)
+        if st:
+            self._call(st)
 
     def dot_mm(self, a, b, out, transa=False, transb=False):
         self._gemm(a, b, out, transa, transb, 0.0)
@@ -1058,42 +1106,58 @@ class HipHandler(Handler):
     def rel(self, x, y):
         if x.size != y.size:
             raise _mismatch("rel", x, y)
-        self._call(self._lib.bship_unary_f32(REL, x.ptr, y.ptr, y.size))
+        st = self._unary(REL, x.ptr, y.ptr, y.size)
+        if st:
+            self._call(st)
 
     def rel_deriv(self, x, y, dy, dx):
         if y.size != dx.size or dy.size != dx.size:
             raise _mismatch("rel_deriv", y, dy, dx)
-        self._call(self._lib.bship_deriv_f32(REL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+        st = self._deriv(REL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size)
+        if st:
+            self._call(st)
 
     def sigmoid(self, x, y):
         if x.size != y.size:
             raise _mismatch("sigmoid", x, y)
-        self._call(self._lib.bship_unary_f32(SIGMOID, x.ptr, y.ptr, y.size))
+        st = self._unary(SIGMOID, x.ptr, y.ptr, y.size)
+        if st:
+            self._call(st)
 
     def sigmoid_deriv(self, x, y, dy, dx):
         if y.size != dx.size or dy.size != dx.size:
             raise _mismatch("sigmoid_deriv", y, dy, dx)
-        self._call(self._lib.bship_deriv_f32(SIGMOID_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+        st = self._deriv(SIGMOID_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size)
+        if st:
+            self._call(st)
 
     def tanh(self, x, y):
         if x.size != y.size:
             raise _mismatch("tanh", x, y)
-        self._call(self._lib.bship_unary_f32(TANH, x.ptr, y.ptr, y.size))
+        st = self._unary(TANH, x.ptr, y.ptr, y.size)
+        if st:
+            self._call(st)
 
     def tanh_deriv(self, x, y, dy, dx):
         if y.size != dx.size or dy.size != dx.size:
             raise _mismatch("tanh_deriv", y, dy, dx)
-        self._call(self._lib.bship_deriv_f32(TANH_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+        st = self._deriv(TANH_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size)
+        if st:
+            self._call(st)
 
     def el(self, x, y):
         if x.size != y.size:
             raise _mismatch("el", x, y)
-        self._call(self._lib.bship_unary_f32(EL, x.ptr, y.ptr, y.size))
+        st = self._unary(EL, x.ptr, y.ptr, y.size)
+        if st:
+            self._call(st)
 
     def el_deriv(self, x, y, dy, dx):
         if y.size != dx.size or dy.size != dx.size:
             raise _mismatch("el_deriv", y, dy, dx)
-        self._call(self._lib.bship_deriv_f32(EL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size))
+        st = self._deriv(EL_DERIV, y.ptr, dy.ptr, dx.ptr, dx.size)
+        if st:
+            self._call(st)
 
     # ------------------------------------------------ fused layer-level steps
     # Extensions beyond the Handler interface. A layer may test for them with

@@ -166,3 +166,23 @@ def test_net_applies_modifiers_where_the_reference_does():
     stepper.run()
     w = net.get("fc1", "parameters", "W")
     assert np.sqrt((w ** 2).sum(axis=1)).max() <= 0.05 * (1 + 1e-9)
+
+
+def test_label_range_is_numpy_indexing():
+    # labels in [-K, -1] count from the last column (numpy_handler.py:101, 203); beyond [-K, K), NaN and
+    # infinities are refused
+    h = NumpyRefHandler(np.float32, seed=0)
+    checked = CheckedHandler(h)
+    m = checked.create_from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4))
+    out = checked.allocate((3, 1))
+    checked.index_m_by_v(m, checked.create_from_numpy(np.array([[-1], [-4], [3]], np.float32)), out)
+    assert np.array_equal(out.ravel(), [3, 4, 11])
+    onehot = checked.allocate((3, 4))
+    checked.binarize_v(checked.create_from_numpy(np.array([[-1], [0], [-4]], np.float32)), onehot)
+    assert np.array_equal(np.argmax(onehot, axis=1), [3, 0, 0])
+    for bad in (-5.0, 4.0, np.nan, np.inf):
+        labels = checked.create_from_numpy(np.array([[0], [bad], [1]], np.float32))
+        with pytest.raises(ContractError, match=r"\[-4, 4\)"):
+            checked.binarize_v(labels, onehot)
+        with pytest.raises(ContractError):
+            checked.index_m_by_v(m, labels, out)

@@ -422,16 +422,17 @@ def test_copy_to_broadcasts_like_numpy(hip, ref):
     rng = np.random.RandomState(19)
     cases = [((1, 7), (5, 7)), ((7,), (5, 7)), ((5, 1), (5, 7)), ((1,), (5, 7)), ((), (3, 4, 5)), ((1, 1), (3, 4)),
              ((3, 1, 1, 6), (3, 4, 5, 6)), ((4, 260), (3, 4, 260)), ((2, 1, 1028), (2, 300, 1028)), ((5, 7), (5, 7)),
-             ((35,), (35,))]
+             ((35,), (35,)),
+             # repeated axes that are not neighbours: one broadcast per run of them, innermost first
+             ((1, 4, 1), (3, 4, 5)), ((4, 1), (3, 4, 5)), ((2, 1, 3, 1), (2, 5, 3, 4)), ((1, 3, 1, 7, 1), (2, 3, 4, 7, 5)),
+             ((1, 1, 5), (1, 1, 5)), ((1, 5), (1, 1, 5))]
     for src_shape, dest_shape in cases:
         operation_check(hip, ref, "copy_to", (rand(rng, src_shape), rand(rng, dest_shape)))
-    for src_shape, dest_shape in [((3,), (5, 7)), ((2, 7), (5, 7)), ((5, 7, 1), (5, 7))]:
+    for src_shape, dest_shape in [((3,), (5, 7)), ((2, 7), (5, 7)), ((5, 7, 1), (5, 7)), ((35,), (5, 7))]:
         with pytest.raises(ValueError):
             hip.copy_to(hip.allocate(src_shape), hip.allocate(dest_shape))
         with pytest.raises(ValueError):
             ref.copy_to(np.zeros(src_shape, F32), np.zeros(dest_shape, F32))
-    with pytest.raises(NotImplementedError):
-        hip.copy_to(hip.allocate((1, 4, 1)), hip.allocate((3, 4, 5)))      # repeats two axes that are not neighbours
 
 
 def test_sum_t_is_deterministic(hip):
