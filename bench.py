@@ -303,11 +303,19 @@ def run_pitched_ops(rows=8192, cols=8192, reps=10):
     return out
 
 
-def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
+def time_net(handler, builder, steps, warmup, sync, recorded=False, fusing=None, **kw):
     """Training steps per second of one network workload (forward + backward + momentum update,
     inputs uploaded once; the per-step loss read-back of a Trainer is included). recorded: the
-    step's handler calls are recorded once (after an ordinary step) and replayed with one launch."""
+    step's handler calls are recorded once (after an ordinary step) and replayed with one launch.
+    fusing: the handler's fusing window on or off for this run (None: as the handler is). The
+    random stream is restarted first, so every variant of a network sees the same dropout masks;
+    "loss" is the loss of the last step, which variants that promise the same bits must share."""
     from brainstorm_amd.drivers.net import MomentumStepper
+    before = getattr(handler, "fusing", None)
+    if fusing is not None:
+        handler.set_fusing(fusing)
+    if hasattr(handler.rnd, "seed"):
+        handler.rnd.seed(0)
     net, data = builder(handler, **kw)
     net.provide_external_data(data)
     stepper = MomentumStepper(0.1, 0.9, fused=bool(kw.get("fused")))
@@ -315,20 +323,23 @@ def time_net(handler, builder, steps, warmup, sync, recorded=False, **kw):
     if recorded:
         stepper.run()
     step = stepper.run_recorded if recorded else stepper.run
-    for _ in range(warmup):
+    for _ in range(warmup - (1 if recorded else 0)):
         step()
         net.get("loss", "outputs", "loss")
     sync()
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
-        net.get("loss", "outputs", "loss")      # device-to-host copy + wait, as trainer.py:100 does
+        loss = net.get("loss", "outputs", "loss")      # device-to-host copy + wait, as trainer.py:100 does
     sync()
     dt = (time.perf_counter() - t0) / steps
     if recorded:
         stepper.release_recorded()
+    if fusing is not None:
+        handler.set_fusing(before)
     samples = data["default"].shape[0] * data["default"].shape[1]
-    return {"ms_per_step": round(dt * 1e3, 3), "samples_per_s": round(samples / dt, 1)}
+    return {"ms_per_step": round(dt * 1e3, 3), "samples_per_s": round(samples / dt, 1),
+            "loss": float(np.asarray(loss).ravel()[0])}
 
 
 def time_net_fast_masks(builder, steps, warmup):
@@ -337,51 +348,72 @@ def time_net_fast_masks(builder, steps, warmup):
     return time_net(handler, builder, steps, warmup, handler.synchronize, recorded=True, fused=True)
 
 
+def same_bits(nets, names):
+    """The variants `names` of one network promise the same bits: their last losses must be one number
+    (a timing of a path that computes something else is not a timing of that network)."""
+    losses = {n: nets[n]["loss"] for n in names}
+    if len({np.float32(v).tobytes() for v in losses.values()}) != 1 or not all(np.isfinite(v) for v in losses.values()):
+        raise AssertionError("variants that must agree bit for bit do not: %r" % losses)
+
+
+def close_to(nets, name, reference, rel):
+    a, b = nets[name]["loss"], nets[reference]["loss"]
+    if not (np.isfinite(a) and abs(a - b) <= rel * abs(b)):
+        raise AssertionError("%s: loss %r is not within %g of %s's %r" % (name, a, rel, reference, b))
+
+
 def run_nets_gpu(hip):
+    """Step times of the four network workloads. The first line of each group is what an UNCHANGED caller
+    gets: the reference layers' primitive call sequences (fused=False drivers) on the default handler, whose
+    fusing window turns them into the fused kernels (same bits). "_window_off": the same calls launched
+    one by one. "_fused...": a handler-aware caller that asks for the fused entry points itself."""
     from brainstorm_amd.drivers import configs
-    return {
-        "mlp_784-1200-1200-10_batch100": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize),
-        # same network, dropout and bias+activation through the fused entry points (same bits)
-        "mlp_784-1200-1200-10_batch100_fused": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize,
-                                                        fused=True),
-        # same network and bits, the step recorded into a HIP graph and replayed
-        "mlp_784-1200-1200-10_batch100_recorded": time_net(hip, configs.build_mlp, 600, 20, hip.synchronize,
-                                                           recorded=True),
-        "mlp_784-1200-1200-10_batch100_fused_recorded": time_net(hip, configs.build_mlp, 600, 20,
-                                                                 hip.synchronize, recorded=True, fused=True),
+    mlp, lstm, cnn, hw = ("mlp_784-1200-1200-10_batch100", "lstm_205-1000-205_T100_batch100", "cnn_32x32x3_batch100",
+                          "highway_bn_50x4096_batch2048")
+    sync = hip.synchronize
+    nets = {
+        mlp: time_net(hip, configs.build_mlp, 600, 20, sync, fusing=True),
+        mlp + "_window_off": time_net(hip, configs.build_mlp, 600, 20, sync, fusing=False),
+        # dropout, bias + activation, softmax cross entropy and the update through the fused entry points
+        mlp + "_fused": time_net(hip, configs.build_mlp, 600, 20, sync, fused=True),
+        # the step recorded into a HIP graph and replayed
+        mlp + "_recorded": time_net(hip, configs.build_mlp, 600, 20, sync, recorded=True),
+        mlp + "_fused_recorded": time_net(hip, configs.build_mlp, 600, 20, sync, recorded=True, fused=True),
         # NOT the reference's masks: dropout masks from the optional counter-based generator
         # (HipHandler(fast_masks=True)), one parallel launch per mask instead of the MT19937 walk
-        "mlp_784-1200-1200-10_batch100_fused_recorded_fast_masks": time_net_fast_masks(configs.build_mlp, 600, 20),
-        "lstm_205-1000-205_T100_batch100": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize),
-        # same network and bits, the ~4000 launches of a step recorded into a HIP graph and replayed
-        "lstm_205-1000-205_T100_batch100_recorded": time_net(hip, configs.build_lstm, 5, 1, hip.synchronize,
-                                                             recorded=True),
-        # same network, the elementwise part of each time step in one launch (same bits)
-        "lstm_205-1000-205_T100_batch100_fused_steps": time_net(hip, configs.build_lstm, 5, 1,
-                                                               hip.synchronize, fused=True),
+        mlp + "_fused_recorded_fast_masks": time_net_fast_masks(configs.build_mlp, 600, 20),
+        lstm: time_net(hip, configs.build_lstm, 5, 2, sync, fusing=True),
+        lstm + "_window_off": time_net(hip, configs.build_lstm, 5, 2, sync, fusing=False),
+        # the ~4000 launches of a step (window off) recorded into a HIP graph and replayed
+        lstm + "_window_off_recorded": time_net(hip, configs.build_lstm, 5, 2, sync, recorded=True, fusing=False),
+        # the elementwise part of each time step in one launch, asked for by the layer
+        lstm + "_fused_steps": time_net(hip, configs.build_lstm, 5, 2, sync, fused=True),
         # ... and the four recurrent matrix products of a step as one over the stacked matrices
-        "lstm_205-1000-205_T100_batch100_fused_packed": time_net(hip, configs.build_lstm, 5, 1,
-                                                                hip.synchronize, fused="packed"),
+        lstm + "_fused_packed": time_net(hip, configs.build_lstm, 5, 2, sync, fused="packed"),
         # ... with the backward recurrent product through the thin-operand kernel (dot_small_tn)
-        "lstm_205-1000-205_T100_batch100_fused_thin": time_net(hip, configs.build_lstm, 5, 1,
-                                                              hip.synchronize, fused="thin"),
+        lstm + "_fused_thin": time_net(hip, configs.build_lstm, 5, 2, sync, fused="thin"),
         # ... and the whole forward recurrence as one persistent launch (weights resident in LDS, one grid
         # barrier per time step); the backward pass is the packed one
-        "lstm_205-1000-205_T100_batch100_fused_sequence": time_net(hip, configs.build_lstm, 5, 1,
-                                                                  hip.synchronize, fused="sequence"),
+        lstm + "_fused_sequence": time_net(hip, configs.build_lstm, 5, 2, sync, fused="sequence"),
         # the convolutional workload (conv 5x5x32, max pool 3x3/2, conv 5x5x64, max pool, 1000, 10)
-        "cnn_32x32x3_batch100": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize),
-        # same network and bits, the step recorded into a HIP graph and replayed
-        "cnn_32x32x3_batch100_recorded": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize, recorded=True),
-        # ... with the fused entry points (bias + activation, softmax cross entropy, momentum update; same bits)
-        "cnn_32x32x3_batch100_fused": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize, fused=True),
-        "cnn_32x32x3_batch100_fused_recorded": time_net(hip, configs.build_cnn, 200, 10, hip.synchronize,
-                                                        recorded=True, fused=True),
+        cnn: time_net(hip, configs.build_cnn, 200, 10, sync, fusing=True),
+        cnn + "_window_off": time_net(hip, configs.build_cnn, 200, 10, sync, fusing=False),
+        cnn + "_recorded": time_net(hip, configs.build_cnn, 200, 10, sync, recorded=True),
+        cnn + "_fused": time_net(hip, configs.build_cnn, 200, 10, sync, fused=True),
+        cnn + "_fused_recorded": time_net(hip, configs.build_cnn, 200, 10, sync, recorded=True, fused=True),
         # the bandwidth-stress workload: 50 Highway + batch normalisation blocks of width 4096
-        "highway_bn_50x4096_batch2048": time_net(hip, configs.build_highway, 3, 1, hip.synchronize),
-        "highway_bn_50x4096_batch2048_fused": time_net(hip, configs.build_highway, 3, 1, hip.synchronize,
-                                                       fused=True),
+        hw: time_net(hip, configs.build_highway, 3, 1, sync, fusing=True),
+        hw + "_window_off": time_net(hip, configs.build_highway, 3, 1, sync, fusing=False),
+        hw + "_fused": time_net(hip, configs.build_highway, 3, 1, sync, fused=True),
     }
+    # a timing of a broken path must fail: same-bits variants share their last loss, the others are close to it
+    same_bits(nets, [mlp, mlp + "_window_off", mlp + "_fused", mlp + "_recorded", mlp + "_fused_recorded"])
+    same_bits(nets, [lstm, lstm + "_window_off", lstm + "_window_off_recorded", lstm + "_fused_steps"])
+    for variant in ("_fused_packed", "_fused_thin", "_fused_sequence"):      # other summation orders in the products
+        close_to(nets, lstm + variant, lstm, 1e-4)
+    same_bits(nets, [cnn, cnn + "_window_off", cnn + "_recorded", cnn + "_fused", cnn + "_fused_recorded"])
+    same_bits(nets, [hw, hw + "_window_off", hw + "_fused"])
+    return nets
 
 
 def run_nets_cpu(ref):
@@ -456,6 +488,10 @@ def main():
                     if args.size == 16384 and dominant in MEASURED_TRAFFIC_MIB_2P28 else None),
         "alg_bytes_per_launch": ab[dominant], "ms_per_launch": ops[dominant]["ms"],
     }
+    # the graded kernel furthest below the roofline in the timed sweep (index_m_by_v is a latency-bound gather
+    # of one element per row and is reported in microseconds, not graded against the bandwidth)
+    lowest = min((n for n in ops if n != "index_m_by_v"), key=lambda n: ops[n]["frac"])
+    roofline["lowest"] = {"kernel": lowest, "frac": ops[lowest]["frac"]}
     out = {
         "metric": "handler-op HBM GB/s", "value": round(value, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -467,7 +503,6 @@ def main():
                                   int(round(np.log2(args.size * args.size)))),
                    "device": dev_name, "compute_units": cus},
         "roofline": roofline,
-        "ops": ops,
     }
     if not args.no_2p26 and args.size != 8192:
         # the same sweep at 2^26 elements per tensor, the smallest size the throughput targets are
@@ -506,6 +541,12 @@ def main():
         if not args.no_nets:
             from oracle.numpy_ref_handler import NumpyRefHandler
             out["cpu_baseline"]["nets"] = run_nets_cpu(NumpyRefHandler(F32, seed=0))
+    # the per-operation tables go last, the headline sweep's at the very end, so that a reader who keeps
+    # only the end of the line still has the figures the headline value is made of
+    for key in ("image_ops", "pitched_ops", "note_256mb_tensors", "ops_2p26"):
+        if key in out:
+            out[key] = out.pop(key)
+    out["ops"] = ops
     print(json.dumps(out))
 
 

@@ -78,6 +78,14 @@ int window_flush();
 static inline bool window_takes() {
     return g_window_on.load(std::memory_order_relaxed) != 0 && !t_window_emitting;
 }
+// For code that holds one of the library's own locks while it calls public entry points: those calls
+// must not go for the window's lock (the window takes that lock first and the other one inside when it
+// enqueues a held operation). What the window held was enqueued by the outer entry point already.
+struct WindowBypass {
+    bool before;
+    WindowBypass() : before(t_window_emitting) { t_window_emitting = true; }
+    ~WindowBypass() { t_window_emitting = before; }
+};
 
 #define BSHIP_REQUIRE_INIT_NO_FLUSH()                                            \
     do {                                                                         \

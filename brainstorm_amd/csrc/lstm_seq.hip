@@ -39,12 +39,27 @@
 
 #include <cstdlib>
 
+#include <cerrno>
+#include <mutex>
+
 #include "buffer_loads.h"
 #include "common.h"
 #include "functors.h"
 #include "lstm_cell.h"
 
 namespace bship {
+
+// The value of an environment variable that must be a whole number in [0, most]; `fallback` when it is
+// unset, empty, not a number, followed by anything, or too large.
+static unsigned long long env_number(const char* name, unsigned long long fallback, unsigned long long most) {
+    const char* text = getenv(name);
+    if (!text || !text[0]) return fallback;
+    char* end = nullptr;
+    errno = 0;
+    const unsigned long long v = strtoull(text, &end, 10);
+    if (errno != 0 || end == text || *end != 0 || text[0] == '-' || v > most) return fallback;
+    return v;
+}
 
 constexpr int kSeqSetThreads = 256;               // the four wavefronts (K quarters) of one row set
 constexpr int kSeqUnits = 4;                      // hidden units per workgroup
@@ -315,14 +330,18 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
     int kpitch = k16;                                  // covers every k a wavefront reads
     if ((kpitch / 4) % 2 == 0) kpitch += 4;            // an odd number of 16-byte units per row spreads the rows over the banks
     a.kpitch = kpitch;
-    const char* spins = getenv("BSHIP_GRID_BARRIER_SPINS");
-    a.spin_limit = spins && spins[0] ? static_cast<unsigned>(strtoul(spins, nullptr, 10)) : (1u << 21);
+    // BSHIP_GRID_BARRIER_SPINS: polls a workgroup spends at a barrier before it gives up. A value that is
+    // not a whole number is ignored; 0 is the test hook that makes every barrier fail at once.
+    a.spin_limit = static_cast<unsigned>(env_number("BSHIP_GRID_BARRIER_SPINS", 1u << 21, 0xffffffffull));
     const size_t lds = (static_cast<size_t>(kSeqCols) * kpitch + 4 * kSeqMaxBatch * kSeqCols) * sizeof(float);
-    static bool lds_granted = false;
-    if (!lds_granted) {
-        BSHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(lstm_fwd_sequence_kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024));
-        lds_granted = true;
+    {
+        static std::once_flag lds_once;
+        static hipError_t lds_status = hipSuccess;
+        std::call_once(lds_once, [] {
+            lds_status = hipFuncSetAttribute(reinterpret_cast<const void*>(lstm_fwd_sequence_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
+        });
+        BSHIP_HIP(lds_status);
     }
     // More than half of a compute unit's LDS, so that two workgroups never share one: a second one would
     // take matrix-core time from the first without shortening anybody's step.
@@ -340,8 +359,11 @@ extern "C" int bship_lstm_fwd_sequence_f32(int act, int64_t time_steps, int64_t 
     // the failure flag, 256 bytes on the flags of both groups (zero-filled), 4 KB on the transposed buffers:
     // one per time step and one for y[-1] if that stays below 256 MB, else as many as do (at least two)
     const size_t one = static_cast<size_t>(a.krows) * kSeqMaxBatch * sizeof(float);
-    const char* cap_mb = getenv("BSHIP_LSTM_SEQ_SCRATCH_MB");       // default 256; small values force buffers to be reused
-    const size_t cap = static_cast<size_t>(cap_mb && cap_mb[0] ? strtoul(cap_mb, nullptr, 10) : 256) << 20;
+    // BSHIP_LSTM_SEQ_SCRATCH_MB: default 256; small values force buffers to be reused (anything that is not a
+    // whole number of at least 1 is ignored)
+    size_t cap_mb = static_cast<size_t>(env_number("BSHIP_LSTM_SEQ_SCRATCH_MB", 256, 1u << 20));
+    if (cap_mb < 1) cap_mb = 256;
+    const size_t cap = cap_mb << 20;
     int64_t nbuf = time_steps + 1;
     if (static_cast<size_t>(nbuf) * one > cap) nbuf = static_cast<int64_t>(cap / one) < 2 ? 2 : static_cast<int64_t>(cap / one);
     a.nbuf = static_cast<int>(nbuf);

@@ -796,6 +796,7 @@ static void prefetch_maybe_start() {
 
 int rng_graph_begin(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     int st = ensure_side_stream();
     if (st == 0 && g_state) st = prefetch_flush(true);
     if (st == 0 && g_state) st = graph_masks_unprime();
@@ -809,6 +810,7 @@ int rng_graph_begin(int id) {
 // The recording is complete: one buffer for the raw words of a round of its masks (a block of the recording's own).
 int rng_graph_end(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     g_recording_masks = 0;
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
@@ -823,6 +825,7 @@ int rng_graph_end(int id) {
 
 int rng_graph_before_launch(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
     {
@@ -871,6 +874,7 @@ static int draw_next_round(GraphMasks& gm) {
 
 int rng_graph_after_launch(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end() || it->second.slots.empty()) return 0;
     const int st = draw_next_round(it->second);
@@ -884,6 +888,7 @@ int rng_graph_after_launch(int id) {
 
 void rng_graph_destroyed(int id) {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     auto it = g_graph_masks.find(id);
     if (it == g_graph_masks.end()) return;
     if (g_primed_graph == id) (void)graph_masks_unprime();
@@ -1094,6 +1099,7 @@ static int launch_fast_mask(const float* in, float* mask, float* out, size_t n, 
 
 void rng_release() {
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (g_side) (void)hipStreamSynchronize(g_side);
     free_round(g_round[0]);
     free_round(g_round[1]);
@@ -1143,6 +1149,7 @@ static int rng_seed_impl(int generator, uint32_t seed) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1166,6 +1173,7 @@ static int rng_get_state_impl(int generator, uint32_t* key_host, int* pos_host, 
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1191,6 +1199,7 @@ static int prob_mask_pitched_f32_impl(int generator, float* mask, int64_t ld_mas
     BSHIP_REQUIRE_PTR(mask);
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1218,6 +1227,7 @@ static int dropout_fwd_f32_impl(int generator, const float* in, float* mask, flo
     const size_t tiles = (n + static_cast<size_t>(kBlock) * 4 - 1) / (static_cast<size_t>(kBlock) * 4);
     if (tiles > 0x7fffffffu) return set_error(BSHIP_ERR_BAD_DIMENSION, "%s: %zu elements exceed one launch", "bship_dropout_fwd_f32", n);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1248,6 +1258,7 @@ static int fill_gaussian_f32_impl(int generator, float* out, size_t n, double me
     BSHIP_REQUIRE_PTR(out);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1316,6 +1327,7 @@ static int fast_rng_seed_impl(int generator, unsigned long long seed) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1334,6 +1346,7 @@ static int fast_rng_get_state_impl(int generator, unsigned long long* seed_host,
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_EAGER();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1353,6 +1366,7 @@ static int prob_mask_fast_f32_impl(int generator, float* mask, size_t n, double 
     BSHIP_REQUIRE_PTR(mask);
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1372,6 +1386,7 @@ static int dropout_fwd_fast_f32_impl(int generator, const float* in, float* mask
     BSHIP_REQUIRE_F32_ALIGNED(mask);
     BSHIP_REQUIRE_F32_ALIGNED(out);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator >= 0) {
         int sel_st = select_generator_locked(generator);
         if (sel_st != 0) return sel_st;
@@ -1386,6 +1401,7 @@ int bship_rng_create(int* generator_id) {
     BSHIP_REQUIRE_INIT();
     BSHIP_REQUIRE_PTR(generator_id);
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     *generator_id = g_next_generator++;
     g_generators[*generator_id] = Generator();
     return 0;
@@ -1399,12 +1415,14 @@ int bship_rng_select(int generator_id) {
     }
     BSHIP_FLUSH_PENDING();       // masks that the fusing window holds are drawn from the generator selected so far
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     return select_generator_locked(generator_id);
 }
 
 int bship_rng_destroy(int generator_id) {
     BSHIP_REQUIRE_INIT();
     std::lock_guard<std::mutex> lock(g_rng_mutex);
+    WindowBypass bypass;      // entry points called from here neither flush nor feed the fusing window (lock order)
     if (generator_id == 0) return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator 0 is the library's own");
     if (g_generators.find(generator_id) == g_generators.end())
         return set_error(BSHIP_ERR_BAD_DIMENSION, "bship_rng_destroy: generator %d does not exist", generator_id);

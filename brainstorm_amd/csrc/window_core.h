@@ -367,58 +367,63 @@ inline bool ranges_overlap(const char* a, size_t alen, const char* b, size_t ble
     return alen != 0 && blen != 0 && a < b + blen && b < a + alen;
 }
 
+// Does call r agree with element i of the pattern, given the operands met so far (m)? Binds the
+// operands it meets for the first time.
+inline bool match_call(const Pattern& P, int i, const Rec& r, Match& m) {
+    const Elem& e = P.e[i];
+    if (r.kind != e.kind) return false;
+    if (e.op == OP_ANY_ACT || e.op == OP_ANY_ACT_DERIV) {
+        const int a = e.op == OP_ANY_ACT ? act_of_unary(r.op) : act_of_deriv(r.op);
+        if (a < 0) return false;
+        if (m.act < 0) m.act = a;
+        else if (m.act != a) return false;
+    } else if (e.kind != K_MASK && e.kind != K_FILL && e.kind != K_CLIP && e.kind != K_MULT_ADD_TT &&
+               e.kind != K_SOFTMAX && e.kind != K_INDEX && e.kind != K_BINARIZE) {
+        if (r.op != e.op) return false;
+    }
+    if (e.kind == K_MV && r.flags != e.flags) return false;
+    switch (e.check) {
+        case C_ONE: if (r.s0 != 1.0f) return false; break;
+        case C_MINUS_ONE: if (r.s0 != -1.0f) return false; break;
+        case C_CE_CLIP: if (r.s0 != 1e-6f || r.s1 != 1.0f) return false; break;
+        default: break;
+    }
+    if (has_shape(e.kind)) {
+        if (m.M < 0) {
+            if (m.total >= 0 && r.M * r.N != m.total) return false;
+            m.M = r.M; m.N = r.N; m.total = r.M * r.N;
+        } else if (r.M != m.M || r.N != m.N) {
+            return false;
+        }
+    } else {
+        int64_t want = e.size == S_MN ? m.total : (e.size == S_M ? m.M : m.N);
+        if (want < 0) {
+            if (e.size != S_MN) return false;
+            m.total = want = static_cast<int64_t>(r.n);
+        }
+        if (static_cast<int64_t>(r.n) != want) return false;
+    }
+    for (int s = 0; s < r.nptr; ++s) {
+        const int id = e.v[s];
+        if (id < 0) return false;
+        Var& v = m.v[id];
+        if (!v.bound) {
+            v.p = r.p[s]; v.len = r.len[s]; v.bound = true;
+        } else if (v.p != r.p[s] || v.len != r.len[s]) {
+            return false;
+        }
+        if ((r.wr >> s) & 1) v.written = true;
+    }
+    return true;
+}
+
 // How many of the first min(count, P.len) queued calls agree with the pattern: that number if all
 // of them do (m then holds the operands met so far), else -1.
 inline int match_prefix(const Pattern& P, const Rec* q, int count, Match& m) {
     m = Match();
     const int k = count < P.len ? count : P.len;
-    for (int i = 0; i < k; ++i) {
-        const Elem& e = P.e[i];
-        const Rec& r = q[i];
-        if (r.kind != e.kind) return -1;
-        if (e.op == OP_ANY_ACT || e.op == OP_ANY_ACT_DERIV) {
-            const int a = e.op == OP_ANY_ACT ? act_of_unary(r.op) : act_of_deriv(r.op);
-            if (a < 0) return -1;
-            if (m.act < 0) m.act = a;
-            else if (m.act != a) return -1;
-        } else if (e.kind != K_MASK && e.kind != K_FILL && e.kind != K_CLIP && e.kind != K_MULT_ADD_TT &&
-                   e.kind != K_SOFTMAX && e.kind != K_INDEX && e.kind != K_BINARIZE) {
-            if (r.op != e.op) return -1;
-        }
-        if (e.kind == K_MV && r.flags != e.flags) return -1;
-        switch (e.check) {
-            case C_ONE: if (r.s0 != 1.0f) return -1; break;
-            case C_MINUS_ONE: if (r.s0 != -1.0f) return -1; break;
-            case C_CE_CLIP: if (r.s0 != 1e-6f || r.s1 != 1.0f) return -1; break;
-            default: break;
-        }
-        if (has_shape(e.kind)) {
-            if (m.M < 0) {
-                if (m.total >= 0 && r.M * r.N != m.total) return -1;
-                m.M = r.M; m.N = r.N; m.total = r.M * r.N;
-            } else if (r.M != m.M || r.N != m.N) {
-                return -1;
-            }
-        } else {
-            int64_t want = e.size == S_MN ? m.total : (e.size == S_M ? m.M : m.N);
-            if (want < 0) {
-                if (e.size != S_MN) return -1;
-                m.total = want = static_cast<int64_t>(r.n);
-            }
-            if (static_cast<int64_t>(r.n) != want) return -1;
-        }
-        for (int s = 0; s < r.nptr; ++s) {
-            const int id = e.v[s];
-            if (id < 0) return -1;
-            Var& v = m.v[id];
-            if (!v.bound) {
-                v.p = r.p[s]; v.len = r.len[s]; v.bound = true;
-            } else if (v.p != r.p[s] || v.len != r.len[s]) {
-                return -1;
-            }
-            if ((r.wr >> s) & 1) v.written = true;
-        }
-    }
+    for (int i = 0; i < k; ++i)
+        if (!match_call(P, i, q[i], m)) return -1;
     return k;
 }
 
@@ -495,6 +500,8 @@ public:
             if (st == 0) st = s;
         }
         count_ = 0;
+        ncands_ = 0;
+        judged_ = 0;
         return st;
     }
 
@@ -536,6 +543,13 @@ public:
     void count_overtaken() { ++stats_.overtaken; }
 
 private:
+    // A pattern that agrees with the held calls so far (all of them, or its whole length).
+    struct Candidate {
+        int pattern;
+        int matched;
+        Match m;
+    };
+
     int emit_fused(const Pattern& P, const Match& m, Sink& sink) {
         const int st = sink.fused(P, m, q_);
         ++stats_.fused;
@@ -548,32 +562,80 @@ private:
     void drop_front(int k) {
         if (k < count_) memmove(static_cast<void*>(q_), static_cast<const void*>(q_ + k), sizeof(Rec) * size_t(count_ - k));
         count_ -= k;
+        ncands_ = 0;        // the candidates were anchored at the old first call
+        judged_ = 0;
+    }
+
+    // Brings the candidates up to date with the held calls: from scratch when the first held call has
+    // changed, else by looking at the calls that arrived since (one, as a rule).
+    void update_candidates() {
+        const Pattern* table = patterns();
+        if (judged_ == 0) {
+            ncands_ = 0;
+            for (int k = 0; k < P_COUNT; ++k) {
+                const Pattern& P = table[k];
+                if (P.e[0].kind != q_[0].kind) continue;      // most sequences open with another kind of call
+                Candidate& c = cands_[ncands_];
+                const int got = match_prefix(P, q_, count_, c.m);
+                if (got < 0) continue;
+                c.pattern = k;
+                c.matched = got;
+                ++ncands_;
+            }
+        } else {
+            int kept = 0;
+            for (int k = 0; k < ncands_; ++k) {
+                Candidate& c = cands_[k];
+                const Pattern& P = table[c.pattern];
+                bool alive = true;
+                while (alive && c.matched < count_ && c.matched < P.len) {
+                    alive = match_call(P, c.matched, q_[c.matched], c.m);
+                    if (alive) ++c.matched;
+                }
+                if (!alive) continue;
+                if (kept != k) cands_[kept] = c;
+                ++kept;
+            }
+            ncands_ = kept;
+        }
+        judged_ = count_;
     }
 
     int settle(Sink& sink) {
         int st = 0;
+        const Pattern* table = patterns();
         while (count_ > 0) {
+            update_candidates();
             bool partial = false, emitted = false;
-            for (int k = 0; k < P_COUNT && !emitted; ++k) {
-                const Pattern& P = patterns()[k];
-                Match m;
-                const int got = match_prefix(P, q_, count_, m);
-                if (got < 0) continue;
-                if (got < P.len) { partial = true; continue; }
-                if (!fusable(P, m, q_)) continue;
+            for (int k = 0; k < ncands_ && !emitted; ++k) {
+                Candidate& c = cands_[k];
+                const Pattern& P = table[c.pattern];
+                if (c.matched < P.len) { partial = true; continue; }
+                if (!fusable(P, c.m, q_)) { c.matched = -1; continue; }
                 if (P.ntemps > 0) {
-                    if (count_ != P.len) continue;       // calls follow: the temporaries are still alive
-                    pending_ = k;
-                    pending_match_ = m;
+                    if (count_ != P.len) { c.matched = -1; continue; }     // calls follow: the temporaries are still alive
+                    pending_ = c.pattern;
+                    pending_match_ = c.m;
                     dead_ = 0;
                     return st;
                 }
+                const Match m = c.m;      // emit_fused drops the candidates
                 const int s = emit_fused(P, m, sink);
                 if (st == 0) st = s;
                 emitted = true;
             }
             if (emitted) continue;
-            if (partial) return st;
+            if (partial) {
+                // complete candidates that cannot be fused are done with
+                int kept = 0;
+                for (int k = 0; k < ncands_; ++k)
+                    if (cands_[k].matched >= 0 && cands_[k].matched < table[cands_[k].pattern].len) {
+                        if (kept != k) cands_[kept] = cands_[k];
+                        ++kept;
+                    }
+                ncands_ = kept;
+                return st;
+            }
             const int s = sink.primitive(q_[0]);
             ++stats_.unfused;
             if (st == 0) st = s;
@@ -584,6 +646,9 @@ private:
 
     Rec q_[kQueue];
     int count_ = 0;
+    Candidate cands_[P_COUNT];
+    int ncands_ = 0;
+    int judged_ = 0;           // held calls that the candidates have been compared with (0: candidates not built)
     int pending_ = -1;         // pattern that is complete and waits for its temporaries to be freed
     Match pending_match_;
     unsigned dead_ = 0;

@@ -293,10 +293,23 @@ class Lstm(Layer):
 
         R_all = self._stacked_recurrent(Rz, Ri, Rf, Ro)
         if (R_all is not None and self.fused in ("sequence", "thin") and hasattr(_h, "lstm_forward_sequence")
-                and Za.shape[0] == time_size + 1
-                and _h.lstm_forward_sequence(self.activation, R_all, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y,
-                                             pi, pf, po, bz, bi, bf, bo)):
-            return
+                and Za.shape[0] == time_size + 1):
+            try:
+                if _h.lstm_forward_sequence(self.activation, R_all, Za, Zb, Ia, Ib, Fa, Fb, Oa, Ob, Ca, Cb, y,
+                                            pi, pf, po, bz, bi, bf, bo):
+                    return
+            except RuntimeError as err:
+                # the workgroups did not meet at a time step's barrier within the kernel's bound (other work
+                # kept some of them off the device): every workgroup has left, the buffers hold an unfinished
+                # pass. The kernel accumulates in place, so the input products are formed again, then the
+                # step-by-step path below runs the recurrence.
+                if getattr(err, "status", None) != getattr(_h, "ERR_TIMEOUT", None):
+                    raise
+                self.sequence_fallbacks = getattr(self, "sequence_fallbacks", 0) + 1
+                _h.dot_mm(flat_x, Wz, flatten_time(Za[:-1]), transb=True)
+                _h.dot_mm(flat_x, Wi, flatten_time(Ia[:-1]), transb=True)
+                _h.dot_mm(flat_x, Wf, flatten_time(Fa[:-1]), transb=True)
+                _h.dot_mm(flat_x, Wo, flatten_time(Oa[:-1]), transb=True)
         if R_all is not None:
             rec = _h.allocate((x.shape[1], 4 * n))
             for t in range(time_size):

@@ -1,11 +1,13 @@
 """Runs training steps of one network workload on HipHandler: the program to put under a profiler.
 
-    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded]
+    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded] [window_off]
 
-``fused`` is passed to the workload's builder ("0" for single handler operations, "1" for the fused
-entry points; for the LSTM "packed" (stacked recurrent product), "thin" (packed, backward product
-through the thin-operand kernel) or "sequence" (packed, forward recurrence in one launch)). With a fourth argument "recorded"
-the step is recorded after one ordinary step and replayed. One step = forward + backward + momentum
+``fused`` is passed to the workload's builder: "0" for the reference layers' primitive call sequences
+(what an unchanged caller issues), "1" for a handler-aware caller that asks for the fused entry points;
+for the LSTM "packed" (stacked recurrent product), "thin" (packed, backward product through the
+thin-operand kernel) or "sequence" (packed, forward recurrence in one launch). With "recorded" the step
+is recorded after one ordinary step and replayed. With "window_off" the handler's fusing window is
+switched off, so that primitive calls are launched one by one. One step = forward + backward + momentum
 update.
 """
 import sys
@@ -20,10 +22,10 @@ def main(argv):
     steps = int(argv[2]) if len(argv) > 2 else 3
     fused = argv[3] if len(argv) > 3 else ""
     kw = {}
-    recorded = len(argv) > 4 and argv[4] == "recorded"
+    recorded = "recorded" in argv[4:]
     if fused and fused != "0":
         kw["fused"] = fused if fused in ("packed", "thin", "sequence") else True
-    handler = HipHandler(seed=0)
+    handler = HipHandler(seed=0, fusing="window_off" not in argv[4:])
     net, data = getattr(configs, "build_" + name)(handler, **kw)
     net.provide_external_data(data)
     stepper = MomentumStepper(0.1, 0.9, fused=bool(kw.get("fused")))

@@ -197,6 +197,7 @@ class HipHandler(Handler):
     __undescribed__ = {'context', 'dtype', 'EMPTY', 'rnd'}
 
     array_type = DeviceArray
+    ERR_TIMEOUT = _lib.ERR_TIMEOUT      # status of the BshipError that lstm_forward_sequence raises when a barrier ran out
 
     def __init__(self, seed=None, device=0, pitched_views=False, fast_masks=False, fusing=True):
         # fusing: the library's fusing window. brainstorm's layers issue primitive operations only; with

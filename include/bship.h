@@ -397,8 +397,9 @@ int bship_avgpool_bwd_nhwc_f32(const float* out_deltas, float* in_deltas,
  * are adjacent in the layer's parameter vector). The recurrent weights stay in LDS for the whole
  * sequence, one workgroup per 4 hidden units on a compute unit of its own (a batch above 64 rows
  * is two row sets of four wavefronts each in the same workgroup), and the workgroups meet at one
- * grid barrier per time step whose wait is bounded (BSHIP_GRID_BARRIER_SPINS polls, default 2^21):
- * if it runs out, e.g. because other work kept some workgroups off the device, every workgroup
+ * grid barrier per time step whose wait is bounded (BSHIP_GRID_BARRIER_SPINS polls, default 2^21;
+ * a value that is not a whole number is ignored, and 0 is kept as the test hook that makes every
+ * barrier fail at once): if it runs out, e.g. because other work kept some workgroups off the device, every workgroup
  * exits, the call returns BSHIP_ERR_TIMEOUT and the buffers hold an unfinished pass. Needs
  * n % 4 == 0, batch <= 128, n <= 1024 and n / 4 workgroups resident together (one per compute
  * unit); otherwise BSHIP_ERR_UNSUPPORTED before anything is launched.

@@ -195,3 +195,53 @@ def test_barrier_timeout_is_reported_and_the_device_stays_usable():
     assert res.returncode == 0, res.stderr
     assert "STATUS %d" % ERR_TIMEOUT in res.stdout, res.stdout + res.stderr
     assert "AFTER 30.0" in res.stdout, res.stdout
+
+
+_FALLBACK_SCRIPT = r"""
+import sys
+import numpy as np
+sys.path.insert(0, %r)
+from brainstorm_amd import HipHandler
+from brainstorm_amd.drivers import configs
+from oracle.numpy_ref_handler import NumpyRefHandler
+shape = dict(time_steps=6, batch=20, symbols=9, hidden=64)
+h = HipHandler(seed=0)
+net, data = configs.build_lstm(h, fused="sequence", **shape)
+net.provide_external_data(data)
+net.forward_pass(training_pass=True)
+net.backward_pass()
+print("FALLBACKS", net.layers["lstm"].sequence_fallbacks)
+ref, _ = configs.build_lstm(NumpyRefHandler(np.float32, seed=0), **shape)
+ref.provide_external_data(data)
+ref.forward_pass(training_pass=True)
+ref.backward_pass()
+worst = 0.0
+for group, key in (("outputs", "default"), ("internals", "Ca"), ("internals", "Ob"), ("internals", "dZa")):
+    got, want = net.get("lstm", group, key), ref.get("lstm", group, key)
+    worst = max(worst, float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-30)))
+got, want = h.get_numpy_copy(net.gradients), ref.gradients
+worst = max(worst, float(np.max(np.abs(got - want)) / np.max(np.abs(want))))
+print("WORST %%.3e" %% worst)
+"""
+
+
+def test_the_layer_takes_the_step_loop_when_the_sequence_kernel_times_out():
+    # every barrier of the sequence kernel fails at once (spin limit 0, forced from the host; the kernel exits
+    # normally): the layer forms the input products again and runs the recurrence step by step
+    env = dict(os.environ, BSHIP_GRID_BARRIER_SPINS="0")
+    res = subprocess.run([sys.executable, "-c", _FALLBACK_SCRIPT % REPO], env=env, capture_output=True, text=True,
+                         timeout=110)
+    assert res.returncode == 0, res.stderr
+    assert "FALLBACKS 1" in res.stdout, res.stdout + res.stderr
+    worst = float(res.stdout.split("WORST")[1].split()[0])
+    assert worst <= 1e-5, res.stdout
+
+
+def test_unparsable_spin_limits_are_ignored():
+    # "abc" or "12x" must not become a spin limit of 0 (which fails every barrier)
+    for value in ("abc", "12x", "-3", ""):
+        env = dict(os.environ, BSHIP_GRID_BARRIER_SPINS=value)
+        res = subprocess.run([sys.executable, "-c", _TIMEOUT_SCRIPT % REPO], env=env, capture_output=True, text=True,
+                             timeout=110)
+        assert res.returncode == 0, res.stderr
+        assert "NO ERROR" in res.stdout, (value, res.stdout + res.stderr)
