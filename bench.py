@@ -384,6 +384,9 @@ def run_nets_gpu(hip):
         mlp + "_fused_recorded_fast_masks": time_net_fast_masks(configs.build_mlp, 600, 20),
         lstm: time_net(hip, configs.build_lstm, 5, 2, sync, fusing=True),
         lstm + "_window_off": time_net(hip, configs.build_lstm, 5, 2, sync, fusing=False),
+        # the same unchanged caller with the window also stacking the four recurrent products of a time step
+        # into one (HipHandler(fusing="stacked")): another summation order inside the products, not the same bits
+        lstm + "_window_stacked": time_net(hip, configs.build_lstm, 5, 2, sync, fusing="stacked"),
         # the ~4000 launches of a step (window off) recorded into a HIP graph and replayed
         lstm + "_window_off_recorded": time_net(hip, configs.build_lstm, 5, 2, sync, recorded=True, fusing=False),
         # the elementwise part of each time step in one launch, asked for by the layer
@@ -409,7 +412,7 @@ def run_nets_gpu(hip):
     # a timing of a broken path must fail: same-bits variants share their last loss, the others are close to it
     same_bits(nets, [mlp, mlp + "_window_off", mlp + "_fused", mlp + "_recorded", mlp + "_fused_recorded"])
     same_bits(nets, [lstm, lstm + "_window_off", lstm + "_window_off_recorded", lstm + "_fused_steps"])
-    for variant in ("_fused_packed", "_fused_thin", "_fused_sequence"):      # other summation orders in the products
+    for variant in ("_window_stacked", "_fused_packed", "_fused_thin", "_fused_sequence"):      # other summation orders in the products
         close_to(nets, lstm + variant, lstm, 1e-4)
     same_bits(nets, [cnn, cnn + "_window_off", cnn + "_recorded", cnn + "_fused", cnn + "_fused_recorded"])
     same_bits(nets, [hw, hw + "_window_off", hw + "_fused"])

@@ -71,10 +71,11 @@ extern std::atomic<int> g_deferred_fill_count;   // read without the list's lock
 // while window_takes(); every other entry point first enqueues what is held (BSHIP_REQUIRE_INIT),
 // so the order of effects stays the order of the calls. While the window itself enqueues kernels
 // through the public entry points, t_window_emitting keeps them from coming back to it.
-extern std::atomic<int> g_window_on;       // bship_fusing_set
+extern std::atomic<int> g_window_on;       // bship_fusing_set: 0 off, 1 on (same bits), 2 products of an LSTM step stacked as well
 extern std::atomic<int> g_window_held;     // operations held right now
 extern thread_local bool t_window_emitting;
 int window_flush();
+void window_other_work();
 static inline bool window_takes() {
     return g_window_on.load(std::memory_order_relaxed) != 0 && !t_window_emitting;
 }
@@ -101,6 +102,9 @@ struct WindowBypass {
 // still go first.
 #define BSHIP_FLUSH_PENDING()                                                    \
     do {                                                                         \
+        if (::bship::g_window_on.load(std::memory_order_relaxed) == 2 &&         \
+            !::bship::t_window_emitting)                                         \
+            ::bship::window_other_work();                                        \
         if (::bship::g_window_held.load(std::memory_order_relaxed) != 0 &&       \
             !::bship::t_window_emitting) {                                       \
             int flush_st_ = ::bship::window_flush();                             \

@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kBlock) void lstm_bwd_step_kernel(LstmBwdArgs a, in
     if (e >= total) return;
     const unsigned j = static_cast<unsigned>(e % n);
     float dy = ldg(a.dy + e);
-    if (PACKED) {
+    if (PACKED && a.deltas != nullptr) {     // without deltas, dy is complete already and only the packed copy is added
         dy = ldg(a.deltas + e) + dy;
         a.dy_out[e] = dy;
     }
@@ -600,7 +600,7 @@ int lstm_bwd_launch(const char* fn, bool packed, int act, int64_t batch, int64_t
                     const LstmBwdArgs& a) {
     const void* ptrs[] = {a.dy, a.Zb, a.Ib, a.Fb, a.Ob, a.Cb, a.Ca_prev, a.Fb_next, a.dIa_next,
                           a.dFa_next, a.dCa_next, a.dZa, a.dZb, a.dIa, a.dIb, a.dFa, a.dFb, a.dOa,
-                          a.dOb, a.dCa, a.dCb, a.pi, a.pf, a.po, a.deltas, a.packed_out};
+                          a.dOb, a.dCa, a.dCb, a.pi, a.pf, a.po, a.deltas ? a.deltas : a.dy, a.packed_out};
     int st = check_step_args(fn, act, batch, n, ptrs, packed ? 26 : 24);
     const int64_t total = batch * n;
     if (st != 0 || total == 0) return st;

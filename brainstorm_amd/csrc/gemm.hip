@@ -254,6 +254,8 @@ extern "C" int bship_gemm_f32(int transa, int transb, int64_t M, int64_t N, int6
     BSHIP_REQUIRE_PTR(B);
     BSHIP_REQUIRE_DIM(lda >= (transa ? M : K));
     BSHIP_REQUIRE_DIM(ldb >= (transb ? K : N));
+    if (g_window_on.load(std::memory_order_relaxed) == 2 && window_takes())      // mode "stacked": products are held too
+        return window_push(window::rec_gemm(transa != 0, transb != 0, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc));
     if (g_window_held.load(std::memory_order_relaxed) != 0 && !t_window_emitting) {
         // A layer's products lie between its elementwise calls (lstm_layer.py:121-145). The product goes
         // ahead of the operations the fusing window holds when it shares no operand with them that either

@@ -461,11 +461,15 @@ int bship_d2h(void* dst_host, const void* src, size_t nbytes) {
 }
 
 int bship_d2d(void* dst, const void* src, size_t nbytes) {
-    BSHIP_REQUIRE_INIT();
+    BSHIP_REQUIRE_INIT_NO_FLUSH();
     if (nbytes == 0 || dst == src) return 0;
     BSHIP_REQUIRE_PTR(dst);
     BSHIP_REQUIRE_PTR(src);
     uintptr_t bits = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | nbytes;
+    // a copy opens an LSTM layer's backward time step (lstm_layer.py:175): held in mode "stacked"
+    if ((bits & 3u) == 0 && g_window_on.load(std::memory_order_relaxed) == 2 && window_takes())
+        return window_push(window::rec_copy(src, dst, nbytes / 4));
+    BSHIP_FLUSH_PENDING();
     if (bits & 3u) {  // not float-granular: let the runtime copy bytes
         BSHIP_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, ctx().stream));
         return 0;

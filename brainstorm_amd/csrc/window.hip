@@ -40,6 +40,13 @@ int window_push(const window::Rec& r) {
     return st;
 }
 
+void window_other_work() {
+    // an entry point that does not go through the window is about to enqueue something: it may write the arrays
+    // that the packed copy of the last backward step's gate deltas mirrors (mode "stacked")
+    std::lock_guard<std::mutex> lock(g_window_mutex);
+    window::packed_deltas().forget();
+}
+
 int window_flush() {
     std::lock_guard<std::mutex> lock(g_window_mutex);
     Emitting guard;
@@ -80,9 +87,13 @@ using namespace bship;
 
 extern "C" {
 
-int bship_fusing_set(int on) {
+int bship_fusing_set(int mode) {
     BSHIP_REQUIRE_INIT();          // what is held is enqueued before the mode changes
-    g_window_on.store(on ? 1 : 0, std::memory_order_relaxed);
+    BSHIP_REQUIRE_DIM(mode >= 0 && mode <= 2);
+    std::lock_guard<std::mutex> lock(g_window_mutex);
+    g_matcher.set_stacked(mode == 2);
+    if (mode != 2) window::packed_deltas().release();
+    g_window_on.store(mode, std::memory_order_relaxed);
     return 0;
 }
 

@@ -47,10 +47,12 @@ enum Kind : uint8_t {
     K_INDEX,        // p0 = m, p1 = v, p2 = out; M, N (= K columns)
     K_BINARIZE,     // p0 = v, p1 = out; M, N (= K columns)
     K_MASK,         // p0 = mask; d = probability; gen = generator; flags F_FAST
+    K_GEMM,         // p0 = A, p1 = B, p2 = C; flags F_TRANSA, F_TRANSB; M, N, K, ld[]; s0 = alpha, s1 = beta
+    K_COPY,         // p0 = source, p1 = destination; n elements
     K_KINDS
 };
 
-enum : uint8_t { F_COL = 1, F_ACC = 2, F_FAST = 1 };
+enum : uint8_t { F_COL = 1, F_ACC = 2, F_FAST = 1, F_TRANSA = 1, F_TRANSB = 2 };
 
 // operation codes of include/bship.h that the patterns name
 enum { OP_ADD = 0, OP_SUB = 1, OP_MUL = 2, OP_DIV = 3 };
@@ -72,6 +74,7 @@ struct Rec {
     size_t len[kMaxPtrs] = {0, 0, 0};  // bytes
     size_t n = 0;                      // elements of the elementwise kinds
     int64_t M = 0, N = 0;              // rows and columns of the matrix kinds
+    int64_t K = 0, ld[kMaxPtrs] = {0, 0, 0};   // matrix products: inner dimension, row pitches of A, B, C
     float s0 = 0.0f, s1 = 0.0f;
     double d = 0.0;
     int gen = 0;
@@ -155,11 +158,32 @@ inline Rec rec_mask(void* mask, size_t n, double p, int gen, bool fast) {
     return r;
 }
 
+inline Rec rec_gemm(bool transa, bool transb, int64_t M, int64_t N, int64_t K, float alpha, const void* A, int64_t lda,
+                    const void* B, int64_t ldb, float beta, void* C, int64_t ldc) {
+    Rec r; r.kind = K_GEMM; r.M = M; r.N = N; r.K = K; r.n = size_t(M) * size_t(N); r.s0 = alpha; r.s1 = beta;
+    r.flags = uint8_t((transa ? F_TRANSA : 0) | (transb ? F_TRANSB : 0));
+    r.ld[0] = lda; r.ld[1] = ldb; r.ld[2] = ldc;
+    const int64_t a_rows = transa ? K : M, a_cols = transa ? M : K, b_rows = transb ? N : K, b_cols = transb ? K : N;
+    set_ptr(r, 0, A, size_t((a_rows - 1) * lda + a_cols) * 4, true, false);
+    set_ptr(r, 1, B, size_t((b_rows - 1) * ldb + b_cols) * 4, true, false);
+    set_ptr(r, 2, C, size_t((M - 1) * ldc + N) * 4, beta != 0.0f, true);
+    return r;
+}
+inline Rec rec_copy(const void* src, void* dst, size_t n) {
+    Rec r; r.kind = K_COPY; r.n = n;
+    set_ptr(r, 0, src, n * 4, true, false); set_ptr(r, 1, dst, n * 4, false, true);
+    return r;
+}
+
 // ------------------------------------------------------------------ patterns
 enum PatternId {
     P_LSTM_FWD, P_LSTM_BWD, P_BIAS_ACT, P_DROPOUT, P_SOFTMAX_CE_FWD, P_SOFTMAX_CE_BWD, P_MOMENTUM,
-    P_HIGHWAY_FWD, P_HIGHWAY_BWD, P_BN_FWD, P_BN_INFER, P_BN_BWD, P_COUNT
+    P_HIGHWAY_FWD, P_HIGHWAY_BWD, P_BN_FWD, P_BN_INFER, P_BN_BWD,
+    // with matrix products held as well (mode "stacked"): a whole LSTM time step including its four
+    // recurrent products, which then run as one product over the stacked matrices
+    P_LSTM_FWD_STACKED, P_LSTM_BWD_STACKED, P_COUNT
 };
+constexpr int kPlainPatterns = P_LSTM_FWD_STACKED;     // the patterns of the same-bits mode come first
 
 enum : int8_t { OP_ANY_ACT = -2, OP_ANY_ACT_DERIV = -3 };   // an activation; the same one throughout a pattern
 enum Size : uint8_t { S_MN, S_M, S_N };                       // elements of an elementwise call: M*N, M or N
@@ -174,8 +198,8 @@ struct Elem {
     uint8_t check;
 };
 
-constexpr int kMaxVars = 24;
-constexpr int kMaxElems = 16;
+constexpr int kMaxVars = 32;
+constexpr int kMaxElems = 20;
 
 struct Pattern {
     int id;
@@ -323,6 +347,53 @@ inline const Pattern* patterns() {
           W_E(K_MV, OP_MUL, 0, 2, 3, 2, S_MN, C_NONE),
           W_E(K_BINARY, OP_ADD, 0, 2, 8, 8, S_MN, C_NONE)},
          2, {2, 3}, {-1, -1}},
+        // lstm_layer.py:121-145 with its four dot_add_mm(y[t-1], R*, *a[t], transb=True).
+        // operands 0-18 as in lstm_forward_step; yprev19 Rz20 Ri21 Rf22 Ro23
+        {P_LSTM_FWD_STACKED, "lstm_forward_step_with_products", 19,
+         {W_E(K_GEMM, 0, F_TRANSB, 19, 20, 0, S_MN, C_NONE),
+          W_E(K_MV, OP_ADD, 0, 0, 15, 0, S_MN, C_NONE),
+          W_E(K_UNARY, OP_ANY_ACT, 0, 0, 1, -1, S_MN, C_NONE),
+          W_E(K_GEMM, 0, F_TRANSB, 19, 21, 2, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 10, 12, 2, S_MN, C_NONE),
+          W_E(K_MV, OP_ADD, 0, 2, 16, 2, S_MN, C_NONE),
+          W_E(K_UNARY, OP_SIGMOID, 0, 2, 3, -1, S_MN, C_NONE),
+          W_E(K_GEMM, 0, F_TRANSB, 19, 22, 4, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 10, 13, 4, S_MN, C_NONE),
+          W_E(K_MV, OP_ADD, 0, 4, 17, 4, S_MN, C_NONE),
+          W_E(K_UNARY, OP_SIGMOID, 0, 4, 5, -1, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 3, 1, 8, S_MN, C_NONE),
+          W_E(K_MULT_ADD_TT, 0, 0, 5, 10, 8, S_MN, C_NONE),
+          W_E(K_GEMM, 0, F_TRANSB, 19, 23, 6, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 8, 14, 6, S_MN, C_NONE),
+          W_E(K_MV, OP_ADD, 0, 6, 18, 6, S_MN, C_NONE),
+          W_E(K_UNARY, OP_SIGMOID, 0, 6, 7, -1, S_MN, C_NONE),
+          W_E(K_UNARY, OP_ANY_ACT, 0, 8, 9, -1, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 7, 9, 11, S_MN, C_NONE)},
+         0, {-1, -1}, {-1, -1}},
+        // lstm_layer.py:173-205: copy_to(deltas[t], dy[t]), the four dot_add_mm into dy[t], the elementwise part.
+        // operands 0-23 as in lstm_backward_step; deltas24 Ri25 Rf26 Ro27 Rz28 dOan29 dZan30
+        {P_LSTM_BWD_STACKED, "lstm_backward_step_with_products", 20,
+         {W_E(K_COPY, 0, 0, 24, 0, -1, S_MN, C_NONE),
+          W_E(K_GEMM, 0, 0, 8, 25, 0, S_MN, C_NONE),
+          W_E(K_GEMM, 0, 0, 9, 26, 0, S_MN, C_NONE),
+          W_E(K_GEMM, 0, 0, 29, 27, 0, S_MN, C_NONE),
+          W_E(K_GEMM, 0, 0, 30, 28, 0, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 8, 21, 19, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 9, 22, 19, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 0, 5, 18, S_MN, C_NONE),
+          W_E(K_DERIV, OP_SIGMOID_DERIV, 0, 4, 18, 17, S_MN, C_NONE),
+          W_E(K_MV, OP_MUL, F_ACC, 17, 23, 19, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 0, 4, 20, S_MN, C_NONE),
+          W_E(K_DERIV, OP_ANY_ACT_DERIV, 0, 5, 20, 20, S_MN, C_NONE),
+          W_E(K_BINARY, OP_ADD, 0, 19, 20, 19, S_MN, C_NONE),
+          W_E(K_MULT_ADD_TT, 0, 0, 10, 7, 19, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 19, 6, 16, S_MN, C_NONE),
+          W_E(K_DERIV, OP_SIGMOID_DERIV, 0, 3, 16, 15, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 19, 1, 14, S_MN, C_NONE),
+          W_E(K_DERIV, OP_SIGMOID_DERIV, 0, 2, 14, 13, S_MN, C_NONE),
+          W_E(K_BINARY, OP_MUL, 0, 19, 2, 12, S_MN, C_NONE),
+          W_E(K_DERIV, OP_ANY_ACT_DERIV, 0, 1, 12, 11, S_MN, C_NONE)},
+         0, {-1, -1}, {-1, -1}},
     };
     return table;
 }
@@ -360,7 +431,7 @@ inline int act_of_deriv(int op) {
 }
 
 inline bool has_shape(uint8_t kind) {
-    return kind == K_MV || kind == K_SUM || kind == K_SOFTMAX || kind == K_INDEX || kind == K_BINARIZE;
+    return kind == K_MV || kind == K_SUM || kind == K_SOFTMAX || kind == K_INDEX || kind == K_BINARIZE || kind == K_GEMM;
 }
 
 inline bool ranges_overlap(const char* a, size_t alen, const char* b, size_t blen) {
@@ -378,10 +449,14 @@ inline bool match_call(const Pattern& P, int i, const Rec& r, Match& m) {
         if (m.act < 0) m.act = a;
         else if (m.act != a) return false;
     } else if (e.kind != K_MASK && e.kind != K_FILL && e.kind != K_CLIP && e.kind != K_MULT_ADD_TT &&
-               e.kind != K_SOFTMAX && e.kind != K_INDEX && e.kind != K_BINARIZE) {
+               e.kind != K_SOFTMAX && e.kind != K_INDEX && e.kind != K_BINARIZE && e.kind != K_GEMM && e.kind != K_COPY) {
         if (r.op != e.op) return false;
     }
-    if (e.kind == K_MV && r.flags != e.flags) return false;
+    if ((e.kind == K_MV || e.kind == K_GEMM) && r.flags != e.flags) return false;
+    if (e.kind == K_GEMM) {
+        // a recurrent product of an LSTM layer: square weights, dense operands, accumulated into its result
+        if (r.s0 != 1.0f || r.s1 != 1.0f || r.K != r.N || r.ld[0] != r.K || r.ld[1] != r.K || r.ld[2] != r.N) return false;
+    }
     switch (e.check) {
         case C_ONE: if (r.s0 != 1.0f) return false; break;
         case C_MINUS_ONE: if (r.s0 != -1.0f) return false; break;
@@ -451,7 +526,7 @@ inline bool fusable(const Pattern& P, const Match& m, const Rec* q) {
     switch (P.id) {
         case P_BN_BWD: return q[3].s0 == q[7].s0 && m.M >= 1;     // one 1/m for both statistics
         case P_BN_FWD: return m.M >= 1;
-        case P_LSTM_FWD: case P_LSTM_BWD: return m.N <= 0x3fffffff;
+        case P_LSTM_FWD: case P_LSTM_BWD: case P_LSTM_FWD_STACKED: case P_LSTM_BWD_STACKED: return m.N <= 0x3fffffff;
         default: return true;
     }
 }
@@ -477,6 +552,9 @@ constexpr int kQueue = 32;
 class Matcher {
 public:
     int held() const { return count_; }
+    // With `stacked`, the patterns that hold matrix products are in play as well (the caller then hands
+    // products and copies to push() instead of letting them pass).
+    void set_stacked(bool on) { npatterns_ = on ? int(P_COUNT) : int(kPlainPatterns); }
     const Stats& stats() const { return stats_; }
     void reset_stats() { stats_ = Stats(); }
 
@@ -572,7 +650,7 @@ private:
         const Pattern* table = patterns();
         if (judged_ == 0) {
             ncands_ = 0;
-            for (int k = 0; k < P_COUNT; ++k) {
+            for (int k = 0; k < npatterns_; ++k) {
                 const Pattern& P = table[k];
                 if (P.e[0].kind != q_[0].kind) continue;      // most sequences open with another kind of call
                 Candidate& c = cands_[ncands_];
@@ -648,6 +726,7 @@ private:
     int count_ = 0;
     Candidate cands_[P_COUNT];
     int ncands_ = 0;
+    int npatterns_ = kPlainPatterns;
     int judged_ = 0;           // held calls that the candidates have been compared with (0: candidates not built)
     int pending_ = -1;         // pattern that is complete and waits for its temporaries to be freed
     Match pending_match_;

@@ -204,8 +204,11 @@ class HipHandler(Handler):
         # the window on, the library recognises the layers' call sequences (an LSTM time step, a batch
         # normalisation pass, bias + activation, dropout, softmax cross entropy, Highway, the momentum
         # update) and runs each as one fused kernel with the same float32 operations in the same order,
-        # so results are the same bits as with fusing=False. The switch is the library's: it holds for
-        # every handler of the process (the last handler created decides).
+        # so results are the same bits as with fusing=False. fusing="stacked" additionally runs the four
+        # recurrent matrix products of an LSTM time step as one product over the stacked weight matrices
+        # (adjacent in brainstorm's parameter vector): faster, and equal to the other modes up to the order in
+        # which a matrix product sums (about 1e-6 relative), not bit for bit. The switch is the library's: it
+        # holds for every handler of the process (the last handler created, or set_fusing, decides).
         # fast_masks: dropout masks from a counter-based generator (Philox4x32-10) instead of
         # NumPy's MT19937 stream. One parallel launch per mask instead of a sequential walk, but
         # NOT the masks NumpyHandler draws for the same seed (the reference's own GPU handler does
@@ -235,8 +238,7 @@ class HipHandler(Handler):
         self._free = self._lib.bship_free
         self.EMPTY = DeviceArray(0, (0,), None, self)
         self.fast_masks = bool(fast_masks)
-        self.fusing = bool(fusing)
-        self._call(self._lib.bship_fusing_set(int(self.fusing)))
+        self.set_fusing(fusing)
         self.rnd = HipRandomState(self, seed)
 
     def __describe__(self):
@@ -249,7 +251,7 @@ class HipHandler(Handler):
         self.__init__(device=int(description.get('device', 0)),
                       pitched_views=bool(description.get('pitched_views', False)),
                       fast_masks=bool(description.get('fast_masks', False)),
-                      fusing=bool(description.get('fusing', True)))
+                      fusing=description.get('fusing', True))
 
     # ------------------------------------------------------------- plumbing
     # parameters an operation writes (everything else is only read); operations that are not
@@ -554,10 +556,13 @@ class HipHandler(Handler):
         """Waits until every operation issued so far has finished."""
         self._call(self._lib.bship_sync())
 
-    def set_fusing(self, on):
-        """Switches the library's fusing window on or off (what it holds is enqueued first)."""
-        self.fusing = bool(on)
-        self._call(self._lib.bship_fusing_set(int(self.fusing)))
+    def set_fusing(self, mode):
+        """Switches the library's fusing window: False, True (same bits as False) or "stacked" (see the
+        constructor). What the window holds is enqueued first."""
+        if mode not in (True, False, "stacked"):
+            raise ValueError('fusing must be True, False or "stacked", not %r' % (mode,))
+        self._call(self._lib.bship_fusing_set(2 if mode == "stacked" else int(mode)))
+        self.fusing = mode
 
     def fusing_stats(self, reset=False):
         """Counters of the fusing window since the last reset: operations that entered it, operations

@@ -528,6 +528,8 @@ int bship_lstm_bwd_step_f32(int act, int64_t batch, int64_t n, const float* dy,
  *  - backward: dy holds packed[t+1] [Rz;Ri;Rf;Ro] on entry and receives
  *    deltas + that (lstm_layer.py 181-185); packed_out (batch, 4n) receives
  *    [dZa|dIa|dFa|dOa] of this step, the left operand of the next product.
+ *    deltas may be NULL: dy is then complete on entry (bship_lstm_bwd_step_f32's
+ *    meaning) and the call only adds the packed copy of the step's gate deltas.
  * The elementwise arithmetic is the same; the matrix products sum in another
  * order than four separate ones, so results agree to rounding, not bit for bit. */
 int bship_lstm_fwd_step_packed_f32(int act, int64_t batch, int64_t n,
@@ -651,8 +653,16 @@ int bship_batchnorm_bwd_f32(const float* out_deltas, const float* x_hat,
  * Matrix products are never held; they overtake held calls that share no operand with them which
  * either side writes. Every other entry point (copies to the host, bship_sync, allocation,
  * recording, ...) first enqueues what is held. Errors of a held call are reported by the call that
- * causes it to be enqueued. The switch belongs to the library, not to a handler object. */
-int bship_fusing_set(int on);
+ * causes it to be enqueued. The switch belongs to the library, not to a handler object.
+ * mode 0: off. mode 1: as described (same bits as mode 0). mode 2 ("stacked") additionally holds
+ * the matrix products and copies of an LSTM time step (lstm_layer.py:117-145, 173-205): the four
+ * recurrent products of a step, whose weight matrices lie back to back in brainstorm's parameter
+ * vector, run as ONE product over the stacked matrix [Rz;Ri;Rf;Ro] (forward: into a scratch matrix
+ * that the step kernel adds; backward: from a packed copy of the previous step's gate deltas that
+ * the step kernel leaves behind), which is what bship_lstm_*_step_packed_f32 offer a handler-aware
+ * caller. The products then sum in another order, so results agree with modes 0 and 1 to rounding
+ * (1e-6 relative), not bit for bit. */
+int bship_fusing_set(int mode);
 int bship_fusing_get(int* on_host);
 /* Enqueues what the window holds. */
 int bship_fusing_flush(void);

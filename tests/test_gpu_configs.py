@@ -214,6 +214,39 @@ def test_lstm_full_size_forward_backward(hip):
     assert scaled_err(net_s.get("lstm", "outputs", "default"), net_r.get("lstm", "outputs", "default")) <= 1e-5
     print("lstm, whole-sequence forward kernel: worst internal %.2e" % worst_s)
 
+    def whole_pass_against_oracle(label, fused, fusing):
+        before = hip.fusing
+        hip.set_fusing(fusing)
+        try:
+            hip.rnd.seed(22)
+            net, data = configs.build_lstm(hip, fused=fused)
+            net.provide_external_data(data)
+            net.forward_pass(training_pass=True)
+            net.backward_pass()
+            loss = net.get("loss", "outputs", "loss")[0]
+            assert abs(loss - loss_r) <= 1e-5 * abs(loss_r), (label, loss, loss_r)
+            for key in ("Za", "Zb", "Ia", "Ib", "Fa", "Fb", "Oa", "Ob", "Ca", "Cb"):
+                err = scaled_err(net.get("lstm", "internals", key), net_r.get("lstm", "internals", key))
+                assert err <= 1e-5, (label, key, err)
+            g = hip.get_numpy_copy(net.gradients)
+            worst = 0.0
+            for name, (a, b, _) in net_r.parameter_slices().items():
+                err = scaled_err(g[a:b], g_r[a:b])
+                worst = max(worst, err)
+                assert err <= 1e-4, (label, name, err)
+            err = scaled_err(net.get("Input", "output_deltas", "default"), net_r.get("Input", "output_deltas", "default"))
+            assert err <= 1e-4, (label, err)
+            print("lstm, %s: worst gradient block %.2e, input deltas %.2e" % (label, worst, err))
+        finally:
+            hip.set_fusing(before)
+
+    # the layer asking for the per-step kernels itself, products as the reference issues them
+    whole_pass_against_oracle("fused time steps, four products per step", "steps", False)
+    # an unchanged caller: primitive calls only, through the fusing window ...
+    whole_pass_against_oracle("primitive calls through the fusing window", False, True)
+    # ... and with the window stacking the four recurrent products of a step into one
+    whole_pass_against_oracle("primitive calls, window stacking the recurrent products", False, "stacked")
+
 
 @pytest.mark.parametrize("fused", [False, True], ids=["primitives", "fused"])
 def test_highway_batchnorm_blocks(hip, fused):

@@ -185,3 +185,36 @@ def test_errors_of_held_calls_surface(hip):
     assert hip.fusing_stats()["calls"] >= 1
     hip.synchronize()                            # enqueues it; nothing to report
     assert np.array_equal(hip.get_numpy_copy(a), np.zeros((4, 6), F32))
+
+
+@pytest.mark.parametrize("kw", [dict(time_steps=9, batch=7, symbols=11, hidden=13),
+                                dict(time_steps=12, batch=33, symbols=50, hidden=257),
+                                dict(time_steps=6, batch=100, symbols=30, hidden=512)])
+def test_stacked_products_agree_to_rounding(hip, kw):
+    # fusing="stacked": one product over [Rz;Ri;Rf;Ro] per time step instead of four; only the order in which the
+    # products sum changes, so every buffer agrees with the window-off run to rounding
+    results = {}
+    for mode in (False, "stacked"):
+        hip.set_fusing(mode)
+        hip.rnd.seed(7)
+        net, data = configs.build_lstm(hip, **kw)
+        net.provide_external_data(data)
+        stepper = MomentumStepper(0.05, 0.9)
+        stepper.start(net)
+        hip.fusing_stats(reset=True)
+        for _ in range(2):
+            stepper.run()
+        stats = hip.fusing_stats()
+        results[mode] = ({(group, key): net.get("lstm", group, key) for group in ("outputs", "internals", "output_deltas")
+                          for key in getattr(net.buffers["lstm"], group)},
+                         hip.get_numpy_copy(net.gradients), hip.get_numpy_copy(net.parameters), stats)
+        del net, stepper
+    plain, stacked = results[False], results["stacked"]
+    T = kw["time_steps"]
+    assert stacked[3]["fused_launches"] == 2 * (2 * T + 3)
+    for key, want in plain[0].items():
+        scale = float(np.max(np.abs(want))) or 1.0
+        assert float(np.max(np.abs(stacked[0][key] - want))) <= 2e-5 * scale, key
+    for k, what in ((1, "gradients"), (2, "parameters")):
+        scale = float(np.max(np.abs(plain[k])))
+        assert float(np.max(np.abs(stacked[k] - plain[k]))) <= 2e-5 * scale, what

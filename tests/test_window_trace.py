@@ -22,7 +22,9 @@ def canonical(log, base, size):
         for tok in line.split():
             if tok.startswith("@"):
                 addr = int(tok[1:])
-                if base <= addr < base + size:
+                if addr < 0:
+                    tok = "@null"
+                elif base <= addr < base + size:
                     tok = "@net+%d" % (addr - base)
                 else:
                     tok = "@other%d" % seen.setdefault(addr, len(seen))
@@ -198,3 +200,63 @@ def test_products_that_touch_held_operands_do_not_overtake(trace):
     h.dot_add_mm(out, w, b)                      # shares nothing with the held call: goes first
     h.tanh(a, a)
     assert names(trace.trace_log().decode().splitlines()) == ["gemm", "bias_act"]
+
+
+def test_stacked_mode_runs_one_product_per_lstm_time_step(trace):
+    from brainstorm_amd.drivers import configs
+    T, B, n = 5, 3, 6
+    kw = dict(time_steps=T, batch=B, symbols=4, hidden=n)
+    plain, _, _ = run_step(trace, configs.build_lstm, fusing=True, fused=False, **kw)
+    stacked, stats, _ = run_step(trace, configs.build_lstm, fusing="stacked", fused=False, **kw)
+    got = names(stacked)
+    assert got.count("lstm_fwd_step_packed") == T and got.count("lstm_bwd_step_packed") == T
+    assert "lstm_fwd_step" not in got and "lstm_bwd_step" not in got
+    # forward: the four recurrent products of a step are one product with 4n result columns
+    fwd_products = [l.split() for l in stacked if l.startswith("gemm 0 1 %d %d %d " % (B, 4 * n, n))]
+    assert len(fwd_products) == T
+    # backward: the first step has no packed deltas to read (copy + four products), every later step one product over K = 4n
+    bwd_products = [l.split() for l in stacked if l.startswith("gemm 0 0 %d %d %d " % (B, n, 4 * n))]
+    assert len(bwd_products) == T - 1
+    assert got.count("d2d") == 1
+    # the packed copy that a backward step reads is the one the step before it wrote
+    steps = [l.split() for l in stacked if l.startswith("lstm_bwd_step_packed")]
+    assert steps[0][4] == "@null"                                # no deltas: dy was complete
+    for before, product, after in zip(steps, bwd_products, steps[1:]):
+        assert product[7] == before[6]                            # A of the product = packed_out of the step before
+        assert after[4] != "@null" and after[6] != before[6]     # deltas added by the kernel, the other buffer written
+    # everything that is not part of a time step is unchanged
+    keep = ("sum", "softmax_ce_fwd", "softmax_ce_bwd", "momentum", "fill")
+    same = lambda log: [l for l in log if l.split()[0] in keep and "@other" not in l]    # temporaries are numbered per run
+    assert same(plain) == same(stacked) and len(same(plain)) > 10
+    assert len([l for l in stacked if l.startswith("gemm")]) == len([l for l in plain if l.startswith("gemm")]) - 3 * T - 3 * (T - 1)
+
+
+def test_stacked_mode_forgets_the_packed_deltas_when_something_else_runs(trace):
+    # two backward steps with an unrelated call between them: the second one must form its four products itself
+    from brainstorm_amd import HipHandler
+    from brainstorm_amd.drivers import configs
+    h = HipHandler(seed=1, fusing="stacked")
+    net, data = configs.build_lstm(h, time_steps=3, batch=2, symbols=3, hidden=4)
+    net.provide_external_data(data)
+    net.forward_pass(training_pass=True)
+    layer, buffers = net.layers["lstm"], net.buffers["lstm"]
+
+    class Nosy(type(h)):
+        """The same handler, poking an unrelated array after every backward time step."""
+    other = h.allocate((4,))
+    calls = {"n": 0}
+    original = h.tanh_deriv
+
+    def tanh_deriv(x, y, dy, dx):
+        original(x, y, dy, dx)
+        calls["n"] += 1
+        if calls["n"] % 2 == 0:                  # the step's last call (the block input's derivative)
+            h.fill(other, 3.0)
+    h.tanh_deriv = tanh_deriv
+    h.act_func_deriv["tanh"] = tanh_deriv
+    trace.trace_reset()
+    net.backward_pass()
+    log = names(trace.trace_log().decode().splitlines())
+    assert log.count("lstm_bwd_step_packed") == 3
+    assert log.count("d2d") == 3                 # no step could use the packed copy of the one before
+    h.set_fusing(True)

@@ -24,7 +24,8 @@ uintptr_t g_next = kBase;
 std::map<uintptr_t, size_t> g_blocks;
 std::string g_log;
 char g_error[256] = "";
-bool g_on = false, g_emitting = false;
+int g_on = 0;              // bship_fusing_set: 0, 1 or 2 ("stacked")
+bool g_emitting = false;
 Matcher g_matcher;
 
 long long rel(const void* p) { return p ? static_cast<long long>(reinterpret_cast<uintptr_t>(p) - kBase) : -1; }   // printed as @<offset>
@@ -44,7 +45,11 @@ struct Emitting {
     ~Emitting() { g_emitting = false; }
 };
 
-bool takes() { return g_on && !g_emitting; }
+bool takes() { return g_on != 0 && !g_emitting; }
+
+void other_work() {       // what BSHIP_FLUSH_PENDING does in mode "stacked"
+    if (g_on == 2 && !g_emitting) packed_deltas().forget();
+}
 
 int push(const Rec& r) {
     Emitting guard;
@@ -53,6 +58,7 @@ int push(const Rec& r) {
 }
 
 int flush() {
+    other_work();
     if (g_emitting || g_matcher.held() == 0) return 0;
     Emitting guard;
     DeviceSink sink;
@@ -70,6 +76,17 @@ int set_error(int code, const char* fmt, ...) {
     return code;
 }
 int flush_deferred_fills() { return 0; }
+int pool_alloc_raw(size_t nbytes, void** out) {
+    const size_t sz = (nbytes + 255) / 256 * 256;
+    *out = reinterpret_cast<void*>(g_next);
+    g_blocks[g_next] = sz;
+    g_next += sz;
+    return 0;
+}
+int pool_free_raw(void* p) {
+    g_blocks.erase(reinterpret_cast<uintptr_t>(p));
+    return 0;
+}
 int batchnorm_fwd_train_launch(const float* inputs, const float* gamma, const float* beta, float* mu, float* sigma,
                                float* sigma_b, float* centered, float* x_hat, float* out, int64_t M, int64_t N,
                                float neg_inv_m, float decay_mu, float rest_mu, float inv_m, float eps,
@@ -143,8 +160,9 @@ int bship_d2h(void* dst, const void* src, size_t nbytes) {
     return 0;
 }
 int bship_d2d(void* dst, const void* src, size_t nbytes) {
-    flush();
     if (nbytes == 0 || dst == src) return 0;
+    if (g_on == 2 && takes() && nbytes % 4 == 0) return push(rec_copy(src, dst, nbytes / 4));
+    flush();
     logf("d2d @%lld @%lld %zu", P(dst), P(src), nbytes);
     return 0;
 }
@@ -242,6 +260,8 @@ int bship_prob_mask_fast_on_f32(int gen, float* m, size_t n, double p) { return 
 int bship_gemm_f32(int ta, int tb, int64_t M, int64_t N, int64_t K, float alpha, const float* A, int64_t lda,
                    const float* B, int64_t ldb, float beta, float* C, int64_t ldc) {
     if (M == 0 || N == 0) return 0;
+    if (g_on == 2 && takes()) return push(rec_gemm(ta != 0, tb != 0, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc));
+    other_work();
     if (g_matcher.held() != 0 && !g_emitting) {
         const int64_t ar = ta ? K : M, ac = ta ? M : K, br = tb ? N : K, bc = tb ? K : N;
         const char* rd[3] = {reinterpret_cast<const char*>(A), reinterpret_cast<const char*>(B),
@@ -285,6 +305,29 @@ int bship_lstm_bwd_step_f32(int act, int64_t batch, int64_t n, const float* dy, 
          act, (long long)batch, (long long)n, P(dy), P(Zb), P(Ib), P(Fb), P(Ob), P(Cb), P(Ca_prev), P(Fb_next),
          P(dIa_next), P(dFa_next), P(dCa_next), P(dZa), P(dZb), P(dIa), P(dIb), P(dFa), P(dFb), P(dOa), P(dOb), P(dCa),
          P(dCb), P(pi), P(pf), P(po));
+    return 0;
+}
+int bship_lstm_fwd_step_packed_f32(int act, int64_t batch, int64_t n, const float* rec, float* Za, float* Zb, float* Ia,
+                                   float* Ib, float* Fa, float* Fb, float* Oa, float* Ob, float* Ca, float* Cb,
+                                   const float* Ca_prev, float* y, const float* pi, const float* pf, const float* po,
+                                   const float* bz, const float* bi, const float* bf, const float* bo) {
+    flush();
+    logf("lstm_fwd_step_packed %d %lld %lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld",
+         act, (long long)batch, (long long)n, P(rec), P(Za), P(Zb), P(Ia), P(Ib), P(Fa), P(Fb), P(Oa), P(Ob), P(Ca), P(Cb),
+         P(Ca_prev), P(y), P(pi), P(pf), P(po), P(bz), P(bi), P(bf), P(bo));
+    return 0;
+}
+int bship_lstm_bwd_step_packed_f32(int act, int64_t batch, int64_t n, const float* deltas, float* dy, float* packed_out,
+                                   const float* Zb, const float* Ib, const float* Fb, const float* Ob, const float* Cb,
+                                   const float* Ca_prev, const float* Fb_next, const float* dIa_next,
+                                   const float* dFa_next, const float* dCa_next, float* dZa, float* dZb, float* dIa,
+                                   float* dIb, float* dFa, float* dFb, float* dOa, float* dOb, float* dCa, float* dCb,
+                                   const float* pi, const float* pf, const float* po) {
+    flush();
+    logf("lstm_bwd_step_packed %d %lld %lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld @%lld",
+         act, (long long)batch, (long long)n, P(deltas), P(dy), P(packed_out), P(Zb), P(Ib), P(Fb), P(Ob), P(Cb),
+         P(Ca_prev), P(Fb_next), P(dIa_next), P(dFa_next), P(dCa_next), P(dZa), P(dZb), P(dIa), P(dIb), P(dFa), P(dFb),
+         P(dOa), P(dOb), P(dCa), P(dCb), P(pi), P(pf), P(po));
     return 0;
 }
 int bship_bias_act_f32(int act, const float* in, const float* bias, float* out, int64_t M, int64_t N) {
@@ -403,8 +446,14 @@ int bship_rng_select(int) { return flush(); }
 int bship_rng_destroy(int) { return 0; }
 int bship_rng_seed_on(int, uint32_t) { return flush(); }
 int bship_fast_rng_seed_on(int, unsigned long long) { return flush(); }
-int bship_fusing_set(int on) { flush(); g_on = on != 0; return 0; }
-int bship_fusing_get(int* on) { *on = g_on ? 1 : 0; return 0; }
+int bship_fusing_set(int mode) {
+    flush();
+    g_on = mode;
+    g_matcher.set_stacked(mode == 2);
+    if (mode != 2) packed_deltas().release();
+    return 0;
+}
+int bship_fusing_get(int* on) { *on = g_on; return 0; }
 int bship_fusing_flush(void) { return flush(); }
 int bship_fusing_stats(unsigned long long* calls, unsigned long long* unfused, unsigned long long* fused_calls,
                        unsigned long long* fused_launches, unsigned long long* overtaken, int reset) {
