@@ -103,6 +103,8 @@ SIGNATURES = {
     "bship_fusing_stats": [POINTER(ctypes.c_ulonglong)] * 5 + [c_int],
     "bship_gemm_f32": [c_int, c_int, _I64, _I64, _I64, c_float, _P, _I64, _P, _I64, c_float, _P, _I64],
     "bship_gemm_bias_f32": [c_int, c_int, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P, _I64],
+    "bship_conv2d_fwd_thin_f32": [_P, _I64, _P, _P, _P, _I64] + [c_int] * 9,
+    "bship_conv2d_bwd_thin_f32": [_P, _I64, _P, _P, _P, _I64, _P, _P, _I64] + [c_int] * 9,
     "bship_im2col_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
     "bship_col2im_nhwc_f32": [_P, _P, _I64] + [c_int] * 8,
     "bship_maxpool_fwd_nhwc_f32": [_P, _P, _P, _I64] + [c_int] * 10,

@@ -219,6 +219,7 @@ class HipHandler(Handler):
         # check in front of every operation.
         self.pitched_views = bool(pitched_views)
         self.native_pitched = True      # False: every call on a pitched view goes through dense temporaries
+        self.thin_convolutions = True   # False: convolutions with thin filters take the im2col path like all others
         if self.pitched_views:
             self._install_pitched_wrappers()        # before the activation tables bind the methods
         super(HipHandler, self).__init__()
@@ -1021,8 +1022,17 @@ class HipHandler(Handler):
             raise _mismatch("conv2d_forward_batch", inputs, weights, bias)
         kc = kh * kw * c
         rows = n * oh * ow
-        col = self._scratch((rows, kc))       # im2col writes every element
         p_in, ld_in = self._images(inputs)
+        if self.thin_convolutions and kc <= 128 and f % 16 == 0 and f <= 64 and tuple(stride) == (1, 1) and rows:
+            # thin filters (an image network's first layer): the matrix cores read the windows out of a copy
+            # of the image rows in LDS, no col matrix
+            status = self._lib.bship_conv2d_fwd_thin_f32(p_in, ld_in, weights.ptr, bias.ptr, outputs.ptr, n, h, w, c,
+                                                         f, kh, kw, padding, 1, 1)
+            if status == 0:
+                return
+            if status != _lib.ERR_UNSUPPORTED:
+                self._call(status)
+        col = self._scratch((rows, kc))       # im2col writes every element
         self._call(self._lib.bship_im2col_nhwc_pitched_f32(p_in, ld_in, col.ptr, n, h, w, c, kh, kw,
                                                            padding, stride[0], stride[1]))
         # product and bias in one call (the bias goes into the product's epilogue)
@@ -1044,15 +1054,23 @@ class HipHandler(Handler):
             raise _mismatch("conv2d_backward_batch", inputs, weights, in_deltas, weight_deltas, bias_deltas)
         kc = kh * kw * c
         rows = n * oh * ow
-        col = self._scratch((rows, kc))       # im2col writes every element
         p_in, ld_in = self._images(inputs)
+        p_din, ld_din = self._images(in_deltas)
+        if self.thin_convolutions and kc <= 127 and f % 16 == 0 and f <= 64 and tuple(stride) == (1, 1) and rows:
+            status = self._lib.bship_conv2d_bwd_thin_f32(p_in, ld_in, weights.ptr, out_deltas.ptr, p_din, ld_din,
+                                                         weight_deltas.ptr, bias_deltas.ptr, n, h, w, c, f, kh, kw,
+                                                         padding, 1, 1)
+            if status == 0:
+                return
+            if status != _lib.ERR_UNSUPPORTED:
+                self._call(status)
+        col = self._scratch((rows, kc))       # im2col writes every element
         self._call(self._lib.bship_im2col_nhwc_pitched_f32(p_in, ld_in, col.ptr, n, h, w, c, kh, kw,
                                                            padding, stride[0], stride[1]))
         dy = out_deltas.reshape((rows, f))
         self._gemm(dy, col, weight_deltas.reshape((f, kc)), True, False, 0.0)
         self._call(self._lib.bship_sum_f32(dy.ptr, bias_deltas.ptr, rows, f, 0))
         self._gemm(dy, weights.reshape((f, kc)), col, False, False, 0.0)
-        p_din, ld_din = self._images(in_deltas)
         self._call(self._lib.bship_col2im_nhwc_pitched_f32(col.ptr, p_din, ld_din, n, h, w, c, kh, kw,
                                                            padding, stride[0], stride[1]))
 

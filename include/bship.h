@@ -355,6 +355,31 @@ int bship_gemm_bias_f32(int transa, int transb, int64_t M, int64_t N, int64_t K,
                         const float* A, int64_t lda, const float* B, int64_t ldb,
                         const float* bias, float* C, int64_t ldc);
 
+/* conv2d_forward_batch (numpy 149-171) without the col matrix, for thin filters: stride 1, any
+ * padding, kh*kw*c <= 128, f a multiple of 16 up to 64 (the first layer of an image network).
+ * in: n images of (h, w, c), in_pitch floats apart; weights (f, kh, kw, c); bias (f); out (n, out_h,
+ * out_w, f) dense. A workgroup stages the image rows of a band of output rows in LDS and the matrix
+ * cores read the filter windows out of that copy. Any other geometry: BSHIP_ERR_UNSUPPORTED with
+ * nothing launched (the caller then runs bship_im2col_nhwc_f32 + bship_gemm_bias_f32). Products sum
+ * in k order in float32: equal to the im2col path up to the summation order. */
+int bship_conv2d_fwd_thin_f32(const float* in, int64_t in_pitch, const float* weights,
+                              const float* bias, float* out, int64_t n, int h, int w, int c, int f,
+                              int kh, int kw, int pad, int stride_h, int stride_w);
+
+/* conv2d_backward_batch (numpy 110-147) without the col matrix, for the same thin filters (and
+ * kh*kw*c <= 127, a row of out_deltas times f within 4096 floats): weight_deltas (f, kh, kw, c) and
+ * bias_deltas (f) are overwritten, in_deltas (n images of (h, w, c), in_deltas_pitch floats apart)
+ * accumulated; out_deltas (n, out_h, out_w, f) dense. Three launches: the weights' and the bias's
+ * deltas as per-workgroup partial sums over bands of images (the matrix cores read the filter
+ * windows out of a copy of the image rows in LDS; the bias is a window entry that is always one),
+ * their sum in workgroup order, and the inputs' deltas (out_deltas x weights into LDS per band, every
+ * element of in_deltas adding the entries that fall on it in a fixed order: no atomics, the same
+ * bits every time). Any other geometry: BSHIP_ERR_UNSUPPORTED with nothing launched. */
+int bship_conv2d_bwd_thin_f32(const float* in, int64_t in_pitch, const float* weights,
+                              const float* out_deltas, float* in_deltas, int64_t in_deltas_pitch,
+                              float* weight_deltas, float* bias_deltas, int64_t n, int h, int w,
+                              int c, int f, int kh, int kw, int pad, int stride_h, int stride_w);
+
 /* im2col of a whole NHWC batch (_cpuop 251-277 applied per image by numpy
  * 158-166): col is (n*out_h*out_w, kh*kw*c). */
 int bship_im2col_nhwc_f32(const float* in, float* col, int64_t n, int h, int w,

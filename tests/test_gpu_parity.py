@@ -900,6 +900,104 @@ def test_conv2d_forward_backward(hip, ref):
         assert np.max(np.abs(dbd.get() - db) / (np.sqrt(n * oh * ow) + np.abs(db))) <= 1e-5
 
 
+THIN_CASES = [  # n, h, w, c, f, kh, kw, pad: stride 1, kh*kw*c <= 128, f a multiple of 16 up to 64
+    (10, 32, 32, 3, 32, 5, 5, 2), (3, 28, 28, 1, 16, 5, 5, 0), (2, 9, 7, 3, 16, 3, 3, 1), (5, 17, 13, 2, 48, 5, 3, 2),
+    (1, 5, 5, 4, 64, 5, 5, 4), (4, 6, 150, 3, 32, 3, 3, 1), (2, 40, 3, 5, 16, 5, 5, 2), (7, 8, 8, 8, 32, 4, 4, 0),
+    (300, 12, 12, 3, 32, 5, 5, 2), (2, 10, 10, 128, 16, 1, 1, 0), (3, 11, 9, 1, 32, 1, 1, 3)]
+
+
+# of these, backward keeps to the im2col path: a row of out_deltas x f beyond 4096 floats
+THIN_FORWARD_ONLY = {(4, 6, 150, 3, 32, 3, 3, 1)}
+
+
+def test_thin_filter_convolutions_forward(hip, ref):
+    # filters of at most 128 entries are convolved without a col matrix (bship_conv2d_fwd_thin_f32): against the
+    # oracle at the bar of the products, and against the im2col path of the same handler
+    rng = np.random.RandomState(261)
+    assert hip.thin_convolutions
+    for n, h, w, c, f, kh, kw, pad in THIN_CASES:
+        oh, ow = _out_size(h, kh, pad, 1), _out_size(w, kw, pad, 1)
+        x, wts, bias = rand(rng, (n, h, w, c)), rand(rng, (f, kh, kw, c)), rand(rng, (f,))
+        out = np.zeros((n, oh, ow, f), F32)
+        ref.conv2d_forward_batch(x, wts, bias, out, pad, (1, 1))
+        xd, wd, bd = hip.create_from_numpy(x), hip.create_from_numpy(wts), hip.create_from_numpy(bias)
+        outd = hip.create_from_numpy(np.full(out.shape, 7.0, F32))
+        status = hip._lib.bship_conv2d_fwd_thin_f32(xd.ptr, h * w * c, wd.ptr, bd.ptr, outd.ptr, n, h, w, c, f, kh, kw,
+                                                    pad, 1, 1)
+        assert status == 0, (n, h, w, c, f, kh, kw, pad)
+        got = outd.get()
+        scale = np.sqrt(kh * kw * c) + np.abs(out)
+        assert np.max(np.abs(got - out) / scale) <= 1e-5, ("thin conv", n, h, w, c, f, kh, kw, pad)
+        hip.thin_convolutions = False
+        try:
+            other = hip.allocate(out.shape)
+            hip.conv2d_forward_batch(xd, wd, bd, other, pad, (1, 1))
+        finally:
+            hip.thin_convolutions = True
+        assert np.max(np.abs(got - other.get()) / scale) <= 2e-6
+        hip.conv2d_forward_batch(xd, wd, bd, other, pad, (1, 1))          # and through the handler: the same kernel
+        assert_bit_equal(other.get(), got, "handler route")
+    # geometries the kernel does not take are refused with nothing done
+    lib = hip._lib
+    a = hip.allocate((2, 8, 8, 3))
+    for f, kh, kw, c, stride in ((20, 3, 3, 3, 1), (80, 3, 3, 3, 1), (16, 7, 7, 3, 1), (16, 3, 3, 3, 2)):
+        assert lib.bship_conv2d_fwd_thin_f32(a.ptr, 192, a.ptr, a.ptr, a.ptr, 2, 8, 8, c, f, kh, kw, 1, stride, stride) == -6
+
+
+def test_thin_filter_convolutions_backward(hip, ref):
+    # the same filters backward without a col matrix (bship_conv2d_bwd_thin_f32): weight and bias deltas
+    # overwritten, input deltas accumulated; against the oracle at the bar of the products, against the im2col
+    # path of the same handler, and the same bits on a second call (sums in a fixed order, no atomics)
+    rng = np.random.RandomState(262)
+    lib = hip._lib
+    for n, h, w, c, f, kh, kw, pad in THIN_CASES:
+        if kh * kw * c > 127:
+            continue
+        oh, ow = _out_size(h, kh, pad, 1), _out_size(w, kw, pad, 1)
+        x, wts, dout, din = rand(rng, (n, h, w, c)), rand(rng, (f, kh, kw, c)), rand(rng, (n, oh, ow, f)), rand(rng, (n, h, w, c))
+        want_din, dw, db = din.copy(), np.full_like(wts, 5.0), np.full((f,), 5.0, F32)
+        ref.conv2d_backward_batch(x, wts, pad, (1, 1), want_din, dout, dw, db)
+        xd, wd, doutd = hip.create_from_numpy(x), hip.create_from_numpy(wts), hip.create_from_numpy(dout)
+        results = []
+        for _ in range(2):
+            dind = hip.create_from_numpy(din)
+            dwd, dbd = hip.create_from_numpy(np.full_like(wts, 5.0)), hip.create_from_numpy(np.full((f,), 5.0, F32))
+            status = lib.bship_conv2d_bwd_thin_f32(xd.ptr, h * w * c, wd.ptr, doutd.ptr, dind.ptr, h * w * c, dwd.ptr,
+                                                   dbd.ptr, n, h, w, c, f, kh, kw, pad, 1, 1)
+            if (n, h, w, c, f, kh, kw, pad) in THIN_FORWARD_ONLY:
+                assert status == -6
+                break
+            assert status == 0, (n, h, w, c, f, kh, kw, pad, status)
+            results.append((dind.get(), dwd.get(), dbd.get()))
+        if not results:
+            continue
+        case = ("thin conv backward", n, h, w, c, f, kh, kw, pad)
+        got_din, got_dw, got_db = results[0]
+        assert np.max(np.abs(got_din - want_din) / (np.sqrt(f * kh * kw) + np.abs(want_din))) <= 1e-5, case
+        assert np.max(np.abs(got_dw - dw) / (np.sqrt(n * oh * ow) + np.abs(dw))) <= 1e-5, case
+        assert np.max(np.abs(got_db - db) / (np.sqrt(n * oh * ow) + np.abs(db))) <= 1e-5, case
+        for first, second in zip(results[0], results[1]):
+            assert_bit_equal(second, first, "second call")
+        hip.thin_convolutions = False
+        try:
+            dind = hip.create_from_numpy(din)
+            dwd, dbd = hip.allocate(wts.shape), hip.allocate((f,))
+            hip.conv2d_backward_batch(xd, wd, pad, (1, 1), dind, doutd, dwd, dbd)
+        finally:
+            hip.thin_convolutions = True
+        assert np.max(np.abs(got_din - dind.get()) / (np.sqrt(f * kh * kw) + np.abs(want_din))) <= 4e-6, case
+        assert np.max(np.abs(got_dw - dwd.get()) / (np.sqrt(n * oh * ow) + np.abs(dw))) <= 4e-6, case
+        dind = hip.create_from_numpy(din)
+        hip.conv2d_backward_batch(xd, wd, pad, (1, 1), dind, doutd, dwd, dbd)   # through the handler: the same kernels
+        assert_bit_equal(dind.get(), got_din, "handler route, input deltas")
+        assert_bit_equal(dwd.get(), got_dw, "handler route, weight deltas")
+        assert_bit_equal(dbd.get(), got_db, "handler route, bias deltas")
+    a = hip.allocate((2, 8, 8, 3))
+    for f, kh, kw, c, stride in ((20, 3, 3, 3, 1), (80, 3, 3, 3, 1), (16, 7, 7, 3, 1), (16, 3, 3, 3, 2), (16, 8, 8, 2, 1)):
+        assert lib.bship_conv2d_bwd_thin_f32(a.ptr, 192, a.ptr, a.ptr, a.ptr, 192, a.ptr, a.ptr, 2, 8, 8, c, f, kh, kw, 1,
+                                             stride, stride) == -6
+
+
 def test_im2col_col2im_exact(hip, ref):
     # through the C ABI directly: the batched kernels against the oracle's per-image routines
     rng = np.random.RandomState(27)

@@ -393,6 +393,18 @@ int bship_batchnorm_bwd_f32(const float* dout, const float* x_hat, const float* 
          P(dgamma), P(dbeta), P(din), (long long)M, (long long)N);
     return 0;
 }
+int bship_conv2d_fwd_thin_f32(const float* in, int64_t, const float* w, const float* bias, float* out, int64_t n, int, int, int,
+                              int, int, int, int, int, int) {
+    flush();
+    logf("conv_fwd_thin @%lld @%lld @%lld @%lld %lld", P(in), P(w), P(bias), P(out), (long long)n);
+    return 0;
+}
+int bship_conv2d_bwd_thin_f32(const float* in, int64_t, const float* w, const float* dy, float* din, int64_t, float* dw, float* db,
+                              int64_t n, int, int, int, int, int, int, int, int, int) {
+    flush();
+    logf("conv_bwd_thin @%lld @%lld @%lld @%lld @%lld @%lld %lld", P(in), P(w), P(dy), P(din), P(dw), P(db), (long long)n);
+    return 0;
+}
 int bship_im2col_nhwc_pitched_f32(const float* in, int64_t, float* col, int64_t n, int, int, int, int, int, int, int, int) {
     flush();
     logf("im2col @%lld @%lld %lld", P(in), P(col), (long long)n);
