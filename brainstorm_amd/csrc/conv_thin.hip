@@ -27,6 +27,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <mutex>
 
 namespace bship {
 
@@ -61,17 +62,18 @@ constexpr int kStageChunk = kThinThreads * kStageAhead;
 
 // Elements [c0, c0 + kStageChunk) of the band: the image rows [y0 - pad, y0 - pad + br) x all columns, zero beyond
 // the image.
-__device__ __forceinline__ void band_chunk_load(const ThinGeom& g, const float* __restrict__ src, int y0, int c0, int total,
+__device__ __forceinline__ void band_chunk_load(const FastDiv& by_band_row, const FastDiv& by_c, int pad, int h, int w, int c,
+                                                const float* __restrict__ src, int y0, int c0, int total,
                                                 float (&v)[kStageAhead]) {
 #pragma unroll
     for (int u = 0; u < kStageAhead; ++u) {
         const int i = c0 + threadIdx.x + u * kThinThreads;
         uint32_t by, rest, bx, ch;
-        g.by_band_row.divmod(static_cast<uint32_t>(i < total ? i : 0), by, rest);
-        g.by_c.divmod(rest, bx, ch);
-        const int y = y0 - g.pad + static_cast<int>(by), x = static_cast<int>(bx) - g.pad;
-        const bool inside = i < total && y >= 0 && y < g.h && x >= 0 && x < g.w;
-        const int64_t at = inside ? (static_cast<int64_t>(y) * g.w + x) * g.c + ch : 0;
+        by_band_row.divmod(static_cast<uint32_t>(i < total ? i : 0), by, rest);
+        by_c.divmod(rest, bx, ch);
+        const int y = y0 - pad + static_cast<int>(by), x = static_cast<int>(bx) - pad;
+        const bool inside = i < total && y >= 0 && y < h && x >= 0 && x < w;
+        const int64_t at = inside ? (static_cast<int64_t>(y) * w + x) * c + ch : 0;
         const float loaded = src[at];                  // element 0 of the image for the lanes with nothing to fetch
         v[u] = inside ? loaded : 0.0f;
     }
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_fwd_kernel(ThinGeom g,
     // the band and the weights (W is (f, K): read in order, stored transposed) are requested together
     for (int c = 0; c < max(band_floats, w_floats); c += kStageChunk) {
         float bv[kStageAhead], wv[kStageAhead];
-        if (c < band_floats) band_chunk_load(g, src, y0, c, band_floats, bv);
+        if (c < band_floats) band_chunk_load(g.by_band_row, g.by_c, g.pad, g.h, g.w, g.c, src, y0, c, band_floats, bv);
         if (c < w_floats) flat_chunk_load(W, c, w_floats, wv);
         if (c < band_floats) chunk_store(band, c, band_floats, bv);
         if (c < w_floats) {
@@ -469,9 +471,10 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
 // bias_deltas[f] = sum_pixels out_deltas[pixel][f] (a window entry that is always one). A workgroup walks over
 // bands of images (unit = image x band of output rows; unit, unit + gridDim.x, ...), keeps its sums in the
 // accumulators throughout and writes them once: partial[workgroup][f][KT * 16]. Tiles are 16 filters x 16
-// window entries, pixels in steps of 4; a wavefront owns one tile of filters (all KT tiles of window entries,
-// which share the out_deltas operand) and, where there are fewer than four filter tiles, every so-manyth step.
-template <int KT>
+// window entries, pixels in steps of 4. A wavefront owns all FT x KT tiles and every fourth step: per step it
+// reads FT values of out_deltas and KT of the image for FT x KT products, which keeps the matrix cores busier
+// than the reads and the address arithmetic keep the issue slots.
+template <int KT, int FT>
 __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom g, const float* __restrict__ in,
                                                                     int64_t in_pitch, const float* __restrict__ dy,
                                                                     float* __restrict__ partial, int64_t units) {
@@ -482,10 +485,6 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom
     float* dyb = lds + band_floats;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = lane & 15, q4 = lane >> 4;
-    const int ftiles = g.f / 16;
-    const int parts = 4 / ftiles;                   // wavefronts per filter tile (3 filter tiles: one idles)
-    const bool works = wave < ftiles * parts;
-    const int ft = wave % ftiles, part = wave / ftiles;
     int koff[KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
@@ -493,9 +492,12 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom
         koff[kt] = k < g.K ? (k / (g.kw * g.c)) * g.bw * g.c + k % (g.kw * g.c) : 0;
     }
     const bool one = (KT - 1) * 16 + m == g.K, none = (KT - 1) * 16 + m > g.K;      // in the last tile of entries
-    v4f acc[KT];
+    v4f acc[FT][KT];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) acc[kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int ft = 0; ft < FT; ++ft) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) acc[ft][kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     for (int64_t unit = blockIdx.x; unit < units; unit += gridDim.x) {
         const int64_t img = unit / g.bands;
         const int y0 = static_cast<int>(unit % g.bands) * g.rows;
@@ -508,17 +510,7 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom
         const float* src = in + img * in_pitch;
         for (int c0 = 0; c0 < band_floats; c0 += kStageChunk) {
             float v[kStageAhead];
-#pragma unroll
-            for (int u = 0; u < kStageAhead; ++u) {
-                const int i = c0 + threadIdx.x + u * kThinThreads;
-                uint32_t by, rest, bx, ch;
-                g.by_band_row.divmod(static_cast<uint32_t>(i < band_floats ? i : 0), by, rest);
-                g.by_c.divmod(rest, bx, ch);
-                const int y = y0 - g.pad + static_cast<int>(by), x = static_cast<int>(bx) - g.pad;
-                const bool inside = i < band_floats && y >= 0 && y < g.h && x >= 0 && x < g.w;
-                const float loaded = src[inside ? (static_cast<int64_t>(y) * g.w + x) * g.c + ch : 0];
-                v[u] = inside ? loaded : 0.0f;
-            }
+            band_chunk_load(g.by_band_row, g.by_c, g.pad, g.h, g.w, g.c, src, y0, c0, band_floats, v);
             chunk_store(band, c0, band_floats, v);
         }
         for (int r0 = 0; r0 < band_rows; r0 += g.chunk_rows) {
@@ -530,42 +522,50 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom
             dy_chunk_load(dy_band + static_cast<int64_t>(r_next < band_rows ? r_next : 0) * g.ow * g.f, ahead_count, ahead);
             const int px_c = rows_c * g.ow;
             const int steps = (px_c + 3) / 4;
-            if (works && part < steps) {
-                // Steps go in pairs: a pair's operands are read from LDS while the 2 x KT products of the pair
-                // before are issued, which covers the LDS latency. A step past the end reads pixel 0 and
-                // multiplies by zero, like the pixels past the chunk in the last step.
-                auto read_step = [&](int s, float& a, float (&b)[KT]) {
+            if (wave < steps) {
+                // Steps go in pairs: a pair's operands are read from LDS while the 2 x FT x KT products of the
+                // pair before are issued. A step past the end reads pixel 0 and multiplies by zero, like the
+                // pixels past the chunk in the last step.
+                auto read_step = [&](int s, float (&a)[FT], float (&b)[KT]) {
                     const int p = 4 * s + q4;
                     const bool valid = p < px_c;
                     uint32_t py, px;
                     g.by_ow.divmod(static_cast<uint32_t>(valid ? p : 0), py, px);
-                    const float a_read = dyb[(valid ? p : 0) * g.fp + ft * 16 + m];
-                    a = valid ? a_read : 0.0f;
+                    const float* from = dyb + (valid ? p : 0) * g.fp + m;
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) {
+                        const float a_read = from[ft * 16];
+                        a[ft] = valid ? a_read : 0.0f;
+                    }
                     const float* at = band + (static_cast<int>(r0 + py) * g.bw + static_cast<int>(px)) * g.c;
 #pragma unroll
                     for (int kt = 0; kt < KT; ++kt) b[kt] = at[koff[kt]];
                     b[KT - 1] = one ? 1.0f : (none ? 0.0f : b[KT - 1]);
                 };
-                float a_next[2], b_next[2][KT];
-                read_step(part, a_next[0], b_next[0]);
-                read_step(part + parts, a_next[1], b_next[1]);
-                for (int s = part; s < steps; s += 2 * parts) {
-                    float a_now[2], b_now[2][KT];
+                float a_next[2][FT], b_next[2][KT];
+                read_step(wave, a_next[0], b_next[0]);
+                read_step(wave + 4, a_next[1], b_next[1]);
+                for (int s = wave; s < steps; s += 8) {
+                    float a_now[2][FT], b_now[2][KT];
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        a_now[j] = a_next[j];
+#pragma unroll
+                        for (int ft = 0; ft < FT; ++ft) a_now[j][ft] = a_next[j][ft];
 #pragma unroll
                         for (int kt = 0; kt < KT; ++kt) b_now[j][kt] = b_next[j][kt];
                     }
                     __builtin_amdgcn_sched_barrier(0);
-                    read_step(s + 2 * parts, a_next[0], b_next[0]);
-                    read_step(s + 3 * parts, a_next[1], b_next[1]);
+                    read_step(s + 8, a_next[0], b_next[0]);
+                    read_step(s + 12, a_next[1], b_next[1]);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
 #pragma unroll
-                        for (int kt = 0; kt < KT; ++kt)
-                            acc[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_now[j], b_now[j][kt], acc[kt], 0, 0, 0);
+                        for (int ft = 0; ft < FT; ++ft) {
+#pragma unroll
+                            for (int kt = 0; kt < KT; ++kt)
+                                acc[ft][kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_now[j][ft], b_now[j][kt], acc[ft][kt], 0, 0, 0);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -573,24 +573,31 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dw_kernel(ThinBackGeom
             __syncthreads();                        // before the next chunk replaces this one
         }
     }
-    // The parts of one filter tile are added in part order: red[wave][kt][component q][lane]
+    // The four wavefronts' sums are added in wavefront order: red[tile][component q][lane]
     float* red = lds;
-    __syncthreads();
+    for (int w = 0; w < 4; ++w) {
+        __syncthreads();
+        if (wave == w) {
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+            for (int ft = 0; ft < FT; ++ft) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) red[((wave * KT + kt) * 4 + q) * 64 + lane] = acc[kt][q];
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float* at = red + ((ft * KT + kt) * 4 + q) * 64 + lane;
+                        *at = w == 0 ? acc[ft][kt][q] : *at + acc[ft][kt][q];
+                    }
+                }
+            }
+        }
     }
     __syncthreads();
     float* mine = partial + static_cast<int64_t>(blockIdx.x) * g.f * KW;
-    for (int i = threadIdx.x; i < ftiles * KT * 256; i += kThinThreads) {
-        const int e = i & 255, tile = i >> 8;
-        const int kt = tile % KT, t = tile / KT;
-        float sum = 0.0f;
-        for (int pa = 0; pa < parts; ++pa) sum += red[(((pa * ftiles + t) * KT + kt) * 256) + e];
-        // component q of lane l: filter t * 16 + 4 * (l / 16) + q, window entry kt * 16 + l % 16
-        const int q = e >> 6, l = e & 63;
-        mine[(t * 16 + 4 * (l >> 4) + q) * KW + kt * 16 + (l & 15)] = sum;
+    for (int i = threadIdx.x; i < FT * KT * 256; i += kThinThreads) {
+        // component q of lane l of tile (ft, kt): filter ft * 16 + 4 * (l / 16) + q, window entry kt * 16 + l % 16
+        const int l = i & 63, q = (i >> 6) & 3, tile = i >> 8;
+        const int kt = tile % KT, ft = tile / KT;
+        mine[(ft * 16 + 4 * (l >> 4) + q) * KW + kt * 16 + (l & 15)] = red[i];
     }
 }
 
@@ -671,11 +678,46 @@ static void launch_dx(const ThinBackGeom& g, int64_t n, size_t lds, const float*
                        ctx().stream, g, W, dy, din, din_pitch);
 }
 
+// Workgroups of the weights' kernel that one compute unit holds at a time (registers and LDS decide): the
+// launch has that many per unit at most, and each walks over the units that are left.
+template <int KT, int FT>
+static int dw_resident(size_t lds) {
+    static std::mutex guard;
+    static size_t asked_lds = ~size_t(0);
+    static int answer = 1;
+    std::lock_guard<std::mutex> lock(guard);
+    if (lds != asked_lds) {                      // asked once per kernel and LDS size: the query is a driver call
+        int blocks = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, conv_thin_dw_kernel<KT, FT>, kThinThreads, lds) != hipSuccess) {
+            (void)hipGetLastError();
+            blocks = 1;
+        }
+        answer = std::max(1, std::min(blocks, 4));
+        asked_lds = lds;
+    }
+    return answer;
+}
+
+template <int KT>
+static int dw_resident_for(int ftiles, size_t lds) {
+    switch (ftiles) {
+        case 1: return dw_resident<KT, 1>(lds);
+        case 2: return dw_resident<KT, 2>(lds);
+        case 3: return dw_resident<KT, 3>(lds);
+        default: return dw_resident<KT, 4>(lds);
+    }
+}
+
 template <int KT>
 static void launch_dw(const ThinBackGeom& g, unsigned grid, size_t lds, const float* in, int64_t in_pitch, const float* dy,
                       float* partial, int64_t units) {
-    hipLaunchKernelGGL(conv_thin_dw_kernel<KT>, dim3(grid), dim3(kThinThreads), lds, ctx().stream, g, in, in_pitch, dy,
-                       partial, units);
+    const dim3 blocks(grid), threads(kThinThreads);
+    switch (g.f / 16) {
+        case 1: hipLaunchKernelGGL((conv_thin_dw_kernel<KT, 1>), blocks, threads, lds, ctx().stream, g, in, in_pitch, dy, partial, units); break;
+        case 2: hipLaunchKernelGGL((conv_thin_dw_kernel<KT, 2>), blocks, threads, lds, ctx().stream, g, in, in_pitch, dy, partial, units); break;
+        case 3: hipLaunchKernelGGL((conv_thin_dw_kernel<KT, 3>), blocks, threads, lds, ctx().stream, g, in, in_pitch, dy, partial, units); break;
+        default: hipLaunchKernelGGL((conv_thin_dw_kernel<KT, 4>), blocks, threads, lds, ctx().stream, g, in, in_pitch, dy, partial, units); break;
+    }
 }
 
 #define BSHIP_THIN_FOR_KT(kt, CALL)                                                     \
@@ -745,8 +787,8 @@ int bship_conv2d_bwd_thin_f32(const float* in, int64_t in_pitch, const float* we
     }
     if (ok) {
         // deltas of the weights: bands of output rows; the LDS holds the band of the inputs and the chunk, and at
-        // the end the four wavefronts' accumulators
-        const size_t chunk = static_cast<size_t>(gw.chunk_px) * gw.fp, sums = static_cast<size_t>(4) * kt_dw * 256;
+        // the end the sum of the four wavefronts' accumulators
+        const size_t chunk = static_cast<size_t>(gw.chunk_px) * gw.fp, sums = static_cast<size_t>(f / 16) * kt_dw * 256;
         int max_rows = gw.oh;
         while (max_rows > 1 && static_cast<size_t>(max_rows + kh - 1) * gw.bw * c + chunk > kThinLdsFloats) --max_rows;
         ok = static_cast<size_t>(max_rows + kh - 1) * gw.bw * c + chunk <= kThinLdsFloats && sums <= kThinLdsFloats;
@@ -757,8 +799,13 @@ int bship_conv2d_bwd_thin_f32(const float* in, int64_t in_pitch, const float* we
             gw.br = gw.rows + kh - 1;
             lds_w = std::max(static_cast<size_t>(gw.br) * gw.bw * c + chunk, sums) * sizeof(float);
             units = n * gw.bands;
-            // up to four workgroups per compute unit: beyond that the partial sums cost more than the units waiting
-            grid_w = static_cast<unsigned>(std::min<int64_t>(units, 4 * static_cast<int64_t>(ctx().num_cus)));
+            // as many workgroups as the device holds at a time, up to four per compute unit (beyond that the
+            // partial sums cost more than the waiting units)
+            int resident = 1;
+#define BSHIP_THIN_RESIDENT(KT) resident = dw_resident_for<KT>(f / 16, lds_w)
+            BSHIP_THIN_FOR_KT(kt_dw, BSHIP_THIN_RESIDENT)
+#undef BSHIP_THIN_RESIDENT
+            grid_w = static_cast<unsigned>(std::min<int64_t>(units, resident * static_cast<int64_t>(ctx().num_cus)));
         }
     }
     if (!ok) return set_error(BSHIP_ERR_UNSUPPORTED, "%s: not a thin-filter convolution these kernels take", __func__);
@@ -790,6 +837,7 @@ int bship_conv2d_bwd_thin_f32(const float* in, int64_t in_pitch, const float* we
 #undef BSHIP_THIN_DX
     return check_launch("conv2d_backward_batch (thin filters, inputs)");
 }
+
 
 
 }  // extern "C"
