@@ -31,6 +31,7 @@ import time
 import numpy as np
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+F32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense float32 matrix cores, published
 F32 = np.float32
 
 
@@ -223,6 +224,34 @@ def run_image_ops(hip, n_img=2048, reps=10):
         report("col2im_" + tag, timed(lambda: hip._call(lib.bship_col2im_nhwc_f32(
             col.ptr, dx.ptr, n_img, h, w, c, k, k, pad, 1, 1))), 4 * (2 * x.size + col.size))
         del col, dx, x
+    # The CNN workload's first convolution (5 x 5 x 3 filters, 32 of them) forward and backward: without a col
+    # matrix (thin filters: the handler's choice) and through im2col + the matrix-product library + col2im.
+    # Matrix-core work: TFLOP/s of the 2 * pixels * 75 * 32 flops forward and twice that backward, and their
+    # fraction of the float32 matrix peak.
+    for batch, n_reps in ((n_img, reps), (100, 20 * reps)):
+        x, dy = filled((batch, 32, 32, 3)), filled((batch, 32, 32, 32))
+        wts, bias = filled((32, 5, 5, 3)), filled((32,))
+        y, dx, dw, db = hip.allocate((batch, 32, 32, 32)), hip.allocate((batch, 32, 32, 3)), hip.allocate((32, 5, 5, 3)), hip.allocate((32,))
+        flops = 2.0 * batch * 32 * 32 * 75 * 32
+        for thin, route in ((True, "thin"), (False, "im2col")):
+            hip.thin_convolutions = thin
+            try:
+                for name, work, fn in (("fwd", flops, lambda: hip.conv2d_forward_batch(x, wts, bias, y, 2, (1, 1))),
+                                       ("bwd", 2 * flops, lambda: hip.conv2d_backward_batch(x, wts, 2, (1, 1), dx, dy, dw, db))):
+                    for _ in range(2):
+                        fn()
+                    lib.bship_event_record(0)
+                    for _ in range(n_reps):
+                        fn()
+                    lib.bship_event_record(1)
+                    hip._call(lib.bship_event_elapsed_ms(0, 1, ctypes.byref(ms)))
+                    us = ms.value * 1e3 / n_reps
+                    out["conv1_%s_%s_batch%d" % (name, route, batch)] = {
+                        "us": round(us, 1), "tflops": round(work / us / 1e6, 1),
+                        "frac_of_f32_matrix_peak": round(work / us / 1e6 / F32_MATRIX_PEAK_TFLOPS, 4)}
+            finally:
+                hip.thin_convolutions = True
+        del x, dy, y, dx
     for h, w, c, k, s, tag in ((32, 32, 32, 3, 2, "pool1_32x32x32_k3s2"), (15, 15, 64, 3, 2, "pool2_15x15x64_k3s2")):
         x = filled((n_img, h, w, c))
         oh, ow = (h - k) // s + 1, (w - k) // s + 1

@@ -1,13 +1,14 @@
 """Runs training steps of one network workload on HipHandler: the program to put under a profiler.
 
-    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded] [window_off]
+    python3 -m brainstorm_amd.drivers.run_workload mlp|lstm|highway|cnn [steps] [fused] [recorded] [window_off] [im2col]
 
 ``fused`` is passed to the workload's builder: "0" for the reference layers' primitive call sequences
 (what an unchanged caller issues), "1" for a handler-aware caller that asks for the fused entry points;
 for the LSTM "packed" (stacked recurrent product), "thin" (packed, backward product through the
 thin-operand kernel) or "sequence" (packed, forward recurrence in one launch). With "recorded" the step
 is recorded after one ordinary step and replayed. With "window_off" the handler's fusing window is
-switched off, so that primitive calls are launched one by one. One step = forward + backward + momentum
+switched off, so that primitive calls are launched one by one. With "im2col" convolutions with thin filters
+take the col matrix and the matrix-product library like all others. One step = forward + backward + momentum
 update.
 """
 import sys
@@ -26,6 +27,7 @@ def main(argv):
     if fused and fused != "0":
         kw["fused"] = fused if fused in ("packed", "thin", "sequence") else True
     handler = HipHandler(seed=0, fusing="window_off" not in argv[4:])
+    handler.thin_convolutions = "im2col" not in argv[4:]
     net, data = getattr(configs, "build_" + name)(handler, **kw)
     net.provide_external_data(data)
     stepper = MomentumStepper(0.1, 0.9, fused=bool(kw.get("fused")))
