@@ -297,6 +297,17 @@ __device__ __forceinline__ void dy_chunk_load(const float* __restrict__ src, int
 }
 
 __device__ __forceinline__ void dy_chunk_store(const ThinBackGeom& g, float* dyb, int count, const float (&v)[kDyRegs]) {
+    if (kThinThreads % g.f == 0) {           // 16, 32 or 64 filters: a thread's elements lie 256 / f pixels apart
+        uint32_t px, ff;
+        g.by_f.divmod(threadIdx.x, px, ff);
+        float* to = dyb + px * g.fp + ff;
+        const int step = (kThinThreads / g.f) * g.fp;
+#pragma unroll
+        for (int u = 0; u < kDyRegs; ++u) {
+            if (static_cast<int>(threadIdx.x) + u * kThinThreads < count) to[u * step] = v[u];
+        }
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < kDyRegs; ++u) {
         const int i = threadIdx.x + u * kThinThreads;
@@ -324,6 +335,7 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
     float* dyb = wl + g.f * g.wp;                  // the chunk (chunk_px, fp)
     float* dcol = dyb + g.chunk_px * g.fp;         // (chunk_rows, owp, dp): rows of out_deltas between zero pixels
     float* dxb = dcol + g.chunk_rows * g.owp * g.dp;   // the band's sums (rows, w * c)
+    float* zeros = dxb + g.rows * g.w * g.c;           // what a row of out_deltas outside an element's windows reads
     const int wc = g.w * g.c;
     const int64_t img = blockIdx.x / g.bands;
     const int y0 = static_cast<int>(blockIdx.x % g.bands) * g.rows;
@@ -352,6 +364,8 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
         }
     }
     for (int i = threadIdx.x; i < band_rows * wc; i += kThinThreads) dxb[i] = 0.0f;
+    const int zero_floats = (g.kw - 1) * (g.dp - g.c) + 1;
+    for (int i = threadIdx.x; i < zero_floats; i += kThinThreads) zeros[i] = 0.0f;
     // the zero pixels either side of dcol's rows: windows that hang over the edge of out_deltas read them
     for (int i = threadIdx.x; i < g.chunk_rows * 2 * g.margin * g.dp; i += kThinThreads) {
         const int col = i % g.dp, slot = i / g.dp;
@@ -386,6 +400,7 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) b_next[j][kt] = bp[j * 4 * g.wp + kt * 16];
             }
+#pragma unroll 2
             for (int s0 = 0; s0 < steps; s0 += 4) {
                 float a_now[4], b_now[4][KT];
 #pragma unroll
@@ -412,15 +427,18 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
                 __builtin_amdgcn_sched_barrier(0);
             }
             // component q: pixel pt * 16 + 4 * (lane / 16) + q, window entry kt * 16 + lane % 16
+            uint32_t r, ox;
+            g.by_ow.divmod(static_cast<uint32_t>(pt * 16 + 4 * q4), r, ox);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int px = pt * 16 + 4 * q4 + q;
-                if (px < rows_c * g.ow) {
-                    uint32_t r, ox;
-                    g.by_ow.divmod(static_cast<uint32_t>(px), r, ox);
+                if (pt * 16 + 4 * q4 + q < rows_c * g.ow) {
                     float* to = dcol + (r * g.owp + ox + g.margin) * g.dp + m;
 #pragma unroll
                     for (int kt = 0; kt < KT; ++kt) to[kt * 16] = acc[kt][q];
+                }
+                if (++ox == static_cast<uint32_t>(g.ow)) {       // the next pixel starts a row of out_deltas
+                    ox = 0;
+                    ++r;
                 }
             }
         }
@@ -436,26 +454,21 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
             // entry (ky, kx, ch) of pixel (r, x + pad - kx): from kx to kx + 1 one pixel back and one entry on
             const float* at = dcol + (static_cast<int>(x) + g.pad + g.margin) * g.dp + ch;
             const int next = g.c - g.dp;
-            // two rows of out_deltas x eight kx at a time: all sixteen reads are under way before the first is
-            // added (those beyond the rows, the window or kw read a valid address and add zero)
-            for (int r0 = 0; r0 < rows_c; r0 += 2) {
-                for (int kx0 = 0; kx0 < g.kw; kx0 += 8) {
-                    float v[2][8];
-                    bool row_counts[2];
-#pragma unroll
-                    for (int jr = 0; jr < 2; ++jr) {
-                        const int r = r0 + jr, ky = static_cast<int>(t) - r;
-                        row_counts[jr] = r < rows_c && ky >= 0 && ky < g.kh;
-                        const float* p = row_counts[jr] ? at + (r * g.owp) * g.dp + ky * g.kw * g.c : at;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) v[jr][j] = p[min(kx0 + j, g.kw - 1) * next];
-                    }
-#pragma unroll
-                    for (int jr = 0; jr < 2; ++jr) {
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) sum += row_counts[jr] && kx0 + j < g.kw ? v[jr][j] : 0.0f;
-                    }
+            // kx in fours: four reads under way before the first is added. A row of out_deltas whose windows
+            // do not hold this element's row reads zeros instead, so the loops are the same for every lane.
+            const float* zero_at = zeros + (g.kw - 1) * (g.dp - g.c);
+            for (int r = 0; r < rows_c; ++r) {
+                const int ky = static_cast<int>(t) - r;
+                const float* p = ky >= 0 && ky < g.kh ? at + (r * g.owp) * g.dp + ky * g.kw * g.c : zero_at;
+                int kx = 0;
+                for (; kx + 4 <= g.kw; kx += 4) {
+                    const float v0 = p[kx * next], v1 = p[(kx + 1) * next], v2 = p[(kx + 2) * next], v3 = p[(kx + 3) * next];
+                    sum += v0;
+                    sum += v1;
+                    sum += v2;
+                    sum += v3;
                 }
+                for (; kx < g.kw; ++kx) sum += p[kx * next];
             }
             dxb[(y - y0) * wc + static_cast<int>(e)] += sum;
         }
@@ -769,7 +782,7 @@ int bship_conv2d_bwd_thin_f32(const float* in, int64_t in_pitch, const float* we
         const size_t wc = static_cast<size_t>(w) * c;
         auto fixed_floats = [&]() {
             return static_cast<size_t>(f) * gx.wp + static_cast<size_t>(gx.chunk_px) * gx.fp +
-                   static_cast<size_t>(gx.chunk_rows) * gx.owp * gx.dp;
+                   static_cast<size_t>(gx.chunk_rows) * gx.owp * gx.dp + static_cast<size_t>(kw - 1) * (gx.dp - c) + 1;
         };
         // narrow images: fewer rows per chunk where their products (with the zero pixels either side) do not fit
         while (gx.chunk_rows > 1 && fixed_floats() + std::min<size_t>(h, 4) * wc > kThinLdsFloats)
