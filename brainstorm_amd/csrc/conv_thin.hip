@@ -17,12 +17,15 @@
 //
 // Sums inside a product are float32 accumulations of the matrix cores in k order (forward), pixel order
 // (weights) and filter order (inputs); the handler's bar for products is 1e-5 relative to the result's scale,
-// as for the hipBLASLt path. Nothing depends on which workgroup finishes first: the weight gradients are
-// per-band partial sums in a scratch buffer that a second kernel adds in band order.
+// as for the hipBLASLt path. Nothing depends on which workgroup finishes first: the weights' deltas are
+// per-workgroup partial sums in a scratch buffer that a second kernel adds in workgroup order, and every element
+// of the inputs' deltas is summed by one thread in a fixed order. With finite operands, that is: where a tile has
+// fewer than 16 pixels the spare rows are multiplied by zero, which an infinity in the image turns into NaN
+// (is_fully_finite reports either).
 //
-// Taken for stride 1, any padding, kh * kw * c <= 128, filters a multiple of 16 up to 64, and images whose
-// band fits the LDS; everything else returns BSHIP_ERR_UNSUPPORTED with nothing launched and the caller
-// takes the im2col path.
+// Taken for stride 1, any padding, kh * kw * c <= 128 (127 backward: the bias takes a window entry), filters a
+// multiple of 16 up to 64, and images whose band fits the LDS; everything else returns BSHIP_ERR_UNSUPPORTED
+// with nothing launched and the caller takes the im2col path.
 #include "common.h"
 
 #include <algorithm>
@@ -241,8 +244,7 @@ static int thin_rows(int64_t n, int extent, int ow, int max_rows, double tiles_p
 }
 
 static bool thin_geometry(ThinGeom& g, int64_t n, int h, int w, int c, int f, int kh, int kw, int pad, int sh, int sw,
-                          size_t extra_lds_floats_per_pixel, size_t fixed_lds_floats, double tiles_per_pixel_tile,
-                          size_t* lds_bytes) {
+                          size_t fixed_lds_floats, double tiles_per_pixel_tile, size_t* lds_bytes) {
     if (sh != 1 || sw != 1 || n < 1 || h < 1 || w < 1 || c < 1 || kh < 1 || kw < 1 || pad < 0) return false;
     const int64_t K = static_cast<int64_t>(kh) * kw * c;
     if (K > kThinMaxK || f < 16 || f > kThinMaxF || f % 16 != 0) return false;
@@ -254,9 +256,7 @@ static bool thin_geometry(ThinGeom& g, int64_t n, int h, int w, int c, int f, in
     g.bw = w + 2 * pad;
     const size_t budget = 60 * 1024 / sizeof(float);
     int max_rows = g.oh;
-    while (max_rows > 1 && static_cast<size_t>(max_rows + kh - 1) * g.bw * c + fixed_lds_floats +
-                               extra_lds_floats_per_pixel * static_cast<size_t>(max_rows) * g.ow > budget)
-        --max_rows;
+    while (max_rows > 1 && static_cast<size_t>(max_rows + kh - 1) * g.bw * c + fixed_lds_floats > budget) --max_rows;
     int rows = thin_rows(n, g.oh, g.ow, max_rows, tiles_per_pixel_tile);
     g.rows = rows;
     g.bands = (g.oh + rows - 1) / rows;
@@ -266,9 +266,7 @@ static bool thin_geometry(ThinGeom& g, int64_t n, int h, int w, int c, int f, in
     g.by_ow = FastDiv(static_cast<uint32_t>(g.ow));
     g.by_K = FastDiv(static_cast<uint32_t>(g.K));
     g.by_window_row = FastDiv(static_cast<uint32_t>(kw * c));
-    const size_t floats = static_cast<size_t>(g.br) * g.bw * c + fixed_lds_floats +
-                          extra_lds_floats_per_pixel * static_cast<size_t>(rows) * g.ow;
-    *lds_bytes = floats * sizeof(float);
+    *lds_bytes = (static_cast<size_t>(g.br) * g.bw * c + fixed_lds_floats) * sizeof(float);
     return *lds_bytes <= 64 * 1024 && n * g.bands <= 0x7fffffff;
 }
 
@@ -283,7 +281,7 @@ struct ThinBackGeom {
     int margin, owp;        // dcol: zero pixels either side of a row of out_deltas (kw - 1 - pad), and a row with them
     int wp, dp, fp;         // LDS row pitches in floats: weights, dcol, the chunk of out_deltas
     int bw, br;             // staged band of the inputs (the weights' deltas): columns, rows
-    FastDiv by_f, by_wc, by_c, by_ow, by_band_row, by_window_row;
+    FastDiv by_f, by_wc, by_c, by_ow, by_band_row;
 };
 
 constexpr int kDyRegs = 16;          // floats of a chunk per thread: chunk_px * f <= kDyRegs * kThinThreads
@@ -387,10 +385,10 @@ __global__ __launch_bounds__(kThinThreads) void conv_thin_dx_kernel(ThinBackGeom
             v4f acc[KT];
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) acc[kt] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            // rows of the tile beyond the chunk's pixels hold whatever LDS held: their products are not kept
-            // f is a multiple of 16: steps come in groups of four, and a group's operands (4 values of
+            // Rows of the tile beyond the chunk's pixels hold whatever LDS held: their products are not kept.
+            // f is a multiple of 16, so steps come in groups of four: a group's operands (4 values of
             // out_deltas, 4 x KT weights) are read from LDS while the 4 x KT products of the group before are
-            // issued, which covers the LDS latency
+            // issued.
             const float* ap = dyb + (pt * 16 + m) * g.fp + q4;
             const float* bp = wl + q4 * g.wp + m;
             float a_next[4], b_next[4][KT];
@@ -673,12 +671,13 @@ static bool thin_back_geometry(ThinBackGeom& g, int64_t n, int h, int w, int c, 
     g.dp = KW + ((c % 32) - (KW % 32) + 32) % 32;
     g.fp = for_weights ? (f % 32 == 16 ? f : f + 16) : f + 2;
     g.bw = w + 2 * pad;
+    g.br = 0;               // set with the rows per band, for the weights' deltas
+    g.rows = g.bands = 0;
     g.by_f = FastDiv(static_cast<uint32_t>(f));
     g.by_wc = FastDiv(static_cast<uint32_t>(w * c));
     g.by_c = FastDiv(static_cast<uint32_t>(c));
     g.by_ow = FastDiv(static_cast<uint32_t>(g.ow));
     g.by_band_row = FastDiv(static_cast<uint32_t>(g.bw * c));
-    g.by_window_row = FastDiv(static_cast<uint32_t>(kw * c));
     return true;
 }
 
@@ -752,7 +751,7 @@ int bship_conv2d_fwd_thin_f32(const float* in, int64_t in_pitch, const float* we
     ThinGeom g;
     size_t lds = 0;
     const int64_t K = static_cast<int64_t>(kh) * kw * c;
-    if (!thin_geometry(g, n, h, w, c, f, kh, kw, pad, stride_h, stride_w, 0,
+    if (!thin_geometry(g, n, h, w, c, f, kh, kw, pad, stride_h, stride_w,
                        static_cast<size_t>((K + 3) & ~int64_t(3)) * static_cast<size_t>(f > 0 ? f + 2 : 0), f / 16, &lds))
         return set_error(BSHIP_ERR_UNSUPPORTED, "%s: not a thin-filter convolution this kernel takes", __func__);
     BSHIP_REQUIRE_PTR(in);
