@@ -903,11 +903,12 @@ def test_conv2d_forward_backward(hip, ref):
 THIN_CASES = [  # n, h, w, c, f, kh, kw, pad: stride 1, kh*kw*c <= 128, f a multiple of 16 up to 64
     (10, 32, 32, 3, 32, 5, 5, 2), (3, 28, 28, 1, 16, 5, 5, 0), (2, 9, 7, 3, 16, 3, 3, 1), (5, 17, 13, 2, 48, 5, 3, 2),
     (1, 5, 5, 4, 64, 5, 5, 4), (4, 6, 150, 3, 32, 3, 3, 1), (2, 40, 3, 5, 16, 5, 5, 2), (7, 8, 8, 8, 32, 4, 4, 0),
-    (300, 12, 12, 3, 32, 5, 5, 2), (2, 10, 10, 128, 16, 1, 1, 0), (3, 11, 9, 1, 32, 1, 1, 3)]
+    (300, 12, 12, 3, 32, 5, 5, 2), (2, 10, 10, 128, 16, 1, 1, 0), (3, 11, 9, 1, 32, 1, 1, 3),
+    (2, 64, 64, 1, 16, 7, 7, 3), (1, 96, 96, 3, 16, 3, 3, 1), (2, 33, 65, 2, 32, 3, 5, 1), (5, 7, 100, 1, 64, 1, 9, 4)]
 
 
 # of these, backward keeps to the im2col path: a row of out_deltas x f beyond 4096 floats
-THIN_FORWARD_ONLY = {(4, 6, 150, 3, 32, 3, 3, 1)}
+THIN_FORWARD_ONLY = {(4, 6, 150, 3, 32, 3, 3, 1), (5, 7, 100, 1, 64, 1, 9, 4)}
 
 
 def test_thin_filter_convolutions_forward(hip, ref):
