@@ -269,6 +269,38 @@ def run_image_ops(hip, n_img=2048, reps=10):
     return out
 
 
+def run_host_call_cost(hip, calls=20000):
+    """What one handler call costs on the host, in us: `add_tt` on 100x1200 arrays issued back to back
+    (a call no pattern of the fusing window begins with: it goes into the window and out again), with the
+    window on and off, and for comparison the same entry point through ctypes alone."""
+    lib = hip._lib
+    a, b, o = hip.allocate((100, 1200)), hip.allocate((100, 1200)), hip.allocate((100, 1200))
+    out = {"calls": calls, "arrays": "100x1200 float32"}
+
+    def issue(fn):
+        for _ in range(200):
+            fn()
+        hip.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        dt = time.perf_counter() - t0
+        hip.synchronize()
+        return round(dt / calls * 1e6, 3)
+
+    before = hip.fusing
+    try:
+        for on, tag in ((True, "window_on"), (False, "window_off")):
+            hip.set_fusing(on)
+            out["add_tt_%s_us" % tag] = issue(lambda: hip.add_tt(a, b, o))
+        from brainstorm_amd._lib import ADD
+        ap, bp, op, n = a.ptr, b.ptr, o.ptr, o.size
+        out["bship_binary_f32_through_ctypes_us"] = issue(lambda: lib.bship_binary_f32(ADD, ap, bp, op, n))
+    finally:
+        hip.set_fusing(before)
+    return out
+
+
 def run_pitched_ops(rows=8192, cols=8192, reps=10):
     """Operations on row-pitched views: three (rows, cols) feature slices of one (rows, 3*cols) hub,
     as the layers writing side by side into a hub see them (buffer_structure.py:232-245). For each
@@ -557,6 +589,7 @@ def main():
     if not args.no_nets:
         # second part of the metric: training samples/s of the MLP and LSTM workloads
         out["nets"] = run_nets_gpu(hip)
+        out["host_call_cost"] = run_host_call_cost(hip)
     if not args.no_cpu:
         passes, cpu_s = run_cpu(args.cpu_size, args.cpu_seconds)
         cab = alg_bytes(args.cpu_size, args.cpu_size)
